@@ -1,0 +1,3 @@
+from .model import CausalLM, EntryView
+from .step import StepEntry, StepContext, StepFunction, GroupView
+from .engine import Engine, parse_dtype, write_random_model

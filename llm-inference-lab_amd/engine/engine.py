@@ -1,0 +1,126 @@
+"""The engine: a model folder (or a configuration and a seed) becomes a model
+bound to kernels, a cache manager and a step function.
+
+Option names follow the reference's command line where it has them
+(rust/engine/examples/qwen2.rs:38-73): ``dtype`` ("bf16" or "f32": weights,
+activations and cache storage; reductions stay in 32 bits), ``model_dir``,
+``max_batch_tokens`` (most uncached input tokens per step, shared by decode and
+prefill, default 512).
+"""
+from __future__ import annotations
+
+import os
+import tempfile
+from typing import Callable, Dict, List, Optional, Sequence
+
+import torch
+
+from .. import architectures  # noqa: F401  (registers the known architectures)
+from ..cache.manager import CacheManager, GroupLayout, RequestCache, pages_for_tokens
+from ..config.errors import ConfigError
+from ..config.registry import get_architecture, read_config
+from ..weights.loader import load_tensors, place_tensors
+from ..weights.random_init import random_tensors, write_model_dir
+from .model import CausalLM
+from .step import StepEntry, StepFunction
+
+_DTYPES = {
+    "bf16": torch.bfloat16, "bfloat16": torch.bfloat16,
+    "f32": torch.float32, "fp32": torch.float32, "float32": torch.float32,
+}
+
+
+def parse_dtype(name) -> torch.dtype:
+    if isinstance(name, torch.dtype):
+        if name not in (torch.bfloat16, torch.float32):
+            raise ConfigError(f"dtype must be bfloat16 or float32, got {name}")
+        return name
+    try:
+        return _DTYPES[str(name).lower()]
+    except KeyError:
+        raise ConfigError(f"dtype must be one of {sorted(_DTYPES)}, got {name!r}") from None
+
+
+def default_ops(device):
+    """The HIP kernel set.  There is no other: without a GPU or without the
+    compiled extension this raises."""
+    from ..kernels.hip_ops import HipOps
+    return HipOps(device)
+
+
+class Engine:
+    """Model + cache + step function on one GPU."""
+
+    def __init__(self, model_dir: Optional[str] = None, *, config=None, seed: int = 0,
+                 dtype="bf16", device: str = "cuda:0", ops=None, page_size: int = 64,
+                 max_cache_tokens: Optional[int] = None, num_pages: Optional[int] = None,
+                 max_requests: int = 64, max_batch_tokens: int = 512,
+                 max_seq_len: Optional[int] = None, tensors=None,
+                 progress: Optional[Callable[[str], None]] = None):
+        self.dtype = parse_dtype(dtype)
+        self.ops = ops if ops is not None else default_ops(device)
+        self.device = self.ops.device
+        if model_dir is not None:
+            self.architecture, self.config = read_config(model_dir)
+        elif config is not None:
+            arch_name = getattr(config, "architecture", None) or getattr(config, "ARCHITECTURE")
+            self.architecture, self.config = get_architecture(arch_name), config
+        else:
+            raise ValueError("give a model_dir or a config")
+        self.spec = self.architecture.build_spec(self.config)
+        self.model = CausalLM(self.spec)
+        expected = self.model.tensor_specs()
+        if model_dir is not None:
+            loaded = load_tensors(model_dir, expected, self.dtype, self.device, progress)
+        elif tensors is not None:
+            loaded = place_tensors(tensors, expected, self.dtype, self.device)
+        else:
+            loaded = place_tensors(random_tensors(expected, seed, torch.bfloat16), expected,
+                                   self.dtype, self.device, "random weights")
+        self.model.bind(loaded, self.ops, self.dtype)
+        del loaded
+        # ------------------------------------------------------------- cache
+        self.page_size = int(page_size)
+        self.max_requests = int(max_requests)
+        self.max_batch_tokens = int(max_batch_tokens)
+        self.max_seq_len = int(max_seq_len or self.spec.max_positions)
+        self.max_seq_len = min(self.max_seq_len, self.spec.max_positions)
+        groups, state_specs = self.model.cache_layout()
+        if num_pages is None:
+            tokens = max_cache_tokens if max_cache_tokens is not None else \
+                self.max_requests * self.max_seq_len
+            num_pages = pages_for_tokens(int(tokens), self.page_size)
+        for g in groups:
+            g.num_pages = int(num_pages)
+        self.cache = CacheManager(groups, self.page_size, self.max_requests, self.max_seq_len,
+                                  state_specs, self.dtype, self.device)
+        self.model.attach_cache(self.cache)
+        self.step_fn = StepFunction(self.model, self.cache, self.ops, self.max_batch_tokens)
+
+    # ------------------------------------------------------------- requests
+    def open(self, request_id) -> RequestCache:
+        """Give a new request a row in the cache manager."""
+        return self.cache.admit(request_id)
+
+    def close(self, request: RequestCache) -> None:
+        """The request has ended: everything it holds is given back."""
+        self.cache.release(request)
+
+    def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        return self.step_fn(entries)
+
+    # ------------------------------------------------------------------ info
+    def weight_bytes_per_step(self) -> int:
+        return self.model.weight_bytes_per_step()
+
+    def metrics(self) -> Dict[str, object]:
+        return {"steps": self.step_fn.steps, "rows": self.step_fn.rows_total,
+                "cache": self.cache.metrics()}
+
+
+def write_random_model(model_dir: str, config, seed: int, dtype=torch.bfloat16) -> str:
+    """Random-weights mode: write ``config.json`` and ``model.safetensors``."""
+    arch_name = getattr(config, "architecture", None) or getattr(config, "ARCHITECTURE")
+    arch = get_architecture(arch_name)
+    expected = CausalLM(arch.build_spec(config)).tensor_specs()
+    return write_model_dir(model_dir, config, expected, seed, dtype)

@@ -1,0 +1,138 @@
+"""A causal language model put together from a ``ModelSpec``.
+
+Nothing here names an architecture: the embedding, the blocks, the final norm
+and the head are built from the spec's records through the parts registry, and
+the blocks run in the order of ``spec.schedule``.  The reference's counterpart
+is a struct written for one architecture
+(rust/engine/src/runner/model/qwen2/engine.rs:235-252) whose forward body is
+``submit_forward_kernels`` (engine.rs:916-1130).
+"""
+from __future__ import annotations
+
+import dataclasses
+from typing import Dict, List, Optional, Tuple
+
+import torch
+
+from ..cache.manager import CacheManager, GroupLayout
+from ..config.spec import ModelSpec
+from ..parts.registry import build_part, part_class
+from ..weights.loader import TensorSpec
+
+
+@dataclasses.dataclass
+class EntryView:
+    """What one run of a block sees of the cache manager."""
+
+    index: int                      # position in the schedule
+    block: int
+    group: Optional[int] = None     # cache group, None if the mixer keeps no cache
+    slot: Optional[int] = None      # which of the group's layers
+    writes_cache: bool = False
+    k_cache: Optional[torch.Tensor] = None     # [pages, kv_heads, page_size, head_dim]
+    v_cache: Optional[torch.Tensor] = None     # [pages, kv_heads, head_dim, page_size]
+    state: Dict[str, torch.Tensor] = dataclasses.field(default_factory=dict)
+
+
+class CausalLM:
+    def __init__(self, spec: ModelSpec):
+        spec.validate()
+        self.spec = spec
+        self.embedding = build_part("embedding", spec.embedding)
+        self.blocks = [
+            part_class("block", b.kind)(norm1=b.norm1, mixer=b.mixer, norm2=b.norm2,
+                                        feed_forward=b.feed_forward, **dict(b.params))
+            for b in spec.blocks]
+        self.final_norm = build_part("norm", spec.final_norm)
+        self.head = build_part("head", spec.head)
+        self.entries: List[EntryView] = [EntryView(i, e.block) for i, e in enumerate(spec.schedule)]
+        self.ops = None
+        self.dtype = None
+
+    # ---------------------------------------------------------------- weights
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        specs: Dict[str, TensorSpec] = {}
+
+        def add(new):
+            for name, s in new.items():
+                if name in specs and specs[name] != s:
+                    raise ValueError(f"tensor '{name}' is asked for with two shapes: "
+                                     f"{specs[name]} and {s}")
+                specs[name] = s
+        add(self.embedding.tensor_specs())
+        for b in self.blocks:
+            add(b.tensor_specs())
+        add(self.final_norm.tensor_specs())
+        add(self.head.tensor_specs())
+        return specs
+
+    def bind(self, tensors: Dict[str, torch.Tensor], ops, dtype: torch.dtype) -> None:
+        self.ops, self.dtype = ops, dtype
+        self.embedding.bind(tensors, ops, dtype)
+        for b in self.blocks:
+            b.bind(tensors, ops, dtype)
+        self.final_norm.bind(tensors, ops, dtype)
+        self.head.bind(tensors, ops, dtype)
+
+    def weight_bytes_per_step(self) -> int:
+        """Bytes of weights that one step reads once (every run of a block reads
+        its block's weights; the embedding table is read by rows only)."""
+        total = sum(self.blocks[e.block].weight_bytes() for e in self.entries)
+        return total + self.final_norm.weight_bytes() + self.head.weight_bytes()
+
+    # ------------------------------------------------------------------ cache
+    def cache_layout(self) -> Tuple[List[GroupLayout], Dict[int, dict]]:
+        """Groups of cache-owning runs by equal need, and per-run state specs."""
+        groups: List[GroupLayout] = []
+        by_spec: Dict[object, int] = {}
+        state_specs: Dict[int, dict] = {}
+        for view, entry in zip(self.entries, self.spec.schedule):
+            mixer = self.blocks[entry.block].mixer_part()
+            need = mixer.cache_spec()
+            if need is not None:
+                if entry.cache_of is None:
+                    if need not in by_spec:
+                        by_spec[need] = len(groups)
+                        groups.append(GroupLayout(need, []))
+                    view.group = by_spec[need]
+                    view.slot = len(groups[view.group].entries)
+                    view.writes_cache = True
+                    groups[view.group].entries.append(view.index)
+                else:
+                    owner = self.entries[entry.cache_of]
+                    owner_need = self.blocks[self.spec.schedule[entry.cache_of].block].mixer_part().cache_spec()
+                    if owner_need != need:
+                        raise ValueError(
+                            f"schedule[{view.index}] reads the cache of schedule[{entry.cache_of}], "
+                            f"whose need {owner_need} differs from its own {need}")
+                    view.group, view.slot, view.writes_cache = owner.group, owner.slot, False
+            elif entry.cache_of is not None:
+                raise ValueError(f"schedule[{view.index}] names a cache but its mixer keeps none")
+            st = mixer.state_spec()
+            if st:
+                state_specs[view.index] = dict(st)
+        return groups, state_specs
+
+    def attach_cache(self, cache: CacheManager) -> None:
+        for view in self.entries:
+            if view.group is not None:
+                view.k_cache = cache.keys[view.group][view.slot]
+                view.v_cache = cache.values[view.group][view.slot]
+            view.state = cache.state.get(view.index, {})
+
+    # ---------------------------------------------------------------- forward
+    def forward(self, ctx) -> Optional[torch.Tensor]:
+        """Run this step's rows through every scheduled block; returns float32
+        logits ``[wanted, vocab]`` for ``ctx.want_rows`` (None if none wanted)."""
+        rows, hidden = ctx.n_rows, self.spec.hidden_size
+        x = ctx.scratch("model.residual", (rows, hidden), torch.float32)
+        self.embedding.forward(ctx.token_ids, x)
+        for view in self.entries:
+            self.blocks[view.block].forward(x, ctx, view)
+        if ctx.n_want == 0:
+            return None
+        h = ctx.scratch("model.final_normed", (ctx.n_want, hidden), self.dtype)
+        self.final_norm.forward(x, h, ctx.want_rows)
+        logits = ctx.scratch("model.logits", (ctx.n_want, self.spec.vocab_size), torch.float32)
+        self.head.forward(h, logits)
+        return logits

@@ -1,0 +1,227 @@
+"""The step function: one packed, ragged batch from the cache to logits.
+
+A step takes, for each request in it, the request's next tokens (a portion of
+its prompt, cut anywhere, or one decoded token) and the places among those
+tokens whose logits are wanted.  All rows of all requests run as one batch;
+keys and values of the new positions go to the request's pages; earlier
+positions are read from there.  Only the given tokens are computed.
+
+The reference's counterpart is ``CausalModel::forward`` over
+``ModelInput{token_ids, kv}`` (rust/engine/src/runner/model/api.rs:11-16,
+203-207): rows packed in input order with per-row (context row, position)
+metadata and per-request last-row indices
+(rust/engine/src/runner/model/qwen2/engine.rs:936-969, 1794-1851).  It returns
+one prediction per request; this one returns logits at the wanted places.
+"""
+from __future__ import annotations
+
+import dataclasses
+from typing import Dict, List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from ..cache.manager import CacheManager, RequestCache
+from .model import CausalLM
+
+
+@dataclasses.dataclass
+class StepEntry:
+    """One request's share of a step."""
+
+    request: RequestCache
+    tokens: Sequence[int]
+    want: Sequence[int] = ()        # indices into ``tokens`` whose logits are returned
+
+
+@dataclasses.dataclass
+class GroupView:
+    block_table: torch.Tensor       # int32 [max_requests, max_pages_per_request], row b = b-th request of the step
+    page_size: int
+    window: Optional[int]
+
+
+class StepContext:
+    """What the parts see of a step.  Device tensors (int32):
+
+    ``token_ids [rows]``, ``positions [rows]`` (absolute position of each row in
+    its request), ``row_req [rows]`` (which request of the step a row belongs
+    to), ``q_start [reqs + 1]`` (first row of each request; rows of a request are
+    adjacent), ``start_pos [reqs]`` (tokens already cached before this step),
+    ``req_rows [reqs]`` (the request's row in the state slots), ``want_rows
+    [wanted]``.  Host-side: ``n_rows``, ``n_reqs``, ``n_want``, ``max_q_len``,
+    ``max_ctx_len``, ``host_q_start``, ``host_start_pos``, ``host_req_rows``."""
+
+    def __init__(self, ops, device, max_rows: int, max_reqs: int, groups: List[Tuple[int, Optional[int]]],
+                 max_pages_per_request: int):
+        self.ops = ops
+        self.device = device
+        self.max_rows, self.max_reqs = int(max_rows), int(max_reqs)
+        self.max_pages = int(max_pages_per_request)
+        r, b = self.max_rows, self.max_reqs
+        # One int32 buffer, fixed offsets: the addresses never change, so a
+        # captured graph of a step stays valid while only the contents move.
+        sizes = [("token_ids", r), ("positions", r), ("row_req", r), ("q_start", b + 1),
+                 ("start_pos", b), ("req_rows", b), ("want_rows", r)]
+        self._offsets: Dict[str, Tuple[int, int]] = {}
+        at = 0
+        for name, n in sizes:
+            self._offsets[name] = (at, n)
+            at += n
+        self._meta_len = at
+        self._table_at = []
+        for _ in groups:
+            self._table_at.append(at)
+            at += b * self.max_pages
+        pin = (torch.device(device).type == "cuda")
+        self._host = torch.zeros(at, dtype=torch.int32, pin_memory=pin)
+        self._host_np = self._host.numpy()
+        self._dev = torch.zeros(at, dtype=torch.int32, device=device)
+        self._groups = [
+            GroupView(self._dev[t:t + b * self.max_pages].view(b, self.max_pages), page_size, window)
+            for t, (page_size, window) in zip(self._table_at, groups)]
+        self._scratch: Dict[Tuple[str, torch.dtype], torch.Tensor] = {}
+        self.scratch_version = 0
+        self.n_rows = self.n_reqs = self.n_want = 0
+        self.max_q_len = self.max_ctx_len = 0
+        self.host_q_start: List[int] = []
+        self.host_start_pos: List[int] = []
+        self.host_req_rows: List[int] = []
+        self._set_views()
+
+    def _view(self, name: str, count: int) -> torch.Tensor:
+        at, cap = self._offsets[name]
+        return self._dev[at:at + count]
+
+    def _set_views(self) -> None:
+        self.token_ids = self._view("token_ids", self.n_rows)
+        self.positions = self._view("positions", self.n_rows)
+        self.row_req = self._view("row_req", self.n_rows)
+        self.q_start = self._view("q_start", self.n_reqs + 1)
+        self.start_pos = self._view("start_pos", self.n_reqs)
+        self.req_rows = self._view("req_rows", self.n_reqs)
+        self.want_rows = self._view("want_rows", self.n_want)
+
+    def group(self, index: int) -> GroupView:
+        return self._groups[index]
+
+    def scratch(self, name: str, shape: Tuple[int, ...], dtype: torch.dtype) -> torch.Tensor:
+        """A reusable buffer: the same name and dtype give the same memory on
+        every step, grown when a larger shape is asked for."""
+        count = 1
+        for s in shape:
+            count *= int(s)
+        key = (name, dtype)
+        buf = self._scratch.get(key)
+        if buf is None or buf.numel() < count:
+            buf = torch.empty(max(count, 1), dtype=dtype, device=self.device)
+            self._scratch[key] = buf
+            self.scratch_version += 1
+        return buf[:count].view(shape)
+
+    # ------------------------------------------------------------------ fill
+    def fill(self, entries: Sequence[StepEntry], cache: CacheManager) -> None:
+        n_rows = sum(len(e.tokens) for e in entries)
+        n_reqs = len(entries)
+        if n_rows > self.max_rows:
+            raise ValueError(f"a step of {n_rows} tokens exceeds max_batch_tokens {self.max_rows}")
+        if n_reqs > self.max_reqs:
+            raise ValueError(f"a step of {n_reqs} requests exceeds max_requests {self.max_reqs}")
+        h = self._host_np
+        o = {k: v[0] for k, v in self._offsets.items()}
+        row = 0
+        want: List[int] = []
+        self.host_q_start, self.host_start_pos, self.host_req_rows = [], [], []
+        max_q = max_ctx = 0
+        for b, e in enumerate(entries):
+            n = len(e.tokens)
+            start = e.request.computed_len
+            h[o["token_ids"] + row:o["token_ids"] + row + n] = np.asarray(e.tokens, dtype=np.int32)
+            h[o["positions"] + row:o["positions"] + row + n] = np.arange(start, start + n, dtype=np.int32)
+            h[o["row_req"] + row:o["row_req"] + row + n] = b
+            h[o["q_start"] + b] = row
+            h[o["start_pos"] + b] = start
+            h[o["req_rows"] + b] = e.request.row
+            for w in e.want:
+                if not 0 <= w < n:
+                    raise ValueError(f"request {e.request.request_id!r}: wanted place {w} is not "
+                                     f"among its {n} tokens of this step")
+                want.append(row + int(w))
+            self.host_q_start.append(row)
+            self.host_start_pos.append(start)
+            self.host_req_rows.append(e.request.row)
+            max_q = max(max_q, n)
+            max_ctx = max(max_ctx, start + n)
+            row += n
+        h[o["q_start"] + n_reqs] = row
+        self.host_q_start.append(row)
+        if want:
+            h[o["want_rows"]:o["want_rows"] + len(want)] = np.asarray(want, dtype=np.int32)
+        self.n_rows, self.n_reqs, self.n_want = n_rows, n_reqs, len(want)
+        self.max_q_len, self.max_ctx_len = max_q, max_ctx
+        used_pages = (max_ctx + cache.page_size - 1) // cache.page_size
+        for gi, at in enumerate(self._table_at):
+            table = h[at:at + self.max_reqs * self.max_pages].reshape(self.max_reqs, self.max_pages)
+            for b, e in enumerate(entries):
+                table[b, :used_pages] = cache.tables[gi][e.request.row, :used_pages]
+        self._upload(n_reqs)
+        self._set_views()
+
+    def _upload(self, n_reqs: int) -> None:
+        self._dev[:self._meta_len].copy_(self._host[:self._meta_len], non_blocking=True)
+        for at in self._table_at:
+            n = n_reqs * self.max_pages
+            self._dev[at:at + n].copy_(self._host[at:at + n], non_blocking=True)
+
+
+class StepFunction:
+    """Owns the step's buffers; ``__call__`` runs one step."""
+
+    def __init__(self, model: CausalLM, cache: CacheManager, ops, max_batch_tokens: int):
+        self.model = model
+        self.cache = cache
+        self.ops = ops
+        self.max_batch_tokens = int(max_batch_tokens)
+        self.ctx = StepContext(
+            ops, cache.device, self.max_batch_tokens, cache.max_requests,
+            [(cache.page_size, g.window) for g in cache.groups], cache.max_pages_per_request)
+        self.steps = 0
+        self.rows_total = 0
+
+    def __call__(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        """Reserve pages, run the rows, commit.  Returns float32 logits
+        ``[wanted, vocab]`` in the order of the entries and of their ``want``
+        (None when nothing is wanted).  The tensor is reused by the next step."""
+        if not entries:
+            return None
+        vocab, max_pos = self.model.spec.vocab_size, self.model.spec.max_positions
+        seen = set()
+        for e in entries:
+            if id(e.request) in seen:
+                raise ValueError(f"request {e.request.request_id!r} appears twice in one step")
+            seen.add(id(e.request))
+            if len(e.tokens) == 0:
+                raise ValueError(f"request {e.request.request_id!r} brings no token")
+            for t in e.tokens:
+                if not 0 <= int(t) < vocab:
+                    raise ValueError(f"token id {t} is outside the vocabulary of {vocab}")
+            if e.request.computed_len + len(e.tokens) > max_pos:
+                raise ValueError(
+                    f"request {e.request.request_id!r}: position "
+                    f"{e.request.computed_len + len(e.tokens) - 1} exceeds max_position_embeddings {max_pos}")
+        reserved: List[RequestCache] = []
+        try:
+            for e in entries:
+                self.cache.reserve(e.request, len(e.tokens))
+                reserved.append(e.request)
+            self.ctx.fill(entries, self.cache)
+        except Exception:
+            for r in reserved:
+                self.cache.cancel_reservation(r)
+            raise
+        logits = self.model.forward(self.ctx)
+        for e in entries:
+            self.cache.commit(e.request)
+        self.steps += 1
+        self.rows_total += self.ctx.n_rows
+        return logits

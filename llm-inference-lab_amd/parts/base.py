@@ -1,0 +1,107 @@
+"""Interfaces of the parts.
+
+Data flow through a block: the residual stream ``x`` is a float32 tensor
+``[rows, hidden]`` (rows = all tokens of the step, packed); a norm reads it and
+writes activations in the compute dtype; a mixer or feed-forward reads those
+activations and ADDS its result into the residual stream in float32.
+
+Every part states which tensors of the model file it needs (``tensor_specs``),
+receives them in ``bind``, and takes its sizes and constants as constructor
+arguments.  No part knows which model it is in.
+"""
+from __future__ import annotations
+
+import dataclasses
+from typing import Dict, Optional, Tuple
+
+import torch
+
+from ..weights.loader import TensorSpec
+
+
+@dataclasses.dataclass(frozen=True)
+class KVCacheSpec:
+    """What a mixer keeps for each token: ``num_kv_heads * head_dim`` keys and as
+    many values.  ``window``: how many of the latest positions (the current one
+    included) it ever reads, or ``None`` for all.  Mixers with equal specs share
+    one group of pages and one block table."""
+
+    num_kv_heads: int
+    head_dim: int
+    window: Optional[int] = None
+
+
+class Part:
+    """Common base: tensors by role, bound after loading."""
+
+    def __init__(self, tensors: Optional[Dict[str, str]] = None):
+        self.tensor_names: Dict[str, str] = dict(tensors or {})
+        self.ops = None
+        self.dtype = None
+
+    def tensor_specs(self) -> Dict[str, TensorSpec]:
+        """Tensor name in the model file -> expected shape and kind."""
+        return {}
+
+    def bind(self, tensors: Dict[str, torch.Tensor], ops, dtype: torch.dtype) -> None:
+        """Receive the loaded tensors (by file name), the kernel set and the
+        compute dtype.  A part may rearrange its tensors here (fuse, interleave)."""
+        self.ops = ops
+        self.dtype = dtype
+
+    def weight_bytes(self) -> int:
+        """Bytes of weights one forward reads (for roofline accounting)."""
+        return 0
+
+
+class Norm(Part):
+    def forward(self, x: torch.Tensor, out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> None:
+        """``out[i] = norm(x[rows[i]])`` (all rows in order when ``rows`` is None).
+        ``x`` float32, ``out`` compute dtype."""
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    def rotary_table(self) -> Optional[torch.Tensor]:
+        """``inv_freq [rotary_dim/2]`` float32 if this is a split-half rotation
+        that the fused projection epilogue can apply; None otherwise."""
+        return None
+
+    def apply(self, q: torch.Tensor, k: torch.Tensor, positions: torch.Tensor) -> None:
+        """Encode positions into ``q [rows, heads, dim]`` and ``k`` in place."""
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    def cache_spec(self) -> Optional[KVCacheSpec]:
+        """Per-token cache need, or None."""
+        return None
+
+    def state_spec(self) -> Dict[str, Tuple[Tuple[int, ...], torch.dtype]]:
+        """Fixed-size per-request state: name -> (shape, dtype).  The cache
+        manager keeps ``[max_requests, *shape]`` per name, zeroed at admission."""
+        return {}
+
+    def forward(self, h: torch.Tensor, residual: torch.Tensor, ctx, entry) -> None:
+        """``residual += mixer(h)``; ``h`` are the normed activations of this
+        step's rows, ``ctx`` the step's batch description, ``entry`` this run's
+        cache and state (``EntryView``)."""
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, h: torch.Tensor, residual: torch.Tensor, ctx) -> None:
+        """``residual += feed_forward(h)``."""
+        raise NotImplementedError
+
+
+class Block(Part):
+    def parts(self):
+        """The parts this block is made of (for tensor lists and binding)."""
+        raise NotImplementedError
+
+    def mixer_part(self) -> Mixer:
+        raise NotImplementedError
+
+    def forward(self, residual: torch.Tensor, ctx, entry) -> None:
+        raise NotImplementedError

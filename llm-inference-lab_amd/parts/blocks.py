@@ -1,0 +1,108 @@
+"""Arrangements of parts in a layer, the embedding and the output head."""
+from __future__ import annotations
+
+from typing import Dict
+
+import torch
+
+from ..config.spec import PartSpec
+from ..weights.loader import TensorSpec, MATRIX
+from .base import Block, Part
+from .registry import register_part, build_part
+
+
+class PreNormBlock(Block):
+    """``x += mixer(norm1(x)); x += feed_forward(norm2(x))``; the sums are taken
+    in float32 on the float32 residual stream.
+
+    Arrangement: rust/engine/src/runner/model/qwen2/engine.rs:1065-1122 (layer
+    loop), 1140-1147 and 1234-1241 (norm before each sublayer)."""
+
+    def __init__(self, hidden_size: int, norm1: PartSpec, mixer: PartSpec, norm2: PartSpec,
+                 feed_forward: PartSpec, tensors: Dict[str, str] = None):
+        super().__init__(tensors)
+        self.hidden_size = int(hidden_size)
+        self.norm1 = build_part("norm", norm1)
+        self.mixer = build_part("mixer", mixer)
+        self.norm2 = build_part("norm", norm2)
+        self.feed_forward = build_part("feed_forward", feed_forward)
+
+    def parts(self):
+        return [self.norm1, self.mixer, self.norm2, self.feed_forward]
+
+    def mixer_part(self):
+        return self.mixer
+
+    def tensor_specs(self):
+        specs = {}
+        for p in self.parts():
+            specs.update(p.tensor_specs())
+        return specs
+
+    def bind(self, tensors, ops, dtype):
+        super().bind(tensors, ops, dtype)
+        for p in self.parts():
+            p.bind(tensors, ops, dtype)
+
+    def forward(self, residual, ctx, entry):
+        rows = residual.shape[0]
+        h = ctx.scratch("block.normed", (rows, self.hidden_size), self.dtype)
+        self.norm1.forward(residual, h)
+        self.mixer.forward(h, residual, ctx, entry)
+        self.norm2.forward(residual, h)
+        self.feed_forward.forward(h, residual, ctx)
+
+    def weight_bytes(self):
+        return sum(p.weight_bytes() for p in self.parts())
+
+
+class TokenEmbedding(Part):
+    """``x[r] = table[id_r]`` into the float32 residual stream
+    (rust/engine/src/runner/model/qwen2/kernels.rs:46-57)."""
+
+    def __init__(self, vocab_size: int, hidden_size: int, tensors: Dict[str, str]):
+        super().__init__(tensors)
+        self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
+        self.table = None
+
+    def tensor_specs(self):
+        return {self.tensor_names["weight"]: TensorSpec((self.vocab_size, self.hidden_size), MATRIX)}
+
+    def bind(self, tensors, ops, dtype):
+        super().bind(tensors, ops, dtype)
+        self.table = tensors[self.tensor_names["weight"]]
+
+    def forward(self, ids, out):
+        self.ops.embed(self.table, ids, out)
+
+    def weight_bytes(self):
+        return 0     # a step reads one row per token, not the table
+
+
+class LinearHead(Part):
+    """``logits = h W^T`` in float32; ``W`` is the embedding table when the
+    names coincide (tied), as in rust/engine/src/runner/model/qwen2/engine.rs:299-303
+    and 1312-1319."""
+
+    def __init__(self, vocab_size: int, hidden_size: int, tensors: Dict[str, str]):
+        super().__init__(tensors)
+        self.vocab_size, self.hidden_size = int(vocab_size), int(hidden_size)
+        self.weight = None
+
+    def tensor_specs(self):
+        return {self.tensor_names["weight"]: TensorSpec((self.vocab_size, self.hidden_size), MATRIX)}
+
+    def bind(self, tensors, ops, dtype):
+        super().bind(tensors, ops, dtype)
+        self.weight = tensors[self.tensor_names["weight"]]
+
+    def forward(self, h, out):
+        self.ops.linear_logits(h, self.weight, out)
+
+    def weight_bytes(self):
+        return self.weight.numel() * self.weight.element_size()
+
+
+register_part("block", "prenorm", PreNormBlock)
+register_part("embedding", "token_embedding", TokenEmbedding)
+register_part("head", "linear_head", LinearHead)

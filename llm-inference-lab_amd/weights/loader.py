@@ -1,0 +1,105 @@
+"""Weights by tensor name.
+
+A model says which tensors it expects (name -> ``TensorSpec``); the loader
+compares that list with the file and raises ONE ``WeightError`` that lists
+every missing name, every unexpected name and every wrong shape.  The
+reference reports the first missing tensor or wrong shape only and ignores
+extra tensors (rust/engine/src/runner/loader.rs:218,
+rust/engine/src/runner/model/qwen2/engine.rs:2223-2241).
+
+Kept dtypes: matrices take the compute dtype (bfloat16, or float32 in the
+32-bit mode); vectors (norm weights, biases) keep their stored width, so a
+vector stored in 32 bits stays in 32 bits also in the bfloat16 mode; integer
+tables become int32.  The reference converts every tensor to the one storage
+type of the engine (loader.rs:57-133).
+"""
+from __future__ import annotations
+
+import dataclasses
+from typing import Callable, Dict, Iterable, Iterator, Optional, Tuple
+
+import torch
+
+from ..config.errors import WeightError
+from .safetensors_io import ModelFiles
+
+MATRIX = "matrix"
+VECTOR = "vector"
+INT_TABLE = "int"
+
+
+@dataclasses.dataclass(frozen=True)
+class TensorSpec:
+    shape: Tuple[int, ...]
+    kind: str = MATRIX
+
+
+def kept_dtype(kind: str, stored: torch.dtype, compute: torch.dtype) -> torch.dtype:
+    """Which dtype a tensor of ``kind`` stored as ``stored`` is held in."""
+    if kind == INT_TABLE:
+        return torch.int32
+    if compute == torch.float32:
+        return torch.float32
+    if kind == VECTOR:
+        return torch.bfloat16 if stored == torch.bfloat16 else torch.float32
+    return torch.bfloat16
+
+
+def check_names_and_shapes(expected: Dict[str, TensorSpec], found: Dict[str, Tuple[Tuple[int, ...], torch.dtype]],
+                           where: str) -> None:
+    missing = sorted(n for n in expected if n not in found)
+    unexpected = sorted(n for n in found if n not in expected)
+    wrong_shape = []
+    wrong_dtype = []
+    for name, spec in expected.items():
+        if name not in found:
+            continue
+        shape, dtype = found[name]
+        if tuple(shape) != tuple(spec.shape):
+            wrong_shape.append((name, tuple(spec.shape), tuple(shape)))
+        is_int = dtype in (torch.int64, torch.int32, torch.int16, torch.int8, torch.uint8, torch.bool)
+        if is_int != (spec.kind == INT_TABLE):
+            wrong_dtype.append((name, "integer" if spec.kind == INT_TABLE else "floating point",
+                                str(dtype)))
+    if not (missing or unexpected or wrong_shape or wrong_dtype):
+        return
+    lines = [f"{where}: the tensors do not match the model"]
+    if missing:
+        lines.append(f"  missing ({len(missing)}): " + ", ".join(missing))
+    if unexpected:
+        lines.append(f"  unexpected ({len(unexpected)}): " + ", ".join(unexpected))
+    if wrong_shape:
+        lines.append(f"  wrong shape ({len(wrong_shape)}): " + ", ".join(
+            f"{n} expected {list(e)} found {list(f)}" for n, e, f in wrong_shape))
+    if wrong_dtype:
+        lines.append(f"  wrong dtype ({len(wrong_dtype)}): " + ", ".join(
+            f"{n} expected {e} found {f}" for n, e, f in wrong_dtype))
+    raise WeightError("\n".join(lines), missing, unexpected, wrong_shape, wrong_dtype)
+
+
+def load_tensors(model_dir: str, expected: Dict[str, TensorSpec], compute_dtype: torch.dtype,
+                 device, progress: Optional[Callable[[str], None]] = None) -> Dict[str, torch.Tensor]:
+    """Read every expected tensor of a model folder onto ``device``."""
+    files = ModelFiles(model_dir)
+    try:
+        found = {n: (files.shape(n), files.dtype(n)) for n in files.names()}
+        check_names_and_shapes(expected, found, model_dir)
+        out: Dict[str, torch.Tensor] = {}
+        for i, (name, spec) in enumerate(expected.items()):
+            host = files.tensor(name)
+            out[name] = host.to(kept_dtype(spec.kind, host.dtype, compute_dtype)).to(device)
+            if progress is not None and i % 64 == 0:
+                progress(f"loaded {i + 1}/{len(expected)} tensors")
+        return out
+    finally:
+        files.close()
+
+
+def place_tensors(tensors: Iterable[Tuple[str, torch.Tensor]], expected: Dict[str, TensorSpec],
+                  compute_dtype: torch.dtype, device, where: str = "tensors") -> Dict[str, torch.Tensor]:
+    """Same checks and dtype rules for tensors that are already in memory."""
+    given = dict(tensors)
+    found = {n: (tuple(t.shape), t.dtype) for n, t in given.items()}
+    check_names_and_shapes(expected, found, where)
+    return {n: given[n].to(kept_dtype(expected[n].kind, given[n].dtype, compute_dtype)).to(device)
+            for n in expected}

@@ -1,0 +1,160 @@
+"""Plain PyTorch references of the kernel set, op by op, on the engine's own
+buffers and layouts (paged cache, block tables, interleaved gate/up rows).
+
+Two uses: the GPU tests compare each HIP kernel with the function of the same
+name here, and the CPU tests plug this object into the engine in place of the
+HIP kernels to exercise the cache manager, the step function and the scheduler
+without a GPU.  It is test code, not a fallback: the product never loads it.
+All arithmetic is float32 whatever the storage dtype.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+
+class EmuOps:
+    def __init__(self, device="cpu"):
+        self.device = torch.device(device)
+        self.calls = {}
+
+    def _count(self, name):
+        self.calls[name] = self.calls.get(name, 0) + 1
+
+    def check_attention_sizes(self, num_heads, num_kv_heads, head_dim, dtype):
+        pass
+
+    def synchronize(self):
+        pass
+
+    # ------------------------------------------------------------ elementwise
+    def embed(self, table, ids, out):
+        self._count("embed")
+        out.copy_(table[ids.long()].float())
+
+    def rmsnorm(self, x, weight, eps, out, rows=None):
+        self._count("rmsnorm")
+        v = x.float() if rows is None else x.float()[rows.long()]
+        inv = torch.rsqrt((v * v).sum(-1, keepdim=True) / v.shape[-1] + eps)
+        out.copy_((v * inv * weight.float()).to(out.dtype))
+
+    # ----------------------------------------------------------------- linear
+    def linear(self, x, w, out, bias=None):
+        self._count("linear")
+        y = x.float() @ w.float().t()
+        if bias is not None:
+            y = y + bias.float()
+        out.copy_(y.to(out.dtype))
+
+    def linear_residual(self, x, w, resid, bias=None):
+        self._count("linear_residual")
+        y = x.float() @ w.float().t()
+        if bias is not None:
+            y = y + bias.float()
+        resid.add_(y)
+
+    def linear_logits(self, x, w, out):
+        self._count("linear_logits")
+        out.copy_(x.float() @ w.float().t())
+
+    def linear_swiglu(self, x, w_gu, out):
+        """w_gu rows alternate in runs of 16: gate rows of 16 outputs, then the
+        up rows of the same outputs."""
+        self._count("linear_swiglu")
+        inter = out.shape[1]
+        y = x.float() @ w_gu.float().t()                       # [M, 2*Ipad]
+        y = y.view(x.shape[0], -1, 2, 16)
+        gate = y[:, :, 0, :].reshape(x.shape[0], -1)[:, :inter]
+        up = y[:, :, 1, :].reshape(x.shape[0], -1)[:, :inter]
+        out.copy_((gate / (1.0 + torch.exp(-gate)) * up).to(out.dtype))
+
+    # ------------------------------------------------------------------- rope
+    @staticmethod
+    def _rotate(x, positions, inv_freq):
+        # x [rows, heads, d] float32
+        half = x.shape[-1] // 2
+        ang = positions.float()[:, None] * inv_freq.float()[None, :]
+        c, s = torch.cos(ang)[:, None, :], torch.sin(ang)[:, None, :]
+        lo, hi = x[..., :half], x[..., half:]
+        return torch.cat([lo * c - hi * s, hi * c + lo * s], dim=-1)
+
+    def rope_inplace(self, x, positions, inv_freq):
+        self._count("rope_inplace")
+        x.copy_(self._rotate(x.float(), positions, inv_freq).to(x.dtype))
+
+    def rope_kv_write(self, qkv, num_heads, num_kv_heads, head_dim, inv_freq, positions, row_req,
+                      block_table, page_size, k_cache, v_cache):
+        self._count("rope_kv_write")
+        rows = qkv.shape[0]
+        qs, ks = num_heads * head_dim, num_kv_heads * head_dim
+        q = qkv[:, :qs].float().view(rows, num_heads, head_dim)
+        k = qkv[:, qs:qs + ks].float().view(rows, num_kv_heads, head_dim)
+        v = qkv[:, qs + ks:].float().view(rows, num_kv_heads, head_dim)
+        if inv_freq is not None:
+            q = self._rotate(q, positions[:rows], inv_freq)
+            k = self._rotate(k, positions[:rows], inv_freq)
+            qkv[:, :qs] = q.reshape(rows, qs).to(qkv.dtype)
+        if k_cache is None:
+            return
+        for r in range(rows):
+            p = int(positions[r])
+            page = int(block_table[int(row_req[r]), p // page_size])
+            assert page >= 0, "write to a position without a page"
+            off = p % page_size
+            k_cache[page, :, off, :] = k[r].to(k_cache.dtype)
+            v_cache[page, :, :, off] = v[r].to(v_cache.dtype)
+
+    # -------------------------------------------------------------- attention
+    def paged_attention(self, qkv, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_table,
+                        page_size, q_start, start_pos, n_reqs, max_q_len, max_ctx_len, window, scale,
+                        out, ctx=None):
+        self._count("paged_attention")
+        group = num_heads // num_kv_heads
+        qs = num_heads * head_dim
+        for b in range(n_reqs):
+            r0, r1 = int(q_start[b]), int(q_start[b + 1])
+            sp = int(start_pos[b])
+            for r in range(r0, r1):
+                p = sp + (r - r0)
+                lo = 0 if window is None else max(0, p - window + 1)
+                js = list(range(lo, p + 1))
+                pages = [int(block_table[b, j // page_size]) for j in js]
+                assert all(pg >= 0 for pg in pages), "read of a position without a page"
+                offs = [j % page_size for j in js]
+                q = qkv[r, :qs].float().view(num_heads, head_dim)
+                for h in range(num_heads):
+                    kvh = h // group
+                    keys = torch.stack([k_cache[pg, kvh, o, :].float() for pg, o in zip(pages, offs)])
+                    vals = torch.stack([v_cache[pg, kvh, :, o].float() for pg, o in zip(pages, offs)])
+                    s = (keys @ q[h]) * scale
+                    pr = torch.softmax(s, dim=0)
+                    out[r, h * head_dim:(h + 1) * head_dim] = (pr @ vals).to(out.dtype)
+
+    # --------------------------------------------------------------- sampling
+    def argmax(self, logits, out):
+        self._count("argmax")
+        for b in range(logits.shape[0]):
+            row = logits[b]
+            if torch.isnan(row).all():
+                out[b] = -1
+                continue
+            row = torch.where(torch.isnan(row), torch.full_like(row, float("-inf")), row)
+            m = row.max()
+            out[b] = int((row == m).nonzero()[0, 0])
+
+    def sample(self, logits, temperatures, uniforms, out):
+        """temperature <= 0: argmax.  Else the smallest index whose cumulative
+        probability under softmax(logits / t) reaches u * total."""
+        self._count("sample")
+        for b in range(logits.shape[0]):
+            t = float(temperatures[b])
+            if t <= 0.0:
+                self.argmax(logits[b:b + 1], out[b:b + 1])
+                continue
+            z = logits[b].double() / t
+            e = torch.exp(z - z.max())
+            target = float(uniforms[b]) * float(e.sum())
+            cum = torch.cumsum(e, dim=0)
+            idx = int(torch.searchsorted(cum, torch.tensor(target, dtype=torch.float64)))
+            out[b] = min(idx, logits.shape[1] - 1)
