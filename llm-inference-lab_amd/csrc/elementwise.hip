@@ -1,0 +1,191 @@
+// Embedding gather, RMSNorm, and rotary position encoding fused with the
+// write of keys and values into the paged cache.  gfx950 only.
+#include "common.h"
+
+extern "C" const char* llmlab_last_error() { return g_llmlab_error; }
+
+extern "C" int llmlab_abi_version() { return 1; }
+
+// --------------------------------------------------------------- embedding
+// out[r, :] = float(table[ids[r], :]); an id outside [0, vocab) is clamped (the
+// host has already refused such ids; the clamp keeps a stale device-side id
+// from reading outside the table).
+template <typename T>
+__global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ ids,
+                             float* __restrict__ out, int hidden, int vocab) {
+  const int r = blockIdx.x;
+  int id = ids[r];
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+  const T* src = table + (size_t)id * hidden;
+  float* dst = out + (size_t)r * hidden;
+  for (int c = threadIdx.x; c < hidden; c += blockDim.x) dst[c] = to_float(src[c]);
+}
+
+extern "C" int llmlab_embed(const void* table, int dtype, const int* ids, float* out, int rows,
+                            int hidden, int vocab, hipStream_t stream) {
+  LLMLAB_REQUIRE(rows >= 0 && hidden > 0 && vocab > 0, "embed: bad sizes rows=%d hidden=%d vocab=%d",
+                 rows, hidden, vocab);
+  if (rows == 0) return 0;
+  dim3 grid(rows), block(256);
+  if (dtype == DT_BF16)
+    hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)table, ids, out,
+                       hidden, vocab);
+  else
+    hipLaunchKernelGGL(embed_kernel<float>, grid, block, 0, stream, (const float*)table, ids, out,
+                       hidden, vocab);
+  LLMLAB_LAUNCH_CHECK("embed");
+  return 0;
+}
+
+// ----------------------------------------------------------------- RMSNorm
+// out[i, :] = x[row_i, :] * rsqrt(mean(x[row_i]^2) + eps) * w, row_i = rows[i] or
+// i.  The square, the mean, the rsqrt and both products are float32; one
+// rounding to T at the end.
+template <typename T>
+__global__ void rmsnorm_kernel(const float* __restrict__ x, const void* __restrict__ w, int w_bf16,
+                               float eps, T* __restrict__ out, const int* __restrict__ rows,
+                               int hidden) {
+  __shared__ float red[17];
+  const int i = blockIdx.x;
+  const int r = rows ? rows[i] : i;
+  const float* src = x + (size_t)r * hidden;
+  float ss = 0.f;
+  for (int c = threadIdx.x; c < hidden; c += blockDim.x) {
+    const float v = src[c];
+    ss += v * v;
+  }
+  ss = block_sum(ss, red);
+  const float inv = rsqrtf(ss / (float)hidden + eps);
+  T* dst = out + (size_t)i * hidden;
+  for (int c = threadIdx.x; c < hidden; c += blockDim.x)
+    dst[c] = from_float<T>(src[c] * inv * load_vec(w, w_bf16, c));
+}
+
+extern "C" int llmlab_rmsnorm(const float* x, const void* w, int w_dtype, float eps, void* out,
+                              int out_dtype, const int* rows, int n_out, int hidden,
+                              hipStream_t stream) {
+  LLMLAB_REQUIRE(n_out >= 0 && hidden > 0, "rmsnorm: bad sizes n=%d hidden=%d", n_out, hidden);
+  if (n_out == 0) return 0;
+  dim3 grid(n_out), block(hidden >= 2048 ? 512 : 256);
+  if (out_dtype == DT_BF16)
+    hipLaunchKernelGGL(rmsnorm_kernel<bf16_t>, grid, block, 0, stream, x, w, w_dtype == DT_BF16, eps,
+                       (bf16_t*)out, rows, hidden);
+  else
+    hipLaunchKernelGGL(rmsnorm_kernel<float>, grid, block, 0, stream, x, w, w_dtype == DT_BF16, eps,
+                       (float*)out, rows, hidden);
+  LLMLAB_LAUNCH_CHECK("rmsnorm");
+  return 0;
+}
+
+// ------------------------------------------------- rotary + cache write
+// One block per (row, head) of the packed projection output
+//   qkv[r] = [q heads | k heads | v heads], each head `d` wide.
+// q heads: rotated in place.  k heads: rotated, written in place and to the
+// key page  K[page][kvh][off][d].  v heads: written to the value page, which is
+// kept transposed,  V[page][kvh][d][off].  page = table[row_req[r]][pos / P],
+// off = pos % P.  Angles, sine and cosine in float32; one rounding to T.
+template <typename T>
+__global__ void rope_kv_write_kernel(T* __restrict__ qkv, int row_stride, int nq, int nkv, int d,
+                                     const float* __restrict__ inv_freq,
+                                     const int* __restrict__ positions,
+                                     const int* __restrict__ row_req, const int* __restrict__ table,
+                                     int table_stride, int page_size, T* __restrict__ kcache,
+                                     T* __restrict__ vcache) {
+  const int r = blockIdx.x, head = blockIdx.y;
+  const int pos = positions[r];
+  T* base = qkv + (size_t)r * row_stride + (size_t)head * d;
+  const bool is_q = head < nq, is_k = !is_q && head < nq + nkv;
+  size_t page = 0;
+  int off = 0;
+  if (!is_q && kcache) {
+    page = (size_t)table[(size_t)row_req[r] * table_stride + pos / page_size];
+    off = pos % page_size;
+  }
+  if (is_q || is_k) {
+    const int half = d >> 1;
+    T* kdst = nullptr;
+    if (is_k && kcache)
+      kdst = kcache + ((page * nkv + (head - nq)) * page_size + off) * (size_t)d;
+    for (int i = threadIdx.x; i < half; i += blockDim.x) {
+      float lo = to_float(base[i]), hi = to_float(base[i + half]);
+      if (inv_freq) {
+        float s, c;
+        sincosf((float)pos * inv_freq[i], &s, &c);
+        const float nlo = lo * c - hi * s, nhi = hi * c + lo * s;
+        lo = nlo;
+        hi = nhi;
+        base[i] = from_float<T>(lo);
+        base[i + half] = from_float<T>(hi);
+      }
+      if (kdst) {
+        kdst[i] = from_float<T>(lo);
+        kdst[i + half] = from_float<T>(hi);
+      }
+    }
+  } else if (vcache) {
+    T* vdst = vcache + ((page * nkv + (head - nq - nkv)) * (size_t)d) * page_size + off;
+    for (int i = threadIdx.x; i < d; i += blockDim.x) vdst[(size_t)i * page_size] = base[i];
+  }
+}
+
+extern "C" int llmlab_rope_kv_write(void* qkv, int dtype, int rows, int row_stride, int nq, int nkv,
+                                    int d, const float* inv_freq, const int* positions,
+                                    const int* row_req, const int* table, int table_stride,
+                                    int page_size, void* kcache, void* vcache, hipStream_t stream) {
+  LLMLAB_REQUIRE(rows >= 0 && nq > 0 && nkv >= 0 && d > 0 && d % 2 == 0,
+                 "rope_kv_write: bad sizes rows=%d nq=%d nkv=%d d=%d", rows, nq, nkv, d);
+  LLMLAB_REQUIRE(row_stride >= (nq + 2 * nkv) * d || (kcache == nullptr && row_stride >= nq * d),
+                 "rope_kv_write: row stride %d is smaller than the heads it holds", row_stride);
+  LLMLAB_REQUIRE((kcache == nullptr) == (vcache == nullptr), "rope_kv_write: need both caches or none");
+  LLMLAB_REQUIRE(kcache == nullptr || (table != nullptr && row_req != nullptr && page_size > 0),
+                 "rope_kv_write: a cache write needs a block table");
+  if (rows == 0) return 0;
+  // Without a cache only q and k heads are rotated (k in place) and v is left alone.
+  const int heads = kcache ? nq + 2 * nkv : (inv_freq ? nq + nkv : 0);
+  if (heads == 0) return 0;
+  dim3 grid(rows, heads), block(64);
+  if (dtype == DT_BF16)
+    hipLaunchKernelGGL(rope_kv_write_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)qkv, row_stride,
+                       nq, nkv, d, inv_freq, positions, row_req, table, table_stride, page_size,
+                       (bf16_t*)kcache, (bf16_t*)vcache);
+  else
+    hipLaunchKernelGGL(rope_kv_write_kernel<float>, grid, block, 0, stream, (float*)qkv, row_stride,
+                       nq, nkv, d, inv_freq, positions, row_req, table, table_stride, page_size,
+                       (float*)kcache, (float*)vcache);
+  LLMLAB_LAUNCH_CHECK("rope_kv_write");
+  return 0;
+}
+
+// Rotation alone, of x[rows, heads, d] with arbitrary row and head strides.
+template <typename T>
+__global__ void rope_inplace_kernel(T* __restrict__ x, long row_stride, long head_stride, int d,
+                                    const float* __restrict__ inv_freq,
+                                    const int* __restrict__ positions) {
+  const int r = blockIdx.x, head = blockIdx.y;
+  const int pos = positions[r];
+  T* base = x + (size_t)r * row_stride + (size_t)head * head_stride;
+  const int half = d >> 1;
+  for (int i = threadIdx.x; i < half; i += blockDim.x) {
+    const float lo = to_float(base[i]), hi = to_float(base[i + half]);
+    float s, c;
+    sincosf((float)pos * inv_freq[i], &s, &c);
+    base[i] = from_float<T>(lo * c - hi * s);
+    base[i + half] = from_float<T>(hi * c + lo * s);
+  }
+}
+
+extern "C" int llmlab_rope_inplace(void* x, int dtype, int rows, int heads, int d, long row_stride,
+                                   long head_stride, const float* inv_freq, const int* positions,
+                                   hipStream_t stream) {
+  LLMLAB_REQUIRE(rows >= 0 && heads > 0 && d > 0 && d % 2 == 0, "rope_inplace: bad sizes");
+  if (rows == 0) return 0;
+  dim3 grid(rows, heads), block(64);
+  if (dtype == DT_BF16)
+    hipLaunchKernelGGL(rope_inplace_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)x, row_stride,
+                       head_stride, d, inv_freq, positions);
+  else
+    hipLaunchKernelGGL(rope_inplace_kernel<float>, grid, block, 0, stream, (float*)x, row_stride,
+                       head_stride, d, inv_freq, positions);
+  LLMLAB_LAUNCH_CHECK("rope_inplace");
+  return 0;
+}

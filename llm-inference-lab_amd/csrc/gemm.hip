@@ -1,0 +1,442 @@
+// Matrix products  out = x . W^T  (x [M, K] and W [N, K], both K-contiguous)
+// for gfx950, with the epilogues the model needs fused in.
+//
+//   bfloat16:  v_mfma_f32_16x16x32_bf16 everywhere.
+//     * tiled kernel (M > 64): 256 threads = 4 waves in 2x2, block tile 128x128 or
+//       64x64, K step 64 staged through LDS (rows padded to 72 elements so that the
+//       16-byte fragment reads of 8 lanes cover all banks), next tile prefetched
+//       into registers while the current one is multiplied.
+//     * skinny kernel (M <= 64, decode): weights stream from HBM straight into MFMA
+//       B fragments, one wave per 16 (or 32) weight rows and K range; the few rows
+//       of x come from cache.  K may be split over blocks; partial sums go to a
+//       float32 workspace and a second kernel reduces them and applies the epilogue
+//       (a fixed order, so results do not depend on timing).
+//   float32: a plain FMA kernel (64x64 tile, 4x4 outputs per thread): true 32-bit
+//     products and sums, no matrix-core shortcut.
+//
+// Fragment layout of the 16x16x32 MFMA (wave of 64 lanes, lane l):
+//   A operand: row l%16, k = 8*(l/16) .. +7      B operand: column l%16, same k
+//   result element i (0..3): row 4*(l/16)+i, column l%16
+//
+// Epilogues: STORE  out[M,N] (T) = acc (+bias)            RESID  out[M,N] (f32) += acc (+bias)
+//            F32    out[M,N] (f32) = acc                   SWIGLU out[M,N/2] (T) = silu(g)*u
+// For SWIGLU the rows of W alternate in runs of 16: gate rows of 16 outputs, then
+// the up rows of the same 16 outputs, so fragments j and j+1 hold gate and up of
+// the same outputs in the same lanes.
+#include "common.h"
+
+enum { EPI_STORE = 0, EPI_RESID = 1, EPI_F32 = 2, EPI_SWIGLU = 3 };
+
+struct EpiArgs {
+  void* out;         // T or float, see above
+  const void* bias;  // may be null
+  int bias_bf16;
+  int ldo;    // row stride of out in elements
+  int n_out;  // logical output columns (SWIGLU: intermediate size; else N)
+};
+
+__device__ __forceinline__ float silu_f(float z) { return z / (1.f + __expf(-z)); }
+
+// One output element (non-SWIGLU).
+template <typename T, int EPI>
+__device__ __forceinline__ void epi_store(const EpiArgs& e, int m, int n, float acc) {
+  if (e.bias) acc += load_vec(e.bias, e.bias_bf16, n);
+  const size_t at = (size_t)m * e.ldo + n;
+  if (EPI == EPI_STORE)
+    ((T*)e.out)[at] = from_float<T>(acc);
+  else if (EPI == EPI_RESID)
+    ((float*)e.out)[at] += acc;
+  else
+    ((float*)e.out)[at] = acc;
+}
+
+// ============================================================ bf16, tiled
+#define LDS_STRIDE 72
+
+template <int BM, int BN, int EPI>
+__global__ __launch_bounds__(256) void gemm_bf16_tiled(const bf16_t* __restrict__ A,
+                                                        const bf16_t* __restrict__ W, EpiArgs e, int M,
+                                                        int N, int K) {
+  constexpr int BK = 64;
+  constexpr int WTM = BM / 2, WTN = BN / 2;  // wave tile
+  constexpr int TM = WTM / 16, TN = WTN / 16;
+  constexpr int A_CHUNKS = BM * 8 / 256, B_CHUNKS = BN * 8 / 256;  // 16-byte chunks per thread
+  __shared__ __attribute__((aligned(16))) bf16_t As[BM * LDS_STRIDE];
+  __shared__ __attribute__((aligned(16))) bf16_t Bs[BN * LDS_STRIDE];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  const int c = lane & 15, g = lane >> 4;
+
+  floatx4 acc[TM][TN];
+#pragma unroll
+  for (int i = 0; i < TM; ++i)
+#pragma unroll
+    for (int j = 0; j < TN; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  bf16x8 ra[A_CHUNKS], rb[B_CHUNKS];
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < A_CHUNKS; ++i) {
+      const int ch = tid + i * 256, row = ch >> 3, kc = (ch & 7) * 8;
+      const int m = m0 + row, k = k0 + kc;
+      ra[i] = (m < M && k < K) ? *(const bf16x8*)(A + (size_t)m * K + k) : zero;
+    }
+#pragma unroll
+    for (int i = 0; i < B_CHUNKS; ++i) {
+      const int ch = tid + i * 256, row = ch >> 3, kc = (ch & 7) * 8;
+      const int n = n0 + row, k = k0 + kc;
+      rb[i] = (n < N && k < K) ? *(const bf16x8*)(W + (size_t)n * K + k) : zero;
+    }
+  };
+  auto stash = [&]() {
+#pragma unroll
+    for (int i = 0; i < A_CHUNKS; ++i) {
+      const int ch = tid + i * 256, row = ch >> 3, kc = (ch & 7) * 8;
+      *(bf16x8*)(As + row * LDS_STRIDE + kc) = ra[i];
+    }
+#pragma unroll
+    for (int i = 0; i < B_CHUNKS; ++i) {
+      const int ch = tid + i * 256, row = ch >> 3, kc = (ch & 7) * 8;
+      *(bf16x8*)(Bs + row * LDS_STRIDE + kc) = rb[i];
+    }
+  };
+
+  const int nk = (K + BK - 1) / BK;
+  fetch(0);
+  for (int kt = 0; kt < nk; ++kt) {
+    stash();
+    __syncthreads();
+    if (kt + 1 < nk) fetch((kt + 1) * BK);
+#pragma unroll
+    for (int ks = 0; ks < 2; ++ks) {
+      bf16x8 a[TM], b[TN];
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+        a[i] = *(const bf16x8*)(As + (wm * WTM + i * 16 + c) * LDS_STRIDE + ks * 32 + g * 8);
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+        b[j] = *(const bf16x8*)(Bs + (wn * WTN + j * 16 + c) * LDS_STRIDE + ks * 32 + g * 8);
+#pragma unroll
+      for (int i = 0; i < TM; ++i)
+#pragma unroll
+        for (int j = 0; j < TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+    }
+    __syncthreads();
+  }
+
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int nb = n0 + wn * WTN + j * 16;
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        const int m = m0 + wm * WTM + i * 16 + g * 4 + x;
+        if (m >= M) continue;
+        if constexpr (EPI == EPI_SWIGLU) {
+          if (j & 1) continue;
+          const int o = (nb >> 5) * 16 + c;
+          if (o < e.n_out)
+            ((bf16_t*)e.out)[(size_t)m * e.ldo + o] =
+                (bf16_t)(silu_f(acc[i][j][x]) * acc[i][j | 1][x]);
+        } else {
+          const int n = nb + c;
+          if (n < N) epi_store<bf16_t, EPI>(e, m, n, acc[i][j][x]);
+        }
+      }
+    }
+  }
+}
+
+// =========================================================== bf16, skinny
+// One wave per NS strips of 16 weight rows and one K range; MB blocks of 16 rows
+// of x.  SPLIT: write float32 partial sums  part[split][m][n]  instead of the
+// epilogue.
+template <int MB, int NS, int EPI, bool SPLIT>
+__global__ __launch_bounds__(256) void gemm_bf16_skinny(const bf16_t* __restrict__ A,
+                                                         const bf16_t* __restrict__ W, EpiArgs e,
+                                                         float* __restrict__ part, int M, int N, int K,
+                                                         int k_per_split) {
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int c = lane & 15, g = lane >> 4;
+  const int n0 = (blockIdx.x * 4 + wave) * (16 * NS);
+  if (n0 >= N) return;
+  const int k_begin = blockIdx.y * k_per_split;
+  const int k_end = min(K, k_begin + k_per_split);
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+
+  floatx4 acc[MB][NS];
+#pragma unroll
+  for (int i = 0; i < MB; ++i)
+#pragma unroll
+    for (int j = 0; j < NS; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+
+  const bf16_t* wrow[NS];
+  bool wok[NS];
+#pragma unroll
+  for (int j = 0; j < NS; ++j) {
+    const int n = n0 + j * 16 + c;
+    wok[j] = n < N;
+    wrow[j] = W + (size_t)(wok[j] ? n : 0) * K;
+  }
+  const bf16_t* arow[MB];
+  bool aok[MB];
+#pragma unroll
+  for (int i = 0; i < MB; ++i) {
+    const int m = i * 16 + c;
+    aok[i] = m < M;
+    arow[i] = A + (size_t)(aok[i] ? m : 0) * K;
+  }
+
+  int k = k_begin;
+  // full groups of 4 steps: 4 independent 16-byte loads per weight strip in flight
+  for (; k + 128 <= k_end; k += 128) {
+    bf16x8 b[4][NS], a[4][MB];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+      const int kk = k + s * 32 + g * 8;
+#pragma unroll
+      for (int j = 0; j < NS; ++j) b[s][j] = wok[j] ? *(const bf16x8*)(wrow[j] + kk) : zero;
+#pragma unroll
+      for (int i = 0; i < MB; ++i) a[s][i] = aok[i] ? *(const bf16x8*)(arow[i] + kk) : zero;
+    }
+#pragma unroll
+    for (int s = 0; s < 4; ++s)
+#pragma unroll
+      for (int i = 0; i < MB; ++i)
+#pragma unroll
+        for (int j = 0; j < NS; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[s][i], b[s][j], acc[i][j], 0, 0, 0);
+  }
+  for (; k < k_end; k += 32) {
+    const int kk = k + g * 8;
+    const bool kok = kk < k_end;
+    bf16x8 b[NS], a[MB];
+#pragma unroll
+    for (int j = 0; j < NS; ++j) b[j] = (wok[j] && kok) ? *(const bf16x8*)(wrow[j] + kk) : zero;
+#pragma unroll
+    for (int i = 0; i < MB; ++i) a[i] = (aok[i] && kok) ? *(const bf16x8*)(arow[i] + kk) : zero;
+#pragma unroll
+    for (int i = 0; i < MB; ++i)
+#pragma unroll
+      for (int j = 0; j < NS; ++j)
+        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+  }
+
+#pragma unroll
+  for (int i = 0; i < MB; ++i) {
+#pragma unroll
+    for (int j = 0; j < NS; ++j) {
+      const int nb = n0 + j * 16;
+#pragma unroll
+      for (int x = 0; x < 4; ++x) {
+        const int m = i * 16 + g * 4 + x;
+        if (m >= M) continue;
+        if constexpr (SPLIT) {
+          const int n = nb + c;
+          if (n < N) part[((size_t)blockIdx.y * M + m) * N + n] = acc[i][j][x];
+        } else if constexpr (EPI == EPI_SWIGLU) {
+          if (j & 1) continue;
+          const int o = (nb >> 5) * 16 + c;
+          if (o < e.n_out)
+            ((bf16_t*)e.out)[(size_t)m * e.ldo + o] =
+                (bf16_t)(silu_f(acc[i][j][x]) * acc[i][j | 1][x]);
+        } else {
+          const int n = nb + c;
+          if (n < N) epi_store<bf16_t, EPI>(e, m, n, acc[i][j][x]);
+        }
+      }
+    }
+  }
+}
+
+// Sum the partial results of the K splits in a fixed order and apply the epilogue.
+template <typename T, int EPI>
+__global__ void splitk_epilogue(const float* __restrict__ part, EpiArgs e, int M, int N, int splits) {
+  const int cols = (EPI == EPI_SWIGLU) ? e.n_out : N;
+  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (idx >= (size_t)M * cols) return;
+  const int m = (int)(idx / cols), o = (int)(idx % cols);
+  if constexpr (EPI == EPI_SWIGLU) {
+    const int ng = (o >> 4) * 32 + (o & 15), nu = ng + 16;
+    float gsum = 0.f, usum = 0.f;
+    for (int s = 0; s < splits; ++s) {
+      gsum += part[((size_t)s * M + m) * N + ng];
+      usum += part[((size_t)s * M + m) * N + nu];
+    }
+    ((T*)e.out)[(size_t)m * e.ldo + o] = from_float<T>(silu_f(gsum) * usum);
+  } else {
+    float sum = 0.f;
+    for (int s = 0; s < splits; ++s) sum += part[((size_t)s * M + m) * N + o];
+    epi_store<T, EPI>(e, m, o, sum);
+  }
+}
+
+// ================================================================ float32
+// 64x64 outputs per block of 256 threads; thread (ty, tx) owns rows ty + 16*i and
+// columns tx + 16*j (i, j in 0..3), so for SWIGLU columns j = 0, 2 are gate and
+// j = 1, 3 the up values of the same outputs.
+template <int EPI>
+__global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__ A,
+                                                        const float* __restrict__ W, EpiArgs e, int M,
+                                                        int N, int K) {
+  constexpr int BK = 16;
+  __shared__ float As[BK][64 + 1];
+  __shared__ float Bs[BK][64 + 1];
+  const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+  const int m0 = blockIdx.y * 64, n0 = blockIdx.x * 64;
+  float acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+  const int lrow = tid >> 2, lk = (tid & 3) * 4;  // this thread loads 4 k values of one row
+  for (int k0 = 0; k0 < K; k0 += BK) {
+#pragma unroll
+    for (int x = 0; x < 4; ++x) {
+      const int k = k0 + lk + x;
+      const int m = m0 + lrow, n = n0 + lrow;
+      As[lk + x][lrow] = (m < M && k < K) ? A[(size_t)m * K + k] : 0.f;
+      Bs[lk + x][lrow] = (n < N && k < K) ? W[(size_t)n * K + k] : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < BK; ++kk) {
+      float a[4], b[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] = As[kk][ty + 16 * i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) b[j] = Bs[kk][tx + 16 * j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int m = m0 + ty + 16 * i;
+    if (m >= M) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      if constexpr (EPI == EPI_SWIGLU) {
+        if (j & 1) continue;
+        const int nb = n0 + 16 * j;
+        const int o = (nb >> 5) * 16 + tx;
+        if (o < e.n_out) {
+          const float z = acc[i][j];
+          ((float*)e.out)[(size_t)m * e.ldo + o] = z / (1.f + expf(-z)) * acc[i][j + 1];
+        }
+      } else {
+        const int n = n0 + tx + 16 * j;
+        if (n < N) epi_store<float, EPI>(e, m, n, acc[i][j]);
+      }
+    }
+  }
+}
+
+// ================================================================ dispatch
+template <int EPI>
+static int launch_bf16(const bf16_t* A, const bf16_t* W, EpiArgs e, int M, int N, int K,
+                       float* workspace, size_t workspace_floats, int num_cus, hipStream_t stream) {
+  if (M > 64) {
+    const long big_tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
+    if (big_tiles >= num_cus) {
+      dim3 grid((N + 127) / 128, (M + 127) / 128);
+      hipLaunchKernelGGL((gemm_bf16_tiled<128, 128, EPI>), grid, dim3(256), 0, stream, A, W, e, M, N, K);
+    } else {
+      dim3 grid((N + 63) / 64, (M + 63) / 64);
+      hipLaunchKernelGGL((gemm_bf16_tiled<64, 64, EPI>), grid, dim3(256), 0, stream, A, W, e, M, N, K);
+    }
+    return 0;
+  }
+  constexpr int NS = (EPI == EPI_SWIGLU) ? 2 : 1;
+  const int strips = (N + 16 * NS - 1) / (16 * NS);
+  const int blocks = (strips + 3) / 4;
+  // Enough waves to keep HBM busy: split K while there are fewer than ~8 per CU.
+  int splits = 1;
+  const int want_waves = num_cus * 8;
+  if (strips < want_waves) {
+    splits = (want_waves + strips - 1) / strips;
+    const int max_splits = K / 128 > 0 ? K / 128 : 1;
+    if (splits > max_splits) splits = max_splits;
+    if (splits > 32) splits = 32;
+    // the partial sums are written and read once: keep that under a quarter of
+    // the weight bytes (4*splits*M*N*2 against 2*N*K)
+    const int traffic_cap = K / (16 * M) > 0 ? K / (16 * M) : 1;
+    if (splits > traffic_cap) splits = traffic_cap;
+    while (splits > 1 && (size_t)splits * M * N > workspace_floats) --splits;
+  }
+  int k_per_split = ((K + splits - 1) / splits + 31) / 32 * 32;
+  splits = (K + k_per_split - 1) / k_per_split;
+  dim3 grid(blocks, splits), block(256);
+  const int mb = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
+#define SKINNY(MB_, SPLIT_)                                                                      \
+  hipLaunchKernelGGL((gemm_bf16_skinny<MB_, NS, EPI, SPLIT_>), grid, block, 0, stream, A, W, e, \
+                     workspace, M, N, K, k_per_split)
+  if (splits > 1) {
+    if (mb == 1) SKINNY(1, true); else if (mb == 2) SKINNY(2, true); else SKINNY(4, true);
+    const int cols = (EPI == EPI_SWIGLU) ? e.n_out : N;
+    const size_t total = (size_t)M * cols;
+    hipLaunchKernelGGL((splitk_epilogue<bf16_t, EPI>), dim3((unsigned)((total + 255) / 256)), dim3(256),
+                       0, stream, workspace, e, M, N, splits);
+  } else {
+    if (mb == 1) SKINNY(1, false); else if (mb == 2) SKINNY(2, false); else SKINNY(4, false);
+  }
+#undef SKINNY
+  return 0;
+}
+
+// x [M,K] (dtype), w [N,K] (dtype); epilogue selects what `out` is.  For SWIGLU N
+// is the number of interleaved weight rows (2 * ceil16(n_out)).  `workspace` is
+// float32 scratch for split-K partial sums (may be null: no splitting).
+extern "C" int llmlab_linear(const void* x, const void* w, int dtype, int epilogue, void* out,
+                             const void* bias, int bias_dtype, int M, int N, int K, int ldo, int n_out,
+                             float* workspace, size_t workspace_floats, int num_cus,
+                             hipStream_t stream) {
+  LLMLAB_REQUIRE(M >= 0 && N > 0 && K > 0, "linear: bad sizes M=%d N=%d K=%d", M, N, K);
+  LLMLAB_REQUIRE(epilogue >= 0 && epilogue <= 3, "linear: unknown epilogue %d", epilogue);
+  if (epilogue == EPI_SWIGLU) {
+    LLMLAB_REQUIRE(N % 32 == 0 && n_out > 0 && 2 * ((n_out + 15) / 16 * 16) == N,
+                   "linear(swiglu): %d weight rows do not interleave %d outputs", N, n_out);
+    LLMLAB_REQUIRE(bias == nullptr, "linear(swiglu): no bias");
+  } else {
+    LLMLAB_REQUIRE(n_out == N, "linear: n_out %d != N %d", n_out, N);
+  }
+  LLMLAB_REQUIRE(ldo >= n_out, "linear: output row stride %d < %d columns", ldo, n_out);
+  if (M == 0) return 0;
+  EpiArgs e{out, bias, bias_dtype == DT_BF16, ldo, n_out};
+  if (workspace == nullptr) workspace_floats = 0;
+  if (num_cus <= 0) num_cus = 256;
+  if (dtype == DT_BF16) {
+    LLMLAB_REQUIRE(K % 8 == 0, "linear(bfloat16): inner size %d must be a multiple of 8", K);
+    LLMLAB_REQUIRE(((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0),
+                   "linear(bfloat16): operands must be 16-byte aligned");
+    const bf16_t* A = (const bf16_t*)x;
+    const bf16_t* W = (const bf16_t*)w;
+    switch (epilogue) {
+      case EPI_STORE: launch_bf16<EPI_STORE>(A, W, e, M, N, K, workspace, workspace_floats, num_cus, stream); break;
+      case EPI_RESID: launch_bf16<EPI_RESID>(A, W, e, M, N, K, workspace, workspace_floats, num_cus, stream); break;
+      case EPI_F32: launch_bf16<EPI_F32>(A, W, e, M, N, K, workspace, workspace_floats, num_cus, stream); break;
+      default: launch_bf16<EPI_SWIGLU>(A, W, e, M, N, K, workspace, workspace_floats, num_cus, stream); break;
+    }
+  } else {
+    dim3 grid((N + 63) / 64, (M + 63) / 64), block(256);
+    const float* A = (const float*)x;
+    const float* W = (const float*)w;
+    switch (epilogue) {
+      case EPI_STORE: hipLaunchKernelGGL(gemm_f32_kernel<EPI_STORE>, grid, block, 0, stream, A, W, e, M, N, K); break;
+      case EPI_RESID: hipLaunchKernelGGL(gemm_f32_kernel<EPI_RESID>, grid, block, 0, stream, A, W, e, M, N, K); break;
+      case EPI_F32: hipLaunchKernelGGL(gemm_f32_kernel<EPI_F32>, grid, block, 0, stream, A, W, e, M, N, K); break;
+      default: hipLaunchKernelGGL(gemm_f32_kernel<EPI_SWIGLU>, grid, block, 0, stream, A, W, e, M, N, K); break;
+    }
+  }
+  LLMLAB_LAUNCH_CHECK("linear");
+  return 0;
+}

@@ -1,0 +1,132 @@
+// Token selection over float32 logits [rows, vocab]: greedy argmax and
+// temperature sampling by inverse CDF.  One block of 1024 threads per row; any
+// vocabulary size.  gfx950 only.
+//
+// argmax: the largest value, ties to the smallest index; NaN never wins; a row of
+// nothing but NaN gives -1 (the host turns that into an error).
+// sample: with temperature t <= 0 the argmax; else p = softmax(logits / t) in
+// float32 and the token is the smallest index whose cumulative sum reaches
+// u * total, u in [0, 1) given by the host (a seeded counter-based generator), so
+// a request's choices do not depend on the batch it ran in.  Each thread owns one
+// contiguous stretch of the row, so the cumulative sum has one fixed order.
+#include "common.h"
+
+constexpr int SAMPLE_THREADS = 1024;
+
+struct Best {
+  float v;
+  int i;
+};
+
+__device__ __forceinline__ Best better(Best a, Best b) {
+  // b replaces a if larger, or equal with a smaller index; i < 0 means "none yet"
+  if (b.i < 0) return a;
+  if (a.i < 0) return b;
+  if (b.v > a.v || (b.v == a.v && b.i < a.i)) return b;
+  return a;
+}
+
+__device__ Best block_argmax(const float* __restrict__ row, int vocab, float inv_t, Best* red) {
+  Best best{0.f, -1};
+  for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
+    const float v = row[i] * inv_t;
+    if (v != v) continue;  // NaN
+    best = better(best, Best{v, i});
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    Best o{__shfl_xor(best.v, off, WAVE), __shfl_xor(best.i, off, WAVE)};
+    best = better(best, o);
+  }
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  __syncthreads();
+  if (lane == 0) red[wave] = best;
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    Best t = red[0];
+    for (int w = 1; w < nw; ++w) t = better(t, red[w]);
+    red[16] = t;
+  }
+  __syncthreads();
+  return red[16];
+}
+
+__global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __restrict__ logits,
+                                                                 long row_stride, int vocab,
+                                                                 const float* __restrict__ temperature,
+                                                                 const float* __restrict__ uniform,
+                                                                 int* __restrict__ out) {
+  __shared__ Best red[17];
+  __shared__ float sums[SAMPLE_THREADS];
+  __shared__ float fred[17];
+  __shared__ int chosen;
+  const int b = blockIdx.x;
+  const float* row = logits + (size_t)b * row_stride;
+  const float t = temperature ? temperature[b] : 0.f;
+  if (!(t > 0.f)) {
+    const Best best = block_argmax(row, vocab, 1.f, red);
+    if (threadIdx.x == 0) out[b] = best.i;
+    return;
+  }
+  const float inv_t = 1.f / t;
+  const Best best = block_argmax(row, vocab, inv_t, red);
+  if (best.i < 0) {
+    if (threadIdx.x == 0) out[b] = -1;
+    return;
+  }
+  // contiguous stretch per thread
+  const int per = (vocab + blockDim.x - 1) / blockDim.x;
+  const int begin = min(vocab, (int)threadIdx.x * per), end = min(vocab, begin + per);
+  float mine = 0.f;
+  for (int i = begin; i < end; ++i) {
+    const float v = row[i] * inv_t;
+    if (v == v) mine += __expf(v - best.v);
+  }
+  sums[threadIdx.x] = mine;
+  if (threadIdx.x == 0) chosen = -1;
+  __syncthreads();
+  // thread 0 walks the 1024 partial sums: a fixed order
+  if (threadIdx.x == 0) {
+    float total = 0.f;
+    for (int i = 0; i < (int)blockDim.x; ++i) total += sums[i];
+    const float target = uniform[b] * total;
+    float run = 0.f;
+    int owner = -1;
+    for (int i = 0; i < (int)blockDim.x; ++i) {
+      if (sums[i] > 0.f) owner = i;                 // last non-empty stretch so far
+      if (run + sums[i] >= target && sums[i] > 0.f) { owner = i; break; }
+      run += sums[i];
+    }
+    fred[0] = target - run;   // what is left to cover inside the owner's stretch
+    chosen = owner;
+  }
+  __syncthreads();
+  if ((int)threadIdx.x == chosen) {
+    const float left = fred[0];
+    float run = 0.f;
+    int pick = -1, last = -1;
+    for (int i = begin; i < end; ++i) {
+      const float v = row[i] * inv_t;
+      if (!(v == v)) continue;
+      const float p = __expf(v - best.v);
+      if (p > 0.f) last = i;
+      run += p;
+      if (run >= left && p > 0.f) { pick = i; break; }
+    }
+    out[b] = pick >= 0 ? pick : (last >= 0 ? last : best.i);
+  }
+}
+
+extern "C" int llmlab_sample(const float* logits, long row_stride, int rows, int vocab,
+                             const float* temperature, const float* uniform, int* out,
+                             hipStream_t stream) {
+  LLMLAB_REQUIRE(rows >= 0 && vocab > 0 && row_stride >= vocab, "sample: bad sizes rows=%d vocab=%d",
+                 rows, vocab);
+  LLMLAB_REQUIRE(temperature == nullptr || uniform != nullptr,
+                 "sample: temperatures need uniform numbers");
+  if (rows == 0) return 0;
+  hipLaunchKernelGGL(sample_kernel, dim3(rows), dim3(SAMPLE_THREADS), 0, stream, logits, row_stride,
+                     vocab, temperature, uniform, out);
+  LLMLAB_LAUNCH_CHECK("sample");
+  return 0;
+}

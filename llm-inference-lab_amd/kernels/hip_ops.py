@@ -1,0 +1,316 @@
+"""The kernel set of the engine: thin, checked ctypes calls into the HIP
+libraries.  There is no other implementation on the product path: without a
+GPU, or if a library cannot be built or loaded, constructing ``HipOps`` raises.
+
+Every call checks on the host that dtypes, shapes, strides and devices are what
+the kernel and its grid assume before it launches anything; a size that the
+kernels do not take is refused with ``UnsupportedSizeError``.  Kernels run on
+the current PyTorch stream, so they can be captured into a HIP graph.
+"""
+from __future__ import annotations
+
+import ctypes
+from typing import Dict, Optional
+
+import torch
+
+from ..config.errors import UnsupportedSizeError
+from . import build
+
+DT_F32, DT_BF16 = 0, 1
+EPI_STORE, EPI_RESID, EPI_F32, EPI_SWIGLU = 0, 1, 2, 3
+
+_c_int, _c_long, _c_float, _c_size, _c_ptr = (ctypes.c_int, ctypes.c_long, ctypes.c_float,
+                                              ctypes.c_size_t, ctypes.c_void_p)
+
+
+def _dt(t: torch.Tensor) -> int:
+    if t.dtype == torch.float32:
+        return DT_F32
+    if t.dtype == torch.bfloat16:
+        return DT_BF16
+    raise TypeError(f"kernels take float32 or bfloat16 tensors, got {t.dtype}")
+
+
+class KernelError(RuntimeError):
+    pass
+
+
+class HipOps:
+    WORKSPACE_FLOATS = 16 * 1024 * 1024      # 64 MiB of float32 scratch (split partial sums)
+
+    def __init__(self, device="cuda:0"):
+        if not torch.cuda.is_available():
+            raise RuntimeError(
+                "no GPU is visible: the engine runs on hand-written HIP kernels for gfx950 "
+                "and has no CPU path")
+        self.device = torch.device(device)
+        if self.device.type != "cuda":
+            raise RuntimeError(f"the kernels need a GPU device, got '{device}'")
+        torch.cuda.set_device(self.device)
+        self._core = self._load(build.core_library())
+        self._declare_core()
+        if self._core.llmlab_abi_version() != 1:
+            raise RuntimeError("kernel library and Python bindings disagree on the interface")
+        self._attn: Dict[int, ctypes.CDLL] = {}
+        self.num_cus = int(torch.cuda.get_device_properties(self.device).multi_processor_count)
+        self.workspace = torch.empty(self.WORKSPACE_FLOATS, dtype=torch.float32, device=self.device)
+        self.loaded_libraries = [self._core._name]
+
+    # ---------------------------------------------------------------- loading
+    @staticmethod
+    def _load(path: str) -> ctypes.CDLL:
+        try:
+            return ctypes.CDLL(path)
+        except OSError as e:
+            raise RuntimeError(f"cannot load the kernel library {path}: {e}") from None
+
+    def _declare_core(self) -> None:
+        c = self._core
+        c.llmlab_last_error.restype = ctypes.c_char_p
+        c.llmlab_abi_version.restype = _c_int
+        c.llmlab_embed.argtypes = [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr]
+        c.llmlab_rmsnorm.argtypes = [_c_ptr, _c_ptr, _c_int, _c_float, _c_ptr, _c_int, _c_ptr, _c_int,
+                                     _c_int, _c_ptr]
+        c.llmlab_rope_kv_write.argtypes = [_c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
+                                           _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr,
+                                           _c_ptr, _c_ptr]
+        c.llmlab_rope_inplace.argtypes = [_c_ptr, _c_int, _c_int, _c_int, _c_int, _c_long, _c_long,
+                                          _c_ptr, _c_ptr, _c_ptr]
+        c.llmlab_linear.argtypes = [_c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_int, _c_int,
+                                    _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_size, _c_int, _c_ptr]
+        c.llmlab_sample.argtypes = [_c_ptr, _c_long, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr]
+        for fn in (c.llmlab_embed, c.llmlab_rmsnorm, c.llmlab_rope_kv_write, c.llmlab_rope_inplace,
+                   c.llmlab_linear, c.llmlab_sample):
+            fn.restype = _c_int
+
+    def _attention_lib(self, head_dim: int) -> ctypes.CDLL:
+        lib = self._attn.get(head_dim)
+        if lib is None:
+            lib = self._load(build.attention_library(head_dim))
+            lib.llmlab_last_error.restype = ctypes.c_char_p
+            lib.llmlab_attention_head_dim.restype = _c_int
+            if lib.llmlab_attention_head_dim() != head_dim:
+                raise RuntimeError(f"attention library for head size {head_dim} reports "
+                                   f"{lib.llmlab_attention_head_dim()}")
+            lib.llmlab_paged_attention.argtypes = [
+                _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr,
+                _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_float, _c_ptr, _c_int, _c_ptr, _c_size,
+                _c_int, _c_int, _c_ptr]
+            lib.llmlab_paged_attention.restype = _c_int
+            self._attn[head_dim] = lib
+            self.loaded_libraries.append(lib._name)
+        return lib
+
+    def check_attention_sizes(self, num_heads: int, num_kv_heads: int, head_dim: int, dtype) -> None:
+        if head_dim % 16 != 0 or not 16 <= head_dim <= 256:
+            raise UnsupportedSizeError(
+                f"attention kernels take head sizes that are multiples of 16 from 16 to 256, "
+                f"got {head_dim}")
+        if num_heads % num_kv_heads != 0:
+            raise UnsupportedSizeError(f"{num_heads} heads are not a multiple of {num_kv_heads} kv heads")
+        self._attention_lib(head_dim)
+
+    # ---------------------------------------------------------------- helpers
+    def _stream(self):
+        return _c_ptr(torch.cuda.current_stream(self.device).cuda_stream)
+
+    def _check(self, code: int, lib=None) -> None:
+        if code != 0:
+            msg = (lib or self._core).llmlab_last_error()
+            raise KernelError(msg.decode() if msg else f"kernel call failed with code {code}")
+
+    def _need(self, t: torch.Tensor, name: str, dtype=None, contiguous=True) -> torch.Tensor:
+        if t.device != self.device:
+            raise ValueError(f"{name} is on {t.device}, the kernels run on {self.device}")
+        if dtype is not None and t.dtype != dtype:
+            raise TypeError(f"{name} must be {dtype}, got {t.dtype}")
+        if contiguous and not t.is_contiguous():
+            raise ValueError(f"{name} must be contiguous")
+        return t
+
+    @staticmethod
+    def _ptr(t: Optional[torch.Tensor]):
+        return _c_ptr(t.data_ptr()) if t is not None else _c_ptr(0)
+
+    def synchronize(self) -> None:
+        torch.cuda.synchronize(self.device)
+
+    # ------------------------------------------------------------ elementwise
+    def embed(self, table, ids, out) -> None:
+        self._need(table, "embedding table")
+        self._need(ids, "token ids", torch.int32)
+        self._need(out, "embedding output", torch.float32)
+        rows, hidden = out.shape
+        if ids.numel() != rows or table.shape[1] != hidden:
+            raise ValueError(f"embed: ids {tuple(ids.shape)}, table {tuple(table.shape)}, "
+                             f"out {tuple(out.shape)} do not fit")
+        self._check(self._core.llmlab_embed(self._ptr(table), _dt(table), self._ptr(ids), self._ptr(out),
+                                            rows, hidden, table.shape[0], self._stream()))
+
+    def rmsnorm(self, x, weight, eps, out, rows=None) -> None:
+        self._need(x, "norm input", torch.float32)
+        self._need(weight, "norm weight")
+        self._need(out, "norm output")
+        hidden = x.shape[1]
+        n_out = out.shape[0]
+        if weight.numel() != hidden or out.shape[1] != hidden:
+            raise ValueError(f"rmsnorm: x {tuple(x.shape)}, weight {tuple(weight.shape)}, "
+                             f"out {tuple(out.shape)} do not fit")
+        if rows is None:
+            if n_out != x.shape[0]:
+                raise ValueError("rmsnorm: output rows differ from input rows")
+        else:
+            self._need(rows, "norm row indices", torch.int32)
+            if rows.numel() != n_out:
+                raise ValueError("rmsnorm: one row index per output row")
+        self._check(self._core.llmlab_rmsnorm(self._ptr(x), self._ptr(weight), _dt(weight), float(eps),
+                                              self._ptr(out), _dt(out), self._ptr(rows), n_out, hidden,
+                                              self._stream()))
+
+    # ----------------------------------------------------------------- linear
+    def _linear(self, x, w, out, bias, epilogue, n_out) -> None:
+        self._need(x, "linear input")
+        self._need(w, "linear weight")
+        if x.dtype != w.dtype:
+            raise TypeError(f"linear: input is {x.dtype} but the weight is {w.dtype}")
+        if out.device != self.device or out.stride(-1) != 1:
+            raise ValueError("linear: output must be on the GPU with unit column stride")
+        m, k = x.shape
+        n = w.shape[0]
+        if w.shape[1] != k or out.shape[0] != m or out.shape[1] != n_out:
+            raise ValueError(f"linear: x {tuple(x.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} "
+                             f"do not fit")
+        if x.dtype == torch.bfloat16 and k % 8 != 0:
+            raise UnsupportedSizeError(
+                f"bfloat16 matrix products need an inner size that is a multiple of 8, got {k}")
+        want_out = x.dtype if epilogue in (EPI_STORE, EPI_SWIGLU) else torch.float32
+        if out.dtype != want_out:
+            raise TypeError(f"linear: output must be {want_out}, got {out.dtype}")
+        if bias is not None:
+            self._need(bias, "linear bias")
+            if bias.numel() != n:
+                raise ValueError("linear: bias length differs from the output width")
+        ldo = out.stride(0) if m > 1 else max(out.stride(0), n_out)
+        self._check(self._core.llmlab_linear(
+            self._ptr(x), self._ptr(w), _dt(x), epilogue, self._ptr(out), self._ptr(bias),
+            _dt(bias) if bias is not None else 0, m, n, k, ldo, n_out, self._ptr(self.workspace),
+            self.workspace.numel(), self.num_cus, self._stream()))
+
+    def linear(self, x, w, out, bias=None) -> None:
+        self._linear(x, w, out, bias, EPI_STORE, w.shape[0])
+
+    def linear_residual(self, x, w, resid, bias=None) -> None:
+        self._linear(x, w, resid, bias, EPI_RESID, w.shape[0])
+
+    def linear_logits(self, x, w, out) -> None:
+        self._linear(x, w, out, None, EPI_F32, w.shape[0])
+
+    def linear_swiglu(self, x, w_gate_up, out) -> None:
+        inter = out.shape[1]
+        if w_gate_up.shape[0] != 2 * ((inter + 15) // 16 * 16):
+            raise ValueError(f"linear_swiglu: {w_gate_up.shape[0]} interleaved rows do not belong "
+                             f"to {inter} outputs")
+        self._linear(x, w_gate_up, out, None, EPI_SWIGLU, inter)
+
+    # ------------------------------------------------------------------- rope
+    def rope_inplace(self, x, positions, inv_freq) -> None:
+        rows, heads, d = x.shape
+        if x.stride(2) != 1:
+            raise ValueError("rope: the head dimension must be contiguous")
+        self._need(positions, "positions", torch.int32)
+        self._need(inv_freq, "rotary frequencies", torch.float32)
+        if inv_freq.numel() != d // 2 or positions.numel() < rows:
+            raise ValueError("rope: frequency table or positions do not fit")
+        self._check(self._core.llmlab_rope_inplace(
+            self._ptr(x), _dt(x), rows, heads, d, x.stride(0), x.stride(1), self._ptr(inv_freq),
+            self._ptr(positions), self._stream()))
+
+    def rope_kv_write(self, qkv, num_heads, num_kv_heads, head_dim, inv_freq, positions, row_req,
+                      block_table, page_size, k_cache, v_cache) -> None:
+        self._need(qkv, "qkv", contiguous=False)
+        rows = qkv.shape[0]
+        if qkv.stride(1) != 1 or qkv.shape[1] != (num_heads + 2 * num_kv_heads) * head_dim:
+            raise ValueError(f"rope_kv_write: qkv {tuple(qkv.shape)} does not hold {num_heads}+2*"
+                             f"{num_kv_heads} heads of {head_dim}")
+        self._need(positions, "positions", torch.int32)
+        if positions.numel() < rows:
+            raise ValueError("rope_kv_write: one position per row")
+        if inv_freq is not None:
+            self._need(inv_freq, "rotary frequencies", torch.float32)
+            if inv_freq.numel() != head_dim // 2:
+                raise ValueError("rope_kv_write: the frequency table must hold head_dim/2 entries")
+        table_stride = 0
+        if k_cache is not None:
+            self._need(row_req, "row -> request map", torch.int32)
+            self._need(block_table, "block table", torch.int32)
+            if row_req.numel() < rows:
+                raise ValueError("rope_kv_write: one request index per row")
+            pages = k_cache.shape[0]
+            if (tuple(k_cache.shape) != (pages, num_kv_heads, page_size, head_dim)
+                    or tuple(v_cache.shape) != (pages, num_kv_heads, head_dim, page_size)
+                    or not k_cache.is_contiguous() or not v_cache.is_contiguous()
+                    or k_cache.dtype != qkv.dtype or v_cache.dtype != qkv.dtype):
+                raise ValueError("rope_kv_write: cache tensors do not have the paged layout")
+            table_stride = block_table.stride(0)
+        self._check(self._core.llmlab_rope_kv_write(
+            self._ptr(qkv), _dt(qkv), rows, qkv.stride(0) if rows > 1 else qkv.shape[1], num_heads,
+            num_kv_heads, head_dim, self._ptr(inv_freq), self._ptr(positions), self._ptr(row_req),
+            self._ptr(block_table), table_stride, page_size, self._ptr(k_cache), self._ptr(v_cache),
+            self._stream()))
+
+    # -------------------------------------------------------------- attention
+    def paged_attention(self, qkv, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_table,
+                        page_size, q_start, start_pos, n_reqs, max_q_len, max_ctx_len, window, scale,
+                        out, ctx=None) -> None:
+        lib = self._attention_lib(head_dim)
+        rows = qkv.shape[0]
+        self._need(qkv, "queries", contiguous=False)
+        self._need(out, "attention output")
+        self._need(block_table, "block table", torch.int32)
+        self._need(q_start, "request row starts", torch.int32)
+        self._need(start_pos, "request start positions", torch.int32)
+        pages = k_cache.shape[0]
+        if (tuple(k_cache.shape) != (pages, num_kv_heads, page_size, head_dim)
+                or tuple(v_cache.shape) != (pages, num_kv_heads, head_dim, page_size)
+                or not k_cache.is_contiguous() or not v_cache.is_contiguous()):
+            raise ValueError("attention: cache tensors do not have the paged layout")
+        if not (qkv.dtype == out.dtype == k_cache.dtype == v_cache.dtype):
+            raise TypeError("attention: queries, cache and output must share one dtype")
+        if qkv.stride(1) != 1 or qkv.shape[1] < num_heads * head_dim:
+            raise ValueError("attention: the query rows are too narrow")
+        if tuple(out.shape) != (rows, num_heads * head_dim):
+            raise ValueError(f"attention: output {tuple(out.shape)} != ({rows}, {num_heads * head_dim})")
+        if q_start.numel() < n_reqs + 1 or start_pos.numel() < n_reqs or block_table.shape[0] < n_reqs:
+            raise ValueError("attention: request arrays are shorter than the number of requests")
+        if max_ctx_len > block_table.shape[1] * page_size:
+            raise ValueError("attention: the block table is too narrow for the longest context")
+        if page_size % 16 != 0:
+            raise UnsupportedSizeError(f"page size {page_size} is not a multiple of 16")
+        q_stride = qkv.stride(0) if rows > 1 else qkv.shape[1]
+        self._check(lib.llmlab_paged_attention(
+            self._ptr(qkv), _dt(qkv), q_stride, num_heads, num_kv_heads, self._ptr(k_cache),
+            self._ptr(v_cache), self._ptr(block_table), block_table.stride(0), page_size,
+            self._ptr(q_start), self._ptr(start_pos), n_reqs, max_q_len, max_ctx_len,
+            int(window) if window else 0, float(scale), self._ptr(out), out.stride(0) if rows > 1 else
+            out.shape[1], self._ptr(self.workspace), self.workspace.numel(), rows, self.num_cus,
+            self._stream()), lib)
+
+    # --------------------------------------------------------------- sampling
+    def argmax(self, logits, out) -> None:
+        self.sample(logits, None, None, out)
+
+    def sample(self, logits, temperatures, uniforms, out) -> None:
+        self._need(logits, "logits", torch.float32, contiguous=False)
+        self._need(out, "chosen tokens", torch.int32)
+        rows, vocab = logits.shape
+        if logits.stride(1) != 1 or out.numel() < rows:
+            raise ValueError("sample: logits rows must be contiguous and out must hold one token per row")
+        if temperatures is not None:
+            self._need(temperatures, "temperatures", torch.float32)
+            self._need(uniforms, "uniform numbers", torch.float32)
+            if temperatures.numel() < rows or uniforms.numel() < rows:
+                raise ValueError("sample: one temperature and one uniform number per row")
+        self._check(self._core.llmlab_sample(
+            self._ptr(logits), logits.stride(0) if rows > 1 else vocab, rows, vocab,
+            self._ptr(temperatures), self._ptr(uniforms), self._ptr(out), self._stream()))

@@ -115,21 +115,25 @@ class EmuOps:
         for b in range(n_reqs):
             r0, r1 = int(q_start[b]), int(q_start[b + 1])
             sp = int(start_pos[b])
+            end = sp + (r1 - r0)
+            # the request's positions, read through its block table (a freed or
+            # missing page reads as NaN, so a wrong access shows in the result)
+            keys = torch.full((end, num_kv_heads, head_dim), float("nan"))
+            vals = torch.full((end, num_kv_heads, head_dim), float("nan"))
+            for j in range(end):
+                pg = int(block_table[b, j // page_size])
+                if pg >= 0:
+                    keys[j] = k_cache[pg, :, j % page_size, :].float()
+                    vals[j] = v_cache[pg, :, :, j % page_size].float()
             for r in range(r0, r1):
                 p = sp + (r - r0)
                 lo = 0 if window is None else max(0, p - window + 1)
-                js = list(range(lo, p + 1))
-                pages = [int(block_table[b, j // page_size]) for j in js]
-                assert all(pg >= 0 for pg in pages), "read of a position without a page"
-                offs = [j % page_size for j in js]
                 q = qkv[r, :qs].float().view(num_heads, head_dim)
                 for h in range(num_heads):
                     kvh = h // group
-                    keys = torch.stack([k_cache[pg, kvh, o, :].float() for pg, o in zip(pages, offs)])
-                    vals = torch.stack([v_cache[pg, kvh, :, o].float() for pg, o in zip(pages, offs)])
-                    s = (keys @ q[h]) * scale
+                    s = (keys[lo:p + 1, kvh] @ q[h]) * scale
                     pr = torch.softmax(s, dim=0)
-                    out[r, h * head_dim:(h + 1) * head_dim] = (pr @ vals).to(out.dtype)
+                    out[r, h * head_dim:(h + 1) * head_dim] = (pr @ vals[lo:p + 1, kvh]).to(out.dtype)
 
     # --------------------------------------------------------------- sampling
     def argmax(self, logits, out):

@@ -1,0 +1,331 @@
+"""Each HIP kernel alone against its plain PyTorch reference (tests/emu_ops.py),
+at sizes other than the engine's: widths and vocabularies that are no power of
+two, partial tiles, every head size in steps of 16, odd group counts."""
+import math
+
+import pytest
+import torch
+
+from emu_ops import EmuOps
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from llm_inference_lab_amd.kernels.hip_ops import HipOps
+    return HipOps(DEV)
+
+
+@pytest.fixture(scope="module")
+def emu():
+    return EmuOps("cpu")
+
+
+def rnd(shape, dtype, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype)
+
+
+def close(got, want, dtype, what, scale=1.0):
+    got, want = got.float().cpu(), want.float().cpu()
+    # float32: rounding of sums in another order; bfloat16: one rounding of the result
+    tol = 2e-5 if dtype == torch.float32 else 1.0 / 128
+    bound = tol * max(1.0, scale)
+    err = (got - want).abs().max().item()
+    assert err <= bound, f"{what}: max abs error {err} > {bound}"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,hidden,vocab", [(1, 64, 256), (37, 896, 1000), (5, 100, 33)])
+def test_embed(ops, emu, dtype, rows, hidden, vocab):
+    table = rnd((vocab, hidden), dtype, 1)
+    ids = torch.randint(0, vocab, (rows,), generator=torch.Generator().manual_seed(2)).int()
+    ids[0] = vocab - 1
+    want = torch.empty(rows, hidden)
+    emu.embed(table, ids, want)
+    got = torch.empty(rows, hidden, device=DEV)
+    ops.embed(table.to(DEV), ids.to(DEV), got)
+    assert torch.equal(got.cpu(), want)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("wdtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,hidden,eps", [(1, 64, 1e-6), (19, 896, 1e-5), (7, 3584, 1e-6), (3, 100, 1e-3)])
+def test_rmsnorm(ops, emu, dtype, wdtype, rows, hidden, eps):
+    x = rnd((rows, hidden), torch.float32, 3, 3.0)
+    w = (1 + 0.1 * torch.randn(hidden, generator=torch.Generator().manual_seed(4))).to(wdtype)
+    want = torch.empty(rows, hidden, dtype=dtype)
+    emu.rmsnorm(x, w, eps, want)
+    got = torch.empty(rows, hidden, dtype=dtype, device=DEV)
+    ops.rmsnorm(x.to(DEV), w.to(DEV), eps, got)
+    close(got, want, dtype, "rmsnorm", 4.0)
+    # gathered rows
+    if rows > 2:
+        idx = torch.tensor([rows - 1, 0, rows - 2], dtype=torch.int32)
+        want = torch.empty(3, hidden, dtype=dtype)
+        emu.rmsnorm(x, w, eps, want, idx)
+        got = torch.empty(3, hidden, dtype=dtype, device=DEV)
+        ops.rmsnorm(x.to(DEV), w.to(DEV), eps, got, idx.to(DEV))
+        close(got, want, dtype, "rmsnorm gather", 4.0)
+
+
+LINEAR_SHAPES = [
+    (1, 96, 64), (5, 90, 96), (16, 1152, 896), (17, 65, 104), (33, 200, 64), (64, 896, 4864),
+    (65, 130, 72), (128, 896, 896), (200, 1152, 896), (300, 257, 136), (513, 384, 264),
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("m,n,k", LINEAR_SHAPES)
+def test_linear_bias(ops, emu, dtype, m, n, k):
+    x, w = rnd((m, k), dtype, 5), rnd((n, k), dtype, 6, 0.1)
+    for bias in (None, rnd((n,), torch.float32, 7), rnd((n,), torch.bfloat16, 8)):
+        if dtype == torch.float32 and bias is not None and bias.dtype == torch.bfloat16:
+            continue
+        want = torch.empty(m, n, dtype=dtype)
+        emu.linear(x, w, want, bias)
+        got = torch.empty(m, n, dtype=dtype, device=DEV)
+        ops.linear(x.to(DEV), w.to(DEV), got, None if bias is None else bias.to(DEV))
+        close(got, want, dtype, f"linear {m}x{n}x{k}", want.float().abs().max().item())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("m,n,k", LINEAR_SHAPES)
+def test_linear_residual_and_logits(ops, emu, dtype, m, n, k):
+    x, w = rnd((m, k), dtype, 9), rnd((n, k), dtype, 10, 0.1)
+    resid = rnd((m, n), torch.float32, 11)
+    want = resid.clone()
+    emu.linear_residual(x, w, want)
+    got = resid.clone().to(DEV)
+    ops.linear_residual(x.to(DEV), w.to(DEV), got)
+    close(got, want, torch.float32, f"linear_residual {m}x{n}x{k}", want.abs().max().item())
+    want = torch.empty(m, n)
+    emu.linear_logits(x, w, want)
+    got = torch.empty(m, n, device=DEV)
+    ops.linear_logits(x.to(DEV), w.to(DEV), got)
+    close(got, want, torch.float32, f"linear_logits {m}x{n}x{k}", want.abs().max().item())
+
+
+def test_linear_reference_vectors(ops):
+    """The closed-form vectors of the reference's own linear tests
+    (rust/engine/src/runner/model/qwen2/engine.rs:3574-3612): x = ((i*17 % 31) - 15)/32,
+    W = ((i*7 + part*11) % 29)/64 - 14/64, b = (i + part*7)/128, with partial tiles."""
+    for m, k, n in [(1, 96, 90), (5, 96, 90), (3, 96, 65)]:
+        i = torch.arange(m * k)
+        x = (((i * 17) % 31) - 15).float().view(m, k) / 32
+        j = torch.arange(n * k)
+        w = (((j * 7 + 11) % 29).float() / 64 - 14 / 64).view(n, k)
+        b = (torch.arange(n).float() + 7) / 128
+        want = x.double() @ w.double().t() + b.double()
+        got = torch.empty(m, n, device=DEV)
+        ops.linear(x.to(DEV), w.to(DEV), got, b.to(DEV))
+        assert (got.cpu().double() - want).abs().max().item() < 1e-4
+        # all these values are exact in bfloat16, so that path must agree after one rounding
+        gotb = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
+        ops.linear(x.bfloat16().to(DEV), w.bfloat16().to(DEV), gotb, b.to(DEV))
+        assert torch.equal(gotb.cpu(), want.float().bfloat16())
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("m,inter,k", [(1, 128, 64), (7, 320, 96), (16, 4864, 896), (40, 100, 72),
+                                       (64, 320, 96), (70, 136, 64), (260, 4864, 896), (150, 50, 40)])
+def test_linear_swiglu(ops, emu, dtype, m, inter, k):
+    from llm_inference_lab_amd.parts.feed_forward import interleave_gate_up
+    x = rnd((m, k), dtype, 12)
+    gate, up = rnd((inter, k), dtype, 13, 0.2), rnd((inter, k), dtype, 14, 0.2)
+    w = interleave_gate_up(gate, up)
+    want = torch.empty(m, inter, dtype=dtype)
+    emu.linear_swiglu(x, w, want)
+    # the interleaving itself, against the separate matrices
+    g = x.float() @ gate.float().t()
+    direct = g / (1 + torch.exp(-g)) * (x.float() @ up.float().t())
+    assert (want.float() - direct).abs().max() < 1e-2 * max(1.0, direct.abs().max().item())
+    got = torch.empty(m, inter, dtype=dtype, device=DEV)
+    ops.linear_swiglu(x.to(DEV), w.to(DEV), got)
+    close(got, want, dtype, f"linear_swiglu {m}x{inter}x{k}", want.float().abs().max().item())
+
+
+def make_cache(num_pages, nkv, page, d, dtype, seed):
+    k = rnd((num_pages, nkv, page, d), dtype, seed)
+    v = rnd((num_pages, nkv, d, page), dtype, seed + 1)
+    return k, v
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nq,nkv,d,page", [(4, 2, 16, 16), (3, 1, 32, 32), (14, 2, 64, 64), (6, 3, 48, 16),
+                                           (8, 8, 128, 64)])
+def test_rope_kv_write(ops, emu, dtype, nq, nkv, d, page):
+    rows_per, reqs, num_pages = [5, 1, 9], 3, 12
+    starts = [3, 40, 0]
+    rows = sum(rows_per)
+    qkv = rnd((rows, (nq + 2 * nkv) * d), dtype, 20)
+    positions = torch.cat([torch.arange(s, s + n) for s, n in zip(starts, rows_per)]).int()
+    row_req = torch.cat([torch.full((n,), b) for b, n in enumerate(rows_per)]).int()
+    table = torch.full((reqs, 8), -1, dtype=torch.int32)
+    perm = torch.randperm(num_pages, generator=torch.Generator().manual_seed(21)).int()
+    at = 0
+    for b in range(reqs):
+        need = (starts[b] + rows_per[b] + page - 1) // page
+        table[b, :need] = perm[at:at + need]
+        at += need
+    theta = 1e6
+    inv_freq = (1.0 / (theta ** (torch.arange(0, d, 2, dtype=torch.float64) / d))).float()
+    kc, vc = make_cache(num_pages, nkv, page, d, dtype, 22)
+    want_qkv, want_k, want_v = qkv.clone(), kc.clone(), vc.clone()
+    emu.rope_kv_write(want_qkv, nq, nkv, d, inv_freq, positions, row_req, table, page, want_k, want_v)
+    got_qkv, got_k, got_v = qkv.to(DEV), kc.to(DEV), vc.to(DEV)
+    ops.rope_kv_write(got_qkv, nq, nkv, d, inv_freq.to(DEV), positions.to(DEV), row_req.to(DEV),
+                      table.to(DEV), page, got_k, got_v)
+    close(got_qkv[:, :nq * d], want_qkv[:, :nq * d], dtype, "rope q", 4.0)
+    close(got_k, want_k, dtype, "key cache", 4.0)
+    close(got_v, want_v, dtype, "value cache", 4.0)
+    # untouched places of the cache stay bit-identical
+    untouched = (want_k == kc)
+    assert torch.equal(got_k.cpu()[untouched], kc[untouched])
+
+
+def run_attention(ops, emu, dtype, nq, nkv, d, page, window, reqs_spec, seed=30, scale=None, amplify=None):
+    """reqs_spec: list of (start_pos, q_len)."""
+    reqs = len(reqs_spec)
+    rows = sum(n for _, n in reqs_spec)
+    max_ctx = max(s + n for s, n in reqs_spec)
+    pages_per = (max_ctx + page - 1) // page
+    num_pages = reqs * pages_per + 3
+    qkv = rnd((rows, (nq + 2 * nkv) * d), dtype, seed)
+    kc, vc = make_cache(num_pages, nkv, page, d, dtype, seed + 1)
+    perm = torch.randperm(num_pages, generator=torch.Generator().manual_seed(seed + 2)).int()
+    table = torch.full((reqs, pages_per), -1, dtype=torch.int32)
+    q_start, start_pos = [0], []
+    at = 0
+    for b, (s, n) in enumerate(reqs_spec):
+        need = (s + n + page - 1) // page
+        table[b, :need] = perm[at:at + need]
+        at += need
+        q_start.append(q_start[-1] + n)
+        start_pos.append(s)
+    if amplify is not None:
+        # one far key stands out: scale query and that key so its score dominates
+        b, key_pos, factor = amplify
+        pg, off = int(table[b, key_pos // page]), key_pos % page
+        kc[pg, :, off, :] *= factor
+    # positions past each request's end hold garbage that must not leak in
+    for b, (s, n) in enumerate(reqs_spec):
+        end = s + n
+        if end % page:
+            pg = int(table[b, end // page])
+            kc[pg, :, end % page:, :] = 1e4
+            vc[pg, :, :, end % page:] = -1e4
+    q_start_t = torch.tensor(q_start, dtype=torch.int32)
+    start_pos_t = torch.tensor(start_pos, dtype=torch.int32)
+    scale = scale if scale is not None else 1 / math.sqrt(d)
+    want = torch.zeros(rows, nq * d, dtype=dtype)
+    emu.paged_attention(qkv, nq, nkv, d, kc, vc, table, page, q_start_t, start_pos_t, reqs,
+                        max(n for _, n in reqs_spec), max_ctx, window, scale, want)
+    got = torch.zeros(rows, nq * d, dtype=dtype, device=DEV)
+    ops.paged_attention(qkv.to(DEV), nq, nkv, d, kc.to(DEV), vc.to(DEV), table.to(DEV), page,
+                        q_start_t.to(DEV), start_pos_t.to(DEV), reqs, max(n for _, n in reqs_spec),
+                        max_ctx, window, scale, got)
+    tol = 2e-5 if dtype == torch.float32 else 2e-2
+    err = (got.float().cpu() - want.float()).abs().max().item()
+    assert err <= tol * max(1.0, want.float().abs().max().item()), f"attention error {err}"
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("d", [16, 32, 48, 64, 80, 96, 112, 128])
+def test_attention_head_sizes(ops, emu, dtype, d):
+    run_attention(ops, emu, dtype, 4, 2, d, 16, None, [(0, 37), (21, 1), (5, 12)])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("nq,nkv", [(3, 1), (14, 2), (7, 7), (5, 1), (40, 8), (20, 1)])
+def test_attention_groups(ops, emu, dtype, nq, nkv):
+    run_attention(ops, emu, dtype, nq, nkv, 32, 32, None, [(0, 50), (63, 1), (10, 3)])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("length", [31, 32, 33, 63, 64, 65, 127, 129, 513])
+def test_attention_decode_lengths(ops, emu, dtype, length):
+    """One decoded token over `length` cached keys (the lengths of the reference's
+    attention tests, rust/engine/src/runner/model/qwen2/engine.rs:3209-3435)."""
+    run_attention(ops, emu, dtype, 14, 2, 64, 64, None, [(length - 1, 1)])
+    run_attention(ops, emu, dtype, 4, 2, 64, 16, None, [(length - 1, 1), (7, 1)])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("window", [1, 5, 24, 64, 1000])
+def test_attention_window(ops, emu, dtype, window):
+    run_attention(ops, emu, dtype, 3, 1, 32, 16, window, [(0, 70), (100, 1), (33, 9)])
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_attention_far_key_among_hundreds(ops, emu, dtype):
+    """A single far key carries the whole answer: a kernel that skips, repeats or
+    mis-places a key block cannot hide behind averaged random values."""
+    run_attention(ops, emu, dtype, 4, 2, 64, 64, None, [(900, 1)], amplify=(0, 3, 30.0))
+    run_attention(ops, emu, dtype, 4, 2, 64, 16, None, [(0, 700)], amplify=(0, 130, 30.0))
+    run_attention(ops, emu, dtype, 14, 2, 64, 64, None, [(4000, 1), (2000, 1)], amplify=(1, 1999, 30.0))
+
+
+@pytest.mark.parametrize("vocab", [1, 255, 256, 257, 4095, 4097, 151936])
+def test_argmax(ops, emu, vocab):
+    """Vocabulary sizes and special rows of the reference's argmax tests
+    (rust/engine/src/runner/model/qwen2/engine.rs:2285-2358)."""
+    g = torch.Generator().manual_seed(vocab)
+    logits = torch.randn(5, vocab, generator=g)
+    logits[1, vocab - 1] = 100.0                      # maximum at the last index
+    if vocab > 300:
+        logits[2, 7] = logits[2, 290] = 50.0          # tie across threads: smallest index
+    logits[3, :] = float("-inf")                      # all -inf: index 0
+    logits[4, :] = float("nan")                       # all NaN: -1
+    want = torch.zeros(5, dtype=torch.int32)
+    emu.argmax(logits, want)
+    got = torch.zeros(5, dtype=torch.int32, device=DEV)
+    ops.argmax(logits.to(DEV), got)
+    assert got.cpu().tolist() == want.tolist()
+    assert want[1] == vocab - 1 and want[3] == 0 and want[4] == -1
+    if vocab > 300:
+        assert want[2] == 7
+
+
+def test_sample_temperature(ops, emu):
+    vocab = 1000
+    g = torch.Generator().manual_seed(5)
+    logits = torch.randn(64, vocab, generator=g) * 3
+    temps = torch.full((64,), 0.8)
+    temps[:4] = 0.0
+    u = torch.rand(64, generator=g)
+    got = torch.zeros(64, dtype=torch.int32, device=DEV)
+    ops.sample(logits.to(DEV), temps.to(DEV), u.to(DEV), got)
+    got = got.cpu()
+    for b in range(64):
+        if temps[b] == 0:
+            assert got[b] == logits[b].argmax()
+            continue
+        p = torch.softmax(logits[b].double() / 0.8, dim=0)
+        cdf = torch.cumsum(p, dim=0)
+        t = int(got[b])
+        lo = 0.0 if t == 0 else float(cdf[t - 1])
+        assert lo - 1e-4 <= float(u[b]) <= float(cdf[t]) + 1e-4, (b, t, lo, float(u[b]), float(cdf[t]))
+    # a 4-token vocabulary: the histogram of many draws follows softmax(logits / t)
+    small = torch.tensor([[1.0, 0.0, -1.0, 2.0]]).repeat(4096, 1)
+    u = torch.rand(4096, generator=g)
+    out = torch.zeros(4096, dtype=torch.int32, device=DEV)
+    ops.sample(small.to(DEV), torch.full((4096,), 0.5).to(DEV), u.to(DEV), out)
+    hist = torch.bincount(out.cpu().long(), minlength=4).double() / 4096
+    want = torch.softmax(small[0].double() / 0.5, dim=0)
+    assert (hist - want).abs().max() < 0.03
+
+
+def test_refused_sizes(ops):
+    from llm_inference_lab_amd.config.errors import UnsupportedSizeError
+    with pytest.raises(UnsupportedSizeError):
+        ops.check_attention_sizes(4, 2, 24, torch.bfloat16)
+    with pytest.raises(UnsupportedSizeError):
+        ops.check_attention_sizes(4, 2, 272, torch.bfloat16)
+    x = torch.zeros(2, 100, dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros(8, 100, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(UnsupportedSizeError):
+        ops.linear(x, w, torch.zeros(2, 8, dtype=torch.bfloat16, device=DEV))
