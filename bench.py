@@ -1,0 +1,156 @@
+"""Decode and prefill throughput of the engine on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--context S] [--layers L]
+
+Default: the layer sizes of the Qwen2.5-0.5B shape with seeded random weights,
+batch 8, context 4096, bfloat16.  A "step" is one decode step of the whole
+batch through the scheduler's own path (step function + sampling, tokens fed
+back).  One JSON line is printed: decoded tokens a second as ``value``, plus
+``prefill`` (one 2,048-token prompt), ``roofline`` (bytes the decode step has to
+read over its time against 8 TB/s) and ``points`` (decode at batch 1 and 64).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+PEAK_FLOPS = {"bf16": 2.5e15, "f32": 157.3e12}
+MODEL = dict(
+    architectures=["Qwen2ForCausalLM"], model_type="qwen2", vocab_size=151936, hidden_size=896,
+    intermediate_size=4864, num_hidden_layers=24, num_attention_heads=14, num_key_value_heads=2,
+    head_dim=64, rms_norm_eps=1e-6, rope_theta=1e6, max_position_embeddings=32768,
+    tie_word_embeddings=True, use_sliding_window=False)
+FULL_LAYERS = MODEL["num_hidden_layers"]
+
+
+def prefill_flops(cfg, tokens):
+    h, i, v = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
+    q, kv = cfg.num_attention_heads * cfg.head_dim, cfg.num_key_value_heads * cfg.head_dim
+    per_token_layer = 2 * (h * (q + 2 * kv) + q * h + 3 * h * i)
+    attention_layer = 4 * (tokens * (tokens + 1) // 2) * q
+    return cfg.num_hidden_layers * (tokens * per_token_layer + attention_layer) + 2 * h * v
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=64)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=4096)
+    ap.add_argument("--layers", type=int, default=FULL_LAYERS)
+    ap.add_argument("--dtype", default="bf16", choices=["bf16", "f32"])
+    ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--no-points", action="store_true", help="skip batch 1 / 64 and the prefill")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
+        sys.exit(2)
+
+    import torch
+    import llm_inference_lab_amd as lab
+    from llm_inference_lab_amd.engine.step import StepEntry
+    from llm_inference_lab_amd.sampling import SamplingConfig
+
+    raw = dict(MODEL, num_hidden_layers=args.layers)
+    cfg = lab.Qwen2Config.from_dict(raw)
+    batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
+    max_batch = max(batches)
+    page = 64
+    context = args.context
+    engine = lab.Engine(config=cfg, seed=0, dtype=args.dtype, device="cuda:0", page_size=page,
+                        max_cache_tokens=max_batch * (context + page), max_requests=max_batch,
+                        max_batch_tokens=2048, max_seq_len=context + page, graph=not args.no_graph)
+    gen = torch.Generator().manual_seed(1234)
+
+    def random_ids(n):
+        return torch.randint(0, cfg.vocab_size, (n,), generator=gen).tolist()
+
+    def sync():
+        torch.cuda.synchronize()
+
+    def decode_run(batch, steps, warmup):
+        """Requests with (context - steps - warmup) cached tokens decode to `context`."""
+        prompt_len = context - steps - warmup - 1
+        sched = engine.scheduler(max_batch_tokens=2048)
+        never = cfg.vocab_size  # no token ends a request: a fixed number of outputs, as the reference's bench
+        for b in range(batch):
+            sched.add_request(random_ids(prompt_len),
+                              SamplingConfig(max_new_tokens=steps + warmup + 1, eos_token_id=[]))
+        while any(not r.decoding for r in sched.active) or sched.waiting:
+            sched.step()                      # prefill in portions; ends with every request decoding
+        for _ in range(warmup):
+            sched.step()
+        live_tokens = sum(r.computed for r in sched.active)
+        sync()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            sched.step()
+        sync()
+        seconds = time.perf_counter() - t0
+        live_tokens = (live_tokens + sum(r.computed for r in sched.active)) / 2
+        sched.run()
+        assert engine.cache.live_requests == 0
+        return seconds, live_tokens
+
+    seconds, live_tokens = decode_run(args.batch, args.steps, args.warmup)
+    ms_per_step = seconds / args.steps * 1e3
+    value = args.batch * args.steps / seconds
+    step_bytes = engine.weight_bytes_per_step() + live_tokens * engine.cache.bytes_per_token()
+    achieved = step_bytes / (seconds / args.steps) / 1e9
+
+    result = {
+        "metric": "decode_tokens_per_second", "value": round(value, 1), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": args.dtype, "data": "synthetic",
+        "config": {
+            "model": "Qwen2.5-0.5B shape, random weights", "global_batch": args.batch,
+            "seq_len": context, "parallelism": "single GPU", "layers": args.layers,
+            "layers_of_full_model": FULL_LAYERS, "hidden_size": cfg.hidden_size,
+            "num_attention_heads": cfg.num_attention_heads,
+            "num_key_value_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
+            "intermediate_size": cfg.intermediate_size, "vocab_size": cfg.vocab_size,
+            "tie_word_embeddings": cfg.tie_word_embeddings, "page_size": page,
+            "hip_graph_decode": not args.no_graph, "weights_seed": 0,
+        },
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+                     "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4)},
+    }
+    if not args.no_points:
+        # prefill: one prompt of 2,048 tokens in one step, logits at its last place
+        tokens = 2048
+        times = []
+        for _ in range(4):
+            req = engine.open("prefill")
+            ids = random_ids(tokens)
+            sync()
+            t0 = time.perf_counter()
+            engine.step([StepEntry(req, ids, [tokens - 1])])
+            sync()
+            times.append(time.perf_counter() - t0)
+            engine.close(req)
+        best = min(times[1:])
+        flops = prefill_flops(cfg, tokens)
+        result["prefill"] = {"value": round(tokens / best, 1), "tokens": tokens,
+                             "ms": round(best * 1e3, 3),
+                             "frac": round(flops / best / PEAK_FLOPS[args.dtype], 4)}
+        points = {}
+        for b in (1, 64):
+            if b == args.batch:
+                points[f"decode_b{b}"] = round(value, 1)
+                continue
+            s, _ = decode_run(b, max(8, args.steps // 2), max(2, args.warmup // 2))
+            points[f"decode_b{b}"] = round(b * max(8, args.steps // 2) / s, 1)
+        result["points"] = points
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

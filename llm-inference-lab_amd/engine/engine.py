@@ -55,11 +55,9 @@ class Engine:
                  dtype="bf16", device: str = "cuda:0", ops=None, page_size: int = 64,
                  max_cache_tokens: Optional[int] = None, num_pages: Optional[int] = None,
                  max_requests: int = 64, max_batch_tokens: int = 512,
-                 max_seq_len: Optional[int] = None, tensors=None,
+                 max_seq_len: Optional[int] = None, tensors=None, graph: bool = False,
                  progress: Optional[Callable[[str], None]] = None):
         self.dtype = parse_dtype(dtype)
-        self.ops = ops if ops is not None else default_ops(device)
-        self.device = self.ops.device
         if model_dir is not None:
             self.architecture, self.config = read_config(model_dir)
         elif config is not None:
@@ -68,6 +66,15 @@ class Engine:
         else:
             raise ValueError("give a model_dir or a config")
         self.spec = self.architecture.build_spec(self.config)
+        if ops is None:
+            # compile what this model needs before the GPU is first touched
+            from ..kernels import build
+            build.core_library()
+            for dim in sorted({b.mixer.params["head_dim"] for b in self.spec.blocks
+                               if "head_dim" in b.mixer.params}):
+                build.attention_library(int(dim))
+        self.ops = ops if ops is not None else default_ops(device)
+        self.device = self.ops.device
         self.model = CausalLM(self.spec)
         expected = self.model.tensor_specs()
         if model_dir is not None:
@@ -95,7 +102,10 @@ class Engine:
         self.cache = CacheManager(groups, self.page_size, self.max_requests, self.max_seq_len,
                                   state_specs, self.dtype, self.device)
         self.model.attach_cache(self.cache)
-        self.step_fn = StepFunction(self.model, self.cache, self.ops, self.max_batch_tokens)
+        self.step_fn = StepFunction(self.model, self.cache, self.ops, self.max_batch_tokens,
+                                    graph=graph)
+        self._sampler = None
+        self.last_scheduler = None
 
     # ------------------------------------------------------------- requests
     def open(self, request_id) -> RequestCache:
@@ -108,6 +118,42 @@ class Engine:
 
     def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
         return self.step_fn(entries)
+
+    # ------------------------------------------------------------ generation
+    def scheduler(self, max_batch_tokens: Optional[int] = None, on_token=None, trace=None):
+        """A scheduler over this engine (continuous batching, chunked prefill)."""
+        from ..sampling.sampler import Sampler
+        from .scheduler import Scheduler
+        if self._sampler is None:
+            self._sampler = Sampler(self.ops, self.max_requests)
+        return Scheduler(self, self._sampler, max_batch_tokens or self.max_batch_tokens,
+                         on_token=on_token, trace=trace)
+
+    def generate(self, prompts: Sequence[Sequence[int]], max_new_tokens: int = 8,
+                 temperature: Optional[float] = None, seed: int = 0, eos_token_id=None,
+                 sampling=None, max_batch_tokens: Optional[int] = None, on_token=None,
+                 trace=None) -> List[List[int]]:
+        """Token ids in, generated token ids out, one list per prompt.  ``sampling``
+        (one ``SamplingConfig`` or one per prompt) overrides the scalar options; the
+        i-th prompt draws from the random stream ``seed + i``.  A request that the
+        scheduler refuses raises its error here."""
+        from ..sampling.params import SamplingConfig
+        sched = self.scheduler(max_batch_tokens, on_token, trace)
+        ids = []
+        for i, prompt in enumerate(prompts):
+            if sampling is None:
+                cfg = SamplingConfig(temperature=temperature, max_new_tokens=max_new_tokens,
+                                     eos_token_id=eos_token_id, seed=seed + i,
+                                     do_sample=None if temperature is None else temperature > 0)
+            else:
+                cfg = sampling[i] if isinstance(sampling, (list, tuple)) else sampling
+            ids.append(sched.add_request(prompt, cfg))
+        done = sched.run()
+        self.last_scheduler = sched
+        for i in ids:
+            if done[i].error is not None:
+                raise done[i].error
+        return [list(done[i].generated) for i in ids]
 
     # ------------------------------------------------------------------ info
     def weight_bytes_per_step(self) -> int:

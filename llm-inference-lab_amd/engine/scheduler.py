@@ -1,0 +1,273 @@
+"""The scheduler: admits requests, cuts prompts into portions under a token
+budget, decodes, finishes and frees.
+
+Decisions, all taken from the reference's Runner and its batch policy:
+
+* Admission (rust/engine/src/runner/model_runner.rs:577-694): a request is
+  refused if its prompt is empty, a token id is outside the vocabulary, or
+  ``prompt + max_new_tokens - 1`` exceeds the longest sequence the cache takes.
+  Otherwise it is admitted when a request row is free and every cache group has
+  pages for the WHOLE turn (prompt and all generated tokens but the last) on top
+  of what the active requests are still promised.  So pages never run out in the
+  middle of a request.
+* When pages are short (model_runner.rs:745-756): the request waits while others
+  are active and is tried again every step; requests behind it that fit are
+  admitted meanwhile.  If nothing is active and it still does not fit, it fails
+  with ``CapacityExhausted``.  No preemption, no swapping, no recomputation.
+* The step's plan (rust/engine/src/runner/model_runner/batch_policy.rs:36-88):
+  every decoding request gets one token first (at most ``max_batch_tokens`` of
+  them); what is left of the budget goes to prompts in order of admission, each
+  ``min(rest of the prompt, budget left)``; a request that gets nothing sits
+  the step out.  A request decodes once it has produced a token; the last
+  portion of a prompt, however short, is still prefill.
+* Only a portion that ends the prompt yields a token (model_runner.rs:825);
+  the end-of-sequence token counts as generated and is kept
+  (model_runner.rs:280-321); a request ends at end-of-sequence or at its budget
+  and gives its pages and its row back before the next step.
+"""
+from __future__ import annotations
+
+import collections
+import dataclasses
+import time
+from typing import Callable, Deque, Dict, List, Optional, Sequence, Tuple
+
+from ..sampling.params import SamplingConfig
+from .step import StepEntry
+
+
+class CapacityExhausted(RuntimeError):
+    """The cache cannot hold the request even with nothing else running."""
+
+
+@dataclasses.dataclass
+class Request:
+    request_id: int
+    prompt: List[int]
+    sampling: SamplingConfig
+    tokens: List[int] = dataclasses.field(default_factory=list)     # prompt + generated
+    generated: List[int] = dataclasses.field(default_factory=list)
+    cache: object = None
+    remaining: int = 0
+    promised_pages: List[int] = dataclasses.field(default_factory=list)
+    error: Optional[Exception] = None
+    finish_reason: Optional[str] = None        # "eos", "length", "error"
+    arrival: float = 0.0
+    first_token_time: Optional[float] = None
+    finish_time: Optional[float] = None
+
+    @property
+    def finished(self) -> bool:
+        return self.finish_reason is not None
+
+    @property
+    def decoding(self) -> bool:
+        return len(self.generated) > 0
+
+    @property
+    def computed(self) -> int:
+        return self.cache.computed_len if self.cache is not None else 0
+
+
+@dataclasses.dataclass
+class Planned:
+    request: Request
+    count: int              # tokens of this step
+    yields_token: bool      # the portion ends the request's known tokens
+
+
+def plan_step(active: Sequence[Request], max_batch_tokens: int) -> List[Planned]:
+    """Decode first, then prompts in order, under one token budget."""
+    runnable = [r for r in active if not r.finished and r.remaining > 0]
+    decode_budget = min(sum(1 for r in runnable if r.decoding), max_batch_tokens)
+    prefill_budget = max_batch_tokens - decode_budget
+    plan: List[Planned] = []
+    for r in runnable:
+        ready = r.computed
+        if r.decoding:
+            if decode_budget == 0:
+                continue
+            decode_budget -= 1
+            count = 1
+        else:
+            if prefill_budget == 0:
+                continue
+            count = min(len(r.tokens) - ready, prefill_budget)
+            prefill_budget -= count
+        plan.append(Planned(r, count, ready + count == len(r.tokens)))
+    return plan
+
+
+class Scheduler:
+    """Continuous batching over an engine's step function.
+
+    ``engine`` needs: ``step(entries) -> logits``, ``cache`` (a ``CacheManager``),
+    ``open(id)``, ``close(request_cache)``, ``spec`` (vocab_size, eos_token_ids),
+    ``max_seq_len``.  ``sampler.sample(logits, temperatures, seeds, counters)``
+    picks the tokens."""
+
+    def __init__(self, engine, sampler, max_batch_tokens: Optional[int] = None,
+                 on_token: Optional[Callable[[Request, int], None]] = None,
+                 trace: Optional[Callable[[dict], None]] = None):
+        self.engine = engine
+        self.sampler = sampler
+        self.max_batch_tokens = int(max_batch_tokens or engine.max_batch_tokens)
+        if self.max_batch_tokens <= 0:
+            raise ValueError("max_batch_tokens must be positive")
+        self.waiting: Deque[Request] = collections.deque()
+        self.active: List[Request] = []
+        self.finished: Dict[int, Request] = {}
+        self._next_id = 0
+        self.on_token = on_token
+        self.trace = trace
+        self.steps = 0
+        self.step_log: List[List[Tuple[int, int]]] = []     # per step: (request id, tokens)
+        self.keep_step_log = False
+
+    # ---------------------------------------------------------------- ingress
+    def add_request(self, prompt: Sequence[int], sampling: Optional[SamplingConfig] = None) -> int:
+        request = Request(self._next_id, [int(t) for t in prompt], sampling or SamplingConfig(),
+                          arrival=time.perf_counter())
+        self._next_id += 1
+        request.tokens = list(request.prompt)
+        request.remaining = request.sampling.new_tokens
+        self.waiting.append(request)
+        return request.request_id
+
+    # -------------------------------------------------------------- admission
+    def _promised(self) -> List[int]:
+        """Pages per group that active requests may still take."""
+        cache = self.engine.cache
+        owed = [0] * len(cache.groups)
+        for r in self.active:
+            for g in range(len(cache.groups)):
+                held = sum(1 for p in r.cache.pages[g] if p >= 0)
+                owed[g] += max(0, r.promised_pages[g] - held)
+        return owed
+
+    def _refusal(self, r: Request) -> Optional[Exception]:
+        try:
+            r.sampling.validate()
+        except ValueError as e:
+            return e
+        if not r.prompt:
+            return ValueError("empty prompt")
+        vocab = self.engine.spec.vocab_size
+        for t in r.prompt:
+            if not 0 <= t < vocab:
+                return ValueError(f"token id {t} is outside the vocabulary of {vocab}")
+        end = len(r.prompt) + max(0, r.remaining - 1)
+        if end > self.engine.max_seq_len:
+            return ValueError(f"generation to {end} tokens exceeds the cache's longest "
+                              f"sequence {self.engine.max_seq_len}")
+        return None
+
+    def _fits(self, r: Request) -> Tuple[bool, List[int]]:
+        cache = self.engine.cache
+        end = len(r.prompt) + max(0, r.remaining - 1)
+        need = cache.page_need(end, self.max_batch_tokens)
+        if cache.free_rows == 0:
+            return False, need
+        owed = self._promised()
+        for g in range(len(cache.groups)):
+            if need[g] > cache.free_pages(g) - owed[g]:
+                return False, need
+        return True, need
+
+    def _admit(self) -> None:
+        still_waiting: Deque[Request] = collections.deque()
+        while self.waiting:
+            r = self.waiting.popleft()
+            refusal = self._refusal(r)
+            if refusal is not None:
+                self._finish(r, "error", refusal)
+                continue
+            if r.remaining == 0:
+                self._finish(r, "length")
+                continue
+            fits, need = self._fits(r)
+            if fits:
+                r.cache = self.engine.open(("request", r.request_id))
+                r.promised_pages = need
+                self.active.append(r)
+            elif self.active:
+                still_waiting.append(r)
+            else:
+                self._finish(r, "error", CapacityExhausted(
+                    f"insufficient cache capacity for request {r.request_id}: it needs {need} "
+                    f"pages per group"))
+        self.waiting = still_waiting
+
+    # ------------------------------------------------------------------- step
+    def step(self) -> List[Request]:
+        """Admit, plan, run one step, sample, finish.  Returns the requests that
+        finished in this call."""
+        before = set(self.finished)
+        self._admit()
+        plan = plan_step(self.active, self.max_batch_tokens)
+        if plan:
+            entries = []
+            for p in plan:
+                start = p.request.computed
+                entries.append(StepEntry(p.request.cache, p.request.tokens[start:start + p.count],
+                                         [p.count - 1] if p.yields_token else []))
+            t0 = time.perf_counter()
+            logits = self.engine.step(entries)
+            yielding = [p.request for p in plan if p.yields_token]
+            if yielding:
+                tokens = self.sampler.sample(
+                    logits, [r.sampling.effective_temperature for r in yielding],
+                    [r.sampling.seed for r in yielding], [len(r.generated) for r in yielding])
+                now = time.perf_counter()
+                for r, token in zip(yielding, tokens):
+                    self._accept(r, token, now)
+            self.steps += 1
+            if self.keep_step_log:
+                self.step_log.append([(p.request.request_id, p.count) for p in plan])
+            if self.trace is not None:
+                self.trace({"event": "step_completed", "step": self.steps,
+                            "phase": "decode" if all(p.request.decoding and p.count == 1 for p in plan)
+                            else "prefill",
+                            "requests": len(plan), "tokens": sum(p.count for p in plan),
+                            "seconds": time.perf_counter() - t0})
+        for r in [r for r in self.active if r.finished]:
+            self._release(r)
+        return [self.finished[i] for i in self.finished if i not in before]
+
+    def _accept(self, r: Request, token: int, now: float) -> None:
+        r.generated.append(token)
+        r.tokens.append(token)
+        r.remaining -= 1
+        if r.first_token_time is None:
+            r.first_token_time = now
+        if self.on_token is not None:
+            self.on_token(r, token)
+        eos = r.sampling.eos_ids(self.engine.spec.eos_token_ids)
+        if token in eos:
+            r.remaining = 0
+            r.finish_reason = "eos"
+        elif r.remaining == 0:
+            r.finish_reason = "length"
+
+    def _release(self, r: Request) -> None:
+        self.active.remove(r)
+        if r.cache is not None:
+            self.engine.close(r.cache)
+            r.cache = None
+        r.finish_time = time.perf_counter()
+        self.finished[r.request_id] = r
+
+    def _finish(self, r: Request, reason: str, error: Optional[Exception] = None) -> None:
+        r.finish_reason, r.error, r.remaining = reason, error, 0
+        r.finish_time = time.perf_counter()
+        self.finished[r.request_id] = r
+
+    @property
+    def idle(self) -> bool:
+        return not self.waiting and not self.active
+
+    def run(self) -> Dict[int, Request]:
+        """Step until every request has finished."""
+        while not self.idle:
+            self.step()
+        return self.finished

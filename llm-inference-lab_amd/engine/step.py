@@ -15,6 +15,7 @@ one prediction per request; this one returns logits at the wanted places.
 """
 from __future__ import annotations
 
+import collections
 import dataclasses
 from typing import Dict, List, Optional, Sequence, Tuple
 
@@ -80,6 +81,7 @@ class StepContext:
         self._groups = [
             GroupView(self._dev[t:t + b * self.max_pages].view(b, self.max_pages), page_size, window)
             for t, (page_size, window) in zip(self._table_at, groups)]
+        self._uploaded = torch.cuda.Event() if pin else None
         self._scratch: Dict[Tuple[str, torch.dtype], torch.Tensor] = {}
         self.scratch_version = 0
         self.n_rows = self.n_reqs = self.n_want = 0
@@ -127,6 +129,8 @@ class StepContext:
             raise ValueError(f"a step of {n_rows} tokens exceeds max_batch_tokens {self.max_rows}")
         if n_reqs > self.max_reqs:
             raise ValueError(f"a step of {n_reqs} requests exceeds max_requests {self.max_reqs}")
+        if self._uploaded is not None:
+            self._uploaded.synchronize()      # the staging buffer is free again
         h = self._host_np
         o = {k: v[0] for k, v in self._offsets.items()}
         row = 0
@@ -172,21 +176,63 @@ class StepContext:
         for at in self._table_at:
             n = n_reqs * self.max_pages
             self._dev[at:at + n].copy_(self._host[at:at + n], non_blocking=True)
+        if self._uploaded is not None:
+            self._uploaded.record()
 
 
 class StepFunction:
     """Owns the step's buffers; ``__call__`` runs one step."""
 
-    def __init__(self, model: CausalLM, cache: CacheManager, ops, max_batch_tokens: int):
+    MAX_GRAPHS = 16
+
+    def __init__(self, model: CausalLM, cache: CacheManager, ops, max_batch_tokens: int,
+                 graph: bool = False):
         self.model = model
         self.cache = cache
         self.ops = ops
         self.max_batch_tokens = int(max_batch_tokens)
+        # Pure decode steps (one token and one wanted place per request) can be
+        # replayed from a captured HIP graph: buffers have fixed addresses and
+        # everything that changes from step to step (tokens, positions, block
+        # tables) lives in device memory that is rewritten before the replay.
+        self.use_graph = bool(graph)
+        self._graphs: "collections.OrderedDict" = collections.OrderedDict()
+        self.graph_replays = 0
+        self.graph_captures = 0
         self.ctx = StepContext(
             ops, cache.device, self.max_batch_tokens, cache.max_requests,
             [(cache.page_size, g.window) for g in cache.groups], cache.max_pages_per_request)
         self.steps = 0
         self.rows_total = 0
+
+    def _decode_with_graph(self) -> torch.Tensor:
+        ctx = self.ctx
+        # Grid sizes and split counts are frozen into a graph: take them from a
+        # bucket of the context length, so one graph serves while contexts grow.
+        bucket = 128
+        while bucket < ctx.max_ctx_len:
+            bucket *= 2
+        ctx.max_ctx_len = min(bucket, self.cache.max_pages_per_request * self.cache.page_size)
+        key = (ctx.n_reqs, ctx.max_ctx_len, ctx.scratch_version)
+        hit = self._graphs.get(key)
+        if hit is not None:
+            self._graphs.move_to_end(key)
+            graph, logits = hit
+            graph.replay()
+            self.graph_replays += 1
+            return logits
+        logits = self.model.forward(ctx)       # this step's result; also sizes every scratch buffer
+        if key[2] != ctx.scratch_version:
+            return logits                      # buffers moved: capture at the next step
+        graph = torch.cuda.CUDAGraph()
+        torch.cuda.synchronize(ctx.device)
+        with torch.cuda.graph(graph):
+            captured = self.model.forward(ctx)
+        self._graphs[key] = (graph, captured)
+        self.graph_captures += 1
+        while len(self._graphs) > self.MAX_GRAPHS:
+            self._graphs.popitem(last=False)
+        return logits
 
     def __call__(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
         """Reserve pages, run the rows, commit.  Returns float32 logits
@@ -219,7 +265,10 @@ class StepFunction:
             for r in reserved:
                 self.cache.cancel_reservation(r)
             raise
-        logits = self.model.forward(self.ctx)
+        if self.use_graph and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
+            logits = self._decode_with_graph()
+        else:
+            logits = self.model.forward(self.ctx)
         for e in entries:
             self.cache.commit(e.request)
         self.steps += 1

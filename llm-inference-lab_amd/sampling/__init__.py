@@ -1,0 +1,2 @@
+from .params import SamplingConfig, read_generation_config
+from .sampler import Sampler, uniform

@@ -1,0 +1,62 @@
+"""Token selection on the GPU with host-side, counter-based random numbers.
+
+The n-th token of a request is drawn with the uniform number ``u(seed, n)``, a
+pure function of the request's seed and n.  The choice therefore does not depend
+on which other requests shared the step, on how the prompt was cut, or on the
+order of the batch.  The kernel takes the argmax where the temperature is 0 and
+otherwise the smallest token whose cumulative probability under
+``softmax(logits / temperature)`` reaches ``u``.  The reference selects with a
+two-stage argmax only (rust/engine/src/runner/model/qwen2/kernels.rs:1488-1552).
+"""
+from __future__ import annotations
+
+from typing import List, Sequence
+
+import numpy as np
+import torch
+
+_MASK = (1 << 64) - 1
+
+
+def _splitmix64(x: int) -> int:
+    x = (x + 0x9E3779B97F4A7C15) & _MASK
+    z = x
+    z = ((z ^ (z >> 30)) * 0xBF58476D1CE4E5B9) & _MASK
+    z = ((z ^ (z >> 27)) * 0x94D049BB133111EB) & _MASK
+    return z ^ (z >> 31)
+
+
+def uniform(seed: int, n: int) -> float:
+    """The n-th uniform number in [0, 1) of the stream ``seed`` (24 bits, exact in float32)."""
+    z = _splitmix64(_splitmix64(int(seed) & _MASK) ^ ((int(n) * 0xD1342543DE82EF95) & _MASK))
+    return (z >> 40) / float(1 << 24)
+
+
+class Sampler:
+    def __init__(self, ops, max_requests: int):
+        self.ops = ops
+        self.device = ops.device
+        pin = torch.device(self.device).type == "cuda"
+        self._host = torch.zeros((2, max_requests), dtype=torch.float32, pin_memory=pin)
+        self._dev = torch.zeros((2, max_requests), dtype=torch.float32, device=self.device)
+        self._out = torch.zeros(max_requests, dtype=torch.int32, device=self.device)
+
+    def sample(self, logits: torch.Tensor, temperatures: Sequence[float], seeds: Sequence[int],
+               counters: Sequence[int]) -> List[int]:
+        """One token per row of ``logits``.  Raises if a row holds no finite value."""
+        rows = logits.shape[0]
+        out = self._out[:rows]
+        if all(t <= 0.0 for t in temperatures):
+            self.ops.argmax(logits, out)
+        else:
+            h = self._host.numpy()
+            h[0, :rows] = np.asarray(temperatures, dtype=np.float32)
+            h[1, :rows] = np.asarray([uniform(s, c) for s, c in zip(seeds, counters)], dtype=np.float32)
+            self._dev[0, :rows].copy_(self._host[0, :rows], non_blocking=True)
+            self._dev[1, :rows].copy_(self._host[1, :rows], non_blocking=True)
+            self.ops.sample(logits, self._dev[0, :rows], self._dev[1, :rows], out)
+        tokens = out.cpu().tolist()
+        for t in tokens:
+            if t < 0:
+                raise FloatingPointError("non-finite logits: no token can be chosen")
+        return tokens
