@@ -17,6 +17,7 @@ import os
 import struct
 from typing import Dict, Iterable, List, Tuple
 
+import numpy as np
 import torch
 
 _DTYPES = {
@@ -77,9 +78,8 @@ class SafetensorsFile:
         dtype = _DTYPES[info["dtype"]]
         if end == begin:
             return torch.empty(shape, dtype=dtype)
-        flat = torch.frombuffer(self._map, dtype=torch.uint8, count=end - begin,
-                                offset=self._base + begin)
-        return flat.clone().view(dtype).reshape(shape)
+        flat = np.frombuffer(self._map, dtype=np.uint8, count=end - begin, offset=self._base + begin)
+        return torch.from_numpy(flat.copy()).view(dtype).reshape(shape)
 
     def close(self) -> None:
         try:

@@ -1,0 +1,147 @@
+"""The cache manager: no page lost, held twice or freed twice, under random
+orders of requests; windows; admission arithmetic."""
+import random
+
+import pytest
+import torch
+
+from llm_inference_lab_amd.cache import (CacheManager, GroupLayout, OutOfPages, PagePool,
+                                         group_page_need, pages_for_tokens)
+from llm_inference_lab_amd.parts import KVCacheSpec
+
+
+def manager(pages=(8,), windows=(None,), page_size=16, max_requests=4, max_seq_len=256, state=None):
+    groups = [GroupLayout(KVCacheSpec(1, 16, w), [i], n) for i, (n, w) in enumerate(zip(pages, windows))]
+    return CacheManager(groups, page_size, max_requests, max_seq_len, state or {}, torch.float32, "cpu")
+
+
+def test_pool_hands_out_every_page_once_and_takes_it_back_once():
+    pool = PagePool(5)
+    got = [pool.alloc(owner=1) for _ in range(5)]
+    assert sorted(got) == [0, 1, 2, 3, 4] and pool.free_count == 0
+    with pytest.raises(OutOfPages):
+        pool.alloc(owner=1)
+    pool.free(got[2], owner=1)
+    with pytest.raises(AssertionError, match="freed twice"):
+        pool.free(got[2], owner=1)
+    with pytest.raises(AssertionError, match="held by"):
+        pool.free(got[0], owner=2)
+    assert pool.alloc(owner=3) == got[2]          # a freed page is used again
+    pool.check()
+    assert pool.high_water == 5
+
+
+def test_reserve_commit_release_and_tables():
+    m = manager(pages=(6,))
+    a = m.admit("a")
+    m.reserve(a, 20)
+    assert a.reserved_len == 20 and a.computed_len == 0 and len(a.pages[0]) == 2
+    m.commit(a)
+    assert a.computed_len == 20
+    m.reserve(a, 12)                               # 32 tokens: still two pages
+    m.commit(a)
+    assert len(a.pages[0]) == 2
+    m.reserve(a, 1)                                # crosses a page's edge
+    m.commit(a)
+    assert len(a.pages[0]) == 3
+    assert list(m.tables[0][a.row, :3]) == a.pages[0] and m.tables[0][a.row, 3] == -1
+    m.check()
+    m.release(a)
+    assert m.free_pages(0) == 6 and m.free_rows == 4 and (m.tables[0] == -1).all()
+    with pytest.raises(AssertionError, match="released twice"):
+        m.release(a)
+
+
+def test_failed_reservation_gives_back_what_it_took():
+    m = manager(pages=(4, 2), windows=(None, None))
+    a = m.admit("a")
+    m.reserve(a, 30)
+    m.commit(a)
+    before = (m.free_pages(0), m.free_pages(1))
+    with pytest.raises(OutOfPages):
+        m.reserve(a, 40)                           # group 1 has no page left
+    assert (m.free_pages(0), m.free_pages(1)) == before
+    assert a.reserved_len == a.computed_len == 30
+    m.check()
+
+
+def test_rows_run_out_and_state_slots_start_at_zero():
+    state = {0: {"acc": ((3,), torch.float32)}}
+    m = manager(max_requests=2, state=state)
+    a, b = m.admit("a"), m.admit("b")
+    with pytest.raises(OutOfPages, match="rows"):
+        m.admit("c")
+    with pytest.raises(ValueError, match="already live"):
+        m.admit("a")
+    m.state[0]["acc"][a.row] += 5.0
+    row = a.row
+    m.release(a)
+    c = m.admit("c")
+    assert c.row == row and (m.state[0]["acc"][c.row] == 0).all()
+
+
+def test_window_frees_pages_that_every_later_query_has_passed():
+    m = manager(pages=(8, 8), windows=(None, 20), page_size=16)
+    a = m.admit("a")
+    for step in range(10):
+        m.reserve(a, 10)
+        m.commit(a)
+        m.check()
+        lowest_needed = max(0, a.computed_len - 20 + 1)
+        held = [lp for lp, p in enumerate(a.pages[1]) if p >= 0]
+        assert held[0] == lowest_needed // 16        # nothing older is kept, nothing needed is gone
+        assert held[-1] == (a.computed_len - 1) // 16
+    assert sum(p >= 0 for p in a.pages[0]) == 7 and sum(p >= 0 for p in a.pages[1]) <= 3
+    m.release(a)
+    assert m.free_pages(1) == 8
+
+
+def test_page_need_bounds_what_a_request_ever_holds():
+    for window in (None, 1, 5, 24, 100):
+        for page in (16, 64):
+            for step in (1, 7, 48):
+                m = manager(pages=(64,), windows=(window,), page_size=page, max_seq_len=1024)
+                a = m.admit("a")
+                need = group_page_need(window, page, 500, step)
+                worst = 0
+                while a.computed_len < 500:
+                    n = min(step, 500 - a.computed_len)
+                    m.reserve(a, n)
+                    worst = max(worst, sum(p >= 0 for p in a.pages[0]))
+                    m.commit(a)
+                assert worst <= need, (window, page, step, worst, need)
+                if window is None:
+                    assert need == pages_for_tokens(500, page)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_orders_keep_every_invariant(seed):
+    rng = random.Random(seed)
+    m = manager(pages=(24, 10), windows=(None, 24), page_size=16, max_requests=4, max_seq_len=400)
+    live, names = {}, 0
+    for _ in range(400):
+        action = rng.random()
+        if action < 0.2 and m.free_rows:
+            names += 1
+            live[names] = m.admit(names)
+        elif action < 0.85 and live:
+            req = live[rng.choice(list(live))]
+            n = rng.choice([1, 1, 1, 2, 5, 17, 40])
+            try:
+                m.reserve(req, n)
+                if rng.random() < 0.1:
+                    m.cancel_reservation(req)
+                else:
+                    m.commit(req)
+            except OutOfPages:
+                pass
+            except ValueError:
+                pass                                   # past the longest sequence
+        elif live:
+            key = rng.choice(list(live))
+            m.release(live.pop(key))
+        m.check()
+    for req in live.values():
+        m.release(req)
+    m.check()
+    assert m.free_pages(0) == 24 and m.free_pages(1) == 10 and m.free_rows == 4

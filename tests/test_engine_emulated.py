@@ -1,0 +1,107 @@
+"""The engine's own cache manager, step function and model assembly, run on the
+CPU with the per-kernel PyTorch references in place of the HIP kernels, against
+the plain whole-sequence implementation.  What these tests pin is everything
+around the kernels: block tables, page reuse, windows that free pages, portions,
+mixed batches."""
+import pytest
+import torch
+
+import helpers as H
+from emu_ops import EmuOps
+
+LENGTHS = {"A": [1, 7, 29, 70], "B": [5, 40, 61, 90], "C": [3, 50]}
+
+
+def sequences_of(name, seed=0):
+    cfg = H.config_of(name)
+    return {f"r{i}": H.random_ids(cfg, n, 100 * seed + i) for i, n in enumerate(LENGTHS[name])}
+
+
+def engine_of(name, dtype, **kw):
+    return H.make_engine(name, 1, dtype, ops=EmuOps(), device="cpu", **kw)
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("cut", ["whole", "decode", "portions", "mixed"])
+def test_every_cut_matches_plain(name, cut):
+    seqs = sequences_of(name)
+    want = {rid: H.plain_logits(name, 1, ids) for rid, ids in seqs.items()}
+    # so few pages that finished requests' pages are used again
+    engine = engine_of(name, "f32", page_size=16, num_pages=14, max_requests=4)
+    steps = {"whole": H.steps_whole, "decode": H.steps_prefill_then_decode,
+             "portions": H.steps_portions, "mixed": H.steps_mixed}[cut](seqs)
+    got = H.run_trace(engine, seqs, steps)
+    bad = H.first_wrong(got, want, H.TOL["f32"])
+    assert bad is None, f"first wrong logits at (request, position, error) = {bad}"
+    engine.cache.check()
+    m = engine.cache.metrics()
+    assert m["rows_used"] == 0 and all(g["pages_used"] == 0 for g in m["groups"])
+    if cut == "mixed":
+        assert sum(g["pages_high_water"] for g in m["groups"]) > 0
+
+
+def test_pages_are_reused_in_mixed():
+    seqs = sequences_of("B", seed=3)
+    engine = engine_of("B", "f32", page_size=16, num_pages=10)
+    total_pages_needed = sum((len(v) + 15) // 16 for v in seqs.values())
+    assert total_pages_needed > 10          # cannot all be live at once: reuse is forced
+    steps = H.steps_mixed(seqs, seed=1, max_live=2)
+    got = H.run_trace(engine, seqs, steps)
+    want = {rid: H.plain_logits("B", 1, ids) for rid, ids in seqs.items()}
+    assert H.max_error(got, want) < H.TOL["f32"]
+
+
+def test_window_group_gives_pages_back_early():
+    engine = engine_of("B", "f32", page_size=16, num_pages=12)
+    cfg = H.config_of("B")
+    ids = H.random_ids(cfg, 150, 9)
+    req = engine.open("x")
+    for i in range(0, 150, 10):
+        engine.step([H.lab.StepEntry(req, ids[i:i + 10], [])])
+        engine.cache.check()
+    full, windowed = engine.cache.metrics()["groups"]
+    assert full["window"] is None and windowed["window"] == 24
+    assert full["pages_used"] == 10                      # ceil(150 / 16)
+    assert windowed["pages_used"] <= 3                   # 24 latest positions touch at most 3 pages
+    assert windowed["pages_high_water"] <= 4
+    engine.close(req)
+
+
+def test_step_rejects_bad_input_and_keeps_cache_clean():
+    engine = engine_of("A", "f32", page_size=16, num_pages=2)
+    req = engine.open("x")
+    with pytest.raises(ValueError, match="outside the vocabulary"):
+        engine.step([H.lab.StepEntry(req, [1, 2, 999], [])])
+    with pytest.raises(ValueError, match="not among"):
+        engine.step([H.lab.StepEntry(req, [1, 2], [2])])
+    from llm_inference_lab_amd.cache import OutOfPages
+    with pytest.raises(OutOfPages):
+        engine.step([H.lab.StepEntry(req, list(range(40)), [])])
+    assert req.computed_len == 0 and req.reserved_len == 0
+    engine.cache.check()
+    assert engine.cache.free_pages(0) == 2
+    engine.step([H.lab.StepEntry(req, list(range(30)), [29])])
+    assert req.computed_len == 30
+    engine.close(req)
+    engine.cache.check()
+
+
+def test_schedule_may_repeat_a_block_and_share_a_cache():
+    """The order in which layers run is data: block 0 runs twice (two caches), and a
+    third run of block 1 reads the cache that block 1's first run wrote."""
+    import dataclasses
+    from llm_inference_lab_amd.config import ScheduleEntry
+    cfg = H.config_of("A")
+    arch = H.get_architecture(cfg.architecture)
+    spec = arch.build_spec(cfg)
+    spec = dataclasses.replace(spec, schedule=(ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(0),
+                                               ScheduleEntry(1, cache_of=1)))
+    model = CausalLMFromSpec(spec, cfg)
+    groups, _ = model.cache_layout()
+    assert len(groups) == 1 and groups[0].entries == [0, 1, 2]
+    assert model.entries[3].writes_cache is False and model.entries[3].slot == model.entries[1].slot
+
+
+def CausalLMFromSpec(spec, cfg):
+    from llm_inference_lab_amd.engine.model import CausalLM
+    return CausalLM(spec)

@@ -1,0 +1,251 @@
+"""Each part alone against the plain function of the same name, and a toy mixer
+with state of its own (defined here, not in the framework) registered, built
+and stepped without a change to the framework's files."""
+import dataclasses
+import math
+
+import pytest
+import torch
+
+import helpers as H
+import plain_qwen2 as P
+from llm_inference_lab_amd.config import (BlockSpec, ModelSpec, PartSpec, ScheduleEntry,
+                                          register_architecture, unregister_architecture)
+from llm_inference_lab_amd.parts import (Mixer, RMSNorm, RotaryEmbedding, SwiGLU, TokenEmbedding,
+                                         LinearHead, register_part, build_part)
+from llm_inference_lab_amd.parts.registry import unregister_part
+from llm_inference_lab_amd.weights import TensorSpec, MATRIX
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from llm_inference_lab_amd.kernels.hip_ops import HipOps
+    return HipOps(DEV)
+
+
+class Scratch:
+    """The part of a step context that parts without a cache need."""
+
+    def __init__(self):
+        self.bufs = {}
+
+    def scratch(self, name, shape, dtype):
+        key = (name, tuple(shape), dtype)
+        if key not in self.bufs:
+            self.bufs[key] = torch.empty(shape, dtype=dtype, device=DEV)
+        return self.bufs[key]
+
+
+def rnd(shape, seed, scale=1.0):
+    return torch.randn(shape, generator=torch.Generator().manual_seed(seed)) * scale
+
+
+TOLS = {torch.float32: 2e-5, torch.bfloat16: 2e-2}
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rmsnorm_part(ops, dtype):
+    norm = RMSNorm(size=96, eps=1e-5, tensors={"weight": "w"})
+    w = (1 + 0.1 * rnd((96,), 1)).to(torch.bfloat16)
+    norm.bind({"w": w.to(DEV)}, ops, dtype)
+    x = rnd((11, 96), 2, 2.0)
+    out = torch.empty(11, 96, dtype=dtype, device=DEV)
+    norm.forward(x.to(DEV), out)
+    want = P.rms_norm(x.double(), w.double(), 1e-5)
+    assert (out.double().cpu() - want).abs().max() < TOLS[dtype] * 4
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_rotary_part_general_path(ops, dtype):
+    rope = RotaryEmbedding(dim=32, theta=1e6)
+    rope.bind({}, ops, dtype)
+    q, k = rnd((9, 3, 32), 3).to(dtype), rnd((9, 1, 32), 4).to(dtype)
+    pos = torch.tensor([0, 1, 2, 3, 100, 1000, 4095, 7, 8], dtype=torch.int32)
+    qd, kd = q.to(DEV), k.to(DEV)
+    rope.apply(qd, kd, pos.to(DEV))
+    assert (qd.double().cpu() - P.rope(q.double(), pos.long(), 1e6)).abs().max() < TOLS[dtype] * 4
+    assert (kd.double().cpu() - P.rope(k.double(), pos.long(), 1e6)).abs().max() < TOLS[dtype] * 4
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_swiglu_part(ops, dtype):
+    ffn = SwiGLU(hidden_size=72, intermediate_size=200,
+                 tensors=dict(gate_weight="g", up_weight="u", down_weight="d"))
+    g, u, d = (rnd(s, i, 0.2).to(torch.bfloat16) for i, s in enumerate([(200, 72), (200, 72), (72, 200)]))
+    ffn.bind({"g": g.to(dtype).to(DEV), "u": u.to(dtype).to(DEV), "d": d.to(dtype).to(DEV)}, ops, dtype)
+    x = rnd((13, 72), 5).to(torch.bfloat16)
+    resid = rnd((13, 72), 6)
+    got = resid.clone().to(DEV)
+    ffn.forward(x.to(dtype).to(DEV), got, Scratch())
+    want = resid.double() + P.swiglu_mlp(x.double(), g.double(), u.double(), d.double())
+    assert (got.double().cpu() - want).abs().max() < TOLS[dtype] * 4
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_embedding_and_head_parts(ops, dtype):
+    table = rnd((301, 72), 7).to(torch.bfloat16)
+    emb = TokenEmbedding(vocab_size=301, hidden_size=72, tensors={"weight": "t"})
+    head = LinearHead(vocab_size=301, hidden_size=72, tensors={"weight": "t"})
+    loaded = {"t": table.to(dtype).to(DEV)}
+    emb.bind(loaded, ops, dtype)
+    head.bind(loaded, ops, dtype)
+    assert head.weight.data_ptr() == emb.table.data_ptr()            # tied: one tensor
+    ids = torch.tensor([0, 300, 17, 17], dtype=torch.int32)
+    x = torch.empty(4, 72, device=DEV)
+    emb.forward(ids.to(DEV), x)
+    assert torch.equal(x.cpu(), table.float()[ids.long()])
+    h = rnd((4, 72), 8).to(torch.bfloat16)
+    logits = torch.empty(4, 301, device=DEV)
+    head.forward(h.to(dtype).to(DEV), logits)
+    assert (logits.double().cpu() - P.linear(h.double(), table.double())).abs().max() < 1e-3
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("name,layer", [("A", 0), ("B", 0), ("B", 2), ("C", 1)])
+def test_block_alone(dtype, name, layer):
+    """One decoder layer (norm, attention with its cache, norm, feed-forward) on a
+    random residual stream, in two portions, against the plain layer."""
+    cfg = H.config_of(name)
+    engine = H.make_engine(name, 1, dtype, page_size=16, num_pages=8)
+    tensors = {k: v.double() for k, v in H.make_tensors(cfg, 1).items()}
+    x = rnd((50, cfg.hidden_size), 9, 2.0)
+    want = P.decoder_layer(x.double(), torch.arange(50), tensors, cfg.to_dict(), layer)
+    req = engine.open("x")
+    view = engine.model.entries[layer]
+    block = engine.model.blocks[view.block]
+    outs = []
+    for lo, hi in ((0, 33), (33, 50)):
+        engine.cache.reserve(req, hi - lo)
+        engine.step_fn.ctx.fill([H.lab.StepEntry(req, [0] * (hi - lo), [])], engine.cache)
+        resid = x[lo:hi].clone().to(DEV)
+        block.forward(resid, engine.step_fn.ctx, view)
+        engine.cache.commit(req)
+        outs.append(resid.cpu())
+    got = torch.cat(outs)
+    tol = 2e-4 if dtype == "f32" else 5e-2
+    assert (got.double() - want).abs().max() < tol * max(1.0, want.abs().max().item() / 4)
+    engine.close(req)
+
+
+# ---------------------------------------------------------------- toy mixer
+class RunningMean(Mixer):
+    """A mixer with state of fixed size and no cache: the output at a token is a
+    projection of the mean of all inputs of its request so far.  The state (sum
+    and count) lives in the cache manager's per-request slots."""
+
+    def __init__(self, hidden_size, tensors):
+        super().__init__(tensors)
+        self.hidden_size = hidden_size
+        self.weight = None
+
+    def tensor_specs(self):
+        return {self.tensor_names["weight"]: TensorSpec((self.hidden_size, self.hidden_size), MATRIX)}
+
+    def bind(self, tensors, ops, dtype):
+        super().bind(tensors, ops, dtype)
+        self.weight = tensors[self.tensor_names["weight"]]
+
+    def state_spec(self):
+        return {"sum": ((self.hidden_size,), torch.float32), "count": ((1,), torch.float32)}
+
+    def forward(self, h, residual, ctx, entry):
+        total, count = entry.state["sum"], entry.state["count"]
+        mean = torch.empty(h.shape, dtype=torch.float32, device=h.device)
+        for b in range(ctx.n_reqs):
+            r0, r1, slot = ctx.host_q_start[b], ctx.host_q_start[b + 1], ctx.host_req_rows[b]
+            run = total[slot] + torch.cumsum(h[r0:r1].float(), dim=0)
+            n = count[slot] + torch.arange(1, r1 - r0 + 1, device=h.device, dtype=torch.float32)[:, None]
+            mean[r0:r1] = run / n
+            total[slot] = run[-1]
+            count[slot] = n[-1]
+        self.ops.linear_residual(mean.to(self.dtype), self.weight, residual)
+
+
+@dataclasses.dataclass(frozen=True)
+class ToyConfig:
+    vocab_size: int
+    hidden_size: int
+    eps: float
+    architecture: str = "ToyForCausalLM"
+
+    @classmethod
+    def from_dict(cls, raw, where="config.json"):
+        return cls(raw["vocab_size"], raw["hidden_size"], raw["eps"])
+
+    def to_dict(self):
+        return {"architectures": [self.architecture], "vocab_size": self.vocab_size,
+                "hidden_size": self.hidden_size, "eps": self.eps}
+
+
+def toy_spec(cfg):
+    h = cfg.hidden_size
+    norm = lambda n: PartSpec("rmsnorm", dict(size=h, eps=cfg.eps), dict(weight=n))
+    ffn = lambda p: PartSpec("swiglu", dict(hidden_size=h, intermediate_size=2 * h),
+                             dict(gate_weight=p + "gate", up_weight=p + "up", down_weight=p + "down"))
+    toy = BlockSpec("prenorm", mixer=PartSpec("toy_running_mean", dict(hidden_size=h), dict(weight="l0.mix")),
+                    feed_forward=ffn("l0."), norm1=norm("l0.n1"), norm2=norm("l0.n2"), params=dict(hidden_size=h))
+    attn = BlockSpec("prenorm", mixer=PartSpec(
+        "gqa_attention", dict(hidden_size=h, num_heads=2, num_kv_heads=1, head_dim=h // 2, qkv_bias=False,
+                              position=None, window=None),
+        dict(q_weight="l1.q", k_weight="l1.k", v_weight="l1.v", o_weight="l1.o")),
+        feed_forward=ffn("l1."), norm1=norm("l1.n1"), norm2=norm("l1.n2"), params=dict(hidden_size=h))
+    sizes = dict(vocab_size=cfg.vocab_size, hidden_size=h)
+    return ModelSpec("ToyForCausalLM", cfg.vocab_size, h, 4096,
+                     PartSpec("token_embedding", sizes, dict(weight="embed")), (toy, attn),
+                     # the toy block runs twice: two runs, two states
+                     (ScheduleEntry(0), ScheduleEntry(1), ScheduleEntry(0)),
+                     norm("final"), PartSpec("linear_head", sizes, dict(weight="embed")))
+
+
+def toy_plain(ids, w, cfg):
+    """Whole-sequence reference of the toy model, float64."""
+    h = cfg.hidden_size
+    x = w["embed"][torch.tensor(ids)]
+    t = len(ids)
+    def toy_block(x):
+        n = P.rms_norm(x, w["l0.n1"], cfg.eps)
+        mean = torch.cumsum(n, 0) / torch.arange(1, t + 1, dtype=x.dtype)[:, None]
+        x = x + P.linear(mean, w["l0.mix"])
+        return x + P.swiglu_mlp(P.rms_norm(x, w["l0.n2"], cfg.eps), w["l0.gate"], w["l0.up"], w["l0.down"])
+    x = toy_block(x)
+    n = P.rms_norm(x, w["l1.n1"], cfg.eps)
+    q = P.linear(n, w["l1.q"]).view(t, 2, h // 2)
+    k = P.linear(n, w["l1.k"]).view(t, 1, h // 2)
+    v = P.linear(n, w["l1.v"]).view(t, 1, h // 2)
+    a = P.causal_attention_dense(q, k, v, torch.arange(t)).reshape(t, h)      # no position encoding
+    x = x + P.linear(a, w["l1.o"])
+    x = x + P.swiglu_mlp(P.rms_norm(x, w["l1.n2"], cfg.eps), w["l1.gate"], w["l1.up"], w["l1.down"])
+    x = toy_block(x)
+    return P.linear(P.rms_norm(x, w["final"], cfg.eps), w["embed"])
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_toy_mixer_with_state_is_registered_built_and_stepped(dtype):
+    register_part("mixer", "toy_running_mean", RunningMean, replace=True)
+    register_architecture("ToyForCausalLM", ToyConfig, toy_spec, replace=True)
+    try:
+        cfg = ToyConfig(vocab_size=97, hidden_size=64, eps=1e-5)
+        from llm_inference_lab_amd.engine.model import CausalLM
+        from llm_inference_lab_amd.weights import random_tensors
+        tensors = dict(random_tensors(CausalLM(toy_spec(cfg)).tensor_specs(), 3, torch.bfloat16,
+                                      is_norm=lambda n: n.endswith(("n1", "n2", "final"))))
+        for n in ("embed", "l1.q", "l1.k"):
+            tensors[n] = (tensors[n].float() * 8).to(torch.bfloat16)
+        engine = H.lab.Engine(config=cfg, tensors=tensors.items(), dtype=dtype, page_size=16, num_pages=16,
+                              max_requests=3, max_batch_tokens=128, max_seq_len=256)
+        groups, states = engine.model.cache_layout()
+        assert len(groups) == 1 and groups[0].entries == [1] and sorted(states) == [0, 2]
+        g = torch.Generator().manual_seed(0)
+        seqs = {f"r{i}": torch.randint(0, 97, (n,), generator=g).tolist() for i, n in enumerate([45, 80, 23, 60])}
+        w64 = {k: v.double() for k, v in tensors.items()}
+        want = {rid: toy_plain(ids, w64, cfg) for rid, ids in seqs.items()}
+        for steps in (H.steps_whole(seqs), H.steps_portions(seqs), H.steps_mixed(seqs, seed=2, max_live=3)):
+            got = H.run_trace(engine, seqs, steps)
+            bad = H.first_wrong(got, want, H.TOL[dtype])
+            assert bad is None, f"first wrong logits at (request, position, error) = {bad}"
+    finally:
+        unregister_part("mixer", "toy_running_mean")
+        unregister_architecture("ToyForCausalLM")

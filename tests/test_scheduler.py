@@ -1,0 +1,185 @@
+"""The scheduler's decisions, on the CPU: the plan under a token budget,
+admission by whole-turn page budget, what happens when pages run out, end of
+sequence, and that cutting prompts into portions changes no token."""
+import pytest
+import torch
+
+import helpers as H
+from emu_ops import EmuOps
+from llm_inference_lab_amd.engine.scheduler import (CapacityExhausted, Request, Scheduler, plan_step)
+from llm_inference_lab_amd.sampling import SamplingConfig, Sampler, uniform
+
+
+class FakeCache:
+    def __init__(self, computed):
+        self.computed_len = computed
+
+
+def req(rid, prompt_len, computed=0, generated=0, remaining=4):
+    r = Request(rid, list(range(prompt_len)), SamplingConfig(max_new_tokens=remaining))
+    r.tokens = list(r.prompt) + [0] * generated
+    r.generated = [0] * generated
+    r.remaining = remaining
+    r.cache = FakeCache(computed)
+    return r
+
+
+def shape(plan):
+    return [(p.request.request_id, p.count, p.yields_token) for p in plan]
+
+
+def test_plan_cases_of_the_reference():
+    """rust/engine/src/runner/model_runner.rs:1455-1501."""
+    # budget 1, two prompts: the oldest gets it
+    assert shape(plan_step([req(0, 5), req(1, 3)], 1)) == [(0, 1, False)]
+    # budget 2 with one decoder and one prompt: one token each
+    assert shape(plan_step([req(0, 5, computed=5, generated=1), req(1, 3)], 2)) == [(0, 1, True), (1, 1, False)]
+    # no budget left for prompts: decode only
+    assert shape(plan_step([req(0, 5, computed=5, generated=1), req(1, 3)], 1)) == [(0, 1, True)]
+    # the rest of the budget goes to prompts in order; the last one is cut
+    plan = plan_step([req(0, 10), req(1, 10), req(2, 10, computed=11, generated=2)], 16)
+    assert shape(plan) == [(0, 10, True), (1, 5, False), (2, 1, True)]
+    # a one-token prompt is still prefill: it competes for the prefill budget
+    assert shape(plan_step([req(0, 1), req(1, 4, computed=4, generated=1)], 1)) == [(1, 1, True)]
+    # a finished or exhausted request is not planned
+    done = req(0, 3, computed=3, generated=1, remaining=0)
+    assert plan_step([done], 8) == []
+
+
+def engine_of(name="A", **kw):
+    kw.setdefault("page_size", 16)
+    return H.make_engine(name, 1, "f32", ops=EmuOps(), device="cpu", **kw)
+
+
+def generate(engine, prompts, budget, max_new=5, **kw):
+    out = engine.generate(prompts, max_new_tokens=max_new, max_batch_tokens=budget, **kw)
+    engine.cache.check()
+    m = engine.cache.metrics()
+    assert m["rows_used"] == 0 and all(g["pages_used"] == 0 for g in m["groups"])
+    return out
+
+
+def test_portions_of_any_budget_give_the_same_tokens():
+    """Budgets 1, 2, 3 equal the uncut run (model_runner.rs:1609-1635)."""
+    cfg = H.config_of("A")
+    prompts = [H.random_ids(cfg, n, 40 + n) for n in (1, 7, 13)]
+    engine = engine_of(num_pages=16, max_requests=4)
+    whole = generate(engine, prompts, 512)
+    for budget in (1, 2, 3, 7):
+        assert generate(engine, prompts, budget) == whole
+    # and the plain implementation agrees (greedy, float32)
+    tensors = H.make_tensors(cfg, 1)
+    import plain_qwen2
+    assert whole == [plain_qwen2.greedy_generate(p, 5, tensors, cfg.to_dict()) for p in prompts]
+
+
+def test_decode_runs_beside_portions_of_later_prompts():
+    cfg = H.config_of("A")
+    engine = engine_of(num_pages=16, max_requests=4)
+    sched = engine.scheduler(max_batch_tokens=8)
+    sched.keep_step_log = True
+    sched.add_request(H.random_ids(cfg, 3, 1), SamplingConfig(max_new_tokens=6, eos_token_id=[]))
+    sched.step()                                   # request 0: whole prompt, first token
+    sched.add_request(H.random_ids(cfg, 20, 2), SamplingConfig(max_new_tokens=2, eos_token_id=[]))
+    sched.run()
+    log = sched.step_log
+    assert log[0] == [(0, 3)]
+    assert log[1] == [(0, 1), (1, 7)] and log[2] == [(0, 1), (1, 7)] and log[3] == [(0, 1), (1, 6)]
+    assert all(r.finish_reason == "length" for r in sched.finished.values())
+
+
+def test_end_of_sequence_counts_and_ends_the_request():
+    cfg = H.config_of("A")
+    engine = engine_of(num_pages=16)
+    prompt = H.random_ids(cfg, 9, 3)
+    free_run = generate(engine, [prompt], 64, max_new=6, eos_token_id=[])[0]
+    stop = free_run[2]
+    cut = generate(engine, [prompt], 64, max_new=6, eos_token_id=[stop])[0]
+    assert cut == free_run[:free_run.index(stop) + 1]          # the end token is kept and counted
+    assert engine.last_scheduler.finished[0].finish_reason == "eos"
+
+
+def test_admission_budgets_the_whole_turn():
+    """A holds 1 page and is promised 2 more; of a 4-page pool only a request that
+    needs 1 page fits beside it (model_runner.rs:1755-1794, in pages)."""
+    cfg = H.config_of("A")
+    engine = engine_of(num_pages=4, max_requests=4, max_seq_len=64)
+    sched = engine.scheduler(max_batch_tokens=64)
+    sched.add_request(H.random_ids(cfg, 10, 1), SamplingConfig(max_new_tokens=30, eos_token_id=[]))  # 39 -> 3 pages
+    sched.step()
+    assert len(sched.active) == 1 and engine.cache.free_pages(0) == 3
+    sched.add_request(H.random_ids(cfg, 20, 2), SamplingConfig(max_new_tokens=4, eos_token_id=[]))   # 23 -> 2 pages
+    sched.add_request(H.random_ids(cfg, 5, 3), SamplingConfig(max_new_tokens=4, eos_token_id=[]))    # 8 -> 1 page
+    sched.step()
+    assert sorted(r.request_id for r in sched.active) == [0, 2]       # 1 waits, 2 overtakes it
+    assert [r.request_id for r in sched.waiting] == [1]
+    done = sched.run()
+    assert all(r.error is None for r in done.values()) and len(done[1].generated) == 4
+    # request 1 ran only after pages came back
+    assert done[1].first_token_time > min(done[0].finish_time, done[2].finish_time)
+    engine.cache.check()
+
+
+def test_request_that_can_never_fit_fails_alone():
+    cfg = H.config_of("A")
+    engine = engine_of(num_pages=2, max_requests=2, max_seq_len=512)
+    sched = engine.scheduler()
+    big = sched.add_request(H.random_ids(cfg, 40, 1), SamplingConfig(max_new_tokens=2))
+    ok = sched.add_request(H.random_ids(cfg, 10, 2), SamplingConfig(max_new_tokens=2, eos_token_id=[]))
+    done = sched.run()
+    assert isinstance(done[big].error, CapacityExhausted) and done[big].generated == []
+    assert done[ok].error is None and len(done[ok].generated) == 2
+    engine.cache.check()
+    assert engine.cache.free_pages(0) == 2
+
+
+def test_refused_requests_do_not_hurt_their_peers():
+    cfg = H.config_of("A")
+    engine = engine_of(num_pages=8, max_seq_len=64)
+    sched = engine.scheduler()
+    ids = [sched.add_request([], SamplingConfig(max_new_tokens=2)),
+           sched.add_request([1, 2, 99999], SamplingConfig(max_new_tokens=2)),
+           sched.add_request([1, 2, 3], SamplingConfig(max_new_tokens=200)),
+           sched.add_request([1, 2, 3], SamplingConfig(max_new_tokens=2, top_k=5)),
+           sched.add_request([1, 2, 3], SamplingConfig(max_new_tokens=0)),
+           sched.add_request([1, 2, 3], SamplingConfig(max_new_tokens=3, eos_token_id=[]))]
+    done = sched.run()
+    assert "empty prompt" in str(done[ids[0]].error)
+    assert "vocabulary" in str(done[ids[1]].error)
+    assert "exceeds" in str(done[ids[2]].error)
+    assert "top_k" in str(done[ids[3]].error)
+    assert done[ids[4]].error is None and done[ids[4]].generated == []
+    assert done[ids[5]].error is None and len(done[ids[5]].generated) == 3
+
+
+def test_finished_request_frees_before_the_next_step():
+    cfg = H.config_of("A")
+    engine = engine_of(num_pages=8)
+    sched = engine.scheduler()
+    sched.add_request(H.random_ids(cfg, 4, 1), SamplingConfig(max_new_tokens=1))
+    sched.add_request(H.random_ids(cfg, 4, 2), SamplingConfig(max_new_tokens=3, eos_token_id=[]))
+    finished = sched.step()
+    assert [r.request_id for r in finished] == [0]
+    assert engine.cache.live_requests == 1 and engine.cache.free_pages(0) == 7
+
+
+def test_temperature_stream_does_not_depend_on_the_cut_or_the_batch():
+    cfg = H.config_of("B")
+    prompts = [H.random_ids(cfg, n, 70 + n) for n in (5, 40, 61)]
+    engine = engine_of("B", num_pages=24, max_requests=4)
+    a = generate(engine, prompts, 512, max_new=8, temperature=0.8, seed=11, eos_token_id=[])
+    b = generate(engine, prompts, 8, max_new=8, temperature=0.8, seed=11, eos_token_id=[])
+    alone = [generate(engine, [p], 512, max_new=8, temperature=0.8, seed=11 + i, eos_token_id=[])[0]
+             for i, p in enumerate(prompts)]
+    other = generate(engine, prompts, 512, max_new=8, temperature=0.8, seed=12, eos_token_id=[])
+    assert a == b == alone and a != other
+    greedy = generate(engine, prompts, 512, max_new=8, eos_token_id=[])
+    assert generate(engine, prompts, 512, max_new=8, temperature=0.0, eos_token_id=[]) == greedy
+
+
+def test_uniform_numbers_are_a_pure_function_of_seed_and_count():
+    xs = [uniform(3, n) for n in range(2000)]
+    assert all(0.0 <= x < 1.0 for x in xs) and len(set(xs)) > 1990
+    assert abs(sum(xs) / len(xs) - 0.5) < 0.03
+    assert xs[:5] == [uniform(3, n) for n in range(5)] and uniform(4, 0) != uniform(3, 0)
+    assert all(float(torch.tensor(x, dtype=torch.float32)) == x for x in xs[:100])
