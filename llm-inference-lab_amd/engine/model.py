@@ -16,6 +16,7 @@ import torch
 
 from ..cache.manager import CacheManager, GroupLayout
 from ..config.spec import ModelSpec
+from ..parts.base import NormedInput
 from ..parts.registry import build_part, part_class
 from ..weights.loader import TensorSpec
 
@@ -131,8 +132,8 @@ class CausalLM:
             self.blocks[view.block].forward(x, ctx, view)
         if ctx.n_want == 0:
             return None
-        h = ctx.scratch("model.final_normed", (ctx.n_want, hidden), self.dtype)
-        self.final_norm.forward(x, h, ctx.want_rows)
+        h = NormedInput(self.final_norm, x, ctx, "model.final_normed", self.dtype,
+                        rows=ctx.want_rows, n_rows=ctx.n_want)
         logits = ctx.scratch("model.logits", (ctx.n_want, self.spec.vocab_size), torch.float32)
-        self.head.forward(h, logits)
+        self.head.forward(h if getattr(self.head, "takes_normed_input", False) else h.tensor(), logits)
         return logits

@@ -24,7 +24,7 @@ from typing import Dict, List, Optional, Sequence
 ARCH = "gfx950"
 CSRC = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "csrc")
 LIB_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib")
-CORE_SOURCES = ("elementwise.hip", "gemm.hip", "sampling.hip")
+CORE_SOURCES = ("elementwise.hip", "gemm.hip", "decode.hip", "sampling.hip")
 ATTENTION_SOURCE = "attention.hip"
 HEADERS = ("common.h",)
 FLAGS = ("-O3", "-std=c++17", "-fPIC", "-shared", f"--offload-arch={ARCH}",

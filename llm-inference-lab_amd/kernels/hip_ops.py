@@ -18,7 +18,7 @@ from ..config.errors import UnsupportedSizeError
 from . import build
 
 DT_F32, DT_BF16 = 0, 1
-EPI_STORE, EPI_RESID, EPI_F32, EPI_SWIGLU = 0, 1, 2, 3
+EPI_STORE, EPI_RESID, EPI_F32, EPI_SWIGLU, EPI_QKV = 0, 1, 2, 3, 4
 
 _c_int, _c_long, _c_float, _c_size, _c_ptr = (ctypes.c_int, ctypes.c_long, ctypes.c_float,
                                               ctypes.c_size_t, ctypes.c_void_p)
@@ -80,8 +80,12 @@ class HipOps:
         c.llmlab_linear.argtypes = [_c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_int, _c_int,
                                     _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_size, _c_int, _c_ptr]
         c.llmlab_sample.argtypes = [_c_ptr, _c_long, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr]
+        c.llmlab_skinny_linear.argtypes = [
+            _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_float, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr,
+            _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
+            _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr]
         for fn in (c.llmlab_embed, c.llmlab_rmsnorm, c.llmlab_rope_kv_write, c.llmlab_rope_inplace,
-                   c.llmlab_linear, c.llmlab_sample):
+                   c.llmlab_linear, c.llmlab_sample, c.llmlab_skinny_linear):
             fn.restype = _c_int
 
     def _attention_lib(self, head_dim: int) -> ctypes.CDLL:
@@ -192,6 +196,9 @@ class HipOps:
             if bias.numel() != n:
                 raise ValueError("linear: bias length differs from the output width")
         ldo = out.stride(0) if m > 1 else max(out.stride(0), n_out)
+        if x.dtype == torch.bfloat16 and m <= self.FUSED_MAX_ROWS:
+            self._skinny(x, False, None, None, 0.0, w, bias, epilogue, out, m, n, k, ldo, n_out)
+            return
         self._check(self._core.llmlab_linear(
             self._ptr(x), self._ptr(w), _dt(x), epilogue, self._ptr(out), self._ptr(bias),
             _dt(bias) if bias is not None else 0, m, n, k, ldo, n_out, self._ptr(self.workspace),
@@ -212,6 +219,99 @@ class HipOps:
             raise ValueError(f"linear_swiglu: {w_gate_up.shape[0]} interleaved rows do not belong "
                              f"to {inter} outputs")
         self._linear(x, w_gate_up, out, None, EPI_SWIGLU, inter)
+
+    # ----------------------------------------------- few rows: fused kernels
+    FUSED_MAX_ROWS = 64
+
+    def can_fuse(self, rows: int, dtype) -> bool:
+        """Whether the fused few-row kernels take this step (bfloat16, at most 64 rows)."""
+        return dtype == torch.bfloat16 and 0 < rows <= self.FUSED_MAX_ROWS
+
+    def _skinny(self, x, norm, x_rows, norm_w, eps, w, bias, epilogue, out, m, n, k, ldo, n_out,
+                qkv=None) -> None:
+        q = qkv or {}
+        table = q.get("table")
+        self._check(self._core.llmlab_skinny_linear(
+            self._ptr(x), 1 if norm else 0, self._ptr(x_rows), self._ptr(norm_w),
+            _dt(norm_w) if norm_w is not None else 0, float(eps), self._ptr(w), self._ptr(bias),
+            _dt(bias) if bias is not None else 0, epilogue, self._ptr(out), m, n, k, ldo, n_out,
+            self._ptr(q.get("inv_freq")), self._ptr(q.get("positions")), self._ptr(q.get("row_req")),
+            self._ptr(table), table.stride(0) if table is not None else 0, q.get("page_size", 0),
+            self._ptr(q.get("k_cache")), self._ptr(q.get("v_cache")), q.get("nq", 0), q.get("nkv", 0),
+            q.get("d", 0), self.num_cus, self._stream()))
+
+    def _fused_common(self, x, norm_w, w, rows):
+        self._need(x, "residual stream", torch.float32)
+        self._need(norm_w, "norm weight")
+        self._need(w, "weight", torch.bfloat16)
+        k = x.shape[1]
+        if norm_w.numel() != k or w.shape[1] != k:
+            raise ValueError(f"fused norm + product: x {tuple(x.shape)}, norm weight "
+                             f"{tuple(norm_w.shape)}, w {tuple(w.shape)} do not fit")
+        if k % 8 != 0:
+            raise UnsupportedSizeError(
+                f"bfloat16 matrix products need an inner size that is a multiple of 8, got {k}")
+        if not 0 < rows <= self.FUSED_MAX_ROWS:
+            raise ValueError(f"the fused kernels take 1..{self.FUSED_MAX_ROWS} rows, got {rows}")
+        return k
+
+    def fused_norm_qkv(self, x, norm_w, eps, w_qkv, b_qkv, num_heads, num_kv_heads, head_dim, inv_freq,
+                       positions, row_req, block_table, page_size, k_cache, v_cache, q_out) -> None:
+        """q_out = rotate(norm(x) Wq^T + bq); rotated k and v of the new positions go to
+        their pages (skipped when no cache is given)."""
+        rows = x.shape[0]
+        k = self._fused_common(x, norm_w, w_qkv, rows)
+        n = (num_heads + 2 * num_kv_heads) * head_dim
+        if w_qkv.shape[0] != n or tuple(q_out.shape) != (rows, num_heads * head_dim):
+            raise ValueError("fused_norm_qkv: weight or output shape does not fit the heads")
+        self._need(q_out, "q output", torch.bfloat16)
+        self._need(positions, "positions", torch.int32)
+        if positions.numel() < rows:
+            raise ValueError("fused_norm_qkv: one position per row")
+        if b_qkv is not None and b_qkv.numel() != n:
+            raise ValueError("fused_norm_qkv: bias length")
+        if inv_freq is not None and (inv_freq.dtype != torch.float32 or inv_freq.numel() != head_dim // 2):
+            raise ValueError("fused_norm_qkv: the frequency table must hold head_dim/2 float32 entries")
+        if k_cache is not None:
+            self._need(row_req, "row -> request map", torch.int32)
+            self._need(block_table, "block table", torch.int32)
+            pages = k_cache.shape[0]
+            if (tuple(k_cache.shape) != (pages, num_kv_heads, page_size, head_dim)
+                    or tuple(v_cache.shape) != (pages, num_kv_heads, head_dim, page_size)
+                    or not k_cache.is_contiguous() or not v_cache.is_contiguous()
+                    or k_cache.dtype != torch.bfloat16 or v_cache.dtype != torch.bfloat16
+                    or row_req.numel() < rows):
+                raise ValueError("fused_norm_qkv: cache tensors do not have the paged layout")
+        self._skinny(x, True, None, norm_w, eps, w_qkv, b_qkv, EPI_QKV, q_out, rows, n, k,
+                     q_out.shape[1], n,
+                     dict(inv_freq=inv_freq, positions=positions, row_req=row_req, table=block_table,
+                          page_size=page_size, k_cache=k_cache, v_cache=v_cache, nq=num_heads,
+                          nkv=num_kv_heads, d=head_dim))
+
+    def fused_norm_swiglu(self, x, norm_w, eps, w_gate_up, out) -> None:
+        rows, inter = out.shape
+        k = self._fused_common(x, norm_w, w_gate_up, rows)
+        self._need(out, "SwiGLU output", torch.bfloat16)
+        if x.shape[0] != rows or w_gate_up.shape[0] != 2 * ((inter + 15) // 16 * 16):
+            raise ValueError("fused_norm_swiglu: shapes do not fit")
+        self._skinny(x, True, None, norm_w, eps, w_gate_up, None, EPI_SWIGLU, out, rows,
+                     w_gate_up.shape[0], k, out.shape[1], inter)
+
+    def fused_norm_logits(self, x, rows_index, norm_w, eps, w, out) -> None:
+        """out[i] = norm(x[rows_index[i]]) W^T in float32."""
+        rows, vocab = out.shape
+        k = self._fused_common(x, norm_w, w, rows)
+        self._need(out, "logits", torch.float32)
+        if w.shape[0] != vocab:
+            raise ValueError("fused_norm_logits: weight rows differ from the vocabulary")
+        if rows_index is not None:
+            self._need(rows_index, "row indices", torch.int32)
+            if rows_index.numel() < rows:
+                raise ValueError("fused_norm_logits: one row index per output row")
+        elif x.shape[0] != rows:
+            raise ValueError("fused_norm_logits: rows differ")
+        self._skinny(x, True, rows_index, norm_w, eps, w, None, EPI_F32, out, rows, vocab, k,
+                     out.shape[1], vocab)
 
     # ------------------------------------------------------------------- rope
     def rope_inplace(self, x, positions, inv_freq) -> None:

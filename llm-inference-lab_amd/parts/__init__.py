@@ -1,5 +1,6 @@
 from .registry import register_part, unregister_part, part_class, build_part, FAMILIES
-from .base import Part, Norm, PositionEncoding, Mixer, FeedForward, Block, KVCacheSpec
+from .base import (Part, Norm, NormedInput, PositionEncoding, Mixer, FeedForward, Block,
+                   KVCacheSpec)
 from .norms import RMSNorm
 from .positions import RotaryEmbedding, NoPosition
 from .attention import GQAAttention

@@ -8,7 +8,7 @@ import torch
 
 from ..config.spec import PartSpec
 from ..weights.loader import TensorSpec, MATRIX, VECTOR
-from .base import Mixer, KVCacheSpec
+from .base import Mixer, KVCacheSpec, NormedInput
 from .registry import register_part, build_part
 
 
@@ -28,6 +28,8 @@ class GQAAttention(Mixer):
     rust/engine/src/runner/model/qwen2/kernels.rs:702-853, output projection and
     residual engine.rs:1225-1233.  The window is not in the reference (it
     rejects ``use_sliding_window``, engine.rs:262)."""
+
+    takes_normed_input = True
 
     def __init__(self, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  position: Optional[PartSpec], tensors: Dict[str, str], qkv_bias: bool = True,
@@ -96,23 +98,35 @@ class GQAAttention(Mixer):
     def forward(self, h, residual, ctx, entry):
         ops = self.ops
         rows = h.shape[0]
-        qkv = ctx.scratch("attention.qkv", (rows, self.q_size + 2 * self.kv_size), self.dtype)
-        ops.linear(h, self.w_qkv, qkv, self.b_qkv)
         table = self.position.rotary_table() if self.position is not None else None
-        if self.position is not None and table is None:
-            q = qkv[:, :self.q_size].unflatten(1, (self.num_heads, self.head_dim))
-            k = qkv[:, self.q_size:self.q_size + self.kv_size].unflatten(
-                1, (self.num_kv_heads, self.head_dim))
-            self.position.apply(q, k, ctx.positions[:rows])
         group = ctx.group(entry.group)
-        ops.rope_kv_write(
-            qkv, self.num_heads, self.num_kv_heads, self.head_dim, table,
-            ctx.positions, ctx.row_req, group.block_table, group.page_size,
-            entry.k_cache if entry.writes_cache else None,
-            entry.v_cache if entry.writes_cache else None)
+        k_cache = entry.k_cache if entry.writes_cache else None
+        v_cache = entry.v_cache if entry.writes_cache else None
+        rms = h.rms() if isinstance(h, NormedInput) else None
+        if (rms is not None and ops.can_fuse(rows, self.dtype)
+                and (self.position is None or table is not None)):
+            # few rows: norm, the three projections, bias, rotation and the cache
+            # write are one kernel
+            q = ctx.scratch("attention.q", (rows, self.q_size), self.dtype)
+            ops.fused_norm_qkv(rms[0], rms[2], rms[3], self.w_qkv, self.b_qkv, self.num_heads,
+                               self.num_kv_heads, self.head_dim, table, ctx.positions, ctx.row_req,
+                               group.block_table, group.page_size, k_cache, v_cache, q)
+        else:
+            if isinstance(h, NormedInput):
+                h = h.tensor()
+            q = ctx.scratch("attention.qkv", (rows, self.q_size + 2 * self.kv_size), self.dtype)
+            ops.linear(h, self.w_qkv, q, self.b_qkv)
+            if self.position is not None and table is None:
+                qv = q[:, :self.q_size].unflatten(1, (self.num_heads, self.head_dim))
+                kv = q[:, self.q_size:self.q_size + self.kv_size].unflatten(
+                    1, (self.num_kv_heads, self.head_dim))
+                self.position.apply(qv, kv, ctx.positions[:rows])
+            ops.rope_kv_write(q, self.num_heads, self.num_kv_heads, self.head_dim, table,
+                              ctx.positions, ctx.row_req, group.block_table, group.page_size,
+                              k_cache, v_cache)
         out = ctx.scratch("attention.out", (rows, self.q_size), self.dtype)
         ops.paged_attention(
-            qkv, self.num_heads, self.num_kv_heads, self.head_dim,
+            q, self.num_heads, self.num_kv_heads, self.head_dim,
             entry.k_cache, entry.v_cache, group.block_table, group.page_size,
             ctx.q_start, ctx.start_pos, ctx.n_reqs, ctx.max_q_len, ctx.max_ctx_len,
             self.window, self.scale, out, ctx)

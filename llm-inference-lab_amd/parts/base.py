@@ -60,6 +60,45 @@ class Norm(Part):
         ``x`` float32, ``out`` compute dtype."""
         raise NotImplementedError
 
+    def rms_params(self):
+        """``(weight, eps)`` if this norm is a plain RMSNorm that a following matrix
+        product may fold into itself; None otherwise."""
+        return None
+
+
+class NormedInput:
+    """The input of a mixer, feed-forward or head whose norm has not run yet.
+
+    A consumer that sets ``takes_normed_input = True`` is handed this object
+    instead of a tensor.  It may fold the norm into its first kernel
+    (``rms()`` gives what that kernel needs) or ask for the normed activations
+    with ``tensor()``, which runs the norm once."""
+
+    def __init__(self, norm: Norm, x: torch.Tensor, ctx, name: str, dtype: torch.dtype,
+                 rows: Optional[torch.Tensor] = None, n_rows: Optional[int] = None):
+        self.norm, self.x, self.ctx, self.name, self.dtype = norm, x, ctx, name, dtype
+        self.rows = rows
+        self.n_rows = int(n_rows if n_rows is not None else x.shape[0])
+        self._tensor: Optional[torch.Tensor] = None
+
+    @property
+    def shape(self):
+        return (self.n_rows, self.x.shape[1])
+
+    def rms(self):
+        """``(x, rows, weight, eps)`` for a fused kernel, or None."""
+        params = self.norm.rms_params()
+        if params is None:
+            return None
+        return self.x, self.rows, params[0], params[1]
+
+    def tensor(self) -> torch.Tensor:
+        if self._tensor is None:
+            out = self.ctx.scratch(self.name, (self.n_rows, self.x.shape[1]), self.dtype)
+            self.norm.forward(self.x, out, self.rows)
+            self._tensor = out
+        return self._tensor
+
 
 class PositionEncoding(Part):
     def rotary_table(self) -> Optional[torch.Tensor]:
@@ -73,6 +112,8 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
+    takes_normed_input = False     # True: ``forward`` gets a ``NormedInput`` and may fuse the norm
+
     def cache_spec(self) -> Optional[KVCacheSpec]:
         """Per-token cache need, or None."""
         return None
@@ -90,6 +131,8 @@ class Mixer(Part):
 
 
 class FeedForward(Part):
+    takes_normed_input = False
+
     def forward(self, h: torch.Tensor, residual: torch.Tensor, ctx) -> None:
         """``residual += feed_forward(h)``."""
         raise NotImplementedError

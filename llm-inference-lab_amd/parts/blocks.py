@@ -7,7 +7,7 @@ import torch
 
 from ..config.spec import PartSpec
 from ..weights.loader import TensorSpec, MATRIX
-from .base import Block, Part
+from .base import Block, Part, NormedInput
 from .registry import register_part, build_part
 
 
@@ -45,12 +45,11 @@ class PreNormBlock(Block):
             p.bind(tensors, ops, dtype)
 
     def forward(self, residual, ctx, entry):
-        rows = residual.shape[0]
-        h = ctx.scratch("block.normed", (rows, self.hidden_size), self.dtype)
-        self.norm1.forward(residual, h)
-        self.mixer.forward(h, residual, ctx, entry)
-        self.norm2.forward(residual, h)
-        self.feed_forward.forward(h, residual, ctx)
+        h = NormedInput(self.norm1, residual, ctx, "block.normed", self.dtype)
+        self.mixer.forward(h if self.mixer.takes_normed_input else h.tensor(), residual, ctx, entry)
+        h = NormedInput(self.norm2, residual, ctx, "block.normed", self.dtype)
+        self.feed_forward.forward(h if self.feed_forward.takes_normed_input else h.tensor(),
+                                  residual, ctx)
 
     def weight_bytes(self):
         return sum(p.weight_bytes() for p in self.parts())
@@ -96,8 +95,16 @@ class LinearHead(Part):
         super().bind(tensors, ops, dtype)
         self.weight = tensors[self.tensor_names["weight"]]
 
+    takes_normed_input = True
+
     def forward(self, h, out):
-        self.ops.linear_logits(h, self.weight, out)
+        rms = h.rms() if isinstance(h, NormedInput) else None
+        if rms is not None and self.ops.can_fuse(out.shape[0], self.dtype):
+            self.ops.fused_norm_logits(rms[0], rms[1], rms[2], rms[3], self.weight, out)
+        else:
+            if isinstance(h, NormedInput):
+                h = h.tensor()
+            self.ops.linear_logits(h, self.weight, out)
 
     def weight_bytes(self):
         return self.weight.numel() * self.weight.element_size()

@@ -6,7 +6,7 @@ from typing import Dict
 import torch
 
 from ..weights.loader import TensorSpec, MATRIX
-from .base import FeedForward
+from .base import FeedForward, NormedInput
 from .registry import register_part
 
 PAIR = 16   # rows of the gate matrix and of the up matrix alternate in runs of 16
@@ -61,10 +61,18 @@ class SwiGLU(FeedForward):
         self.w_gate_up = interleave_gate_up(tensors[t["gate_weight"]], tensors[t["up_weight"]])
         self.w_down = tensors[t["down_weight"]].contiguous()
 
+    takes_normed_input = True
+
     def forward(self, h, residual, ctx):
         rows = h.shape[0]
         act = ctx.scratch("swiglu.act", (rows, self.intermediate_size), self.dtype)
-        self.ops.linear_swiglu(h, self.w_gate_up, act)
+        rms = h.rms() if isinstance(h, NormedInput) else None
+        if rms is not None and self.ops.can_fuse(rows, self.dtype):
+            self.ops.fused_norm_swiglu(rms[0], rms[2], rms[3], self.w_gate_up, act)
+        else:
+            if isinstance(h, NormedInput):
+                h = h.tensor()
+            self.ops.linear_swiglu(h, self.w_gate_up, act)
         self.ops.linear_residual(act, self.w_down, residual, None)
 
     def weight_bytes(self):

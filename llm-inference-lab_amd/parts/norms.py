@@ -34,6 +34,9 @@ class RMSNorm(Norm):
     def forward(self, x, out, rows=None):
         self.ops.rmsnorm(x, self.weight, self.eps, out, rows)
 
+    def rms_params(self):
+        return self.weight, self.eps
+
     def weight_bytes(self):
         return self.weight.numel() * self.weight.element_size()
 

@@ -15,9 +15,10 @@ import torch
 
 
 class EmuOps:
-    def __init__(self, device="cpu"):
+    def __init__(self, device="cpu", fuse=True):
         self.device = torch.device(device)
         self.calls = {}
+        self.fuse = fuse
 
     def _count(self, name):
         self.calls[name] = self.calls.get(name, 0) + 1
@@ -68,6 +69,39 @@ class EmuOps:
         gate = y[:, :, 0, :].reshape(x.shape[0], -1)[:, :inter]
         up = y[:, :, 1, :].reshape(x.shape[0], -1)[:, :inter]
         out.copy_((gate / (1.0 + torch.exp(-gate)) * up).to(out.dtype))
+
+    # ------------------------------------------------- fused few-row kernels
+    FUSED_MAX_ROWS = 64
+
+    def can_fuse(self, rows, dtype):
+        return self.fuse and dtype == torch.bfloat16 and 0 < rows <= self.FUSED_MAX_ROWS
+
+    def _normed(self, x, rows_index, norm_w, eps, n):
+        v = x.float() if rows_index is None else x.float()[rows_index[:n].long()]
+        inv = torch.rsqrt((v * v).sum(-1, keepdim=True) / v.shape[-1] + eps)
+        # the kernel rounds x * w to bfloat16 and scales by inv_rms afterwards
+        return (v * norm_w.float()).to(torch.bfloat16).float() * inv
+
+    def fused_norm_qkv(self, x, norm_w, eps, w_qkv, b_qkv, num_heads, num_kv_heads, head_dim, inv_freq,
+                       positions, row_req, block_table, page_size, k_cache, v_cache, q_out):
+        self._count("fused_norm_qkv")
+        rows = x.shape[0]
+        y = self._normed(x, None, norm_w, eps, rows) @ w_qkv.float().t()
+        if b_qkv is not None:
+            y = y + b_qkv.float()
+        qkv = y.clone()                      # float32: the kernel rotates before it rounds
+        self.rope_kv_write(qkv, num_heads, num_kv_heads, head_dim, inv_freq, positions, row_req,
+                           block_table, page_size, k_cache, v_cache)
+        q_out.copy_(qkv[:, :num_heads * head_dim].to(q_out.dtype))
+
+    def fused_norm_swiglu(self, x, norm_w, eps, w_gate_up, out):
+        self._count("fused_norm_swiglu")
+        h = self._normed(x, None, norm_w, eps, x.shape[0])
+        self.linear_swiglu(h, w_gate_up, out)
+
+    def fused_norm_logits(self, x, rows_index, norm_w, eps, w, out):
+        self._count("fused_norm_logits")
+        out.copy_(self._normed(x, rows_index, norm_w, eps, out.shape[0]) @ w.float().t())
 
     # ------------------------------------------------------------------- rope
     @staticmethod

@@ -40,6 +40,24 @@ def test_every_cut_matches_plain(name, cut):
         assert sum(g["pages_high_water"] for g in m["groups"]) > 0
 
 
+@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("cut", ["decode", "mixed"])
+def test_few_row_steps_take_the_fused_operations(name, cut):
+    """bfloat16 steps of at most 64 rows fold the norm, the projections, the
+    rotation and the cache write into one operation each; the result is the same."""
+    seqs = sequences_of(name)
+    want = {rid: H.plain_logits(name, 1, ids) for rid, ids in seqs.items()}
+    engine = engine_of(name, "bf16", page_size=16, num_pages=14, max_requests=4)
+    steps = {"decode": H.steps_prefill_then_decode, "mixed": H.steps_mixed}[cut](seqs)
+    got = H.run_trace(engine, seqs, steps)
+    bad = H.first_wrong(got, want, H.TOL["bf16"])
+    assert bad is None, f"first wrong logits at (request, position, error) = {bad}"
+    calls = engine.ops.calls
+    assert calls["fused_norm_qkv"] > 0 and calls["fused_norm_swiglu"] > 0 and calls["fused_norm_logits"] > 0
+    if cut == "decode" and name == "B":
+        assert calls.get("rmsnorm", 0) > 0          # the long first portions take the general path
+
+
 def test_pages_are_reused_in_mixed():
     seqs = sequences_of("B", seed=3)
     engine = engine_of("B", "f32", page_size=16, num_pages=10)

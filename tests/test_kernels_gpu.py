@@ -148,6 +148,92 @@ def test_linear_swiglu(ops, emu, dtype, m, inter, k):
     close(got, want, dtype, f"linear_swiglu {m}x{inter}x{k}", want.float().abs().max().item())
 
 
+@pytest.mark.parametrize("m", [1, 3, 8, 16, 17, 32, 40, 64])
+@pytest.mark.parametrize("n,k", [(896, 896), (90, 96), (1000, 4864), (151936, 896), (65, 104), (3584, 18944)])
+def test_few_row_products(ops, emu, m, n, k):
+    """bfloat16 products of at most 64 rows take the block kernel with the K split
+    inside the block; every epilogue against the plain reference."""
+    if n * k > 40e6 and m not in (1, 8, 64):
+        pytest.skip("large case: three row counts are enough")
+    dtype = torch.bfloat16
+    x, w = rnd((m, k), dtype, 40), rnd((n, k), dtype, 41, 0.05)
+    bias = rnd((n,), torch.float32, 42)
+    want = torch.empty(m, n, dtype=dtype)
+    emu.linear(x, w, want, bias)
+    got = torch.empty(m, n, dtype=dtype, device=DEV)
+    ops.linear(x.to(DEV), w.to(DEV), got, bias.to(DEV))
+    close(got, want, dtype, "few-row linear", want.float().abs().max().item())
+    resid = rnd((m, n), torch.float32, 43)
+    want = resid.clone()
+    emu.linear_residual(x, w, want)
+    got = resid.clone().to(DEV)
+    ops.linear_residual(x.to(DEV), w.to(DEV), got)
+    close(got, want, torch.float32, "few-row residual", want.abs().max().item() * 4)
+
+
+@pytest.mark.parametrize("wdtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("m", [1, 8, 17, 33, 64])
+@pytest.mark.parametrize("hidden,inter,vocab", [(64, 128, 256), (96, 320, 515), (896, 4864, 3001), (72, 200, 301)])
+def test_fused_norm_products(ops, emu, wdtype, m, hidden, inter, vocab):
+    from llm_inference_lab_amd.parts.feed_forward import interleave_gate_up
+    bf = torch.bfloat16
+    x = rnd((m + 5, hidden), torch.float32, 50, 3.0)
+    nw = (1 + 0.1 * rnd((hidden,), torch.float32, 51)).to(wdtype)
+    eps = 1e-5
+    # SwiGLU
+    w = interleave_gate_up(rnd((inter, hidden), bf, 52, 0.1), rnd((inter, hidden), bf, 53, 0.1))
+    want = torch.empty(m, inter, dtype=bf)
+    emu.fused_norm_swiglu(x[:m], nw, eps, w, want)
+    got = torch.empty(m, inter, dtype=bf, device=DEV)
+    ops.fused_norm_swiglu(x[:m].contiguous().to(DEV), nw.to(DEV), eps, w.to(DEV), got)
+    close(got, want, bf, "fused norm + swiglu", want.float().abs().max().item())
+    # logits of gathered rows
+    head = rnd((vocab, hidden), bf, 54, 0.1)
+    idx = torch.randperm(m + 5, generator=torch.Generator().manual_seed(55))[:m].int()
+    want = torch.empty(m, vocab)
+    emu.fused_norm_logits(x, idx, nw, eps, head, want)
+    got = torch.empty(m, vocab, device=DEV)
+    ops.fused_norm_logits(x.to(DEV), idx.to(DEV), nw.to(DEV), eps, head.to(DEV), got)
+    close(got, want, torch.float32, "fused norm + logits", want.abs().max().item() * 40)
+
+
+@pytest.mark.parametrize("nq,nkv,d,page,hidden", [(4, 2, 16, 16, 64), (3, 1, 32, 32, 96), (14, 2, 64, 64, 896),
+                                                 (6, 3, 48, 16, 72), (8, 8, 128, 64, 256), (2, 1, 256, 16, 64)])
+@pytest.mark.parametrize("rotate", [True, False])
+def test_fused_norm_qkv_rope_write(ops, emu, nq, nkv, d, page, hidden, rotate):
+    bf = torch.bfloat16
+    rows_per, starts, reqs, num_pages = [5, 1, 9], [3, 40, 0], 3, 12
+    rows = sum(rows_per)
+    x = rnd((rows, hidden), torch.float32, 60, 2.0)
+    nw = (1 + 0.1 * rnd((hidden,), torch.float32, 61)).to(bf)
+    n = (nq + 2 * nkv) * d
+    w, b = rnd((n, hidden), bf, 62, 0.2), rnd((n,), bf, 63)
+    positions = torch.cat([torch.arange(s, s + c) for s, c in zip(starts, rows_per)]).int()
+    row_req = torch.cat([torch.full((c,), i) for i, c in enumerate(rows_per)]).int()
+    table = torch.full((reqs, 8), -1, dtype=torch.int32)
+    perm = torch.randperm(num_pages, generator=torch.Generator().manual_seed(64)).int()
+    at = 0
+    for i in range(reqs):
+        need = (starts[i] + rows_per[i] + page - 1) // page
+        table[i, :need] = perm[at:at + need]
+        at += need
+    inv_freq = (1.0 / (1e4 ** (torch.arange(0, d, 2, dtype=torch.float64) / d))).float() if rotate else None
+    kc, vc = make_cache(num_pages, nkv, page, d, bf, 65)
+    want_q, want_k, want_v = torch.empty(rows, nq * d, dtype=bf), kc.clone(), vc.clone()
+    emu.fused_norm_qkv(x, nw, 1e-6, w, b, nq, nkv, d, inv_freq, positions, row_req, table, page,
+                       want_k, want_v, want_q)
+    got_q, got_k, got_v = torch.empty(rows, nq * d, dtype=bf, device=DEV), kc.to(DEV), vc.to(DEV)
+    ops.fused_norm_qkv(x.to(DEV), nw.to(DEV), 1e-6, w.to(DEV), b.to(DEV), nq, nkv, d,
+                       None if inv_freq is None else inv_freq.to(DEV), positions.to(DEV), row_req.to(DEV),
+                       table.to(DEV), page, got_k, got_v, got_q)
+    scale = want_q.float().abs().max().item()
+    close(got_q, want_q, bf, "fused q", scale)
+    close(got_k, want_k, bf, "fused key cache", scale)
+    close(got_v, want_v, bf, "fused value cache", scale)
+    untouched = (want_k == kc)
+    assert torch.equal(got_k.cpu()[untouched], kc[untouched])
+
+
 def make_cache(num_pages, nkv, page, d, dtype, seed):
     k = rnd((num_pages, nkv, page, d), dtype, seed)
     v = rnd((num_pages, nkv, d, page), dtype, seed + 1)
