@@ -21,9 +21,11 @@
 // running maximum, the exponentials and the sums are float32; the softmax works in
 // base 2 (scores pre-multiplied by log2 e).
 //
-// Split keys (decode): blockIdx.y also counts splits of the key range; each split
-// writes its unnormalised sum, maximum and denominator, and a second kernel merges
-// them:  out = sum_s w_s acc_s / sum_s w_s l_s,  w_s = 2^(m_s - m).
+// Decode (at most 16 rows per request and kv head): the waves of a block split the
+// block's keys and merge their unnormalised sums, maxima and denominators through
+// LDS; blockIdx.y also counts splits of the key range over blocks.  Each such block
+// writes its merged partial result, and a second kernel merges the splits in their
+// order:  out = sum_s w_s acc_s / sum_s w_s l_s,  w_s = 2^(m_s - m).
 //
 // float32 kernel: one wave per (token, head), lanes over keys, plain FMA; true
 // 32-bit arithmetic.
@@ -54,10 +56,26 @@ struct AttnArgs {
 };
 
 // ------------------------------------------------------------- bf16, MFMA
-template <int QB>
-__global__ __launch_bounds__(256) void attention_bf16_kernel(AttnArgs a) {
+// The fragments of one step of 32 keys: two blocks of 16 keys, and the values of
+// those keys for every 16-wide block of d.
+template <int DC, int DB>
+struct KeyStep {
+  bf16x8 k[2][DC];
+  bf16x4 v[2][DB];
+  bool ok[2];
+};
+
+// DECODE = false: every wave owns a tile of 16*QB rows and walks all its keys.
+// DECODE = true (QB = 1, at most 16 rows per request and kv head): the waves of a
+// block share one tile and split the block's keys; they merge through LDS, and
+// blocks that split the keys further merge through global memory (see below).
+constexpr int DECODE_WAVES = D <= 64 ? 8 : (D <= 128 ? 4 : 2);
+
+template <int QB, bool DECODE>
+__global__ __launch_bounds__(DECODE ? 64 * DECODE_WAVES : 256) void attention_bf16_kernel(AttnArgs a) {
   constexpr int DC = (D + 31) / 32;  // 32-wide chunks of d for Q.K
   constexpr int DB = D / 16;         // 16-wide blocks of d for P.V
+  constexpr bool PIPE = DECODE;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
   const int c = lane & 15, g = lane >> 4;
   const int b = blockIdx.z;
@@ -65,14 +83,15 @@ __global__ __launch_bounds__(256) void attention_bf16_kernel(AttnArgs a) {
   const int G = a.nq / a.nkv;
   const int r0 = a.q_start[b], qlen = a.q_start[b + 1] - r0, sp = a.start_pos[b];
   const int rows_total = qlen * G;
-  const int row0 = (blockIdx.x * nw + wave) * (16 * QB);
-  if (row0 >= rows_total) return;
+  const int row0 = DECODE ? 0 : (blockIdx.x * nw + wave) * (16 * QB);
+  if (!DECODE && row0 >= rows_total) return;
   const bf16_t* q = (const bf16_t*)a.q;
   const bf16_t* kc = (const bf16_t*)a.kc;
   const bf16_t* vc = (const bf16_t*)a.vc;
   const int P = a.page_size;
   const float scale2 = a.scale * 1.4426950408889634f;
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+  const bf16x4 zero4 = {0, 0, 0, 0};
 
   // this lane's row in each 16-row block
   bool valid[QB];
@@ -94,15 +113,21 @@ __global__ __launch_bounds__(256) void attention_bf16_kernel(AttnArgs a) {
     }
   }
 
-  // keys this tile can see, and this split's share of them in blocks of 32
+  // keys this tile can see, and this split's share of them in steps of 32
   const int last_row = min(row0 + 16 * QB, rows_total) - 1;
   const int p_first = sp + row0 / G, p_last = sp + last_row / G;
   const int key_lo = a.window > 0 ? max(0, p_first - a.window + 1) : 0;
   const int key_hi = p_last;
   const int blk_lo = key_lo >> 5, blk_hi = key_hi >> 5;
   const int per = (blk_hi - blk_lo + 1 + a.splits - 1) / a.splits;
-  const int my_blk0 = blk_lo + split * per;
-  const int my_blk1 = min(my_blk0 + per, blk_hi + 1);
+  int my_blk0 = blk_lo + split * per;
+  int my_blk1 = min(my_blk0 + per, blk_hi + 1);
+  if constexpr (DECODE) {
+    // this wave's share of the block's steps
+    const int per_wave = (max(my_blk1 - my_blk0, 0) + nw - 1) / nw;
+    my_blk0 += wave * per_wave;
+    my_blk1 = min(my_blk0 + per_wave, my_blk1);
+  }
 
   floatx4 o[QB][DB];
   float m[QB], lsum[QB];
@@ -114,36 +139,52 @@ __global__ __launch_bounds__(256) void attention_bf16_kernel(AttnArgs a) {
     for (int db = 0; db < DB; ++db) o[qb][db] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
 
-  for (int blk = my_blk0; blk < my_blk1; ++blk) {
+  // issue the loads of one step: page numbers first, then key and value fragments
+  auto fetch = [&](int blk, KeyStep<DC, DB>& f) {
+    const int kb = blk << 5;
+#pragma unroll
+    for (int h2 = 0; h2 < 2; ++h2) {
+      const int pos16 = kb + h2 * 16;
+      bool ok = pos16 <= key_hi && pos16 + 15 >= key_lo;
+      int page = -1;
+      if (ok) page = a.table[(size_t)b * a.table_stride + pos16 / P];
+      ok = ok && page >= 0;
+      f.ok[h2] = ok;
+      if (ok) {
+        const int off = pos16 % P;
+        const bf16_t* kp = kc + (((size_t)page * a.nkv + kvh) * P + off + c) * D;
+        const bf16_t* vp = vc + ((size_t)page * a.nkv + kvh) * D * P + off + g * 4;
+#pragma unroll
+        for (int dc = 0; dc < DC; ++dc) {
+          const int dd = dc * 32 + g * 8;
+          f.k[h2][dc] = (dd < D) ? *(const bf16x8*)(kp + dd) : zero8;
+        }
+#pragma unroll
+        for (int db = 0; db < DB; ++db) f.v[h2][db] = *(const bf16x4*)(vp + (size_t)(db * 16 + c) * P);
+      } else {
+#pragma unroll
+        for (int dc = 0; dc < DC; ++dc) f.k[h2][dc] = zero8;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) f.v[h2][db] = zero4;
+      }
+    }
+  };
+
+  auto compute = [&](int blk, const KeyStep<DC, DB>& f) {
     const int kb = blk << 5;
     floatx4 s[2][QB];
-    bool ok[2];
-    const bf16_t* vbase[2];
 #pragma unroll
     for (int h2 = 0; h2 < 2; ++h2) {
 #pragma unroll
       for (int qb = 0; qb < QB; ++qb) s[h2][qb] = floatx4{0.f, 0.f, 0.f, 0.f};
-      const int pos16 = kb + h2 * 16;
-      ok[h2] = pos16 <= key_hi && pos16 + 15 >= key_lo;
-      int page = -1;
-      if (ok[h2]) page = a.table[(size_t)b * a.table_stride + pos16 / P];
-      ok[h2] = ok[h2] && page >= 0;
-      vbase[h2] = vc;
-      if (ok[h2]) {
-        const int off = pos16 % P;
-        const bf16_t* kp = kc + (((size_t)page * a.nkv + kvh) * P + off + c) * D;
-        vbase[h2] = vc + ((size_t)page * a.nkv + kvh) * D * P + off;
+      if (f.ok[h2]) {
 #pragma unroll
-        for (int dc = 0; dc < DC; ++dc) {
-          const int dd = dc * 32 + g * 8;
-          const bf16x8 kf = (dd < D) ? *(const bf16x8*)(kp + dd) : zero8;
+        for (int dc = 0; dc < DC; ++dc)
 #pragma unroll
           for (int qb = 0; qb < QB; ++qb)
-            s[h2][qb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf, qf[qb][dc], s[h2][qb], 0, 0, 0);
-        }
+            s[h2][qb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.k[h2][dc], qf[qb][dc], s[h2][qb], 0, 0, 0);
       }
     }
-
     bf16x8 pf[QB];
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
@@ -154,7 +195,7 @@ __global__ __launch_bounds__(256) void attention_bf16_kernel(AttnArgs a) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const int j = kb + h2 * 16 + g * 4 + i;
-          const bool vis = ok[h2] && valid[qb] && j <= pos[qb] && j >= lo[qb];
+          const bool vis = f.ok[h2] && valid[qb] && j <= pos[qb] && j >= lo[qb];
           const float v = vis ? s[h2][qb][i] * scale2 : NEG_INF;
           sv[h2 * 4 + i] = v;
           mx = fmaxf(mx, v);
@@ -176,16 +217,12 @@ __global__ __launch_bounds__(256) void attention_bf16_kernel(AttnArgs a) {
 #pragma unroll
       for (int db = 0; db < DB; ++db) o[qb][db] *= alpha;
     }
-
     // keys past the last written position hold stale values: keep them out of
     // the product even though their probability is zero
     const bool tail = kb + 31 > key_hi;
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
-      bf16x4 v0 = {0, 0, 0, 0}, v1 = {0, 0, 0, 0};
-      const size_t drow = (size_t)(db * 16 + c) * P + g * 4;
-      if (ok[0]) v0 = *(const bf16x4*)(vbase[0] + drow);
-      if (ok[1]) v1 = *(const bf16x4*)(vbase[1] + drow);
+      const bf16x4 v0 = f.v[0][db], v1 = f.v[1][db];
       bf16x8 vf = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
       if (tail) {
 #pragma unroll
@@ -198,55 +235,128 @@ __global__ __launch_bounds__(256) void attention_bf16_kernel(AttnArgs a) {
       for (int qb = 0; qb < QB; ++qb)
         o[qb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[qb], o[qb][db], 0, 0, 0);
     }
+  };
+
+  if constexpr (PIPE) {
+    // the next step's loads are in flight while this one is computed
+    KeyStep<DC, DB> cur, nxt;
+    if (my_blk0 < my_blk1) fetch(my_blk0, cur);
+    for (int blk = my_blk0; blk < my_blk1; ++blk) {
+      if (blk + 1 < my_blk1) fetch(blk + 1, nxt);
+      compute(blk, cur);
+      cur = nxt;
+    }
+  } else {
+    for (int blk = my_blk0; blk < my_blk1; ++blk) {
+      KeyStep<DC, DB> cur;
+      fetch(blk, cur);
+      compute(blk, cur);
+    }
   }
 
+  if constexpr (!DECODE) {
 #pragma unroll
-  for (int qb = 0; qb < QB; ++qb) {
-    float l = lsum[qb];
-    l += __shfl_xor(l, 16, WAVE);
-    l += __shfl_xor(l, 32, WAVE);
-    if (!valid[qb]) continue;
-    const size_t row = (size_t)(r0 + tok[qb]);
-    if (a.splits == 1) {
+    for (int qb = 0; qb < QB; ++qb) {
+      float l = lsum[qb];
+      l += __shfl_xor(l, 16, WAVE);
+      l += __shfl_xor(l, 32, WAVE);
+      if (!valid[qb]) continue;
       const float inv = l > 0.f ? 1.f / l : 0.f;
-      bf16_t* dst = (bf16_t*)a.out + row * a.out_stride + (size_t)head[qb] * D;
+      bf16_t* dst = (bf16_t*)a.out + (size_t)(r0 + tok[qb]) * a.out_stride + (size_t)head[qb] * D;
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
         bf16x4 w = {(bf16_t)(o[qb][db][0] * inv), (bf16_t)(o[qb][db][1] * inv),
                     (bf16_t)(o[qb][db][2] * inv), (bf16_t)(o[qb][db][3] * inv)};
         *(bf16x4*)(dst + db * 16 + g * 4) = w;
       }
-    } else {
-      const size_t at = (row * a.nq + head[qb]) * a.splits + split;
-      float* dst = a.o_part + at * D;
-#pragma unroll
-      for (int db = 0; db < DB; ++db) *(floatx4*)(dst + db * 16 + g * 4) = o[qb][db];
-      if (g == 0) {
-        a.ml_part[at * 2] = m[qb];
-        a.ml_part[at * 2 + 1] = l;
-      }
     }
+  } else {
+    // ---- merge the waves of the block through LDS
+    //   acc = sum_w 2^(m_w - m) acc_w,  l = sum_w 2^(m_w - m) l_w,  m = max_w m_w
+    __shared__ float s_m[DECODE_WAVES][16], s_l[DECODE_WAVES][16];
+    __shared__ __attribute__((aligned(16))) float s_o[DECODE_WAVES][16][D];
+    {
+      float l = lsum[0];
+      l += __shfl_xor(l, 16, WAVE);
+      l += __shfl_xor(l, 32, WAVE);
+      if (g == 0) {
+        s_m[wave][c] = m[0];
+        s_l[wave][c] = l;
+      }
+#pragma unroll
+      for (int db = 0; db < DB; ++db) *(floatx4*)(&s_o[wave][c][db * 16 + g * 4]) = o[0][db];
+    }
+    __syncthreads();
+    const int nrows = rows_total;     // <= 16
+    // sum the `count` entries of s_m / s_l / s_o in their order; write the result
+    // (final: normalised, to `out`; else: as this block's partial result)
+    auto merge = [&](int count, bool final) {
+      for (int idx = threadIdx.x; idx < nrows * D; idx += blockDim.x) {
+        const int r = idx / D, dd = idx - r * D;
+        float mmax = NEG_INF;
+        for (int w = 0; w < count; ++w) mmax = fmaxf(mmax, s_m[w][r]);
+        float num = 0.f, den = 0.f;
+        for (int w = 0; w < count; ++w) {
+          const float wt = s_m[w][r] == NEG_INF ? 0.f : exp2f(s_m[w][r] - mmax);
+          num += wt * s_o[w][r][dd];
+          den += wt * s_l[w][r];
+        }
+        const int t = r / G, hh = kvh * G + r % G;
+        if (final) {
+          ((bf16_t*)a.out)[(size_t)(r0 + t) * a.out_stride + (size_t)hh * D + dd] =
+              (bf16_t)(den > 0.f ? num / den : 0.f);
+        } else {
+          const size_t at = ((size_t)(r0 + t) * a.nq + hh) * a.splits + split;
+          a.o_part[at * D + dd] = num;
+          if (dd == 0) {
+            a.ml_part[at * 2] = mmax;
+            a.ml_part[at * 2 + 1] = den;
+          }
+        }
+      }
+    };
+    merge(nw, a.splits == 1);
   }
 }
 
-// out[row, head, :] = sum_s 2^(m_s - m) acc_s / sum_s 2^(m_s - m) l_s
-template <typename T>
-__global__ void attention_merge_kernel(const float* __restrict__ o_part,
-                                       const float* __restrict__ ml_part, T* __restrict__ out,
-                                       int out_stride, int nq, int splits) {
-  const int row = blockIdx.x, head = blockIdx.y;
-  const size_t base = ((size_t)row * nq + head) * splits;
-  float mmax = NEG_INF;
-  for (int s = 0; s < splits; ++s) mmax = fmaxf(mmax, ml_part[(base + s) * 2]);
-  for (int dd = threadIdx.x; dd < D; dd += blockDim.x) {
-    float num = 0.f, den = 0.f;
-    for (int s = 0; s < splits; ++s) {
-      const float ms = ml_part[(base + s) * 2];
-      const float w = ms == NEG_INF ? 0.f : exp2f(ms - mmax);
-      num += w * o_part[(base + s) * D + dd];
-      den += w * ml_part[(base + s) * 2 + 1];
+// Merge of the key splits of a decode step, one block per (row, head):
+//   out = sum_s w_s acc_s / sum_s w_s l_s,  w_s = 2^(m_s - max m), in the order of s.
+// A kernel of its own: within one kernel, results of blocks on other dies would
+// need device-wide fences, which cost far more than a launch.
+__global__ __launch_bounds__(64) void attention_merge_kernel(const float* __restrict__ o_part,
+                                                             const float* __restrict__ ml_part,
+                                                             bf16_t* __restrict__ out, int out_stride,
+                                                             int nq, int splits) {
+  const int row = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+  const size_t at0 = ((size_t)row * nq + head) * splits;
+  float ms = NEG_INF, ls = 0.f;
+  if (lane < splits) {
+    ms = ml_part[(at0 + lane) * 2];
+    ls = ml_part[(at0 + lane) * 2 + 1];
+  }
+  // every partial sum on its way before the first is used
+  constexpr int PER = (D + 63) / 64;
+  float v[PER][16];
+#pragma unroll
+  for (int p = 0; p < PER; ++p)
+#pragma unroll
+    for (int u = 0; u < 16; ++u) {
+      const int dd = p * 64 + lane;
+      v[p][u] = (u < splits && dd < D) ? o_part[(at0 + u) * D + dd] : 0.f;
     }
-    out[(size_t)row * out_stride + (size_t)head * D + dd] = from_float<T>(den > 0.f ? num / den : 0.f);
+  const float mmax = wave_max(ms);
+  const float w = ms == NEG_INF ? 0.f : exp2f(ms - mmax);
+  const float wl = w * ls;
+  float den = 0.f;
+  for (int s2 = 0; s2 < splits; ++s2) den += __shfl(wl, s2, WAVE);
+  const float inv = den > 0.f ? 1.f / den : 0.f;
+#pragma unroll
+  for (int p = 0; p < PER; ++p) {
+    float num = 0.f;
+#pragma unroll
+    for (int u = 0; u < 16; ++u) num += __shfl(w, u, WAVE) * v[p][u];
+    const int dd = p * 64 + lane;
+    if (dd < D) out[(size_t)row * out_stride + (size_t)head * D + dd] = (bf16_t)(num * inv);
   }
 }
 
@@ -340,31 +450,30 @@ extern "C" int llmlab_paged_attention(const void* q, int dtype, int q_stride, in
   const int G = nq / nkv;
   const long max_rows = (long)max_q_len * G;
   if (max_rows <= 16) {
-    // decode-like step: one wave per (request, kv head, split)
-    int splits = 1;
-    const long base = (long)reqs * nkv;
+    // decode-like step: a block of DECODE_WAVES waves per (request, kv head, split);
+    // a wave gets about two steps of 32 keys, a block's waves merge in LDS, and only
+    // what is left is split over blocks
     const int visible = window > 0 ? min(window, max_ctx_len) : max_ctx_len;
-    const int blocks32 = (visible + 31) / 32 + 1;
-    if (base < 4L * num_cus) {
-      splits = (int)((4L * num_cus + base - 1) / base);
-      const int cap = blocks32 / 4 > 0 ? blocks32 / 4 : 1;   // at least 128 keys per split
-      if (splits > cap) splits = cap;
-      if (splits > 64) splits = 64;
-      const size_t per_split = (size_t)total_rows * nq * (D + 2);
-      while (splits > 1 && per_split * splits > workspace_floats) --splits;
-    }
+    const int steps32 = (visible + 31) / 32 + 1;
+    int splits = (steps32 + 2 * DECODE_WAVES - 1) / (2 * DECODE_WAVES);
+    const long base = (long)reqs * nkv;
+    const long room = (16L * num_cus + base - 1) / base;      // blocks per (request, kv head) worth having
+    if (splits > room) splits = (int)room;
+    if (splits > 16) splits = 16;                               // what the merge kernel takes
+    const size_t per_split = (size_t)total_rows * nq * (D + 2);
+    while (splits > 1 && per_split * splits > workspace_floats) --splits;
+    if (splits < 1) splits = 1;
     a.splits = splits;
     if (splits > 1) {
       a.o_part = workspace;
       a.ml_part = workspace + (size_t)total_rows * nq * splits * D;
     }
-    dim3 grid(1, nkv * splits, reqs), block(64);
-    hipLaunchKernelGGL(attention_bf16_kernel<1>, grid, block, 0, stream, a);
+    dim3 grid(1, nkv * splits, reqs), block(64 * DECODE_WAVES);
+    hipLaunchKernelGGL((attention_bf16_kernel<1, true>), grid, block, 0, stream, a);
     LLMLAB_LAUNCH_CHECK("attention(bfloat16, decode)");
     if (splits > 1) {
-      dim3 mgrid(total_rows, nq), mblock(64);
-      hipLaunchKernelGGL(attention_merge_kernel<bf16_t>, mgrid, mblock, 0, stream, a.o_part, a.ml_part,
-                         (bf16_t*)out, out_stride, nq, splits);
+      hipLaunchKernelGGL(attention_merge_kernel, dim3(total_rows, nq), dim3(64), 0, stream, a.o_part,
+                         a.ml_part, (bf16_t*)out, out_stride, nq, splits);
       LLMLAB_LAUNCH_CHECK("attention merge");
     }
     return 0;
@@ -372,7 +481,7 @@ extern "C" int llmlab_paged_attention(const void* q, int dtype, int q_stride, in
   constexpr int QB = 2;
   const int rows_per_block = 4 * 16 * QB;
   dim3 grid((unsigned)((max_rows + rows_per_block - 1) / rows_per_block), nkv, reqs), block(256);
-  hipLaunchKernelGGL(attention_bf16_kernel<QB>, grid, block, 0, stream, a);
+  hipLaunchKernelGGL((attention_bf16_kernel<QB, false>), grid, block, 0, stream, a);
   LLMLAB_LAUNCH_CHECK("attention(bfloat16, prefill)");
   return 0;
 }

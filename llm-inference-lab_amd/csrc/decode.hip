@@ -9,18 +9,26 @@
 //
 // A block owns `nsb` strips of 16 weight rows (for the q/k/v projection: exactly one
 // head) and splits K over `kw` waves per strip, so blockDim = 64 * nsb * kw.  Every
-// wave streams its slice of W from HBM straight into MFMA B fragments with several
-// 16-byte loads in flight per lane, multiplies with the A fragments of all rows, and
-// leaves its partial sums in LDS; the block adds the partial sums in a fixed order
-// (no atomics, results do not depend on timing) and applies the epilogue.
+// wave streams its slice of W from HBM straight into MFMA B fragments (loads of the
+// next steps are in flight while the current ones are multiplied), and leaves its
+// partial sums in LDS; the block adds the partial sums in a fixed order (no
+// atomics, results do not depend on timing) and applies the epilogue.
 //
-// The norm is folded in without a pass of its own:  norm(x) . W^T  =
-// inv_rms[m] * ((x * w_norm) . W^T).  The waves read x (float32) anyway to build
-// their A fragments, so each also sums the squares of its slice; the block adds
-// those and scales the reduced sums by inv_rms[m] in the epilogue.
+// The rows of x are staged once per block in LDS as bfloat16 when they fit
+// (STAGE), so the strips of a block share them; otherwise every wave reads its
+// slice from global memory.  The norm is folded in without a pass of its own:
+//   norm(x) . W^T = inv_rms[m] * ((x * w_norm) . W^T)
+// x * w_norm is what is staged (or built on the fly), the sum of squares falls out
+// of the same read, and inv_rms[m] scales the reduced sums in the epilogue.
+//
+// What the epilogue needs from global memory (bias, positions, page numbers,
+// rotary frequencies) is fetched into LDS at the start of the kernel, so those
+// latencies overlap the weight stream instead of following it.
 //
 // Fragment layout of v_mfma_f32_16x16x32_bf16 (lane l): A row l%16, B column l%16,
 // k = 8*(l/16)..+7; result element i: row 4*(l/16)+i, column l%16.
+#include <stdlib.h>
+
 #include "common.h"
 
 enum { SK_STORE = 0, SK_RESID = 1, SK_F32 = 2, SK_SWIGLU = 3, SK_QKV = 4 };
@@ -42,30 +50,60 @@ struct SkinnyArgs {
   int M, N, K, ldo, n_out;
   int norm_w_bf16, bias_bf16;
   int nsb, kw;
+  int qsplit;   // QKV: blocks per head (1, or d/32: a block then owns the strips p and p + d/32)
   int nq, nkv, d, table_stride, page_size;
   float eps;
 };
 
 __device__ __forceinline__ float sk_silu(float z) { return z / (1.f + __expf(-z)); }
 
-template <int MB, int EPI, bool NORM>
+constexpr int SK_APAD = 8;   // padding of a staged row, in elements: 16-byte reads of 8 lanes cover all banks
+
+// floats of LDS before the staged rows (host and device must agree)
+__host__ __device__ inline size_t sk_float_words(int nsb, int kw, int mb, int M, int epi) {
+  size_t f = (size_t)kw * nsb * mb * 256;        // partial sums
+  f += (size_t)kw * mb * 16 + (size_t)mb * 16;    // sums of squares, inverse rms
+  f += (size_t)16 * nsb;                          // bias
+  f += (size_t)mb * 16 * 2 + 128;                 // positions, pages, frequencies
+  if (epi == SK_SWIGLU || epi == SK_QKV) f += (size_t)M * 16 * nsb;
+  return (f + 3) & ~(size_t)3;
+}
+
+template <int MB, int EPI, bool NORM, bool STAGE>
 __global__ __launch_bounds__(MB >= 4 ? 512 : 1024) void skinny_block_kernel(SkinnyArgs a) {
   extern __shared__ __attribute__((aligned(16))) float smem[];
-  constexpr int U = (MB >= 2) ? 2 : 4;   // steps of 32 in flight
+  constexpr int U = STAGE ? 4 : (NORM ? (MB >= 2 ? 2 : 4) : (MB >= 4 ? 2 : (MB == 2 ? 4 : 8)));
   const int nsb = a.nsb, kw = a.kw;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
   const int strip = wave % nsb, ks = wave / nsb;
   const int c = lane & 15, g = lane >> 4;
   const int cols = 16 * nsb;
   const int n0 = blockIdx.x * cols;
   const int K = a.K, M = a.M;
-  // LDS: partial sums, then sums of squares, inverse rms, and the output tile
+
   float* part = smem;                                   // [kw*nsb][MB][64][4]
   float* ss_part = part + (size_t)kw * nsb * MB * 256;  // [kw][MB*16]
   float* inv = ss_part + kw * MB * 16;                  // [MB*16]
-  float* tile = inv + MB * 16;                          // [M][cols]   (SWIGLU, QKV)
+  float* s_bias = inv + MB * 16;                        // [cols]
+  int* s_pos = (int*)(s_bias + cols);                   // [MB*16]
+  int* s_page = s_pos + MB * 16;                        // [MB*16]
+  float* s_freq = (float*)(s_page + MB * 16);           // [128]
+  float* tile = s_freq + 128;                           // [M][cols]   (SWIGLU, QKV)
+  bf16_t* As = (bf16_t*)(smem + sk_float_words(nsb, kw, MB, M, EPI));   // [MB*16][K + SK_APAD]
+  const int lda = K + SK_APAD;
 
-  const int n = n0 + strip * 16 + c;
+  // QKV with qsplit > 1: block = (head, p); its two strips are columns p*16.. and
+  // d/2 + p*16.. of the head, i.e. both halves of the rotary pairs
+  int qhead = 0, qp = 0;
+  if constexpr (EPI == SK_QKV) {
+    qhead = blockIdx.x / a.qsplit;
+    qp = blockIdx.x - qhead * a.qsplit;
+  }
+  auto head_col = [&](int col) {   // column of the block -> column of the head
+    if (a.qsplit == 1) return col;
+    return col < 16 ? qp * 16 + col : (a.d >> 1) + qp * 16 + (col - 16);
+  };
+  const int n = (EPI == SK_QKV) ? qhead * a.d + head_col(strip * 16 + c) : n0 + strip * 16 + c;
   const bool wok = n < a.N;
   const bf16_t* wrow = a.W + (size_t)(wok ? n : 0) * K;
   const int steps = (K + 31) >> 5;
@@ -73,100 +111,198 @@ __global__ __launch_bounds__(MB >= 4 ? 512 : 1024) void skinny_block_kernel(Skin
   const int s_begin = ks * per;
   const int s_end = min(steps, s_begin + per);
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  const floatx4 fzero = {0.f, 0.f, 0.f, 0.f};
+
+  // ---- what the epilogue needs from global memory, fetched now
+  for (int i = threadIdx.x; i < cols; i += blockDim.x) {
+    const int nn = (EPI == SK_QKV) ? qhead * a.d + head_col(i) : n0 + i;
+    s_bias[i] = (a.bias && nn < a.N) ? load_vec(a.bias, a.bias_bf16, nn) : 0.f;
+  }
+  if constexpr (EPI == SK_QKV) {
+    const int head = qhead;
+    for (int m = threadIdx.x; m < M; m += blockDim.x) {
+      const int pos = a.positions[m];
+      s_pos[m] = pos;
+      s_page[m] = (a.kcache && head >= a.nq)
+                      ? a.table[(size_t)a.row_req[m] * a.table_stride + pos / a.page_size] : 0;
+    }
+    for (int i = threadIdx.x; i < (a.d >> 1); i += blockDim.x)
+      s_freq[i] = a.inv_freq ? a.inv_freq[i] : 0.f;
+  }
 
   floatx4 acc[MB];
-  float ss[MB];
-  const float* xf[MB];
-  const bf16_t* xb[MB];
-  bool aok[MB];
 #pragma unroll
-  for (int mb = 0; mb < MB; ++mb) {
-    acc[mb] = floatx4{0.f, 0.f, 0.f, 0.f};
-    ss[mb] = 0.f;
-    const int m = mb * 16 + c;
-    aok[mb] = m < M;
-    const size_t row = aok[mb] ? (size_t)((NORM && a.x_rows) ? a.x_rows[m] : m) : 0;
-    xf[mb] = (const float*)a.x + row * K;
-    xb[mb] = (const bf16_t*)a.x + row * K;
-  }
+  for (int mb = 0; mb < MB; ++mb) acc[mb] = fzero;
 
-  for (int s0 = s_begin; s0 < s_end; s0 += U) {
-    bf16x8 b[U];
-    floatx4 x0[U][MB], x1[U][MB];
-    bf16x8 ab[U][MB];
-    floatx4 w0[U], w1[U];
-    bf16x8 wb[U];
+  if constexpr (STAGE) {
+    // ---- first weight fragments on their way, then stage the rows of x
+    bf16x8 bcur[U], bnext[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int kk = (s0 + u) * 32 + g * 8;
-      const bool kok = (s0 + u) < s_end && kk < K;
-      b[u] = (wok && kok) ? *(const bf16x8*)(wrow + kk) : zero;
-      if constexpr (NORM) {
-        if (a.norm_w_bf16) {
-          wb[u] = kok ? *(const bf16x8*)((const bf16_t*)a.norm_w + kk) : zero;
-        } else {
-          w0[u] = kok ? *(const floatx4*)((const float*)a.norm_w + kk) : floatx4{0.f, 0.f, 0.f, 0.f};
-          w1[u] = kok ? *(const floatx4*)((const float*)a.norm_w + kk + 4) : floatx4{0.f, 0.f, 0.f, 0.f};
-        }
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb) {
-          const bool ok = aok[mb] && kok;
-          x0[u][mb] = ok ? *(const floatx4*)(xf[mb] + kk) : floatx4{0.f, 0.f, 0.f, 0.f};
-          x1[u][mb] = ok ? *(const floatx4*)(xf[mb] + kk + 4) : floatx4{0.f, 0.f, 0.f, 0.f};
-        }
-      } else {
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
-          ab[u][mb] = (aok[mb] && kok) ? *(const bf16x8*)(xb[mb] + kk) : zero;
-      }
+      const int kk = (s_begin + u) * 32 + g * 8;
+      bcur[u] = (wok && (s_begin + u) < s_end && kk < K) ? *(const bf16x8*)(wrow + kk) : zero;
+      bnext[u] = zero;
     }
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb) {
-        bf16x8 av;
-        if constexpr (NORM) {
+    const int chunks = K >> 3;
+    for (int r = wave; r < MB * 16; r += nwaves) {
+      bf16_t* dst = As + (size_t)r * lda;
+      if (r >= M) {
+        for (int ch = lane; ch < chunks; ch += 64) *(bf16x8*)(dst + ch * 8) = zero;
+        if (lane == 0) inv[r] = 0.f;
+        continue;
+      }
+      if constexpr (NORM) {
+        const float* src = (const float*)a.x + (size_t)(a.x_rows ? a.x_rows[r] : r) * K;
+        float ssq = 0.f;
+        for (int ch = lane; ch < chunks; ch += 64) {
+          const floatx4 p = *(const floatx4*)(src + ch * 8), q = *(const floatx4*)(src + ch * 8 + 4);
           float wv[8];
           if (a.norm_w_bf16) {
+            const bf16x8 w8 = *(const bf16x8*)((const bf16_t*)a.norm_w + ch * 8);
 #pragma unroll
-            for (int j = 0; j < 8; ++j) wv[j] = (float)wb[u][j];
+            for (int j = 0; j < 8; ++j) wv[j] = (float)w8[j];
           } else {
+            const floatx4 w0 = *(const floatx4*)((const float*)a.norm_w + ch * 8);
+            const floatx4 w1 = *(const floatx4*)((const float*)a.norm_w + ch * 8 + 4);
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-              wv[j] = w0[u][j];
-              wv[4 + j] = w1[u][j];
+              wv[j] = w0[j];
+              wv[4 + j] = w1[j];
             }
           }
+          bf16x8 av;
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            const float p = x0[u][mb][j], q = x1[u][mb][j];
-            ss[mb] += p * p + q * q;
-            av[j] = (bf16_t)(p * wv[j]);
-            av[4 + j] = (bf16_t)(q * wv[4 + j]);
+            ssq += p[j] * p[j] + q[j] * q[j];
+            av[j] = (bf16_t)(p[j] * wv[j]);
+            av[4 + j] = (bf16_t)(q[j] * wv[4 + j]);
+          }
+          *(bf16x8*)(dst + ch * 8) = av;
+        }
+        ssq = wave_sum(ssq);
+        if (lane == 0) inv[r] = rsqrtf(ssq / (float)K + a.eps);
+      } else {
+        const bf16_t* src = (const bf16_t*)a.x + (size_t)r * K;
+        for (int ch = lane; ch < chunks; ch += 64) *(bf16x8*)(dst + ch * 8) = *(const bf16x8*)(src + ch * 8);
+      }
+    }
+    __syncthreads();
+    for (int s0 = s_begin; s0 < s_end; s0 += U) {
+      if (s0 + U < s_end) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const int kk = (s0 + U + u) * 32 + g * 8;
+          bnext[u] = (wok && (s0 + U + u) < s_end && kk < K) ? *(const bf16x8*)(wrow + kk) : zero;
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (s0 + u < s_end) {
+          const int kk = (s0 + u) * 32 + g * 8;
+          const bool kok = kk < K;
+#pragma unroll
+          for (int mb = 0; mb < MB; ++mb) {
+            const bf16x8 av = kok ? *(const bf16x8*)(As + (size_t)(mb * 16 + c) * lda + kk) : zero;
+            acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, bcur[u], acc[mb], 0, 0, 0);
+          }
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) bcur[u] = bnext[u];
+    }
+  } else {
+    // ---- rows of x straight from global memory
+    float ss[MB];
+    const float* xf[MB];
+    const bf16_t* xb[MB];
+    bool aok[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+      ss[mb] = 0.f;
+      const int m = mb * 16 + c;
+      aok[mb] = m < M;
+      const size_t row = aok[mb] ? (size_t)((NORM && a.x_rows) ? a.x_rows[m] : m) : 0;
+      xf[mb] = (const float*)a.x + row * K;
+      xb[mb] = (const bf16_t*)a.x + row * K;
+    }
+    for (int s0 = s_begin; s0 < s_end; s0 += U) {
+      bf16x8 b[U];
+      floatx4 x0[U][MB], x1[U][MB];
+      bf16x8 ab[U][MB];
+      floatx4 w0[U], w1[U];
+      bf16x8 wb[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int kk = (s0 + u) * 32 + g * 8;
+        const bool kok = (s0 + u) < s_end && kk < K;
+        b[u] = (wok && kok) ? *(const bf16x8*)(wrow + kk) : zero;
+        if constexpr (NORM) {
+          if (a.norm_w_bf16) {
+            wb[u] = kok ? *(const bf16x8*)((const bf16_t*)a.norm_w + kk) : zero;
+          } else {
+            w0[u] = kok ? *(const floatx4*)((const float*)a.norm_w + kk) : fzero;
+            w1[u] = kok ? *(const floatx4*)((const float*)a.norm_w + kk + 4) : fzero;
+          }
+#pragma unroll
+          for (int mb = 0; mb < MB; ++mb) {
+            const bool ok = aok[mb] && kok;
+            x0[u][mb] = ok ? *(const floatx4*)(xf[mb] + kk) : fzero;
+            x1[u][mb] = ok ? *(const floatx4*)(xf[mb] + kk + 4) : fzero;
           }
         } else {
-          av = ab[u][mb];
+#pragma unroll
+          for (int mb = 0; mb < MB; ++mb)
+            ab[u][mb] = (aok[mb] && kok) ? *(const bf16x8*)(xb[mb] + kk) : zero;
         }
-        acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, b[u], acc[mb], 0, 0, 0);
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) {
+          bf16x8 av;
+          if constexpr (NORM) {
+            float wv[8];
+            if (a.norm_w_bf16) {
+#pragma unroll
+              for (int j = 0; j < 8; ++j) wv[j] = (float)wb[u][j];
+            } else {
+#pragma unroll
+              for (int j = 0; j < 4; ++j) {
+                wv[j] = w0[u][j];
+                wv[4 + j] = w1[u][j];
+              }
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              const float p = x0[u][mb][j], q = x1[u][mb][j];
+              ss[mb] += p * p + q * q;
+              av[j] = (bf16_t)(p * wv[j]);
+              av[4 + j] = (bf16_t)(q * wv[4 + j]);
+            }
+          } else {
+            av = ab[u][mb];
+          }
+          acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, b[u], acc[mb], 0, 0, 0);
+        }
+      }
+    }
+    if constexpr (NORM) {
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) {
+        float v = ss[mb];
+        v += __shfl_xor(v, 16, WAVE);
+        v += __shfl_xor(v, 32, WAVE);
+        if (strip == 0 && g == 0) ss_part[(ks * MB + mb) * 16 + c] = v;
       }
     }
   }
 
-  // partial sums to LDS
+  // ---- partial sums to LDS
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb)
     *(floatx4*)(part + (((size_t)wave * MB + mb) * 64 + lane) * 4) = acc[mb];
-  if constexpr (NORM) {
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-      float v = ss[mb];
-      v += __shfl_xor(v, 16, WAVE);
-      v += __shfl_xor(v, 32, WAVE);
-      if (strip == 0 && g == 0) ss_part[(ks * MB + mb) * 16 + c] = v;
-    }
-  }
   __syncthreads();
-  if constexpr (NORM) {
+  if constexpr (NORM && !STAGE) {
     if ((int)threadIdx.x < MB * 16) {
       const int mb = threadIdx.x >> 4, cc = threadIdx.x & 15;
       float t = 0.f;
@@ -176,7 +312,7 @@ __global__ __launch_bounds__(MB >= 4 ? 512 : 1024) void skinny_block_kernel(Skin
     __syncthreads();
   }
 
-  // reduce over the K slices in a fixed order; epilogue
+  // ---- reduce over the K slices in a fixed order; epilogue
   for (int idx = threadIdx.x; idx < M * cols; idx += blockDim.x) {
     const int m = idx / cols, col = idx - m * cols;
     const int st = col >> 4, cc = col & 15;
@@ -185,8 +321,8 @@ __global__ __launch_bounds__(MB >= 4 ? 512 : 1024) void skinny_block_kernel(Skin
     for (int k2 = 0; k2 < kw; ++k2)
       sum += part[((((size_t)k2 * nsb + st) * MB + mb) * 64 + gg * 16 + cc) * 4 + xx];
     if constexpr (NORM) sum *= inv[m];
+    sum += s_bias[col];
     const int nn = n0 + col;
-    if (nn < a.N && a.bias) sum += load_vec(a.bias, a.bias_bf16, nn);
     if constexpr (EPI == SK_SWIGLU || EPI == SK_QKV) {
       tile[idx] = sum;
     } else if (nn < a.N) {
@@ -209,16 +345,19 @@ __global__ __launch_bounds__(MB >= 4 ? 512 : 1024) void skinny_block_kernel(Skin
   }
   if constexpr (EPI == SK_QKV) {
     __syncthreads();
-    // this block is head `blockIdx.x` of [q heads | k heads | v heads]
-    const int head = blockIdx.x, d = a.d, half = d >> 1;
+    // this block is (part of) head `qhead` of [q heads | k heads | v heads]; its tile
+    // holds the low halves of its rotary pairs in the first half of its columns
+    const int head = qhead, d = a.d, dhalf = d >> 1, half = cols >> 1;
+    const int i0 = a.qsplit == 1 ? 0 : qp * 16;
     const bool is_q = head < a.nq, is_k = !is_q && head < a.nq + a.nkv;
     for (int idx = threadIdx.x; idx < M * half; idx += blockDim.x) {
-      const int m = idx / half, i = idx - m * half;
-      float lo = tile[m * cols + i], hi = tile[m * cols + i + half];
-      const int pos = a.positions[m];
+      const int m = idx / half, il = idx - m * half;
+      const int i = i0 + il;                      // pair index within the head
+      float lo = tile[m * cols + il], hi = tile[m * cols + il + half];
+      const int pos = s_pos[m];
       if ((is_q || is_k) && a.inv_freq) {
         float s, co;
-        sincosf((float)pos * a.inv_freq[i], &s, &co);
+        sincosf((float)pos * s_freq[i], &s, &co);
         const float nlo = lo * co - hi * s, nhi = hi * co + lo * s;
         lo = nlo;
         hi = nhi;
@@ -226,18 +365,18 @@ __global__ __launch_bounds__(MB >= 4 ? 512 : 1024) void skinny_block_kernel(Skin
       if (is_q) {
         bf16_t* dst = (bf16_t*)a.out + (size_t)m * a.ldo + (size_t)head * d;
         dst[i] = (bf16_t)lo;
-        dst[i + half] = (bf16_t)hi;
+        dst[i + dhalf] = (bf16_t)hi;
       } else if (a.kcache) {
-        const size_t page = (size_t)a.table[(size_t)a.row_req[m] * a.table_stride + pos / a.page_size];
+        const size_t page = (size_t)s_page[m];
         const int off = pos % a.page_size;
         if (is_k) {
           bf16_t* dst = a.kcache + ((page * a.nkv + (head - a.nq)) * a.page_size + off) * (size_t)d;
           dst[i] = (bf16_t)lo;
-          dst[i + half] = (bf16_t)hi;
+          dst[i + dhalf] = (bf16_t)hi;
         } else {
           bf16_t* dst = a.vcache + ((page * a.nkv + (head - a.nq - a.nkv)) * (size_t)d) * a.page_size + off;
           dst[(size_t)i * a.page_size] = (bf16_t)lo;
-          dst[(size_t)(i + half) * a.page_size] = (bf16_t)hi;
+          dst[(size_t)(i + dhalf) * a.page_size] = (bf16_t)hi;
         }
       }
     }
@@ -245,23 +384,114 @@ __global__ __launch_bounds__(MB >= 4 ? 512 : 1024) void skinny_block_kernel(Skin
 }
 
 // ---------------------------------------------------------------- dispatch
-static size_t skinny_lds_bytes(int nsb, int kw, int mb, int M, int epi) {
-  size_t floats = (size_t)kw * nsb * mb * 256 + (size_t)kw * mb * 16 + (size_t)mb * 16;
-  if (epi == SK_SWIGLU || epi == SK_QKV) floats += (size_t)M * 16 * nsb;
-  return floats * sizeof(float);
+static size_t skinny_lds_bytes(int nsb, int kw, int mb, int M, int K, int epi, bool stage) {
+  size_t bytes = sk_float_words(nsb, kw, mb, M, epi) * sizeof(float);
+  if (stage) bytes += (size_t)mb * 16 * (K + SK_APAD) * sizeof(bf16_t);
+  return bytes;
 }
 
-template <int MB, int EPI, bool NORM>
-static void skinny_launch(const SkinnyArgs& a, int blocks, size_t lds, hipStream_t stream) {
-  hipLaunchKernelGGL((skinny_block_kernel<MB, EPI, NORM>), dim3(blocks), dim3(64 * a.nsb * a.kw), lds,
-                     stream, a);
+// Most LDS a block may take (a compute unit of gfx950 has 160 KB).
+static const size_t SK_LDS_LIMIT = 152 * 1024;
+
+template <int MB, int EPI, bool NORM, bool STAGE>
+static int skinny_launch(const SkinnyArgs& a, int blocks, size_t lds, hipStream_t stream) {
+  auto kernel = skinny_block_kernel<MB, EPI, NORM, STAGE>;
+  if (lds > 48 * 1024) {
+    static size_t raised = 0;     // per instantiation
+    if (lds > raised) {
+      if (hipFuncSetAttribute((const void*)kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                              (int)SK_LDS_LIMIT) != hipSuccess) {
+        llmlab_set_error("skinny_linear: cannot raise the LDS limit to %zu bytes", SK_LDS_LIMIT);
+        return 3;
+      }
+      raised = SK_LDS_LIMIT;
+    }
+  }
+  hipLaunchKernelGGL(kernel, dim3(blocks), dim3(64 * a.nsb * a.kw), lds, stream, a);
+  return 0;
+}
+
+template <int EPI, bool NORM, bool STAGE>
+static int skinny_launch_mb(const SkinnyArgs& a, int mb, int blocks, size_t lds, hipStream_t stream) {
+  if (mb == 1) return skinny_launch<1, EPI, NORM, STAGE>(a, blocks, lds, stream);
+  if (mb == 2) return skinny_launch<2, EPI, NORM, STAGE>(a, blocks, lds, stream);
+  return skinny_launch<4, EPI, NORM, STAGE>(a, blocks, lds, stream);
 }
 
 template <int EPI, bool NORM>
-static void skinny_launch_mb(const SkinnyArgs& a, int mb, int blocks, size_t lds, hipStream_t stream) {
-  if (mb == 1) skinny_launch<1, EPI, NORM>(a, blocks, lds, stream);
-  else if (mb == 2) skinny_launch<2, EPI, NORM>(a, blocks, lds, stream);
-  else skinny_launch<4, EPI, NORM>(a, blocks, lds, stream);
+static int skinny_launch_stage(const SkinnyArgs& a, bool stage, int mb, int blocks, size_t lds,
+                               hipStream_t stream) {
+  if (stage) return skinny_launch_mb<EPI, NORM, true>(a, mb, blocks, lds, stream);
+  return skinny_launch_mb<EPI, NORM, false>(a, mb, blocks, lds, stream);
+}
+
+// A choice of block shape can be forced for measurements (0 = choose).
+static int g_force_nsb = 0, g_force_kw = 0, g_force_stage = -1;
+extern "C" void llmlab_skinny_force(int nsb, int kw, int stage) {
+  g_force_nsb = nsb;
+  g_force_kw = kw;
+  g_force_stage = stage;
+}
+
+struct SkinnyShape {
+  int nsb, kw;
+  bool stage;
+  int qsplit;
+};
+
+// Pick strips per block, K slices per strip and staging by an estimate of the
+// kernel's time: a fixed part, plus what the busiest compute unit needs to stream
+// its share of W and of x (a unit sustains far less than 1/256 of the chip's
+// bandwidth would suggest, so spreading the matrix over all units matters most),
+// or the memory round trips of a wave if those take longer.
+static SkinnyShape skinny_choose(int epilogue, bool norm, int mb, int M, int N, int K, int d, int num_cus) {
+  const int steps = (K + 31) / 32;
+  const int strips = (N + 15) / 16;
+  const int max_waves = mb >= 4 ? 8 : 16;
+  SkinnyShape best{0, 0, false, 1};
+  double best_cost = 1e30;
+  int cand[5], ncand = 0;
+  if (epilogue == SK_QKV) {
+    cand[ncand++] = d / 16;                   // a block per head
+    if (d % 32 == 0 && d > 32) cand[ncand++] = 2;   // or d/32 blocks per head, two strips each
+  } else {
+    for (int nsb = (epilogue == SK_SWIGLU ? 2 : 1); nsb <= 16; nsb *= 2) cand[ncand++] = nsb;
+  }
+  for (int ci = 0; ci < ncand; ++ci) {
+    const int nsb = cand[ci];
+    if (nsb > max_waves) continue;
+    for (int kw = 1; kw * nsb <= max_waves && kw <= steps; ++kw) {
+      for (int st = 0; st < 2; ++st) {
+        const bool stage = st == 1;
+        const size_t lds = skinny_lds_bytes(nsb, kw, mb, M, K, epilogue, stage);
+        if (lds > SK_LDS_LIMIT) continue;
+        const int blocks = (strips + nsb - 1) / nsb;     // (for QKV: heads, or heads * d/32)
+        const int per_cu = (blocks + num_cus - 1) / num_cus;       // blocks the busiest unit runs
+        // a compute unit streams about 25 GB/s from HBM (3.5 GB/s per resident wave until
+        // that limit) and about 50 GB/s from L2
+        int resident = 16 / (nsb * kw);
+        if (resident > per_cu) resident = per_cu;
+        const int by_lds = (int)((160 * 1024) / (lds > 1024 ? lds : 1024));
+        if (resident > by_lds) resident = by_lds;
+        if (resident < 1) resident = 1;
+        double rate = 3.5e3 * resident * nsb * kw;
+        if (rate > 25.0e3) rate = 25.0e3;
+        const double t_stream = per_cu * (16.0 * nsb * K * 2.0) / rate;
+        const double x_bytes = (double)(stage ? 1 : nsb) * M * K * (norm ? 4.0 : 2.0);
+        const double t_x = per_cu * x_bytes / 50.0e3;
+        const int per = (steps + kw - 1) / kw;
+        const int u = stage ? 4 : (norm ? (mb >= 2 ? 2 : 4) : (mb >= 4 ? 2 : (mb == 2 ? 4 : 8)));
+        const double trips = stage ? 1.0 + 0.3 * ((per + u - 1) / u - 1) : (double)((per + u - 1) / u);
+        const double busy = t_stream + t_x > 0.8 * trips ? t_stream + t_x : 0.8 * trips;
+        const double cost = 3.0 + (stage ? 0.7 : 0.0) + busy + 0.03 * kw * nsb;
+        if (cost < best_cost) {
+          best_cost = cost;
+          best = SkinnyShape{nsb, kw, stage, (epilogue == SK_QKV && nsb != d / 16) ? d / 32 : 1};
+        }
+      }
+    }
+  }
+  return best;
 }
 
 // One entry point for the whole family.
@@ -280,59 +510,65 @@ extern "C" int llmlab_skinny_linear(const void* x, int norm, const int* x_rows, 
   LLMLAB_REQUIRE(((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0) &&
                  (norm_w == nullptr || (uintptr_t)norm_w % 16 == 0),
                  "skinny_linear: operands must be 16-byte aligned");
+  LLMLAB_REQUIRE(!norm || norm_w != nullptr, "skinny_linear: a norm needs its weight");
   if (M == 0) return 0;
   if (num_cus <= 0) num_cus = 256;
   const int mb = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
-  const int steps = (K + 31) / 32;
-  int nsb;
   if (epilogue == SK_QKV) {
+    LLMLAB_REQUIRE(norm, "skinny_linear(qkv): takes the residual stream and its norm");
     LLMLAB_REQUIRE(d >= 16 && d % 16 == 0 && d <= 256 && N == (nq + 2 * nkv) * d,
                    "skinny_linear(qkv): head size %d / %d rows do not fit", d, N);
+    LLMLAB_REQUIRE(d / 16 <= (mb >= 4 ? 8 : 16), "skinny_linear(qkv): head size %d with %d rows", d, M);
     LLMLAB_REQUIRE((kcache == nullptr) == (vcache == nullptr), "skinny_linear(qkv): both caches or none");
     LLMLAB_REQUIRE(positions != nullptr && (kcache == nullptr || (table && row_req && page_size > 0)),
                    "skinny_linear(qkv): positions and block table are needed");
-    nsb = d / 16;
   } else if (epilogue == SK_SWIGLU) {
     LLMLAB_REQUIRE(N % 32 == 0 && 2 * ((n_out + 15) / 16 * 16) == N && bias == nullptr,
                    "skinny_linear(swiglu): %d rows do not interleave %d outputs", N, n_out);
-    nsb = 2;
   } else {
     LLMLAB_REQUIRE(n_out == N, "skinny_linear: n_out %d != N %d", n_out, N);
-    nsb = (N >= 32 * 2 * num_cus) ? 2 : 1;
   }
   LLMLAB_REQUIRE(ldo >= (epilogue == SK_QKV ? nq * d : n_out), "skinny_linear: output stride too small");
-  const int cols = 16 * nsb;
-  const int blocks = (N + cols - 1) / cols;
-  // enough waves to have the whole matrix in flight, within the block and LDS limits
-  const long want_waves = 12L * num_cus;
-  int kw = (int)((want_waves + (long)blocks * nsb - 1) / ((long)blocks * nsb));
-  if (kw > 16 / nsb) kw = 16 / nsb;
-  if (kw > steps) kw = steps;
-  while (kw > 1 && nsb * kw * mb > 32) --kw;
-  if (kw < 1) kw = 1;
-  const size_t lds = skinny_lds_bytes(nsb, kw, mb, M, epilogue);
-  LLMLAB_REQUIRE(lds <= 64 * 1024, "skinny_linear: %zu bytes of LDS needed", lds);
+  SkinnyShape shape = skinny_choose(epilogue, norm != 0, mb, M, N, K, d, num_cus);
+  if (g_force_nsb > 0 && epilogue != SK_QKV) shape.nsb = g_force_nsb;
+  if (g_force_nsb > 0 && epilogue == SK_QKV && d % 32 == 0 && d > 32) {
+    shape.nsb = g_force_nsb == 2 ? 2 : d / 16;
+    shape.qsplit = g_force_nsb == 2 ? d / 32 : 1;
+  }
+  if (g_force_kw > 0) shape.kw = g_force_kw;
+  if (g_force_stage >= 0) shape.stage = g_force_stage != 0;
+  LLMLAB_REQUIRE(shape.nsb > 0 && shape.kw > 0, "skinny_linear: no block shape fits N=%d K=%d M=%d", N, K, M);
+  const size_t lds = skinny_lds_bytes(shape.nsb, shape.kw, mb, M, K, epilogue, shape.stage);
+  LLMLAB_REQUIRE(lds <= SK_LDS_LIMIT && shape.nsb * shape.kw <= (mb >= 4 ? 8 : 16),
+                 "skinny_linear: block shape %dx%d does not fit", shape.nsb, shape.kw);
+  const int blocks = (N + 16 * shape.nsb - 1) / (16 * shape.nsb);
   SkinnyArgs a;
+  a.qsplit = shape.qsplit;
   a.x = x; a.x_rows = x_rows; a.norm_w = norm_w; a.W = (const bf16_t*)w; a.bias = bias; a.out = out;
   a.inv_freq = inv_freq; a.positions = positions; a.row_req = row_req; a.table = table;
   a.kcache = (bf16_t*)kcache; a.vcache = (bf16_t*)vcache;
   a.M = M; a.N = N; a.K = K; a.ldo = ldo; a.n_out = n_out;
   a.norm_w_bf16 = norm_w_dtype == DT_BF16; a.bias_bf16 = bias_dtype == DT_BF16;
-  a.nsb = nsb; a.kw = kw; a.nq = nq; a.nkv = nkv; a.d = d; a.table_stride = table_stride;
+  a.nsb = shape.nsb; a.kw = shape.kw; a.nq = nq; a.nkv = nkv; a.d = d; a.table_stride = table_stride;
   a.page_size = page_size; a.eps = eps;
-#define SK_CASE(E)                                                          \
-  case E:                                                                   \
-    if (norm) skinny_launch_mb<E, true>(a, mb, blocks, lds, stream);        \
-    else skinny_launch_mb<E, false>(a, mb, blocks, lds, stream);            \
-    break;
-  switch (epilogue) {
-    SK_CASE(SK_STORE)
-    SK_CASE(SK_RESID)
-    SK_CASE(SK_F32)
-    SK_CASE(SK_SWIGLU)
-    SK_CASE(SK_QKV)
+  int rc = 0;
+  if (norm) {
+    switch (epilogue) {
+      case SK_F32: rc = skinny_launch_stage<SK_F32, true>(a, shape.stage, mb, blocks, lds, stream); break;
+      case SK_SWIGLU: rc = skinny_launch_stage<SK_SWIGLU, true>(a, shape.stage, mb, blocks, lds, stream); break;
+      case SK_QKV: rc = skinny_launch_stage<SK_QKV, true>(a, shape.stage, mb, blocks, lds, stream); break;
+      default: LLMLAB_REQUIRE(false, "skinny_linear: epilogue %d has no fused norm", epilogue);
+    }
+  } else {
+    switch (epilogue) {
+      case SK_STORE: rc = skinny_launch_stage<SK_STORE, false>(a, shape.stage, mb, blocks, lds, stream); break;
+      case SK_RESID: rc = skinny_launch_stage<SK_RESID, false>(a, shape.stage, mb, blocks, lds, stream); break;
+      case SK_F32: rc = skinny_launch_stage<SK_F32, false>(a, shape.stage, mb, blocks, lds, stream); break;
+      case SK_SWIGLU: rc = skinny_launch_stage<SK_SWIGLU, false>(a, shape.stage, mb, blocks, lds, stream); break;
+      default: LLMLAB_REQUIRE(false, "skinny_linear: epilogue %d needs the norm", epilogue);
+    }
   }
-#undef SK_CASE
+  if (rc) return rc;
   LLMLAB_LAUNCH_CHECK("skinny_linear");
   return 0;
 }

@@ -117,6 +117,61 @@ __global__ __launch_bounds__(SAMPLE_THREADS) void sample_kernel(const float* __r
   }
 }
 
+// Greedy rows in two stages so that a row's scan is spread over many blocks:
+// each block takes ARGMAX_CHUNK logits and leaves (value, index); one block per
+// row picks among those with the same rule, so ties still go to the smallest index.
+constexpr int ARGMAX_CHUNK = 8192;
+
+__global__ __launch_bounds__(256) void argmax_partial_kernel(const float* __restrict__ logits,
+                                                             long row_stride, int vocab,
+                                                             float* __restrict__ pvals,
+                                                             int* __restrict__ pidx, int chunks) {
+  __shared__ Best red[17];
+  const int b = blockIdx.y, ch = blockIdx.x;
+  const int begin = ch * ARGMAX_CHUNK;
+  const int count = min(ARGMAX_CHUNK, vocab - begin);
+  const Best best = block_argmax(logits + (size_t)b * row_stride + begin, count, 1.f, red);
+  if (threadIdx.x == 0) {
+    pvals[(size_t)b * chunks + ch] = best.v;
+    pidx[(size_t)b * chunks + ch] = best.i < 0 ? -1 : begin + best.i;
+  }
+}
+
+__global__ __launch_bounds__(64) void argmax_final_kernel(const float* __restrict__ pvals,
+                                                          const int* __restrict__ pidx, int chunks,
+                                                          int* __restrict__ out) {
+  const int b = blockIdx.x;
+  Best best{0.f, -1};
+  for (int i = threadIdx.x; i < chunks; i += 64)
+    best = better(best, Best{pvals[(size_t)b * chunks + i], pidx[(size_t)b * chunks + i]});
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    Best o{__shfl_xor(best.v, off, WAVE), __shfl_xor(best.i, off, WAVE)};
+    best = better(best, o);
+  }
+  if (threadIdx.x == 0) out[b] = best.i;
+}
+
+// workspace: at least rows * ceil(vocab / 8192) * 2 words
+extern "C" int llmlab_argmax(const float* logits, long row_stride, int rows, int vocab, int* out,
+                             float* workspace, size_t workspace_floats, hipStream_t stream) {
+  LLMLAB_REQUIRE(rows >= 0 && vocab > 0 && row_stride >= vocab, "argmax: bad sizes rows=%d vocab=%d",
+                 rows, vocab);
+  if (rows == 0) return 0;
+  const int chunks = (vocab + ARGMAX_CHUNK - 1) / ARGMAX_CHUNK;
+  LLMLAB_REQUIRE(workspace != nullptr && (size_t)rows * chunks * 2 <= workspace_floats,
+                 "argmax: workspace too small");
+  LLMLAB_REQUIRE(rows <= 65535, "argmax: too many rows");
+  float* pvals = workspace;
+  int* pidx = (int*)(workspace + (size_t)rows * chunks);
+  hipLaunchKernelGGL(argmax_partial_kernel, dim3(chunks, rows), dim3(256), 0, stream, logits, row_stride,
+                     vocab, pvals, pidx, chunks);
+  LLMLAB_LAUNCH_CHECK("argmax (partial)");
+  hipLaunchKernelGGL(argmax_final_kernel, dim3(rows), dim3(64), 0, stream, pvals, pidx, chunks, out);
+  LLMLAB_LAUNCH_CHECK("argmax (final)");
+  return 0;
+}
+
 extern "C" int llmlab_sample(const float* logits, long row_stride, int rows, int vocab,
                              const float* temperature, const float* uniform, int* out,
                              hipStream_t stream) {

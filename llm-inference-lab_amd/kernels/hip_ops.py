@@ -80,6 +80,8 @@ class HipOps:
         c.llmlab_linear.argtypes = [_c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_int, _c_int,
                                     _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_size, _c_int, _c_ptr]
         c.llmlab_sample.argtypes = [_c_ptr, _c_long, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr]
+        c.llmlab_argmax.argtypes = [_c_ptr, _c_long, _c_int, _c_int, _c_ptr, _c_ptr, _c_size, _c_ptr]
+        c.llmlab_argmax.restype = _c_int
         c.llmlab_skinny_linear.argtypes = [
             _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_float, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr,
             _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
@@ -398,7 +400,14 @@ class HipOps:
 
     # --------------------------------------------------------------- sampling
     def argmax(self, logits, out) -> None:
-        self.sample(logits, None, None, out)
+        self._need(logits, "logits", torch.float32, contiguous=False)
+        self._need(out, "chosen tokens", torch.int32)
+        rows, vocab = logits.shape
+        if logits.stride(1) != 1 or out.numel() < rows:
+            raise ValueError("argmax: logits rows must be contiguous and out must hold one token per row")
+        self._check(self._core.llmlab_argmax(
+            self._ptr(logits), logits.stride(0) if rows > 1 else vocab, rows, vocab, self._ptr(out),
+            self._ptr(self.workspace), self.workspace.numel(), self._stream()))
 
     def sample(self, logits, temperatures, uniforms, out) -> None:
         self._need(logits, "logits", torch.float32, contiguous=False)

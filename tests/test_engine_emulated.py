@@ -55,7 +55,7 @@ def test_few_row_steps_take_the_fused_operations(name, cut):
     calls = engine.ops.calls
     assert calls["fused_norm_qkv"] > 0 and calls["fused_norm_swiglu"] > 0 and calls["fused_norm_logits"] > 0
     if cut == "decode" and name == "B":
-        assert calls.get("rmsnorm", 0) > 0          # the long first portions take the general path
+        assert calls.get("linear_swiglu", 0) > 0    # the long first portions take the general path
 
 
 def test_pages_are_reused_in_mixed():

