@@ -82,8 +82,8 @@ class CacheManager:
     def __init__(self, groups: Sequence[GroupLayout], page_size: int, max_requests: int,
                  max_seq_len: int, state_specs: Dict[int, Dict[str, Tuple[Tuple[int, ...], torch.dtype]]],
                  dtype: torch.dtype, device):
-        if page_size <= 0 or page_size % 16 != 0:
-            raise ValueError(f"page_size must be a positive multiple of 16, got {page_size}")
+        if page_size < 16 or page_size & (page_size - 1):
+            raise ValueError(f"page_size must be a power of two >= 16, got {page_size}")
         self.page_size = int(page_size)
         self.max_requests = int(max_requests)
         self.max_seq_len = int(max_seq_len)

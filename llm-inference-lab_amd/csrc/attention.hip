@@ -5,7 +5,7 @@
 // Cache of one layer:   keys   K[page][kv_head][P][D]
 //                        values V[page][kv_head][D][P]   (transposed)
 // Position p of the b-th request of the step lives in page table[b][p / P] at
-// offset p % P.  The query at position p sees the keys lo..p, lo = max(0, p -
+// offset p % P (P a power of two).  The query at position p sees the keys lo..p, lo = max(0, p -
 // window + 1) with a window and 0 without.
 //
 // bfloat16 kernel (matrix cores).  A tile is 16*QB "rows", a row being a (token,
@@ -40,6 +40,10 @@ static_assert(HEAD_DIM % 16 == 0 && HEAD_DIM >= 16 && HEAD_DIM <= 256,
 constexpr int D = HEAD_DIM;
 constexpr float NEG_INF = -__builtin_huge_valf();
 
+// 2^x for x <= 0 by the hardware instruction (one ulp; results below 2^-126 become 0,
+// which is what a softmax wants of them)
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
 struct AttnArgs {
   const void* q;      // [rows, q_stride], head h at h*D
   const void* kc;     // this layer's key pages
@@ -52,6 +56,7 @@ struct AttnArgs {
   float* ml_part;     // [rows*nq, splits, 2]
   int q_stride, out_stride, table_stride, page_size;
   int nq, nkv, window, splits;
+  int page_shift;     // log2(page_size); page sizes are powers of two
   float scale;
 };
 
@@ -83,12 +88,18 @@ __global__ __launch_bounds__(DECODE ? 64 * DECODE_WAVES : 256) void attention_bf
   const int G = a.nq / a.nkv;
   const int r0 = a.q_start[b], qlen = a.q_start[b + 1] - r0, sp = a.start_pos[b];
   const int rows_total = qlen * G;
-  const int row0 = DECODE ? 0 : (blockIdx.x * nw + wave) * (16 * QB);
-  if (!DECODE && row0 >= rows_total) return;
+  // prefill: the blocks with the longest histories (the last rows) are dispatched first
+  const int xblk = DECODE ? 0 : (int)(gridDim.x - 1 - blockIdx.x);
+  const int row0 = DECODE ? 0 : (xblk * nw + wave) * (16 * QB);
+  if (!DECODE && xblk * nw * (16 * QB) >= rows_total) return;   // the whole block is past the rows
+  const bool wave_live = row0 < rows_total;      // a wave without rows still helps to stage keys
   const bf16_t* q = (const bf16_t*)a.q;
   const bf16_t* kc = (const bf16_t*)a.kc;
   const bf16_t* vc = (const bf16_t*)a.vc;
   const int P = a.page_size;
+  const int pshift = a.page_shift;
+  auto page_index = [&](int pos) { return pos >> pshift; };
+  auto page_offset = [&](int pos) { return pos & (P - 1); };
   const float scale2 = a.scale * 1.4426950408889634f;
   const bf16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
   const bf16x4 zero4 = {0, 0, 0, 0};
@@ -100,7 +111,7 @@ __global__ __launch_bounds__(DECODE ? 64 * DECODE_WAVES : 256) void attention_bf
 #pragma unroll
   for (int qb = 0; qb < QB; ++qb) {
     const int rr = row0 + qb * 16 + c;
-    valid[qb] = rr < rows_total;
+    valid[qb] = wave_live && rr < rows_total;
     tok[qb] = valid[qb] ? rr / G : 0;
     head[qb] = kvh * G + (valid[qb] ? rr % G : 0);
     pos[qb] = sp + tok[qb];
@@ -117,7 +128,9 @@ __global__ __launch_bounds__(DECODE ? 64 * DECODE_WAVES : 256) void attention_bf
   const int last_row = min(row0 + 16 * QB, rows_total) - 1;
   const int p_first = sp + row0 / G, p_last = sp + last_row / G;
   const int key_lo = a.window > 0 ? max(0, p_first - a.window + 1) : 0;
-  const int key_hi = p_last;
+  const int key_hi = wave_live ? p_last : -1;
+  // every key >= full_lo is inside the window of every row of the tile
+  const int full_lo = a.window > 0 ? max(0, p_last - a.window + 1) : 0;
   const int blk_lo = key_lo >> 5, blk_hi = key_hi >> 5;
   const int per = (blk_hi - blk_lo + 1 + a.splits - 1) / a.splits;
   int my_blk0 = blk_lo + split * per;
@@ -147,11 +160,11 @@ __global__ __launch_bounds__(DECODE ? 64 * DECODE_WAVES : 256) void attention_bf
       const int pos16 = kb + h2 * 16;
       bool ok = pos16 <= key_hi && pos16 + 15 >= key_lo;
       int page = -1;
-      if (ok) page = a.table[(size_t)b * a.table_stride + pos16 / P];
+      if (ok) page = a.table[(size_t)b * a.table_stride + page_index(pos16)];
       ok = ok && page >= 0;
       f.ok[h2] = ok;
       if (ok) {
-        const int off = pos16 % P;
+        const int off = page_offset(pos16);
         const bf16_t* kp = kc + (((size_t)page * a.nkv + kvh) * P + off + c) * D;
         const bf16_t* vp = vc + ((size_t)page * a.nkv + kvh) * D * P + off + g * 4;
 #pragma unroll
@@ -185,45 +198,55 @@ __global__ __launch_bounds__(DECODE ? 64 * DECODE_WAVES : 256) void attention_bf
             s[h2][qb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(f.k[h2][dc], qf[qb][dc], s[h2][qb], 0, 0, 0);
       }
     }
+    // all 32 keys visible to every row of the tile (the common case below the diagonal
+    // and inside the window): no comparisons
+    const bool all_visible = f.ok[0] && f.ok[1] && kb + 31 <= p_first && kb >= full_lo;
     bf16x8 pf[QB];
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
+      // raw scores (masked ones -inf); the running maximum m is kept in raw units too,
+      // the scale goes into the exponent:  p = 2^(s * scale2 - m * scale2)
       float sv[8];
-      float mx = NEG_INF;
+      if (all_visible) {
 #pragma unroll
-      for (int h2 = 0; h2 < 2; ++h2)
+        for (int i = 0; i < 8; ++i) sv[i] = s[i >> 2][qb][i & 3];
+      } else {
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const int j = kb + h2 * 16 + g * 4 + i;
+        for (int i = 0; i < 8; ++i) {
+          const int h2 = i >> 2;
+          const int j = kb + h2 * 16 + g * 4 + (i & 3);
           const bool vis = f.ok[h2] && valid[qb] && j <= pos[qb] && j >= lo[qb];
-          const float v = vis ? s[h2][qb][i] * scale2 : NEG_INF;
-          sv[h2 * 4 + i] = v;
-          mx = fmaxf(mx, v);
+          sv[i] = vis ? s[h2][qb][i & 3] : NEG_INF;
         }
+      }
+      float mx = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])),
+                       fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
       mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
       mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
       const float m_new = fmaxf(m[qb], mx);
-      const bool none = m_new == NEG_INF;
-      const float alpha = none ? 1.f : exp2f(m[qb] - m_new);
+      if (__any(m_new != m[qb])) {            // some row's maximum grew: rescale what is summed so far
+        const float alpha = m_new == NEG_INF ? 1.f : fast_exp2((m[qb] - m_new) * scale2);
+        lsum[qb] *= alpha;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) o[qb][db] *= alpha;
+        m[qb] = m_new;
+      }
+      const float neg_m = m_new == NEG_INF ? 0.f : -m_new * scale2;    // no visible key yet: p = 2^-inf = 0
       float psum = 0.f;
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
-        const float p = none ? 0.f : exp2f(sv[i] - m_new);
+        const float p = fast_exp2(__builtin_fmaf(sv[i], scale2, neg_m));
+        psum += p;
         pf[qb][i] = (bf16_t)p;
-        psum += (float)pf[qb][i];   // the denominator sums what the product uses
       }
-      lsum[qb] = lsum[qb] * alpha + psum;
-      m[qb] = m_new;
-#pragma unroll
-      for (int db = 0; db < DB; ++db) o[qb][db] *= alpha;
+      lsum[qb] += psum;
     }
     // keys past the last written position hold stale values: keep them out of
     // the product even though their probability is zero
     const bool tail = kb + 31 > key_hi;
 #pragma unroll
     for (int db = 0; db < DB; ++db) {
-      const bf16x4 v0 = f.v[0][db], v1 = f.v[1][db];
-      bf16x8 vf = {v0[0], v0[1], v0[2], v0[3], v1[0], v1[1], v1[2], v1[3]};
+      bf16x8 vf = __builtin_shufflevector(f.v[0][db], f.v[1][db], 0, 1, 2, 3, 4, 5, 6, 7);
       if (tail) {
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
@@ -247,10 +270,113 @@ __global__ __launch_bounds__(DECODE ? 64 * DECODE_WAVES : 256) void attention_bf
       cur = nxt;
     }
   } else {
-    for (int blk = my_blk0; blk < my_blk1; ++blk) {
-      KeyStep<DC, DB> cur;
-      fetch(blk, cur);
-      compute(blk, cur);
+    // ---- prefill: tiles of 64 keys go through LDS once per block and serve all its
+    // waves; the next tile is fetched into registers while this one is multiplied
+    constexpr int KS = D + 8, VS = 64 + 8;          // padded rows: 16-byte reads of 8 lanes cover all banks
+    constexpr int NCH = D / 16;                     // 16-byte pieces per thread and tile (256 threads)
+    __shared__ __attribute__((aligned(16))) bf16_t Ks[64 * KS];   // [key][d]
+    __shared__ __attribute__((aligned(16))) bf16_t Vs[D * VS];    // [d][key]
+    __shared__ int s_ok[4];
+    constexpr int PAGE_CAP = 2048;
+    __shared__ int s_pages[PAGE_CAP];               // the block's slice of its request's block table
+    const int tid = threadIdx.x;
+    const int blk_row0 = xblk * nw * (16 * QB);
+    const int blk_last = min(blk_row0 + nw * 16 * QB, rows_total) - 1;
+    const int bkey_hi = sp + blk_last / G;
+    const int bkey_lo = a.window > 0 ? max(0, sp + blk_row0 / G - a.window + 1) : 0;
+    // page numbers first, all at once: the tile loop then has one memory round trip
+    // per tile instead of two dependent ones
+    const int page_first = page_index(bkey_lo);
+    const int page_count = min(page_index(bkey_hi) - page_first + 1, PAGE_CAP);
+    for (int i = tid; i < page_count; i += 256)
+      s_pages[i] = a.table[(size_t)b * a.table_stride + page_first + i];
+    __syncthreads();
+    // PD tiles are on their way from memory at any time (a ring of register buffers):
+    // one tile's arithmetic is far shorter than the memory latency
+    constexpr int PD = NCH <= 4 ? 3 : 2;
+    bf16x8 regs[PD][NCH];
+    bool rok[PD][NCH];
+    const int tile_lo = bkey_lo >> 6, tile_hi = bkey_hi >> 6;
+    auto fetch_tile = [&](int slot, int tile) {
+#pragma unroll
+      for (int n = 0; n < NCH; ++n) {
+        const int i = tid + n * 256;
+        const bool is_v = i >= 8 * D;
+        const int j = is_v ? i - 8 * D : i;
+        const int sub = j / (2 * D), rem = j - sub * (2 * D);
+        const int pos16 = tile * 64 + sub * 16;
+        bool ok = tile <= tile_hi && pos16 <= bkey_hi && pos16 + 15 >= bkey_lo;
+        int page = -1;
+        if (ok) {
+          const int pi = page_index(pos16) - page_first;
+          page = pi < PAGE_CAP ? s_pages[pi] : a.table[(size_t)b * a.table_stride + page_index(pos16)];
+        }
+        ok = ok && page >= 0;
+        rok[slot][n] = ok;
+        regs[slot][n] = zero8;
+        if (ok) {
+          const int off = page_offset(pos16);
+          if (!is_v) {
+            const int key = rem / (D / 8), ch = rem - key * (D / 8);
+            regs[slot][n] = *(const bf16x8*)(kc + (((size_t)page * a.nkv + kvh) * P + off + key) * D + ch * 8);
+          } else {
+            const int drow = rem >> 1, half = rem & 1;
+            regs[slot][n] = *(const bf16x8*)(vc + (((size_t)page * a.nkv + kvh) * D + drow) * P + off + half * 8);
+          }
+        }
+      }
+    };
+    auto store_tile = [&](int slot) {
+#pragma unroll
+      for (int n = 0; n < NCH; ++n) {
+        const int i = tid + n * 256;
+        const bool is_v = i >= 8 * D;
+        const int j = is_v ? i - 8 * D : i;
+        const int sub = j / (2 * D), rem = j - sub * (2 * D);
+        if (!is_v) {
+          const int key = rem / (D / 8), ch = rem - key * (D / 8);
+          *(bf16x8*)(Ks + (sub * 16 + key) * KS + ch * 8) = regs[slot][n];
+          if (rem == 0) s_ok[sub] = rok[slot][n];
+        } else {
+          const int drow = rem >> 1, half = rem & 1;
+          *(bf16x8*)(Vs + drow * VS + sub * 16 + half * 8) = regs[slot][n];
+        }
+      }
+    };
+#pragma unroll
+    for (int p = 0; p < PD; ++p) fetch_tile(p, tile_lo + p);
+    for (int tile0 = tile_lo; tile0 <= tile_hi; tile0 += PD) {
+#pragma unroll
+      for (int p = 0; p < PD; ++p) {
+        const int tile = tile0 + p;
+        if (tile <= tile_hi) {
+          store_tile(p);
+          __syncthreads();
+          fetch_tile(p, tile + PD);
+#pragma unroll
+          for (int st = 0; st < 2; ++st) {
+            const int kb = tile * 64 + st * 32;
+            if (kb <= key_hi && kb + 31 >= key_lo) {        // this wave sees some of these keys
+              KeyStep<DC, DB> f;
+#pragma unroll
+              for (int h2 = 0; h2 < 2; ++h2) {
+                const int sub = st * 2 + h2;
+                f.ok[h2] = s_ok[sub] != 0;
+#pragma unroll
+                for (int dc = 0; dc < DC; ++dc) {
+                  const int dd = dc * 32 + g * 8;
+                  f.k[h2][dc] = (dd < D) ? *(const bf16x8*)(Ks + (sub * 16 + c) * KS + dd) : zero8;
+                }
+#pragma unroll
+                for (int db = 0; db < DB; ++db)
+                  f.v[h2][db] = *(const bf16x4*)(Vs + (db * 16 + c) * VS + sub * 16 + g * 4);
+              }
+              compute(kb >> 5, f);
+            }
+          }
+          __syncthreads();
+        }
+      }
     }
   }
 
@@ -280,7 +406,7 @@ __global__ __launch_bounds__(DECODE ? 64 * DECODE_WAVES : 256) void attention_bf
       l += __shfl_xor(l, 16, WAVE);
       l += __shfl_xor(l, 32, WAVE);
       if (g == 0) {
-        s_m[wave][c] = m[0];
+        s_m[wave][c] = m[0] * scale2;      // the merges work in the units of the exponent
         s_l[wave][c] = l;
       }
 #pragma unroll
@@ -382,8 +508,8 @@ __global__ __launch_bounds__(64) void attention_f32_kernel(AttnArgs a) {
   for (int dd = 0; dd < D; ++dd) o[dd] = 0.f;
   float m = NEG_INF, l = 0.f;
   for (int j = lo + lane; j <= p; j += 64) {
-    const int page = a.table[(size_t)b * a.table_stride + j / P];
-    const int off = j % P;
+    const int page = a.table[(size_t)b * a.table_stride + (j >> a.page_shift)];
+    const int off = j & (P - 1);
     const float* kp = kc + (((size_t)page * a.nkv + kvh) * P + off) * D;
     const float* vp = vc + ((size_t)page * a.nkv + kvh) * D * P + off;
     float dot = 0.f;
@@ -426,11 +552,12 @@ extern "C" int llmlab_paged_attention(const void* q, int dtype, int q_stride, in
                                       float* workspace, size_t workspace_floats, int total_rows,
                                       int num_cus, hipStream_t stream) {
   LLMLAB_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0, "attention: %d heads, %d kv heads", nq, nkv);
-  LLMLAB_REQUIRE(page_size > 0 && page_size % 16 == 0, "attention: page size %d is not a multiple of 16",
-                 page_size);
+  LLMLAB_REQUIRE(page_size >= 16 && (page_size & (page_size - 1)) == 0,
+                 "attention: page size %d is not a power of two >= 16", page_size);
   LLMLAB_REQUIRE(q_stride >= nq * D && out_stride >= nq * D, "attention: row strides too small");
   LLMLAB_REQUIRE(reqs >= 0 && reqs <= 65535 && nq <= 65535, "attention: grid too large");
   LLMLAB_REQUIRE(window >= 0, "attention: negative window");
+  LLMLAB_REQUIRE(scale > 0.f, "attention: the score scale must be positive, got %g", (double)scale);
   if (reqs == 0 || max_q_len <= 0) return 0;
   if (num_cus <= 0) num_cus = 256;
   AttnArgs a;
@@ -438,6 +565,8 @@ extern "C" int llmlab_paged_attention(const void* q, int dtype, int q_stride, in
   a.out = out; a.o_part = nullptr; a.ml_part = nullptr;
   a.q_stride = q_stride; a.out_stride = out_stride; a.table_stride = table_stride; a.page_size = page_size;
   a.nq = nq; a.nkv = nkv; a.window = window; a.splits = 1; a.scale = scale;
+  a.page_shift = 0;
+  while ((1 << a.page_shift) < page_size) ++a.page_shift;
   if (dtype == DT_F32) {
     dim3 grid(max_q_len, nq, reqs), block(64);
     hipLaunchKernelGGL(attention_f32_kernel, grid, block, 0, stream, a);
@@ -478,10 +607,20 @@ extern "C" int llmlab_paged_attention(const void* q, int dtype, int q_stride, in
     }
     return 0;
   }
-  constexpr int QB = 2;
-  const int rows_per_block = 4 * 16 * QB;
-  dim3 grid((unsigned)((max_rows + rows_per_block - 1) / rows_per_block), nkv, reqs), block(256);
-  hipLaunchKernelGGL((attention_bf16_kernel<QB, false>), grid, block, 0, stream, a);
+  // rows per wave: 32 when that still gives every compute unit two blocks (or for
+  // nothing smaller), else 16; always 16 for the largest heads (registers)
+  const long blocks32 = ((max_rows + 127) / 128) * nkv * reqs;
+#ifdef LLMLAB_EXP_QB2
+  if (D <= 128) {
+#else
+  if (D <= 128 && blocks32 >= 2L * num_cus) {
+#endif
+    dim3 grid((unsigned)((max_rows + 127) / 128), nkv, reqs), block(256);
+    hipLaunchKernelGGL((attention_bf16_kernel<2, false>), grid, block, 0, stream, a);
+  } else {
+    dim3 grid((unsigned)((max_rows + 63) / 64), nkv, reqs), block(256);
+    hipLaunchKernelGGL((attention_bf16_kernel<1, false>), grid, block, 0, stream, a);
+  }
   LLMLAB_LAUNCH_CHECK("attention(bfloat16, prefill)");
   return 0;
 }

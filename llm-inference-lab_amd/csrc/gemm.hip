@@ -4,8 +4,8 @@
 //   bfloat16:  v_mfma_f32_16x16x32_bf16 everywhere.
 //     * tiled kernel (M > 64): 256 threads = 4 waves in 2x2, block tile 128x128 or
 //       64x64, K step 64 staged through LDS (rows padded to 72 elements so that the
-//       16-byte fragment reads of 8 lanes cover all banks), next tile prefetched
-//       into registers while the current one is multiplied.
+//       16-byte fragment reads of 8 lanes cover all banks); three or four tiles are
+//       on their way from memory in a ring of register buffers while one is multiplied.
 //     * skinny kernel (M <= 64, decode): weights stream from HBM straight into MFMA
 //       B fragments, one wave per 16 (or 32) weight rows and K range; the few rows
 //       of x come from cache.  K may be split over blocks; partial sums go to a
@@ -75,58 +75,68 @@ __global__ __launch_bounds__(256) void gemm_bf16_tiled(const bf16_t* __restrict_
 #pragma unroll
     for (int j = 0; j < TN; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
 
-  bf16x8 ra[A_CHUNKS], rb[B_CHUNKS];
+  // Memory latency is several times the time a tile takes to multiply, so PD tiles
+  // are on their way at any time: a ring of register buffers, refilled as soon as a
+  // buffer has been put into LDS.
+  constexpr int PD = (A_CHUNKS + B_CHUNKS) <= 4 ? 4 : 3;
+  bf16x8 ra[PD][A_CHUNKS], rb[PD][B_CHUNKS];
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
-  auto fetch = [&](int k0) {
+  auto fetch = [&](int slot, int k0) {
 #pragma unroll
     for (int i = 0; i < A_CHUNKS; ++i) {
       const int ch = tid + i * 256, row = ch >> 3, kc = (ch & 7) * 8;
       const int m = m0 + row, k = k0 + kc;
-      ra[i] = (m < M && k < K) ? *(const bf16x8*)(A + (size_t)m * K + k) : zero;
+      ra[slot][i] = (m < M && k < K) ? *(const bf16x8*)(A + (size_t)m * K + k) : zero;
     }
 #pragma unroll
     for (int i = 0; i < B_CHUNKS; ++i) {
       const int ch = tid + i * 256, row = ch >> 3, kc = (ch & 7) * 8;
       const int n = n0 + row, k = k0 + kc;
-      rb[i] = (n < N && k < K) ? *(const bf16x8*)(W + (size_t)n * K + k) : zero;
+      rb[slot][i] = (n < N && k < K) ? *(const bf16x8*)(W + (size_t)n * K + k) : zero;
     }
   };
-  auto stash = [&]() {
+  auto stash = [&](int slot) {
 #pragma unroll
     for (int i = 0; i < A_CHUNKS; ++i) {
       const int ch = tid + i * 256, row = ch >> 3, kc = (ch & 7) * 8;
-      *(bf16x8*)(As + row * LDS_STRIDE + kc) = ra[i];
+      *(bf16x8*)(As + row * LDS_STRIDE + kc) = ra[slot][i];
     }
 #pragma unroll
     for (int i = 0; i < B_CHUNKS; ++i) {
       const int ch = tid + i * 256, row = ch >> 3, kc = (ch & 7) * 8;
-      *(bf16x8*)(Bs + row * LDS_STRIDE + kc) = rb[i];
+      *(bf16x8*)(Bs + row * LDS_STRIDE + kc) = rb[slot][i];
     }
   };
 
   const int nk = (K + BK - 1) / BK;
-  fetch(0);
-  for (int kt = 0; kt < nk; ++kt) {
-    stash();
-    __syncthreads();
-    if (kt + 1 < nk) fetch((kt + 1) * BK);
 #pragma unroll
-    for (int ks = 0; ks < 2; ++ks) {
-      bf16x8 a[TM], b[TN];
+  for (int p = 0; p < PD; ++p) fetch(p, p * BK);      // past K: no load, zeros
+  for (int kt = 0; kt < nk; kt += PD) {
 #pragma unroll
-      for (int i = 0; i < TM; ++i)
-        a[i] = *(const bf16x8*)(As + (wm * WTM + i * 16 + c) * LDS_STRIDE + ks * 32 + g * 8);
+    for (int p = 0; p < PD; ++p) {
+      if (kt + p < nk) {
+        stash(p);
+        __syncthreads();
+        fetch(p, (kt + p + PD) * BK);
 #pragma unroll
-      for (int j = 0; j < TN; ++j)
-        b[j] = *(const bf16x8*)(Bs + (wn * WTN + j * 16 + c) * LDS_STRIDE + ks * 32 + g * 8);
+        for (int ks = 0; ks < 2; ++ks) {
+          bf16x8 a[TM], b[TN];
 #pragma unroll
-      for (int i = 0; i < TM; ++i)
+          for (int i = 0; i < TM; ++i)
+            a[i] = *(const bf16x8*)(As + (wm * WTM + i * 16 + c) * LDS_STRIDE + ks * 32 + g * 8);
 #pragma unroll
-        for (int j = 0; j < TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+          for (int j = 0; j < TN; ++j)
+            b[j] = *(const bf16x8*)(Bs + (wn * WTN + j * 16 + c) * LDS_STRIDE + ks * 32 + g * 8);
+#pragma unroll
+          for (int i = 0; i < TM; ++i)
+#pragma unroll
+            for (int j = 0; j < TN; ++j)
+              acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+        }
+        __syncthreads();
+      }
     }
-    __syncthreads();
   }
 
 #pragma unroll

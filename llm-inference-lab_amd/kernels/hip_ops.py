@@ -387,8 +387,8 @@ class HipOps:
             raise ValueError("attention: request arrays are shorter than the number of requests")
         if max_ctx_len > block_table.shape[1] * page_size:
             raise ValueError("attention: the block table is too narrow for the longest context")
-        if page_size % 16 != 0:
-            raise UnsupportedSizeError(f"page size {page_size} is not a multiple of 16")
+        if page_size < 16 or page_size & (page_size - 1):
+            raise UnsupportedSizeError(f"page size {page_size} is not a power of two >= 16")
         q_stride = qkv.stride(0) if rows > 1 else qkv.shape[1]
         self._check(lib.llmlab_paged_attention(
             self._ptr(qkv), _dt(qkv), q_stride, num_heads, num_kv_heads, self._ptr(k_cache),

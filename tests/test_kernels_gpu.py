@@ -320,9 +320,10 @@ def run_attention(ops, emu, dtype, nq, nkv, d, page, window, reqs_spec, seed=30,
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("d", [16, 32, 48, 64, 80, 96, 112, 128])
+@pytest.mark.parametrize("d", [16, 32, 48, 64, 80, 96, 112, 128, 256])
 def test_attention_head_sizes(ops, emu, dtype, d):
     run_attention(ops, emu, dtype, 4, 2, d, 16, None, [(0, 37), (21, 1), (5, 12)])
+    run_attention(ops, emu, dtype, 4, 2, d, 64, None, [(100, 150), (300, 1)])
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
