@@ -610,11 +610,7 @@ extern "C" int llmlab_paged_attention(const void* q, int dtype, int q_stride, in
   // rows per wave: 32 when that still gives every compute unit two blocks (or for
   // nothing smaller), else 16; always 16 for the largest heads (registers)
   const long blocks32 = ((max_rows + 127) / 128) * nkv * reqs;
-#ifdef LLMLAB_EXP_QB2
-  if (D <= 128) {
-#else
   if (D <= 128 && blocks32 >= 2L * num_cus) {
-#endif
     dim3 grid((unsigned)((max_rows + 127) / 128), nkv, reqs), block(256);
     hipLaunchKernelGGL((attention_bf16_kernel<2, false>), grid, block, 0, stream, a);
   } else {

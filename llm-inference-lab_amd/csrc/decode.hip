@@ -467,23 +467,28 @@ static SkinnyShape skinny_choose(int epilogue, bool norm, int mb, int M, int N, 
         if (lds > SK_LDS_LIMIT) continue;
         const int blocks = (strips + nsb - 1) / nsb;     // (for QKV: heads, or heads * d/32)
         const int per_cu = (blocks + num_cus - 1) / num_cus;       // blocks the busiest unit runs
-        // a compute unit streams about 25 GB/s from HBM (3.5 GB/s per resident wave until
-        // that limit) and about 50 GB/s from L2
-        int resident = 16 / (nsb * kw);
+        int resident = 16 / (nsb * kw);                             // of which so many at a time
         if (resident > per_cu) resident = per_cu;
         const int by_lds = (int)((160 * 1024) / (lds > 1024 ? lds : 1024));
         if (resident > by_lds) resident = by_lds;
         if (resident < 1) resident = 1;
+        const int rounds = (per_cu + resident - 1) / resident;
+        // a compute unit streams about 25 GB/s from HBM (3.5 GB/s per resident wave until
+        // that limit) and about 50 GB/s from L2; rows of x read by every wave on its own
+        // (not staged) come in short strided pieces and cost about twice that
         double rate = 3.5e3 * resident * nsb * kw;
         if (rate > 25.0e3) rate = 25.0e3;
         const double t_stream = per_cu * (16.0 * nsb * K * 2.0) / rate;
-        const double x_bytes = (double)(stage ? 1 : nsb) * M * K * (norm ? 4.0 : 2.0);
+        const double x_bytes = (double)(stage ? 1 : 2 * nsb) * M * K * (norm ? 4.0 : 2.0);
         const double t_x = per_cu * x_bytes / 50.0e3;
         const int per = (steps + kw - 1) / kw;
         const int u = stage ? 4 : (norm ? (mb >= 2 ? 2 : 4) : (mb >= 4 ? 2 : (mb == 2 ? 4 : 8)));
         const double trips = stage ? 1.0 + 0.3 * ((per + u - 1) / u - 1) : (double)((per + u - 1) / u);
         const double busy = t_stream + t_x > 0.8 * trips ? t_stream + t_x : 0.8 * trips;
-        const double cost = 3.0 + (stage ? 0.7 : 0.0) + busy + 0.03 * kw * nsb;
+        // a fixed part per kernel, and again (in part hidden by the neighbours) for every
+        // further round of blocks on the busiest unit
+        const double cost = 3.3 + (stage ? 0.3 : 0.0) + busy + (rounds - 1) * 2.4 / resident +
+                            0.03 * kw * nsb;
         if (cost < best_cost) {
           best_cost = cost;
           best = SkinnyShape{nsb, kw, stage, (epilogue == SK_QKV && nsb != d / 16) ? d / 32 : 1};

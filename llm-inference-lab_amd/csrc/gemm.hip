@@ -2,15 +2,11 @@
 // for gfx950, with the epilogues the model needs fused in.
 //
 //   bfloat16:  v_mfma_f32_16x16x32_bf16 everywhere.
-//     * tiled kernel (M > 64): 256 threads = 4 waves in 2x2, block tile 128x128 or
+//     * tiled kernel: 256 threads = 4 waves in 2x2, block tile 128x128 or
 //       64x64, K step 64 staged through LDS (rows padded to 72 elements so that the
 //       16-byte fragment reads of 8 lanes cover all banks); three or four tiles are
 //       on their way from memory in a ring of register buffers while one is multiplied.
-//     * skinny kernel (M <= 64, decode): weights stream from HBM straight into MFMA
-//       B fragments, one wave per 16 (or 32) weight rows and K range; the few rows
-//       of x come from cache.  K may be split over blocks; partial sums go to a
-//       float32 workspace and a second kernel reduces them and applies the epilogue
-//       (a fixed order, so results do not depend on timing).
+//     (products of few rows, as in decode steps, have kernels of their own in decode.hip)
 //   float32: a plain FMA kernel (64x64 tile, 4x4 outputs per thread): true 32-bit
 //     products and sums, no matrix-core shortcut.
 //
@@ -163,130 +159,6 @@ __global__ __launch_bounds__(256) void gemm_bf16_tiled(const bf16_t* __restrict_
   }
 }
 
-// =========================================================== bf16, skinny
-// One wave per NS strips of 16 weight rows and one K range; MB blocks of 16 rows
-// of x.  SPLIT: write float32 partial sums  part[split][m][n]  instead of the
-// epilogue.
-template <int MB, int NS, int EPI, bool SPLIT>
-__global__ __launch_bounds__(256) void gemm_bf16_skinny(const bf16_t* __restrict__ A,
-                                                         const bf16_t* __restrict__ W, EpiArgs e,
-                                                         float* __restrict__ part, int M, int N, int K,
-                                                         int k_per_split) {
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int c = lane & 15, g = lane >> 4;
-  const int n0 = (blockIdx.x * 4 + wave) * (16 * NS);
-  if (n0 >= N) return;
-  const int k_begin = blockIdx.y * k_per_split;
-  const int k_end = min(K, k_begin + k_per_split);
-  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-
-  floatx4 acc[MB][NS];
-#pragma unroll
-  for (int i = 0; i < MB; ++i)
-#pragma unroll
-    for (int j = 0; j < NS; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
-
-  const bf16_t* wrow[NS];
-  bool wok[NS];
-#pragma unroll
-  for (int j = 0; j < NS; ++j) {
-    const int n = n0 + j * 16 + c;
-    wok[j] = n < N;
-    wrow[j] = W + (size_t)(wok[j] ? n : 0) * K;
-  }
-  const bf16_t* arow[MB];
-  bool aok[MB];
-#pragma unroll
-  for (int i = 0; i < MB; ++i) {
-    const int m = i * 16 + c;
-    aok[i] = m < M;
-    arow[i] = A + (size_t)(aok[i] ? m : 0) * K;
-  }
-
-  int k = k_begin;
-  // full groups of 4 steps: 4 independent 16-byte loads per weight strip in flight
-  for (; k + 128 <= k_end; k += 128) {
-    bf16x8 b[4][NS], a[4][MB];
-#pragma unroll
-    for (int s = 0; s < 4; ++s) {
-      const int kk = k + s * 32 + g * 8;
-#pragma unroll
-      for (int j = 0; j < NS; ++j) b[s][j] = wok[j] ? *(const bf16x8*)(wrow[j] + kk) : zero;
-#pragma unroll
-      for (int i = 0; i < MB; ++i) a[s][i] = aok[i] ? *(const bf16x8*)(arow[i] + kk) : zero;
-    }
-#pragma unroll
-    for (int s = 0; s < 4; ++s)
-#pragma unroll
-      for (int i = 0; i < MB; ++i)
-#pragma unroll
-        for (int j = 0; j < NS; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[s][i], b[s][j], acc[i][j], 0, 0, 0);
-  }
-  for (; k < k_end; k += 32) {
-    const int kk = k + g * 8;
-    const bool kok = kk < k_end;
-    bf16x8 b[NS], a[MB];
-#pragma unroll
-    for (int j = 0; j < NS; ++j) b[j] = (wok[j] && kok) ? *(const bf16x8*)(wrow[j] + kk) : zero;
-#pragma unroll
-    for (int i = 0; i < MB; ++i) a[i] = (aok[i] && kok) ? *(const bf16x8*)(arow[i] + kk) : zero;
-#pragma unroll
-    for (int i = 0; i < MB; ++i)
-#pragma unroll
-      for (int j = 0; j < NS; ++j)
-        acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
-  }
-
-#pragma unroll
-  for (int i = 0; i < MB; ++i) {
-#pragma unroll
-    for (int j = 0; j < NS; ++j) {
-      const int nb = n0 + j * 16;
-#pragma unroll
-      for (int x = 0; x < 4; ++x) {
-        const int m = i * 16 + g * 4 + x;
-        if (m >= M) continue;
-        if constexpr (SPLIT) {
-          const int n = nb + c;
-          if (n < N) part[((size_t)blockIdx.y * M + m) * N + n] = acc[i][j][x];
-        } else if constexpr (EPI == EPI_SWIGLU) {
-          if (j & 1) continue;
-          const int o = (nb >> 5) * 16 + c;
-          if (o < e.n_out)
-            ((bf16_t*)e.out)[(size_t)m * e.ldo + o] =
-                (bf16_t)(silu_f(acc[i][j][x]) * acc[i][j | 1][x]);
-        } else {
-          const int n = nb + c;
-          if (n < N) epi_store<bf16_t, EPI>(e, m, n, acc[i][j][x]);
-        }
-      }
-    }
-  }
-}
-
-// Sum the partial results of the K splits in a fixed order and apply the epilogue.
-template <typename T, int EPI>
-__global__ void splitk_epilogue(const float* __restrict__ part, EpiArgs e, int M, int N, int splits) {
-  const int cols = (EPI == EPI_SWIGLU) ? e.n_out : N;
-  const size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (idx >= (size_t)M * cols) return;
-  const int m = (int)(idx / cols), o = (int)(idx % cols);
-  if constexpr (EPI == EPI_SWIGLU) {
-    const int ng = (o >> 4) * 32 + (o & 15), nu = ng + 16;
-    float gsum = 0.f, usum = 0.f;
-    for (int s = 0; s < splits; ++s) {
-      gsum += part[((size_t)s * M + m) * N + ng];
-      usum += part[((size_t)s * M + m) * N + nu];
-    }
-    ((T*)e.out)[(size_t)m * e.ldo + o] = from_float<T>(silu_f(gsum) * usum);
-  } else {
-    float sum = 0.f;
-    for (int s = 0; s < splits; ++s) sum += part[((size_t)s * M + m) * N + o];
-    epi_store<T, EPI>(e, m, o, sum);
-  }
-}
-
 // ================================================================ float32
 // 64x64 outputs per block of 256 threads; thread (ty, tx) owns rows ty + 16*i and
 // columns tx + 16*j (i, j in 0..3), so for SWIGLU columns j = 0, 2 are gate and
@@ -353,63 +225,25 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__
 
 // ================================================================ dispatch
 template <int EPI>
-static int launch_bf16(const bf16_t* A, const bf16_t* W, EpiArgs e, int M, int N, int K,
-                       float* workspace, size_t workspace_floats, int num_cus, hipStream_t stream) {
-  if (M > 64) {
-    const long big_tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
-    if (big_tiles >= num_cus) {
-      dim3 grid((N + 127) / 128, (M + 127) / 128);
-      hipLaunchKernelGGL((gemm_bf16_tiled<128, 128, EPI>), grid, dim3(256), 0, stream, A, W, e, M, N, K);
-    } else {
-      dim3 grid((N + 63) / 64, (M + 63) / 64);
-      hipLaunchKernelGGL((gemm_bf16_tiled<64, 64, EPI>), grid, dim3(256), 0, stream, A, W, e, M, N, K);
-    }
-    return 0;
-  }
-  constexpr int NS = (EPI == EPI_SWIGLU) ? 2 : 1;
-  const int strips = (N + 16 * NS - 1) / (16 * NS);
-  const int blocks = (strips + 3) / 4;
-  // Enough waves to keep HBM busy: split K while there are fewer than ~8 per CU.
-  int splits = 1;
-  const int want_waves = num_cus * 8;
-  if (strips < want_waves) {
-    splits = (want_waves + strips - 1) / strips;
-    const int max_splits = K / 128 > 0 ? K / 128 : 1;
-    if (splits > max_splits) splits = max_splits;
-    if (splits > 32) splits = 32;
-    // the partial sums are written and read once: keep that under a quarter of
-    // the weight bytes (4*splits*M*N*2 against 2*N*K)
-    const int traffic_cap = K / (16 * M) > 0 ? K / (16 * M) : 1;
-    if (splits > traffic_cap) splits = traffic_cap;
-    while (splits > 1 && (size_t)splits * M * N > workspace_floats) --splits;
-  }
-  int k_per_split = ((K + splits - 1) / splits + 31) / 32 * 32;
-  splits = (K + k_per_split - 1) / k_per_split;
-  dim3 grid(blocks, splits), block(256);
-  const int mb = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
-#define SKINNY(MB_, SPLIT_)                                                                      \
-  hipLaunchKernelGGL((gemm_bf16_skinny<MB_, NS, EPI, SPLIT_>), grid, block, 0, stream, A, W, e, \
-                     workspace, M, N, K, k_per_split)
-  if (splits > 1) {
-    if (mb == 1) SKINNY(1, true); else if (mb == 2) SKINNY(2, true); else SKINNY(4, true);
-    const int cols = (EPI == EPI_SWIGLU) ? e.n_out : N;
-    const size_t total = (size_t)M * cols;
-    hipLaunchKernelGGL((splitk_epilogue<bf16_t, EPI>), dim3((unsigned)((total + 255) / 256)), dim3(256),
-                       0, stream, workspace, e, M, N, splits);
+static int launch_bf16(const bf16_t* A, const bf16_t* W, EpiArgs e, int M, int N, int K, int num_cus,
+                       hipStream_t stream) {
+  // the large tile when it still fills the chip, else the small one
+  const long big_tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
+  if (big_tiles >= num_cus) {
+    dim3 grid((N + 127) / 128, (M + 127) / 128);
+    hipLaunchKernelGGL((gemm_bf16_tiled<128, 128, EPI>), grid, dim3(256), 0, stream, A, W, e, M, N, K);
   } else {
-    if (mb == 1) SKINNY(1, false); else if (mb == 2) SKINNY(2, false); else SKINNY(4, false);
+    dim3 grid((N + 63) / 64, (M + 63) / 64);
+    hipLaunchKernelGGL((gemm_bf16_tiled<64, 64, EPI>), grid, dim3(256), 0, stream, A, W, e, M, N, K);
   }
-#undef SKINNY
   return 0;
 }
 
 // x [M,K] (dtype), w [N,K] (dtype); epilogue selects what `out` is.  For SWIGLU N
-// is the number of interleaved weight rows (2 * ceil16(n_out)).  `workspace` is
-// float32 scratch for split-K partial sums (may be null: no splitting).
+// is the number of interleaved weight rows (2 * ceil16(n_out)).
 extern "C" int llmlab_linear(const void* x, const void* w, int dtype, int epilogue, void* out,
                              const void* bias, int bias_dtype, int M, int N, int K, int ldo, int n_out,
-                             float* workspace, size_t workspace_floats, int num_cus,
-                             hipStream_t stream) {
+                             int num_cus, hipStream_t stream) {
   LLMLAB_REQUIRE(M >= 0 && N > 0 && K > 0, "linear: bad sizes M=%d N=%d K=%d", M, N, K);
   LLMLAB_REQUIRE(epilogue >= 0 && epilogue <= 3, "linear: unknown epilogue %d", epilogue);
   if (epilogue == EPI_SWIGLU) {
@@ -422,7 +256,6 @@ extern "C" int llmlab_linear(const void* x, const void* w, int dtype, int epilog
   LLMLAB_REQUIRE(ldo >= n_out, "linear: output row stride %d < %d columns", ldo, n_out);
   if (M == 0) return 0;
   EpiArgs e{out, bias, bias_dtype == DT_BF16, ldo, n_out};
-  if (workspace == nullptr) workspace_floats = 0;
   if (num_cus <= 0) num_cus = 256;
   if (dtype == DT_BF16) {
     LLMLAB_REQUIRE(K % 8 == 0, "linear(bfloat16): inner size %d must be a multiple of 8", K);
@@ -431,10 +264,10 @@ extern "C" int llmlab_linear(const void* x, const void* w, int dtype, int epilog
     const bf16_t* A = (const bf16_t*)x;
     const bf16_t* W = (const bf16_t*)w;
     switch (epilogue) {
-      case EPI_STORE: launch_bf16<EPI_STORE>(A, W, e, M, N, K, workspace, workspace_floats, num_cus, stream); break;
-      case EPI_RESID: launch_bf16<EPI_RESID>(A, W, e, M, N, K, workspace, workspace_floats, num_cus, stream); break;
-      case EPI_F32: launch_bf16<EPI_F32>(A, W, e, M, N, K, workspace, workspace_floats, num_cus, stream); break;
-      default: launch_bf16<EPI_SWIGLU>(A, W, e, M, N, K, workspace, workspace_floats, num_cus, stream); break;
+      case EPI_STORE: launch_bf16<EPI_STORE>(A, W, e, M, N, K, num_cus, stream); break;
+      case EPI_RESID: launch_bf16<EPI_RESID>(A, W, e, M, N, K, num_cus, stream); break;
+      case EPI_F32: launch_bf16<EPI_F32>(A, W, e, M, N, K, num_cus, stream); break;
+      default: launch_bf16<EPI_SWIGLU>(A, W, e, M, N, K, num_cus, stream); break;
     }
   } else {
     dim3 grid((N + 63) / 64, (M + 63) / 64), block(256);

@@ -78,7 +78,7 @@ class HipOps:
         c.llmlab_rope_inplace.argtypes = [_c_ptr, _c_int, _c_int, _c_int, _c_int, _c_long, _c_long,
                                           _c_ptr, _c_ptr, _c_ptr]
         c.llmlab_linear.argtypes = [_c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_int, _c_int,
-                                    _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_size, _c_int, _c_ptr]
+                                    _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr]
         c.llmlab_sample.argtypes = [_c_ptr, _c_long, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr]
         c.llmlab_argmax.argtypes = [_c_ptr, _c_long, _c_int, _c_int, _c_ptr, _c_ptr, _c_size, _c_ptr]
         c.llmlab_argmax.restype = _c_int
@@ -198,13 +198,14 @@ class HipOps:
             if bias.numel() != n:
                 raise ValueError("linear: bias length differs from the output width")
         ldo = out.stride(0) if m > 1 else max(out.stride(0), n_out)
-        if x.dtype == torch.bfloat16 and m <= self.FUSED_MAX_ROWS:
+        # few rows: the block kernel that splits K inside a block; from 17 rows on only
+        # for narrow outputs (the tiled kernel has too few tiles there), measured
+        if x.dtype == torch.bfloat16 and (m <= 16 or (m <= self.skinny_max_rows and n < 8192)):
             self._skinny(x, False, None, None, 0.0, w, bias, epilogue, out, m, n, k, ldo, n_out)
             return
         self._check(self._core.llmlab_linear(
             self._ptr(x), self._ptr(w), _dt(x), epilogue, self._ptr(out), self._ptr(bias),
-            _dt(bias) if bias is not None else 0, m, n, k, ldo, n_out, self._ptr(self.workspace),
-            self.workspace.numel(), self.num_cus, self._stream()))
+            _dt(bias) if bias is not None else 0, m, n, k, ldo, n_out, self.num_cus, self._stream()))
 
     def linear(self, x, w, out, bias=None) -> None:
         self._linear(x, w, out, bias, EPI_STORE, w.shape[0])
@@ -223,11 +224,14 @@ class HipOps:
         self._linear(x, w_gate_up, out, None, EPI_SWIGLU, inter)
 
     # ----------------------------------------------- few rows: fused kernels
-    FUSED_MAX_ROWS = 64
+    FUSED_MAX_ROWS = 64           # most rows the few-row kernels take at all
+    skinny_max_rows = 64          # plain products up to here may take the few-row kernel
+    fuse_max_rows = 16            # steps up to here take the fused kernels: their rows fit
+                                  # the staging buffer; beyond, norm + tiled product is faster
 
     def can_fuse(self, rows: int, dtype) -> bool:
-        """Whether the fused few-row kernels take this step (bfloat16, at most 64 rows)."""
-        return dtype == torch.bfloat16 and 0 < rows <= self.FUSED_MAX_ROWS
+        """Whether the fused few-row kernels take this step (bfloat16, few rows)."""
+        return dtype == torch.bfloat16 and 0 < rows <= self.fuse_max_rows
 
     def _skinny(self, x, norm, x_rows, norm_w, eps, w, bias, epilogue, out, m, n, k, ldo, n_out,
                 qkv=None) -> None:

@@ -72,9 +72,10 @@ class EmuOps:
 
     # ------------------------------------------------- fused few-row kernels
     FUSED_MAX_ROWS = 64
+    fuse_max_rows = 16
 
     def can_fuse(self, rows, dtype):
-        return self.fuse and dtype == torch.bfloat16 and 0 < rows <= self.FUSED_MAX_ROWS
+        return self.fuse and dtype == torch.bfloat16 and 0 < rows <= self.fuse_max_rows
 
     def _normed(self, x, rows_index, norm_w, eps, n):
         v = x.float() if rows_index is None else x.float()[rows_index[:n].long()]
