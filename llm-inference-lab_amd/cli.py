@@ -3,9 +3,9 @@ tokens, with one JSON object on standard output.
 
 Option names and meanings follow the reference's command line where it has
 them (rust/engine/examples/qwen2.rs:38-73): ``--dtype``, ``--model-dir``,
-``--prompt``, ``--max-new-tokens``, ``--max-batch-tokens``, ``--reference-dir``,
+``--prompt``, ``--max-new-tokens``, ``--max-batch-tokens``, ``--disable-overlap``, ``--reference-dir``,
 ``--repeat``, ``--cuda-graph``, ``--trace-steps``.  Not taken over:
-``--disable-overlap`` and ``--prefix-cache`` (this engine has neither).  Added:
+``--prefix-cache`` (this engine has none).  Added:
 token ids as input, random weights, temperature and seed, cache sizing.
 The output object has the reference's fields (examples/qwen2.rs:262-268).
 """
@@ -32,6 +32,8 @@ def build_parser() -> argparse.ArgumentParser:
     ap.add_argument("--max-new-tokens", type=int, default=8, help="most generated tokens; positive")
     ap.add_argument("--max-batch-tokens", type=int, default=512,
                     help="most uncached input tokens per step, shared by decode and prefill")
+    ap.add_argument("--disable-overlap", action="store_true",
+                    help="wait for the host's token processing before the next step (serial baseline)")
     ap.add_argument("--reference-dir", help="folder with reference.json and logits.f32 to check against")
     ap.add_argument("--repeat", type=int, default=1, help="run the same prompt N times, checking equality")
     ap.add_argument("--cuda-graph", "--graph", dest="graph", action="store_true",
@@ -132,7 +134,8 @@ def main(argv: Optional[List[str]] = None) -> int:
         out = engine.generate(prompts, max_new_tokens=args.max_new_tokens,
                               temperature=args.temperature, seed=args.sampling_seed,
                               max_batch_tokens=args.max_batch_tokens,
-                              trace=trace if args.trace_steps else None)
+                              trace=trace if args.trace_steps else None,
+                              overlap=not args.disable_overlap)
         elapsed = time.perf_counter() - start
         firsts = [r.first_token_time - start for r in engine.last_scheduler.finished.values()
                   if r.first_token_time is not None]

@@ -189,3 +189,23 @@ extern "C" int llmlab_rope_inplace(void* x, int dtype, int rows, int heads, int 
   LLMLAB_LAUNCH_CHECK("rope_inplace");
   return 0;
 }
+
+// ------------------------------------------------------------- token feedback
+// dst[dst_index[i]] = src[src_index[i]]: tokens chosen by the previous step go
+// straight into this step's input rows without a trip through the host.
+__global__ void gather_tokens_kernel(int* __restrict__ dst, const int* __restrict__ dst_index,
+                                     const int* __restrict__ src, const int* __restrict__ src_index,
+                                     int n) {
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) dst[dst_index[i]] = src[src_index[i]];
+}
+
+extern "C" int llmlab_gather_tokens(int* dst, const int* dst_index, const int* src, const int* src_index,
+                                    int n, hipStream_t stream) {
+  LLMLAB_REQUIRE(n >= 0, "gather_tokens: negative count");
+  if (n == 0) return 0;
+  hipLaunchKernelGGL(gather_tokens_kernel, dim3((n + 63) / 64), dim3(64), 0, stream, dst, dst_index, src,
+                     src_index, n);
+  LLMLAB_LAUNCH_CHECK("gather_tokens");
+  return 0;
+}

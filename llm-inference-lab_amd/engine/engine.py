@@ -120,25 +120,26 @@ class Engine:
         return self.step_fn(entries)
 
     # ------------------------------------------------------------ generation
-    def scheduler(self, max_batch_tokens: Optional[int] = None, on_token=None, trace=None):
+    def scheduler(self, max_batch_tokens: Optional[int] = None, on_token=None, trace=None,
+                  overlap: bool = True):
         """A scheduler over this engine (continuous batching, chunked prefill)."""
         from ..sampling.sampler import Sampler
         from .scheduler import Scheduler
         if self._sampler is None:
             self._sampler = Sampler(self.ops, self.max_requests)
         return Scheduler(self, self._sampler, max_batch_tokens or self.max_batch_tokens,
-                         on_token=on_token, trace=trace)
+                         on_token=on_token, trace=trace, overlap=overlap)
 
     def generate(self, prompts: Sequence[Sequence[int]], max_new_tokens: int = 8,
                  temperature: Optional[float] = None, seed: int = 0, eos_token_id=None,
                  sampling=None, max_batch_tokens: Optional[int] = None, on_token=None,
-                 trace=None) -> List[List[int]]:
+                 trace=None, overlap: bool = True) -> List[List[int]]:
         """Token ids in, generated token ids out, one list per prompt.  ``sampling``
         (one ``SamplingConfig`` or one per prompt) overrides the scalar options; the
         i-th prompt draws from the random stream ``seed + i``.  A request that the
         scheduler refuses raises its error here."""
         from ..sampling.params import SamplingConfig
-        sched = self.scheduler(max_batch_tokens, on_token, trace)
+        sched = self.scheduler(max_batch_tokens, on_token, trace, overlap)
         ids = []
         for i, prompt in enumerate(prompts):
             if sampling is None:

@@ -24,6 +24,13 @@ Decisions, all taken from the reference's Runner and its batch policy:
   the end-of-sequence token counts as generated and is kept
   (model_runner.rs:280-321); a request ends at end-of-sequence or at its budget
   and gives its pages and its row back before the next step.
+* Overlap (model_runner.rs:839-896; the reference's ``--disable-overlap`` turns it
+  off): step N+1 is put on the GPU before the tokens of step N are read; a request
+  whose token is still on its way takes it from the GPU's memory as its next input.
+  What the host does between two steps then hides behind the GPU's work.  A request
+  that turns out to have ended at step N (end of sequence) has by then been given
+  one more token in step N+1; that token is dropped.  The tokens are the same as
+  without overlap.
 """
 from __future__ import annotations
 
@@ -52,6 +59,7 @@ class Request:
     promised_pages: List[int] = dataclasses.field(default_factory=list)
     error: Optional[Exception] = None
     finish_reason: Optional[str] = None        # "eos", "length", "error"
+    in_flight: bool = False                    # a token of this request is chosen but not read yet
     arrival: float = 0.0
     first_token_time: Optional[float] = None
     finish_time: Optional[float] = None
@@ -62,7 +70,17 @@ class Request:
 
     @property
     def decoding(self) -> bool:
-        return len(self.generated) > 0
+        return len(self.generated) > 0 or self.in_flight
+
+    @property
+    def budget_left(self) -> int:
+        """Tokens this request may still be given (one is taken by a token in flight)."""
+        return self.remaining - (1 if self.in_flight else 0)
+
+    @property
+    def known_len(self) -> int:
+        """Tokens of the sequence, the one in flight included."""
+        return len(self.tokens) + (1 if self.in_flight else 0)
 
     @property
     def computed(self) -> int:
@@ -78,7 +96,7 @@ class Planned:
 
 def plan_step(active: Sequence[Request], max_batch_tokens: int) -> List[Planned]:
     """Decode first, then prompts in order, under one token budget."""
-    runnable = [r for r in active if not r.finished and r.remaining > 0]
+    runnable = [r for r in active if not r.finished and r.budget_left > 0]
     decode_budget = min(sum(1 for r in runnable if r.decoding), max_batch_tokens)
     prefill_budget = max_batch_tokens - decode_budget
     plan: List[Planned] = []
@@ -94,7 +112,7 @@ def plan_step(active: Sequence[Request], max_batch_tokens: int) -> List[Planned]
                 continue
             count = min(len(r.tokens) - ready, prefill_budget)
             prefill_budget -= count
-        plan.append(Planned(r, count, ready + count == len(r.tokens)))
+        plan.append(Planned(r, count, ready + count == r.known_len))
     return plan
 
 
@@ -108,7 +126,7 @@ class Scheduler:
 
     def __init__(self, engine, sampler, max_batch_tokens: Optional[int] = None,
                  on_token: Optional[Callable[[Request, int], None]] = None,
-                 trace: Optional[Callable[[dict], None]] = None):
+                 trace: Optional[Callable[[dict], None]] = None, overlap: bool = True):
         self.engine = engine
         self.sampler = sampler
         self.max_batch_tokens = int(max_batch_tokens or engine.max_batch_tokens)
@@ -120,6 +138,8 @@ class Scheduler:
         self._next_id = 0
         self.on_token = on_token
         self.trace = trace
+        self.overlap = bool(overlap)
+        self._pending = None            # (requests, PendingTokens) of the step whose tokens are unread
         self.steps = 0
         self.step_log: List[List[Tuple[int, int]]] = []     # per step: (request id, tokens)
         self.keep_step_log = False
@@ -200,39 +220,66 @@ class Scheduler:
 
     # ------------------------------------------------------------------- step
     def step(self) -> List[Request]:
-        """Admit, plan, run one step, sample, finish.  Returns the requests that
-        finished in this call."""
+        """Admit, plan, run one step, choose tokens, finish.  Returns the requests that
+        finished in this call.  With overlap the tokens read in this call are those of
+        the step before the one it starts."""
         before = set(self.finished)
         self._admit()
         plan = plan_step(self.active, self.max_batch_tokens)
+        started = None
         if plan:
             entries = []
             for p in plan:
-                start = p.request.computed
-                entries.append(StepEntry(p.request.cache, p.request.tokens[start:start + p.count],
-                                         [p.count - 1] if p.yields_token else []))
+                r = p.request
+                start = r.computed
+                if r.in_flight:       # its input token is still on the GPU
+                    source = (self._pending[1].device_tokens, self._pending[0].index(r))
+                    entries.append(StepEntry(r.cache, [0], [0] if p.yields_token else [], source))
+                else:
+                    entries.append(StepEntry(r.cache, r.tokens[start:start + p.count],
+                                             [p.count - 1] if p.yields_token else []))
             t0 = time.perf_counter()
             logits = self.engine.step(entries)
             yielding = [p.request for p in plan if p.yields_token]
             if yielding:
-                tokens = self.sampler.sample(
+                counters = [len(r.generated) + (1 if r.in_flight else 0) for r in yielding]
+                started = (yielding, self.sampler.sample_async(
                     logits, [r.sampling.effective_temperature for r in yielding],
-                    [r.sampling.seed for r in yielding], [len(r.generated) for r in yielding])
-                now = time.perf_counter()
-                for r, token in zip(yielding, tokens):
-                    self._accept(r, token, now)
+                    [r.sampling.seed for r in yielding], counters))
             self.steps += 1
             if self.keep_step_log:
                 self.step_log.append([(p.request.request_id, p.count) for p in plan])
             if self.trace is not None:
-                self.trace({"event": "step_completed", "step": self.steps,
+                self.trace({"event": "step_submitted", "step": self.steps,
                             "phase": "decode" if all(p.request.decoding and p.count == 1 for p in plan)
                             else "prefill",
                             "requests": len(plan), "tokens": sum(p.count for p in plan),
-                            "seconds": time.perf_counter() - t0})
+                            "submit_seconds": time.perf_counter() - t0})
+        # the tokens of the step before (with overlap), or of this one
+        self._collect()
+        if started is not None:
+            self._pending = started
+            for r in started[0]:
+                r.in_flight = True
+            if not self.overlap:
+                self._collect()
         for r in [r for r in self.active if r.finished]:
             self._release(r)
         return [self.finished[i] for i in self.finished if i not in before]
+
+    def _collect(self) -> None:
+        """Read the tokens of the pending step and give them to their requests."""
+        if self._pending is None:
+            return
+        requests, handle = self._pending
+        self._pending = None
+        tokens = handle.result()
+        now = time.perf_counter()
+        for r, token in zip(requests, tokens):
+            r.in_flight = False
+            if r.finished:
+                continue            # it ended a step earlier; this token was one too many
+            self._accept(r, token, now)
 
     def _accept(self, r: Request, token: int, now: float) -> None:
         r.generated.append(token)
@@ -264,7 +311,7 @@ class Scheduler:
 
     @property
     def idle(self) -> bool:
-        return not self.waiting and not self.active
+        return not self.waiting and not self.active and self._pending is None
 
     def run(self) -> Dict[int, Request]:
         """Step until every request has finished."""

@@ -33,6 +33,10 @@ class StepEntry:
     request: RequestCache
     tokens: Sequence[int]
     want: Sequence[int] = ()        # indices into ``tokens`` whose logits are returned
+    # The one token of this entry is not known to the host yet: it is element
+    # ``source[1]`` of the int32 device tensor ``source[0]`` (what the sampler wrote
+    # for the previous step).  ``tokens`` then holds one placeholder.
+    source: Optional[Tuple[torch.Tensor, int]] = None
 
 
 @dataclasses.dataclass
@@ -63,7 +67,7 @@ class StepContext:
         # One int32 buffer, fixed offsets: the addresses never change, so a
         # captured graph of a step stays valid while only the contents move.
         sizes = [("token_ids", r), ("positions", r), ("row_req", r), ("q_start", b + 1),
-                 ("start_pos", b), ("req_rows", b), ("want_rows", r)]
+                 ("start_pos", b), ("req_rows", b), ("want_rows", r), ("feed_dst", b), ("feed_src", b)]
         self._offsets: Dict[str, Tuple[int, int]] = {}
         at = 0
         for name, n in sizes:
@@ -135,6 +139,8 @@ class StepContext:
         o = {k: v[0] for k, v in self._offsets.items()}
         row = 0
         want: List[int] = []
+        feeds: List[Tuple[int, int]] = []
+        feed_tensor = None
         self.host_q_start, self.host_start_pos, self.host_req_rows = [], [], []
         max_q = max_ctx = 0
         for b, e in enumerate(entries):
@@ -146,6 +152,13 @@ class StepContext:
             h[o["q_start"] + b] = row
             h[o["start_pos"] + b] = start
             h[o["req_rows"] + b] = e.request.row
+            if e.source is not None:
+                if n != 1:
+                    raise ValueError("an entry fed from the device brings exactly one token")
+                if feed_tensor is not None and feed_tensor is not e.source[0]:
+                    raise ValueError("all device-fed entries of a step share one source tensor")
+                feed_tensor = e.source[0]
+                feeds.append((row, int(e.source[1])))
             for w in e.want:
                 if not 0 <= w < n:
                     raise ValueError(f"request {e.request.request_id!r}: wanted place {w} is not "
@@ -168,8 +181,14 @@ class StepContext:
             table = h[at:at + self.max_reqs * self.max_pages].reshape(self.max_reqs, self.max_pages)
             for b, e in enumerate(entries):
                 table[b, :used_pages] = cache.tables[gi][e.request.row, :used_pages]
+        for i, (dst, src) in enumerate(feeds):
+            h[o["feed_dst"] + i] = dst
+            h[o["feed_src"] + i] = src
         self._upload(n_reqs)
         self._set_views()
+        if feeds:
+            self.ops.gather_tokens(self._view("token_ids", self.max_rows), self._view("feed_dst", len(feeds)),
+                                   feed_tensor, self._view("feed_src", len(feeds)), len(feeds))
 
     def _upload(self, n_reqs: int) -> None:
         self._dev[:self._meta_len].copy_(self._host[:self._meta_len], non_blocking=True)
@@ -248,7 +267,7 @@ class StepFunction:
             seen.add(id(e.request))
             if len(e.tokens) == 0:
                 raise ValueError(f"request {e.request.request_id!r} brings no token")
-            for t in e.tokens:
+            for t in (e.tokens if e.source is None else ()):
                 if not 0 <= int(t) < vocab:
                     raise ValueError(f"token id {t} is outside the vocabulary of {vocab}")
             if e.request.computed_len + len(e.tokens) > max_pos:

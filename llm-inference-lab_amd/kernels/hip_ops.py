@@ -80,6 +80,8 @@ class HipOps:
         c.llmlab_linear.argtypes = [_c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_int, _c_int,
                                     _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr]
         c.llmlab_sample.argtypes = [_c_ptr, _c_long, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr]
+        c.llmlab_gather_tokens.argtypes = [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr]
+        c.llmlab_gather_tokens.restype = _c_int
         c.llmlab_argmax.argtypes = [_c_ptr, _c_long, _c_int, _c_int, _c_ptr, _c_ptr, _c_size, _c_ptr]
         c.llmlab_argmax.restype = _c_int
         c.llmlab_skinny_linear.argtypes = [
@@ -153,6 +155,15 @@ class HipOps:
                              f"out {tuple(out.shape)} do not fit")
         self._check(self._core.llmlab_embed(self._ptr(table), _dt(table), self._ptr(ids), self._ptr(out),
                                             rows, hidden, table.shape[0], self._stream()))
+
+    def gather_tokens(self, dst, dst_index, src, src_index, n) -> None:
+        """dst[dst_index[i]] = src[src_index[i]] for i < n (all int32 on the GPU)."""
+        for t, name in ((dst, "dst"), (dst_index, "dst_index"), (src, "src"), (src_index, "src_index")):
+            self._need(t, f"gather_tokens {name}", torch.int32)
+        if dst_index.numel() < n or src_index.numel() < n:
+            raise ValueError("gather_tokens: index arrays are shorter than the count")
+        self._check(self._core.llmlab_gather_tokens(self._ptr(dst), self._ptr(dst_index), self._ptr(src),
+                                                    self._ptr(src_index), int(n), self._stream()))
 
     def rmsnorm(self, x, weight, eps, out, rows=None) -> None:
         self._need(x, "norm input", torch.float32)

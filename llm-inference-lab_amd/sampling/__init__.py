@@ -1,2 +1,2 @@
 from .params import SamplingConfig, read_generation_config
-from .sampler import Sampler, uniform
+from .sampler import Sampler, PendingTokens, uniform

@@ -32,31 +32,67 @@ def uniform(seed: int, n: int) -> float:
     return (z >> 40) / float(1 << 24)
 
 
+class PendingTokens:
+    """Tokens chosen on the GPU whose copy to the host may still be under way."""
+
+    def __init__(self, device_tokens: torch.Tensor, host_tokens: torch.Tensor, event, rows: int):
+        self.device_tokens = device_tokens      # int32 [rows] on the GPU: the next step may read it there
+        self._host = host_tokens
+        self._event = event
+        self.rows = rows
+
+    def result(self) -> List[int]:
+        """Wait for the copy; raises if a row held no finite logit."""
+        if self._event is not None:
+            self._event.synchronize()
+        tokens = self._host[:self.rows].tolist()
+        for t in tokens:
+            if t < 0:
+                raise FloatingPointError("non-finite logits: no token can be chosen")
+        return tokens
+
+
 class Sampler:
+    SLOTS = 2     # results of two steps can be alive: the one being read and the one in flight
+
     def __init__(self, ops, max_requests: int):
         self.ops = ops
         self.device = ops.device
-        pin = torch.device(self.device).type == "cuda"
-        self._host = torch.zeros((2, max_requests), dtype=torch.float32, pin_memory=pin)
+        self._cuda = torch.device(self.device).type == "cuda"
+        self._host = torch.zeros((2, max_requests), dtype=torch.float32, pin_memory=self._cuda)
         self._dev = torch.zeros((2, max_requests), dtype=torch.float32, device=self.device)
-        self._out = torch.zeros(max_requests, dtype=torch.int32, device=self.device)
+        self._out = [torch.zeros(max_requests, dtype=torch.int32, device=self.device)
+                     for _ in range(self.SLOTS)]
+        self._out_host = [torch.zeros(max_requests, dtype=torch.int32, pin_memory=self._cuda)
+                          for _ in range(self.SLOTS)]
+        self._slot = 0
 
-    def sample(self, logits: torch.Tensor, temperatures: Sequence[float], seeds: Sequence[int],
-               counters: Sequence[int]) -> List[int]:
-        """One token per row of ``logits``.  Raises if a row holds no finite value."""
+    def sample_async(self, logits: torch.Tensor, temperatures: Sequence[float], seeds: Sequence[int],
+                     counters: Sequence[int]) -> PendingTokens:
+        """Choose one token per row of ``logits``; the tokens stay on the GPU and a copy
+        to the host is started.  The buffers are reused after ``SLOTS`` further calls."""
         rows = logits.shape[0]
-        out = self._out[:rows]
+        self._slot = (self._slot + 1) % self.SLOTS
+        out, out_host = self._out[self._slot], self._out_host[self._slot]
         if all(t <= 0.0 for t in temperatures):
-            self.ops.argmax(logits, out)
+            self.ops.argmax(logits, out[:rows])
         else:
             h = self._host.numpy()
             h[0, :rows] = np.asarray(temperatures, dtype=np.float32)
             h[1, :rows] = np.asarray([uniform(s, c) for s, c in zip(seeds, counters)], dtype=np.float32)
             self._dev[0, :rows].copy_(self._host[0, :rows], non_blocking=True)
             self._dev[1, :rows].copy_(self._host[1, :rows], non_blocking=True)
-            self.ops.sample(logits, self._dev[0, :rows], self._dev[1, :rows], out)
-        tokens = out.cpu().tolist()
-        for t in tokens:
-            if t < 0:
-                raise FloatingPointError("non-finite logits: no token can be chosen")
-        return tokens
+            self.ops.sample(logits, self._dev[0, :rows], self._dev[1, :rows], out[:rows])
+        event = None
+        if self._cuda:
+            out_host[:rows].copy_(out[:rows], non_blocking=True)
+            event = torch.cuda.Event()
+            event.record()
+        else:
+            out_host[:rows].copy_(out[:rows])
+        return PendingTokens(out, out_host, event, rows)
+
+    def sample(self, logits: torch.Tensor, temperatures: Sequence[float], seeds: Sequence[int],
+               counters: Sequence[int]) -> List[int]:
+        """One token per row of ``logits``.  Raises if a row holds no finite value."""
+        return self.sample_async(logits, temperatures, seeds, counters).result()

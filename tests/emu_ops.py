@@ -34,6 +34,11 @@ class EmuOps:
         self._count("embed")
         out.copy_(table[ids.long()].float())
 
+    def gather_tokens(self, dst, dst_index, src, src_index, n):
+        self._count("gather_tokens")
+        for i in range(n):
+            dst[int(dst_index[i])] = src[int(src_index[i])]
+
     def rmsnorm(self, x, weight, eps, out, rows=None):
         self._count("rmsnorm")
         v = x.float() if rows is None else x.float()[rows.long()]

@@ -155,12 +155,56 @@ def test_refused_requests_do_not_hurt_their_peers():
 def test_finished_request_frees_before_the_next_step():
     cfg = H.config_of("A")
     engine = engine_of(num_pages=8)
-    sched = engine.scheduler()
+    sched = engine.scheduler(overlap=False)
     sched.add_request(H.random_ids(cfg, 4, 1), SamplingConfig(max_new_tokens=1))
     sched.add_request(H.random_ids(cfg, 4, 2), SamplingConfig(max_new_tokens=3, eos_token_id=[]))
     finished = sched.step()
     assert [r.request_id for r in finished] == [0]
     assert engine.cache.live_requests == 1 and engine.cache.free_pages(0) == 7
+    sched.run()
+    # with overlap its token is read one call later, and it is freed then; it is
+    # never given a second step (its budget is known to be spent)
+    sched = engine.scheduler(overlap=True)
+    sched.keep_step_log = True
+    a = sched.add_request(H.random_ids(cfg, 4, 1), SamplingConfig(max_new_tokens=1))
+    b = sched.add_request(H.random_ids(cfg, 4, 2), SamplingConfig(max_new_tokens=3, eos_token_id=[]))
+    assert sched.step() == []
+    assert [r.request_id for r in sched.step()] == [a]
+    assert engine.cache.live_requests == 1
+    sched.run()
+    assert sched.step_log == [[(a, 4), (b, 4)], [(b, 1)], [(b, 1)]]
+    engine.cache.check()
+
+
+def test_overlap_gives_the_same_tokens_and_steps():
+    cfg = H.config_of("B")
+    prompts = [H.random_ids(cfg, n, 90 + n) for n in (5, 40, 61, 3)]
+    engine = engine_of("B", num_pages=24, max_requests=3)
+    results = {}
+    for overlap in (False, True):
+        sched = engine.scheduler(max_batch_tokens=16, overlap=overlap)
+        sched.keep_step_log = True
+        for i, p in enumerate(prompts):
+            sched.add_request(p, SamplingConfig(max_new_tokens=6 + i, temperature=0.7, seed=i, eos_token_id=[]))
+        done = sched.run()
+        results[overlap] = ([done[i].generated for i in range(len(prompts))], sched.step_log)
+        engine.cache.check()
+        assert engine.cache.live_requests == 0
+    assert results[False][0] == results[True][0]
+    assert results[False][1] == results[True][1]
+
+
+def test_overlap_drops_the_token_after_an_end_of_sequence():
+    cfg = H.config_of("A")
+    engine = engine_of(num_pages=16)
+    prompt = H.random_ids(cfg, 9, 3)
+    free_run = generate(engine, [prompt], 64, max_new=6, eos_token_id=[])[0]
+    stop = free_run[2]
+    for overlap in (False, True):
+        cut = engine.generate([prompt], max_new_tokens=6, eos_token_id=[stop], overlap=overlap)[0]
+        assert cut == free_run[:free_run.index(stop) + 1]
+        engine.cache.check()
+        assert engine.cache.live_requests == 0
 
 
 def test_temperature_stream_does_not_depend_on_the_cut_or_the_batch():
