@@ -41,13 +41,15 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=64)
-    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--layers", type=int, default=FULL_LAYERS)
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "f32"])
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 / 64 and the prefill")
+    ap.add_argument("--only-prefill", action="store_true",
+                    help="run nothing but the 2,048-token prefill (for profiling); prints its numbers")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -99,6 +101,25 @@ def main():
         assert engine.cache.live_requests == 0
         return seconds, live_tokens
 
+    def prefill_run(tokens=2048, repeats=4):
+        times = []
+        for _ in range(repeats):
+            req = engine.open("prefill")
+            ids = random_ids(tokens)
+            sync()
+            t0 = time.perf_counter()
+            engine.step([StepEntry(req, ids, [tokens - 1])])
+            sync()
+            times.append(time.perf_counter() - t0)
+            engine.close(req)
+        best = min(times[1:])
+        return {"value": round(tokens / best, 1), "tokens": tokens, "ms": round(best * 1e3, 3),
+                "frac": round(prefill_flops(cfg, tokens) / best / PEAK_FLOPS[args.dtype], 4)}
+
+    if args.only_prefill:
+        print(json.dumps({"prefill": prefill_run()}))
+        return
+
     seconds, live_tokens = decode_run(args.batch, args.steps, args.warmup)
     ms_per_step = seconds / args.steps * 1e3
     value = args.batch * args.steps / seconds
@@ -125,22 +146,7 @@ def main():
     }
     if not args.no_points:
         # prefill: one prompt of 2,048 tokens in one step, logits at its last place
-        tokens = 2048
-        times = []
-        for _ in range(4):
-            req = engine.open("prefill")
-            ids = random_ids(tokens)
-            sync()
-            t0 = time.perf_counter()
-            engine.step([StepEntry(req, ids, [tokens - 1])])
-            sync()
-            times.append(time.perf_counter() - t0)
-            engine.close(req)
-        best = min(times[1:])
-        flops = prefill_flops(cfg, tokens)
-        result["prefill"] = {"value": round(tokens / best, 1), "tokens": tokens,
-                             "ms": round(best * 1e3, 3),
-                             "frac": round(flops / best / PEAK_FLOPS[args.dtype], 4)}
+        result["prefill"] = prefill_run()
         points = {}
         for b in (1, 64):
             if b == args.batch:
