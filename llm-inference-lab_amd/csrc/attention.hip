@@ -75,6 +75,8 @@ struct KeyStep {
 // block share one tile and split the block's keys; they merge through LDS, and
 // blocks that split the keys further merge through global memory (see below).
 constexpr int DECODE_WAVES = D <= 64 ? 8 : (D <= 128 ? 4 : 2);
+constexpr int SPLIT_FILL = 1;      // blocks per compute unit a decode step aims at
+constexpr int DECODE_RING = 2;     // key steps in flight per wave (deeper rings measured no faster)
 
 template <int QB, bool DECODE>
 __global__ __launch_bounds__(DECODE ? 64 * DECODE_WAVES : 256) void attention_bf16_kernel(AttnArgs a) {
@@ -261,13 +263,22 @@ __global__ __launch_bounds__(DECODE ? 64 * DECODE_WAVES : 256) void attention_bf
   };
 
   if constexpr (PIPE) {
-    // the next step's loads are in flight while this one is computed
-    KeyStep<DC, DB> cur, nxt;
-    if (my_blk0 < my_blk1) fetch(my_blk0, cur);
-    for (int blk = my_blk0; blk < my_blk1; ++blk) {
-      if (blk + 1 < my_blk1) fetch(blk + 1, nxt);
-      compute(blk, cur);
-      cur = nxt;
+    // the loads of the next steps are in flight while this one is computed
+    constexpr int RING = DECODE_RING;
+    KeyStep<DC, DB> ring[RING];
+#pragma unroll
+    for (int p = 0; p < RING; ++p)
+      if (my_blk0 + p < my_blk1) fetch(my_blk0 + p, ring[p]);
+    for (int blk0 = my_blk0; blk0 < my_blk1; blk0 += RING) {
+#pragma unroll
+      for (int p = 0; p < RING; ++p) {
+        const int blk = blk0 + p;
+        if (blk < my_blk1) {
+          const KeyStep<DC, DB> cur = ring[p];
+          if (blk + RING < my_blk1) fetch(blk + RING, ring[p]);
+          compute(blk, cur);
+        }
+      }
     }
   } else {
     // ---- prefill: tiles of 64 keys go through LDS once per block and serve all its
@@ -584,11 +595,15 @@ extern "C" int llmlab_paged_attention(const void* q, int dtype, int q_stride, in
     // what is left is split over blocks
     const int visible = window > 0 ? min(window, max_ctx_len) : max_ctx_len;
     const int steps32 = (visible + 31) / 32 + 1;
-    int splits = (steps32 + 2 * DECODE_WAVES - 1) / (2 * DECODE_WAVES);
+    // about SPLIT_FILL blocks per compute unit: a unit's memory rate is the limit, so
+    // the keys are spread over all of them; but no more blocks than there are steps
+    // for their waves
     const long base = (long)reqs * nkv;
-    const long room = (16L * num_cus + base - 1) / base;      // blocks per (request, kv head) worth having
-    if (splits > room) splits = (int)room;
+    int splits = (int)((SPLIT_FILL * (long)num_cus + base - 1) / base);
+    const int most = (steps32 + DECODE_WAVES - 1) / DECODE_WAVES;      // one step per wave at least
+    if (splits > most) splits = most;
     if (splits > 16) splits = 16;                               // what the merge kernel takes
+    if (splits < 1) splits = 1;
     const size_t per_split = (size_t)total_rows * nq * (D + 2);
     while (splits > 1 && per_split * splits > workspace_floats) --splits;
     if (splits < 1) splits = 1;

@@ -119,6 +119,13 @@ class HipOps:
             raise UnsupportedSizeError(f"{num_heads} heads are not a multiple of {num_kv_heads} kv heads")
         self._attention_lib(head_dim)
 
+    def check_product_sizes(self, inner: int, dtype, what: str) -> None:
+        """Refuse at load time what the matrix product kernels do not take."""
+        if dtype == torch.bfloat16 and inner % 8 != 0:
+            raise UnsupportedSizeError(
+                f"{what}: bfloat16 matrix products need an inner size that is a multiple of 8, "
+                f"got {inner} (the float32 path takes any size)")
+
     # ---------------------------------------------------------------- helpers
     def _stream(self):
         return _c_ptr(torch.cuda.current_stream(self.device).cuda_stream)

@@ -79,6 +79,8 @@ class GQAAttention(Mixer):
     def bind(self, tensors, ops, dtype):
         super().bind(tensors, ops, dtype)
         ops.check_attention_sizes(self.num_heads, self.num_kv_heads, self.head_dim, dtype)
+        ops.check_product_sizes(self.hidden_size, dtype, "attention projections (hidden size)")
+        ops.check_product_sizes(self.q_size, dtype, "attention output projection (heads * head size)")
         t = self.tensor_names
         # One projection instead of three: the rows of Wq, Wk, Wv stacked.
         self.w_qkv = torch.cat([tensors[t["q_weight"]], tensors[t["k_weight"]],

@@ -93,6 +93,7 @@ class LinearHead(Part):
 
     def bind(self, tensors, ops, dtype):
         super().bind(tensors, ops, dtype)
+        ops.check_product_sizes(self.hidden_size, dtype, "output head (hidden size)")
         self.weight = tensors[self.tensor_names["weight"]]
 
     takes_normed_input = True

@@ -57,6 +57,8 @@ class SwiGLU(FeedForward):
 
     def bind(self, tensors, ops, dtype):
         super().bind(tensors, ops, dtype)
+        ops.check_product_sizes(self.hidden_size, dtype, "feed-forward (hidden size)")
+        ops.check_product_sizes(self.intermediate_size, dtype, "feed-forward (intermediate size)")
         t = self.tensor_names
         self.w_gate_up = interleave_gate_up(tensors[t["gate_weight"]], tensors[t["up_weight"]])
         self.w_down = tensors[t["down_weight"]].contiguous()

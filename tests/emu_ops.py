@@ -26,6 +26,9 @@ class EmuOps:
     def check_attention_sizes(self, num_heads, num_kv_heads, head_dim, dtype):
         pass
 
+    def check_product_sizes(self, inner, dtype, what):
+        pass
+
     def synchronize(self):
         pass
 

@@ -412,6 +412,9 @@ def test_refused_sizes(ops):
         ops.check_attention_sizes(4, 2, 24, torch.bfloat16)
     with pytest.raises(UnsupportedSizeError):
         ops.check_attention_sizes(4, 2, 272, torch.bfloat16)
+    with pytest.raises(UnsupportedSizeError, match="multiple of 8"):
+        ops.check_product_sizes(100, torch.bfloat16, "test")
+    ops.check_product_sizes(100, torch.float32, "test")
     x = torch.zeros(2, 100, dtype=torch.bfloat16, device=DEV)
     w = torch.zeros(8, 100, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(UnsupportedSizeError):
