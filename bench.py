@@ -1,6 +1,7 @@
 """Decode and prefill throughput of the engine on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--context S] [--layers L]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--context S]
+                    [--shape 0.5b|7b|32b] [--layers L]
 
 Default: the layer sizes of the Qwen2.5-0.5B shape with seeded random weights,
 batch 8, context 4096, bfloat16.  A "step" is one decode step of the whole
@@ -20,13 +21,21 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0
+FILL_TOKENS = 8192       # token budget of the steps that fill the caches before decoding is timed
 PEAK_FLOPS = {"bf16": 2.5e15, "f32": 157.3e12}
-MODEL = dict(
-    architectures=["Qwen2ForCausalLM"], model_type="qwen2", vocab_size=151936, hidden_size=896,
-    intermediate_size=4864, num_hidden_layers=24, num_attention_heads=14, num_key_value_heads=2,
-    head_dim=64, rms_norm_eps=1e-6, rope_theta=1e6, max_position_embeddings=32768,
-    tie_word_embeddings=True, use_sliding_window=False)
-FULL_LAYERS = MODEL["num_hidden_layers"]
+COMMON = dict(architectures=["Qwen2ForCausalLM"], model_type="qwen2", rms_norm_eps=1e-6, rope_theta=1e6,
+              max_position_embeddings=32768, use_sliding_window=False)
+SHAPES = {   # layer sizes of the published Qwen2.5 checkpoints; weights are random
+    "0.5b": dict(COMMON, vocab_size=151936, hidden_size=896, intermediate_size=4864,
+                 num_hidden_layers=24, num_attention_heads=14, num_key_value_heads=2, head_dim=64,
+                 tie_word_embeddings=True),
+    "7b": dict(COMMON, vocab_size=152064, hidden_size=3584, intermediate_size=18944,
+               num_hidden_layers=28, num_attention_heads=28, num_key_value_heads=4, head_dim=128,
+               tie_word_embeddings=False),
+    "32b": dict(COMMON, vocab_size=152064, hidden_size=5120, intermediate_size=27648,
+                num_hidden_layers=64, num_attention_heads=40, num_key_value_heads=8, head_dim=128,
+                tie_word_embeddings=False),
+}
 
 
 def prefill_flops(cfg, tokens):
@@ -44,7 +53,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=4096)
-    ap.add_argument("--layers", type=int, default=FULL_LAYERS)
+    ap.add_argument("--shape", default="0.5b", choices=sorted(SHAPES),
+                    help="layer sizes: those of Qwen2.5-0.5B (default), 7B or 32B")
+    ap.add_argument("--layers", type=int, default=None,
+                    help="run fewer layers than the shape has (both numbers are reported)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "f32"])
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 / 64 and the prefill")
@@ -60,7 +72,9 @@ def main():
     from llm_inference_lab_amd.engine.step import StepEntry
     from llm_inference_lab_amd.sampling import SamplingConfig
 
-    raw = dict(MODEL, num_hidden_layers=args.layers)
+    full_layers = SHAPES[args.shape]["num_hidden_layers"]
+    layers = args.layers or full_layers
+    raw = dict(SHAPES[args.shape], num_hidden_layers=layers)
     cfg = lab.Qwen2Config.from_dict(raw)
     batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
     max_batch = max(batches)
@@ -68,7 +82,7 @@ def main():
     context = args.context
     engine = lab.Engine(config=cfg, seed=0, dtype=args.dtype, device="cuda:0", page_size=page,
                         max_cache_tokens=max_batch * (context + page), max_requests=max_batch,
-                        max_batch_tokens=2048, max_seq_len=context + page, graph=not args.no_graph)
+                        max_batch_tokens=FILL_TOKENS, max_seq_len=context + page, graph=not args.no_graph)
     gen = torch.Generator().manual_seed(1234)
 
     def random_ids(n):
@@ -78,17 +92,27 @@ def main():
         torch.cuda.synchronize()
 
     def decode_run(batch, steps, warmup):
-        """Requests with (context - steps - warmup) cached tokens decode to `context`."""
-        prompt_len = context - steps - warmup - 1
-        sched = engine.scheduler(max_batch_tokens=2048)
-        never = cfg.vocab_size  # no token ends a request: a fixed number of outputs, as the reference's bench
-        for b in range(batch):
+        """`batch` requests decode side by side and reach `context` tokens at the end.
+
+        The scheduler decodes for requests whose prompts are in while it still
+        fills the others, so every request gets outputs enough for the fill, the
+        warm-up and the timed steps, and a prompt shorter by as much; none ends
+        before the timed steps are over (checked below).
+        """
+        fill_tokens = FILL_TOKENS
+        fill_steps = batch * context // fill_tokens + 2
+        outputs = fill_steps + warmup + steps + 1
+        prompt_len = context - outputs
+        assert prompt_len > 0, "context too short for this many steps"
+        sched = engine.scheduler(max_batch_tokens=fill_tokens)
+        for b in range(batch):      # no token ends a request: a fixed number of outputs, as the reference's bench
             sched.add_request(random_ids(prompt_len),
-                              SamplingConfig(max_new_tokens=steps + warmup + 1, eos_token_id=[]))
+                              SamplingConfig(max_new_tokens=outputs, eos_token_id=[]))
         while any(not r.decoding for r in sched.active) or sched.waiting:
             sched.step()                      # prefill in portions; ends with every request decoding
         for _ in range(warmup):
             sched.step()
+        assert len(sched.active) == batch
         live_tokens = sum(r.computed for r in sched.active)
         sync()
         t0 = time.perf_counter()
@@ -96,6 +120,7 @@ def main():
             sched.step()
         sync()
         seconds = time.perf_counter() - t0
+        assert len(sched.active) == batch, "a request ended inside the timed steps"
         live_tokens = (live_tokens + sum(r.computed for r in sched.active)) / 2
         sched.run()
         assert engine.cache.live_requests == 0
@@ -132,9 +157,9 @@ def main():
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": args.dtype, "data": "synthetic",
         "config": {
-            "model": "Qwen2.5-0.5B shape, random weights", "global_batch": args.batch,
-            "seq_len": context, "parallelism": "single GPU", "layers": args.layers,
-            "layers_of_full_model": FULL_LAYERS, "hidden_size": cfg.hidden_size,
+            "model": f"Qwen2.5-{args.shape.upper()} shape, random weights", "global_batch": args.batch,
+            "seq_len": context, "parallelism": "single GPU", "layers": layers,
+            "layers_of_full_model": full_layers, "hidden_size": cfg.hidden_size,
             "num_attention_heads": cfg.num_attention_heads,
             "num_key_value_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
             "intermediate_size": cfg.intermediate_size, "vocab_size": cfg.vocab_size,
