@@ -7,16 +7,22 @@
 //   ->  epilogue: bias / add into the residual / float32 logits / SwiGLU /
 //                 rotary + write of q, and of k and v into their cache pages
 //
-// A block owns `nsb` strips of 16 weight rows (for the q/k/v projection: exactly one
-// head) and splits K over `kw` waves per strip, so blockDim = 64 * nsb * kw.  Every
-// wave streams its slice of W from HBM straight into MFMA B fragments (loads of the
-// next steps are in flight while the current ones are multiplied), and leaves its
-// partial sums in LDS; the block adds the partial sums in a fixed order (no
-// atomics, results do not depend on timing) and applies the epilogue.
+// W comes packed in MFMA fragment order (see llmlab_pack_weight): the 16 rows x 32
+// columns a wave multiplies in one step are 1 KB of consecutive memory, lane l
+// owning bytes 16 l .. 16 l + 15, and the steps of a strip follow each other.  A
+// wave therefore streams one contiguous run of memory with full cache lines,
+// which at these sizes is worth a factor of two over rows of 64 bytes each.
 //
-// The rows of x are staged once per block in LDS as bfloat16 when they fit
-// (STAGE), so the strips of a block share them; otherwise every wave reads its
-// slice from global memory.  The norm is folded in without a pass of its own:
+// A block owns `nsb` strips of 16 weight rows (for the q/k/v projection: one head,
+// or two strips of one) and splits K over `kw` waves per strip, so blockDim =
+// 64 * nsb * kw.  Every wave streams its slice of W from HBM straight into MFMA B
+// fragments through a ring of registers, and leaves its partial sums in LDS; the
+// block adds the partial sums in a fixed order (no atomics, results do not depend
+// on timing) and applies the epilogue.
+//
+// The rows of x are staged once per block in LDS as bfloat16 (STAGE), so the strips
+// of a block share them; or every wave reads its slice from global memory (plain
+// products only).  The norm is folded in without a pass of its own:
 //   norm(x) . W^T = inv_rms[m] * ((x * w_norm) . W^T)
 // x * w_norm is what is staged (or built on the fly), the sum of squares falls out
 // of the same read, and inv_rms[m] scales the reduced sums in the epilogue.
@@ -57,12 +63,26 @@ struct SkinnyArgs {
 
 __device__ __forceinline__ float sk_silu(float z) { return z / (1.f + __expf(-z)); }
 
+// Loads of W (and of x where it is not staged) run R steps ahead of the MFMAs in a
+// ring of registers that is refilled slot by slot, so a wave always has R loads
+// in flight and never waits for all of them at once.  Measured at depths 4, 8 and
+// 12: no difference once the stream is continuous, so the shallow ring it is.
+#ifndef SK_RING_STAGE
+#define SK_RING_STAGE 4
+#endif
+#ifndef SK_RING_DIRECT
+#define SK_RING_DIRECT 4
+#endif
+__host__ __device__ constexpr int sk_ring(int mb, bool stage) {
+  return stage ? SK_RING_STAGE : (mb >= 4 ? SK_RING_DIRECT / 2 : SK_RING_DIRECT);
+}
+
 constexpr int SK_APAD = 8;   // padding of a staged row, in elements: 16-byte reads of 8 lanes cover all banks
 
 // floats of LDS before the staged rows (host and device must agree)
 __host__ __device__ inline size_t sk_float_words(int nsb, int kw, int mb, int M, int epi) {
   size_t f = (size_t)kw * nsb * mb * 256;        // partial sums
-  f += (size_t)kw * mb * 16 + (size_t)mb * 16;    // sums of squares, inverse rms
+  f += (size_t)mb * 16;                           // inverse rms
   f += (size_t)16 * nsb;                          // bias
   f += (size_t)mb * 16 * 2 + 128;                 // positions, pages, frequencies
   if (epi == SK_SWIGLU || epi == SK_QKV) f += (size_t)M * 16 * nsb;
@@ -71,8 +91,9 @@ __host__ __device__ inline size_t sk_float_words(int nsb, int kw, int mb, int M,
 
 template <int MB, int EPI, bool NORM, bool STAGE>
 __global__ __launch_bounds__(MB >= 4 ? 512 : 1024) void skinny_block_kernel(SkinnyArgs a) {
+  static_assert(STAGE || !NORM, "the fused norm needs the staged rows");
   extern __shared__ __attribute__((aligned(16))) float smem[];
-  constexpr int U = STAGE ? 4 : (NORM ? (MB >= 2 ? 2 : 4) : (MB >= 4 ? 2 : (MB == 2 ? 4 : 8)));
+  constexpr int R = sk_ring(MB, STAGE);   // K steps whose loads a wave keeps in flight
   const int nsb = a.nsb, kw = a.kw;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nwaves = blockDim.x >> 6;
   const int strip = wave % nsb, ks = wave / nsb;
@@ -80,17 +101,17 @@ __global__ __launch_bounds__(MB >= 4 ? 512 : 1024) void skinny_block_kernel(Skin
   const int cols = 16 * nsb;
   const int n0 = blockIdx.x * cols;
   const int K = a.K, M = a.M;
+  const int steps = (K + 31) >> 5;      // K steps of 32; W is packed and zero-padded to this
 
   float* part = smem;                                   // [kw*nsb][MB][64][4]
-  float* ss_part = part + (size_t)kw * nsb * MB * 256;  // [kw][MB*16]
-  float* inv = ss_part + kw * MB * 16;                  // [MB*16]
+  float* inv = part + (size_t)kw * nsb * MB * 256;      // [MB*16]
   float* s_bias = inv + MB * 16;                        // [cols]
   int* s_pos = (int*)(s_bias + cols);                   // [MB*16]
   int* s_page = s_pos + MB * 16;                        // [MB*16]
   float* s_freq = (float*)(s_page + MB * 16);           // [128]
   float* tile = s_freq + 128;                           // [M][cols]   (SWIGLU, QKV)
-  bf16_t* As = (bf16_t*)(smem + sk_float_words(nsb, kw, MB, M, EPI));   // [MB*16][K + SK_APAD]
-  const int lda = K + SK_APAD;
+  bf16_t* As = (bf16_t*)(smem + sk_float_words(nsb, kw, MB, M, EPI));   // [M][steps*32 + SK_APAD]
+  const int lda = steps * 32 + SK_APAD;
 
   // QKV with qsplit > 1: block = (head, p); its two strips are columns p*16.. and
   // d/2 + p*16.. of the head, i.e. both halves of the rotary pairs
@@ -103,10 +124,11 @@ __global__ __launch_bounds__(MB >= 4 ? 512 : 1024) void skinny_block_kernel(Skin
     if (a.qsplit == 1) return col;
     return col < 16 ? qp * 16 + col : (a.d >> 1) + qp * 16 + (col - 16);
   };
-  const int n = (EPI == SK_QKV) ? qhead * a.d + head_col(strip * 16 + c) : n0 + strip * 16 + c;
-  const bool wok = n < a.N;
-  const bf16_t* wrow = a.W + (size_t)(wok ? n : 0) * K;
-  const int steps = (K + 31) >> 5;
+  // the strip of 16 weight rows this wave multiplies (past the last one: the last
+  // one again, and what comes of it is dropped by the epilogue)
+  int wstrip = (EPI == SK_QKV) ? (qhead * a.d + head_col(strip * 16)) >> 4 : blockIdx.x * nsb + strip;
+  wstrip = min(wstrip, ((a.N + 15) >> 4) - 1);
+  const bf16_t* wp = a.W + (size_t)wstrip * steps * 512 + lane * 8;
   const int per = (steps + kw - 1) / kw;
   const int s_begin = ks * per;
   const int s_end = min(steps, s_begin + per);
@@ -134,23 +156,19 @@ __global__ __launch_bounds__(MB >= 4 ? 512 : 1024) void skinny_block_kernel(Skin
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) acc[mb] = fzero;
 
+  // Loads in the ring are unconditional (a step past the end reads the last tile
+  // again and is multiplied by zeros): a load under a branch makes the compiler wait
+  // for every load in flight at the join, and the stream stalls once per round.
+  auto wload = [&](int st) { return *(const bf16x8*)(wp + (size_t)max(0, min(st, steps - 1)) * 512); };
+  bf16x8 b[R];
+
   if constexpr (STAGE) {
-    // ---- first weight fragments on their way, then stage the rows of x
-    bf16x8 bcur[U], bnext[U];
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int kk = (s_begin + u) * 32 + g * 8;
-      bcur[u] = (wok && (s_begin + u) < s_end && kk < K) ? *(const bf16x8*)(wrow + kk) : zero;
-      bnext[u] = zero;
-    }
-    const int chunks = K >> 3;
-    for (int r = wave; r < MB * 16; r += nwaves) {
+    for (int u = 0; u < R; ++u) b[u] = wload(min(s_begin + u, s_end - 1));
+    // ---- the first weight tiles are on their way; stage the rows of x
+    const int chunks = K >> 3, chunks_pad = steps * 4;
+    for (int r = wave; r < M; r += nwaves) {
       bf16_t* dst = As + (size_t)r * lda;
-      if (r >= M) {
-        for (int ch = lane; ch < chunks; ch += 64) *(bf16x8*)(dst + ch * 8) = zero;
-        if (lane == 0) inv[r] = 0.f;
-        continue;
-      }
       if constexpr (NORM) {
         const float* src = (const float*)a.x + (size_t)(a.x_rows ? a.x_rows[r] : r) * K;
         float ssq = 0.f;
@@ -185,115 +203,78 @@ __global__ __launch_bounds__(MB >= 4 ? 512 : 1024) void skinny_block_kernel(Skin
         const bf16_t* src = (const bf16_t*)a.x + (size_t)r * K;
         for (int ch = lane; ch < chunks; ch += 64) *(bf16x8*)(dst + ch * 8) = *(const bf16x8*)(src + ch * 8);
       }
+      for (int ch = chunks + lane; ch < chunks_pad; ch += 64) *(bf16x8*)(dst + ch * 8) = zero;
     }
     __syncthreads();
-    for (int s0 = s_begin; s0 < s_end; s0 += U) {
-      if (s0 + U < s_end) {
+    // rows past M are not staged: their lanes read the last row, and what they
+    // compute lands in rows of the result that nobody reads
+    const bf16_t* arow[MB];
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-          const int kk = (s0 + U + u) * 32 + g * 8;
-          bnext[u] = (wok && (s0 + U + u) < s_end && kk < K) ? *(const bf16x8*)(wrow + kk) : zero;
-        }
-      }
+    for (int mb = 0; mb < MB; ++mb) arow[mb] = As + (size_t)min(mb * 16 + c, M - 1) * lda + g * 8;
+    int s0 = s_begin;
+    for (; s0 + R < s_end; s0 += R) {       // rounds that refill the ring
 #pragma unroll
-      for (int u = 0; u < U; ++u) {
-        if (s0 + u < s_end) {
-          const int kk = (s0 + u) * 32 + g * 8;
-          const bool kok = kk < K;
-#pragma unroll
-          for (int mb = 0; mb < MB; ++mb) {
-            const bf16x8 av = kok ? *(const bf16x8*)(As + (size_t)(mb * 16 + c) * lda + kk) : zero;
-            acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, bcur[u], acc[mb], 0, 0, 0);
-          }
-        }
-      }
-#pragma unroll
-      for (int u = 0; u < U; ++u) bcur[u] = bnext[u];
-    }
-  } else {
-    // ---- rows of x straight from global memory
-    float ss[MB];
-    const float* xf[MB];
-    const bf16_t* xb[MB];
-    bool aok[MB];
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-      ss[mb] = 0.f;
-      const int m = mb * 16 + c;
-      aok[mb] = m < M;
-      const size_t row = aok[mb] ? (size_t)((NORM && a.x_rows) ? a.x_rows[m] : m) : 0;
-      xf[mb] = (const float*)a.x + row * K;
-      xb[mb] = (const bf16_t*)a.x + row * K;
-    }
-    for (int s0 = s_begin; s0 < s_end; s0 += U) {
-      bf16x8 b[U];
-      floatx4 x0[U][MB], x1[U][MB];
-      bf16x8 ab[U][MB];
-      floatx4 w0[U], w1[U];
-      bf16x8 wb[U];
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const int kk = (s0 + u) * 32 + g * 8;
-        const bool kok = (s0 + u) < s_end && kk < K;
-        b[u] = (wok && kok) ? *(const bf16x8*)(wrow + kk) : zero;
-        if constexpr (NORM) {
-          if (a.norm_w_bf16) {
-            wb[u] = kok ? *(const bf16x8*)((const bf16_t*)a.norm_w + kk) : zero;
-          } else {
-            w0[u] = kok ? *(const floatx4*)((const float*)a.norm_w + kk) : fzero;
-            w1[u] = kok ? *(const floatx4*)((const float*)a.norm_w + kk + 4) : fzero;
-          }
-#pragma unroll
-          for (int mb = 0; mb < MB; ++mb) {
-            const bool ok = aok[mb] && kok;
-            x0[u][mb] = ok ? *(const floatx4*)(xf[mb] + kk) : fzero;
-            x1[u][mb] = ok ? *(const floatx4*)(xf[mb] + kk + 4) : fzero;
-          }
-        } else {
-#pragma unroll
-          for (int mb = 0; mb < MB; ++mb)
-            ab[u][mb] = (aok[mb] && kok) ? *(const bf16x8*)(xb[mb] + kk) : zero;
-        }
-      }
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
+      for (int u = 0; u < R; ++u) {
+        const int st = s0 + u;
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) {
-          bf16x8 av;
-          if constexpr (NORM) {
-            float wv[8];
-            if (a.norm_w_bf16) {
-#pragma unroll
-              for (int j = 0; j < 8; ++j) wv[j] = (float)wb[u][j];
-            } else {
-#pragma unroll
-              for (int j = 0; j < 4; ++j) {
-                wv[j] = w0[u][j];
-                wv[4 + j] = w1[u][j];
-              }
-            }
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              const float p = x0[u][mb][j], q = x1[u][mb][j];
-              ss[mb] += p * p + q * q;
-              av[j] = (bf16_t)(p * wv[j]);
-              av[4 + j] = (bf16_t)(q * wv[4 + j]);
-            }
-          } else {
-            av = ab[u][mb];
-          }
+          const bf16x8 av = *(const bf16x8*)(arow[mb] + st * 32);
           acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, b[u], acc[mb], 0, 0, 0);
         }
+        b[u] = wload(min(st + R, s_end - 1));
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
-    if constexpr (NORM) {
+#pragma unroll
+    for (int u = 0; u < R; ++u) {           // the last round drains it
+      const int st = s0 + u;
+      const bf16x8 bu = st < s_end ? b[u] : zero;
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb) {
-        float v = ss[mb];
-        v += __shfl_xor(v, 16, WAVE);
-        v += __shfl_xor(v, 32, WAVE);
-        if (strip == 0 && g == 0) ss_part[(ks * MB + mb) * 16 + c] = v;
+        const bf16x8 av = *(const bf16x8*)(arow[mb] + min(st, steps - 1) * 32);
+        acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(av, bu, acc[mb], 0, 0, 0);
       }
+    }
+  } else {
+    // ---- rows of x (bfloat16) straight from global memory, in the same ring; a
+    // piece past K or a row past M reads a valid piece instead: it meets zeros of
+    // the padded W, or lands in a row of the result that nobody reads
+    const bf16_t* xb[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) xb[mb] = (const bf16_t*)a.x + (size_t)min(mb * 16 + c, M - 1) * K;
+    auto xload = [&](int st, int mb) {
+      return *(const bf16x8*)(xb[mb] + min(max(0, min(st, steps - 1)) * 32 + g * 8, K - 8));
+    };
+    bf16x8 ab[R][MB];
+#pragma unroll
+    for (int u = 0; u < R; ++u) {     // in the order in which the loop below refills the ring
+      const int st = min(s_begin + u, s_end - 1);
+      b[u] = wload(st);
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb) ab[u][mb] = xload(st, mb);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    int s0 = s_begin;
+    for (; s0 + R < s_end; s0 += R) {       // rounds that refill the ring
+#pragma unroll
+      for (int u = 0; u < R; ++u) {
+        const int st = s0 + u;
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+          acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ab[u][mb], b[u], acc[mb], 0, 0, 0);
+        const int nx = min(st + R, s_end - 1);
+        b[u] = wload(nx);
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) ab[u][mb] = xload(nx, mb);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < R; ++u) {           // the last round drains it
+      const bf16x8 bu = s0 + u < s_end ? b[u] : zero;
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb)
+        acc[mb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ab[u][mb], bu, acc[mb], 0, 0, 0);
     }
   }
 
@@ -302,16 +283,6 @@ __global__ __launch_bounds__(MB >= 4 ? 512 : 1024) void skinny_block_kernel(Skin
   for (int mb = 0; mb < MB; ++mb)
     *(floatx4*)(part + (((size_t)wave * MB + mb) * 64 + lane) * 4) = acc[mb];
   __syncthreads();
-  if constexpr (NORM && !STAGE) {
-    if ((int)threadIdx.x < MB * 16) {
-      const int mb = threadIdx.x >> 4, cc = threadIdx.x & 15;
-      float t = 0.f;
-      for (int k2 = 0; k2 < kw; ++k2) t += ss_part[(k2 * MB + mb) * 16 + cc];
-      inv[threadIdx.x] = rsqrtf(t / (float)K + a.eps);
-    }
-    __syncthreads();
-  }
-
   // ---- reduce over the K slices in a fixed order; epilogue
   for (int idx = threadIdx.x; idx < M * cols; idx += blockDim.x) {
     const int m = idx / cols, col = idx - m * cols;
@@ -386,7 +357,7 @@ __global__ __launch_bounds__(MB >= 4 ? 512 : 1024) void skinny_block_kernel(Skin
 // ---------------------------------------------------------------- dispatch
 static size_t skinny_lds_bytes(int nsb, int kw, int mb, int M, int K, int epi, bool stage) {
   size_t bytes = sk_float_words(nsb, kw, mb, M, epi) * sizeof(float);
-  if (stage) bytes += (size_t)mb * 16 * (K + SK_APAD) * sizeof(bf16_t);
+  if (stage) bytes += (size_t)M * ((K + 31) / 32 * 32 + SK_APAD) * sizeof(bf16_t);
   return bytes;
 }
 
@@ -421,8 +392,12 @@ static int skinny_launch_mb(const SkinnyArgs& a, int mb, int blocks, size_t lds,
 template <int EPI, bool NORM>
 static int skinny_launch_stage(const SkinnyArgs& a, bool stage, int mb, int blocks, size_t lds,
                                hipStream_t stream) {
-  if (stage) return skinny_launch_mb<EPI, NORM, true>(a, mb, blocks, lds, stream);
-  return skinny_launch_mb<EPI, NORM, false>(a, mb, blocks, lds, stream);
+  if constexpr (NORM) {
+    return skinny_launch_mb<EPI, true, true>(a, mb, blocks, lds, stream);   // the norm is staged always
+  } else {
+    if (stage) return skinny_launch_mb<EPI, false, true>(a, mb, blocks, lds, stream);
+    return skinny_launch_mb<EPI, false, false>(a, mb, blocks, lds, stream);
+  }
 }
 
 // A choice of block shape can be forced for measurements (0 = choose).
@@ -461,7 +436,7 @@ static SkinnyShape skinny_choose(int epilogue, bool norm, int mb, int M, int N, 
     const int nsb = cand[ci];
     if (nsb > max_waves) continue;
     for (int kw = 1; kw * nsb <= max_waves && kw <= steps; ++kw) {
-      for (int st = 0; st < 2; ++st) {
+      for (int st = norm ? 1 : 0; st < 2; ++st) {
         const bool stage = st == 1;
         const size_t lds = skinny_lds_bytes(nsb, kw, mb, M, K, epilogue, stage);
         if (lds > SK_LDS_LIMIT) continue;
@@ -482,7 +457,7 @@ static SkinnyShape skinny_choose(int epilogue, bool norm, int mb, int M, int N, 
         const double x_bytes = (double)(stage ? 1 : 2 * nsb) * M * K * (norm ? 4.0 : 2.0);
         const double t_x = per_cu * x_bytes / 50.0e3;
         const int per = (steps + kw - 1) / kw;
-        const int u = stage ? 4 : (norm ? (mb >= 2 ? 2 : 4) : (mb >= 4 ? 2 : (mb == 2 ? 4 : 8)));
+        const int u = sk_ring(mb, stage);
         const double trips = stage ? 1.0 + 0.3 * ((per + u - 1) / u - 1) : (double)((per + u - 1) / u);
         const double busy = t_stream + t_x > 0.8 * trips ? t_stream + t_x : 0.8 * trips;
         // a fixed part per kernel, and again (in part hidden by the neighbours) for every
@@ -541,8 +516,10 @@ extern "C" int llmlab_skinny_linear(const void* x, int norm, const int* x_rows, 
     shape.qsplit = g_force_nsb == 2 ? d / 32 : 1;
   }
   if (g_force_kw > 0) shape.kw = g_force_kw;
-  if (g_force_stage >= 0) shape.stage = g_force_stage != 0;
-  LLMLAB_REQUIRE(shape.nsb > 0 && shape.kw > 0, "skinny_linear: no block shape fits N=%d K=%d M=%d", N, K, M);
+  if (g_force_stage >= 0) shape.stage = norm || g_force_stage != 0;
+  LLMLAB_REQUIRE(shape.nsb > 0 && shape.kw > 0,
+                 "skinny_linear: no block shape fits N=%d K=%d M=%d (rows of x to stage: %zu bytes of LDS)",
+                 N, K, M, (size_t)M * ((K + 31) / 32 * 32 + SK_APAD) * sizeof(bf16_t));
   const size_t lds = skinny_lds_bytes(shape.nsb, shape.kw, mb, M, K, epilogue, shape.stage);
   LLMLAB_REQUIRE(lds <= SK_LDS_LIMIT && shape.nsb * shape.kw <= (mb >= 4 ? 8 : 16),
                  "skinny_linear: block shape %dx%d does not fit", shape.nsb, shape.kw);

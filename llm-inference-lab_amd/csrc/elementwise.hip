@@ -4,7 +4,7 @@
 
 extern "C" const char* llmlab_last_error() { return g_llmlab_error; }
 
-extern "C" int llmlab_abi_version() { return 1; }
+extern "C" int llmlab_abi_version() { return 2; }
 
 // --------------------------------------------------------------- embedding
 // out[r, :] = float(table[ids[r], :]); an id outside [0, vocab) is clamped (the
@@ -21,13 +21,36 @@ __global__ void embed_kernel(const T* __restrict__ table, const int* __restrict_
   for (int c = threadIdx.x; c < hidden; c += blockDim.x) dst[c] = to_float(src[c]);
 }
 
-extern "C" int llmlab_embed(const void* table, int dtype, const int* ids, float* out, int rows,
+// The same from a bfloat16 table packed in MFMA fragment order (see
+// llmlab_pack_weight): row `id` is lane column id % 16 of strip id / 16, its
+// columns 8 ch .. 8 ch + 7 the 16 bytes of lane (ch % 4) * 16 + id % 16 in tile ch / 4.
+__global__ void embed_packed_kernel(const bf16_t* __restrict__ table, const int* __restrict__ ids,
+                                    float* __restrict__ out, int hidden, int vocab) {
+  const int r = blockIdx.x;
+  int id = ids[r];
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+  const int tiles = (hidden + 31) >> 5;
+  const bf16_t* strip = table + (size_t)(id >> 4) * tiles * 512;
+  float* dst = out + (size_t)r * hidden;
+  for (int ch = threadIdx.x; ch < (hidden >> 3); ch += blockDim.x) {
+    const bf16x8 v = *(const bf16x8*)(strip + (size_t)(ch >> 2) * 512 + (((ch & 3) << 4) + (id & 15)) * 8);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) dst[ch * 8 + j] = (float)v[j];
+  }
+}
+
+// dtype DT_BF16 + packed != 0: the table is in fragment order (hidden a multiple of 8).
+extern "C" int llmlab_embed(const void* table, int dtype, int packed, const int* ids, float* out, int rows,
                             int hidden, int vocab, hipStream_t stream) {
   LLMLAB_REQUIRE(rows >= 0 && hidden > 0 && vocab > 0, "embed: bad sizes rows=%d hidden=%d vocab=%d",
                  rows, hidden, vocab);
+  LLMLAB_REQUIRE(!packed || (dtype == DT_BF16 && hidden % 8 == 0), "embed: a packed table is bfloat16, %d wide", hidden);
   if (rows == 0) return 0;
   dim3 grid(rows), block(256);
-  if (dtype == DT_BF16)
+  if (packed)
+    hipLaunchKernelGGL(embed_packed_kernel, grid, dim3(128), 0, stream, (const bf16_t*)table, ids, out,
+                       hidden, vocab);
+  else if (dtype == DT_BF16)
     hipLaunchKernelGGL(embed_kernel<bf16_t>, grid, block, 0, stream, (const bf16_t*)table, ids, out,
                        hidden, vocab);
   else
@@ -207,5 +230,40 @@ extern "C" int llmlab_gather_tokens(int* dst, const int* dst_index, const int* s
   hipLaunchKernelGGL(gather_tokens_kernel, dim3((n + 63) / 64), dim3(64), 0, stream, dst, dst_index, src,
                      src_index, n);
   LLMLAB_LAUNCH_CHECK("gather_tokens");
+  return 0;
+}
+
+// ------------------------------------------------------------ weight packing
+// A bfloat16 matrix W [N, K] in MFMA fragment order: strips of 16 rows, each strip
+// a run of K/32 tiles (K padded to a multiple of 32, N to a multiple of 16, with
+// zeros); a tile is the B operand of one v_mfma_f32_16x16x32_bf16, 1 KB, lane l
+// (row l % 16 of the strip, columns 8 * (l / 16) .. + 7 of the tile) owning bytes
+// 16 l .. 16 l + 15.  Every product kernel reads W in this order, one or two
+// contiguous KB per wave instruction, instead of 16 rows of 64 bytes each.
+__global__ __launch_bounds__(256) void pack_weight_kernel(const bf16_t* __restrict__ src,
+                                                           bf16_t* __restrict__ dst, int N, int K,
+                                                           int tiles_per_strip, long chunks) {
+  const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= chunks) return;
+  const long tile = idx >> 6;
+  const int l = (int)(idx & 63), c = l & 15, g = l >> 4;
+  const int n = (int)(tile / tiles_per_strip) * 16 + c;
+  const int k = (int)(tile % tiles_per_strip) * 32 + g * 8;
+  const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+  *(bf16x8*)(dst + idx * 8) = (n < N && k < K) ? *(const bf16x8*)(src + (size_t)n * K + k) : zero;
+}
+
+extern "C" long llmlab_packed_elements(int N, int K) {
+  return (long)((N + 15) / 16) * ((K + 31) / 32) * 512;
+}
+
+extern "C" int llmlab_pack_weight(const void* src, void* dst, int N, int K, hipStream_t stream) {
+  LLMLAB_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "pack_weight: bad sizes N=%d K=%d (K must be a multiple of 8)", N, K);
+  LLMLAB_REQUIRE(((uintptr_t)src % 16 == 0) && ((uintptr_t)dst % 16 == 0), "pack_weight: operands must be 16-byte aligned");
+  const int tiles = (K + 31) / 32;
+  const long chunks = (long)((N + 15) / 16) * tiles * 64;
+  hipLaunchKernelGGL(pack_weight_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, stream,
+                     (const bf16_t*)src, (bf16_t*)dst, N, K, tiles, chunks);
+  LLMLAB_LAUNCH_CHECK("pack_weight");
   return 0;
 }

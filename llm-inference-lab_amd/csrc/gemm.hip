@@ -1,4 +1,5 @@
-// Matrix products  out = x . W^T  (x [M, K] and W [N, K], both K-contiguous)
+// Matrix products  out = x . W^T  (x [M, K] K-contiguous; W [N, K], in bfloat16
+// packed in MFMA fragment order by llmlab_pack_weight, in float32 K-contiguous)
 // for gfx950, with the epilogues the model needs fused in.
 //
 //   bfloat16:  v_mfma_f32_16x16x32_bf16 everywhere.
@@ -78,18 +79,25 @@ __global__ __launch_bounds__(256) void gemm_bf16_tiled(const bf16_t* __restrict_
   bf16x8 ra[PD][A_CHUNKS], rb[PD][B_CHUNKS];
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
+  // Loads are unconditional (a load under a branch makes the compiler wait for every
+  // load in flight where the branch ends).  Rows of x past M and pieces past K read
+  // a valid piece instead: they meet zeros of the padded W or land in rows nobody
+  // stores.  W is packed in fragment order: the 64 columns of a strip of 16 rows
+  // are 2 KB of consecutive memory, thread p of a strip's 128 reading bytes 16 p...
+  const int T = (K + 31) >> 5, nstrips = (N + 15) >> 4;
   auto fetch = [&](int slot, int k0) {
 #pragma unroll
     for (int i = 0; i < A_CHUNKS; ++i) {
       const int ch = tid + i * 256, row = ch >> 3, kc = (ch & 7) * 8;
-      const int m = m0 + row, k = k0 + kc;
-      ra[slot][i] = (m < M && k < K) ? *(const bf16x8*)(A + (size_t)m * K + k) : zero;
+      const int m = min(m0 + row, M - 1), k = min(k0 + kc, K - 8);
+      ra[slot][i] = *(const bf16x8*)(A + (size_t)m * K + k);
     }
 #pragma unroll
     for (int i = 0; i < B_CHUNKS; ++i) {
-      const int ch = tid + i * 256, row = ch >> 3, kc = (ch & 7) * 8;
-      const int n = n0 + row, k = k0 + kc;
-      rb[slot][i] = (n < N && k < K) ? *(const bf16x8*)(W + (size_t)n * K + k) : zero;
+      const int ch = tid + i * 256, sl = ch >> 7, step = (k0 >> 5) + ((ch >> 6) & 1);
+      const int strip = min((n0 >> 4) + sl, nstrips - 1);
+      const bf16x8 v = *(const bf16x8*)(W + ((size_t)strip * T + min(step, T - 1)) * 512 + (ch & 63) * 8);
+      rb[slot][i] = step < T ? v : zero;
     }
   };
   auto stash = [&](int slot) {
@@ -100,21 +108,25 @@ __global__ __launch_bounds__(256) void gemm_bf16_tiled(const bf16_t* __restrict_
     }
 #pragma unroll
     for (int i = 0; i < B_CHUNKS; ++i) {
-      const int ch = tid + i * 256, row = ch >> 3, kc = (ch & 7) * 8;
+      const int ch = tid + i * 256, l = ch & 63;
+      const int row = (ch >> 7) * 16 + (l & 15), kc = ((ch >> 6) & 1) * 32 + (l >> 4) * 8;
       *(bf16x8*)(Bs + row * LDS_STRIDE + kc) = rb[slot][i];
     }
   };
 
   const int nk = (K + BK - 1) / BK;
 #pragma unroll
-  for (int p = 0; p < PD; ++p) fetch(p, p * BK);      // past K: no load, zeros
+  for (int p = 0; p < PD; ++p) fetch(p, p * BK);      // past K: zeros for W
   for (int kt = 0; kt < nk; kt += PD) {
 #pragma unroll
     for (int p = 0; p < PD; ++p) {
-      if (kt + p < nk) {
+      const bool live = kt + p < nk;
+      if (live) {
         stash(p);
         __syncthreads();
-        fetch(p, (kt + p + PD) * BK);
+      }
+      fetch(p, (kt + p + PD) * BK);
+      if (live) {
 #pragma unroll
         for (int ks = 0; ks < 2; ++ks) {
           bf16x8 a[TM], b[TN];
@@ -239,7 +251,7 @@ static int launch_bf16(const bf16_t* A, const bf16_t* W, EpiArgs e, int M, int N
   return 0;
 }
 
-// x [M,K] (dtype), w [N,K] (dtype); epilogue selects what `out` is.  For SWIGLU N
+// x [M,K] (dtype), w [N,K] (float32: row-major; bfloat16: packed); epilogue selects what `out` is.  For SWIGLU N
 // is the number of interleaved weight rows (2 * ceil16(n_out)).
 extern "C" int llmlab_linear(const void* x, const void* w, int dtype, int epilogue, void* out,
                              const void* bias, int bias_dtype, int M, int N, int K, int ldo, int n_out,

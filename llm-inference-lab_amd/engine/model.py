@@ -74,6 +74,7 @@ class CausalLM:
             b.bind(tensors, ops, dtype)
         self.final_norm.bind(tensors, ops, dtype)
         self.head.bind(tensors, ops, dtype)
+        ops.release_shared()
 
     def weight_bytes_per_step(self) -> int:
         """Bytes of weights that one step reads once (every run of a block reads

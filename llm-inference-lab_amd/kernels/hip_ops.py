@@ -36,6 +36,33 @@ class KernelError(RuntimeError):
     pass
 
 
+class PackedWeight:
+    """A bfloat16 matrix [n, k] in the order the matrix cores read it: strips of 16
+    rows, a strip a run of 1 KB tiles (16 rows x 32 columns, one MFMA B operand,
+    lane l owning 16 bytes), zero-padded to whole tiles.  Made by
+    ``HipOps.prepare_weight``; the product kernels take nothing else in bfloat16."""
+
+    __slots__ = ("data", "shape", "dtype", "device")
+
+    def __init__(self, data: torch.Tensor, n: int, k: int):
+        self.data = data
+        self.shape = (n, k)
+        self.dtype = data.dtype
+        self.device = data.device
+
+    def data_ptr(self) -> int:
+        return self.data.data_ptr()
+
+    def is_contiguous(self) -> bool:
+        return True
+
+    def numel(self) -> int:
+        return self.shape[0] * self.shape[1]
+
+    def element_size(self) -> int:
+        return self.data.element_size()
+
+
 class HipOps:
     WORKSPACE_FLOATS = 16 * 1024 * 1024      # 64 MiB of float32 scratch (split partial sums)
 
@@ -50,9 +77,10 @@ class HipOps:
         torch.cuda.set_device(self.device)
         self._core = self._load(build.core_library())
         self._declare_core()
-        if self._core.llmlab_abi_version() != 1:
+        if self._core.llmlab_abi_version() != 2:
             raise RuntimeError("kernel library and Python bindings disagree on the interface")
         self._attn: Dict[int, ctypes.CDLL] = {}
+        self._shared: Dict[int, tuple] = {}
         self.num_cus = int(torch.cuda.get_device_properties(self.device).multi_processor_count)
         self.workspace = torch.empty(self.WORKSPACE_FLOATS, dtype=torch.float32, device=self.device)
         self.loaded_libraries = [self._core._name]
@@ -69,7 +97,7 @@ class HipOps:
         c = self._core
         c.llmlab_last_error.restype = ctypes.c_char_p
         c.llmlab_abi_version.restype = _c_int
-        c.llmlab_embed.argtypes = [_c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr]
+        c.llmlab_embed.argtypes = [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr]
         c.llmlab_rmsnorm.argtypes = [_c_ptr, _c_ptr, _c_int, _c_float, _c_ptr, _c_int, _c_ptr, _c_int,
                                      _c_int, _c_ptr]
         c.llmlab_rope_kv_write.argtypes = [_c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
@@ -82,6 +110,10 @@ class HipOps:
         c.llmlab_sample.argtypes = [_c_ptr, _c_long, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr]
         c.llmlab_gather_tokens.argtypes = [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr]
         c.llmlab_gather_tokens.restype = _c_int
+        c.llmlab_packed_elements.argtypes = [_c_int, _c_int]
+        c.llmlab_packed_elements.restype = _c_long
+        c.llmlab_pack_weight.argtypes = [_c_ptr, _c_ptr, _c_int, _c_int, _c_ptr]
+        c.llmlab_pack_weight.restype = _c_int
         c.llmlab_argmax.argtypes = [_c_ptr, _c_long, _c_int, _c_int, _c_ptr, _c_ptr, _c_size, _c_ptr]
         c.llmlab_argmax.restype = _c_int
         c.llmlab_skinny_linear.argtypes = [
@@ -126,6 +158,49 @@ class HipOps:
                 f"{what}: bfloat16 matrix products need an inner size that is a multiple of 8, "
                 f"got {inner} (the float32 path takes any size)")
 
+    def prepare_weight(self, w: torch.Tensor, shared: bool = False):
+        """What the product kernels take for the matrix ``w`` [n, k]: float32 as it is,
+        bfloat16 packed in fragment order (a copy; ``w`` itself is not kept).
+
+        ``shared``: parts that may be bound to one and the same tensor (an embedding
+        and an output head with tied weights) get one packed copy between them;
+        the model calls ``release_shared()`` when all its parts are bound."""
+        if shared and id(w) in self._shared:
+            return self._shared[id(w)][1]
+        packed = self._prepare(w)
+        if shared:
+            self._shared[id(w)] = (w, packed)       # w is held so that its id stays its own
+        return packed
+
+    def release_shared(self) -> None:
+        self._shared.clear()
+
+    def _prepare(self, w: torch.Tensor):
+        self._need(w, "weight")
+        if w.dim() != 2:
+            raise ValueError(f"a weight matrix has two dimensions, got {tuple(w.shape)}")
+        if w.dtype == torch.float32:
+            return w
+        if w.dtype != torch.bfloat16:
+            raise TypeError(f"weights are float32 or bfloat16, got {w.dtype}")
+        n, k = w.shape
+        self.check_product_sizes(k, w.dtype, "weight matrix")
+        data = torch.empty(self._core.llmlab_packed_elements(n, k), dtype=torch.bfloat16, device=self.device)
+        self._check(self._core.llmlab_pack_weight(self._ptr(w), self._ptr(data), n, k, self._stream()))
+        return PackedWeight(data, n, k)
+
+    def _weight(self, w, name: str):
+        """The weight operand of a product: packed if bfloat16."""
+        if isinstance(w, PackedWeight):
+            if w.device != self.device:
+                raise ValueError(f"{name} is on {w.device}, the kernels run on {self.device}")
+            return w
+        self._need(w, name)
+        if w.dtype == torch.bfloat16:
+            raise TypeError(f"{name}: bfloat16 weights go through prepare_weight() once, when the "
+                            f"part is bound; the product kernels read the packed order only")
+        return w
+
     # ---------------------------------------------------------------- helpers
     def _stream(self):
         return _c_ptr(torch.cuda.current_stream(self.device).cuda_stream)
@@ -153,15 +228,19 @@ class HipOps:
 
     # ------------------------------------------------------------ elementwise
     def embed(self, table, ids, out) -> None:
-        self._need(table, "embedding table")
+        """Rows of ``table`` (float32, bfloat16, or bfloat16 packed by prepare_weight)."""
+        packed = isinstance(table, PackedWeight)
+        if not packed:
+            self._need(table, "embedding table")
         self._need(ids, "token ids", torch.int32)
         self._need(out, "embedding output", torch.float32)
         rows, hidden = out.shape
         if ids.numel() != rows or table.shape[1] != hidden:
             raise ValueError(f"embed: ids {tuple(ids.shape)}, table {tuple(table.shape)}, "
                              f"out {tuple(out.shape)} do not fit")
-        self._check(self._core.llmlab_embed(self._ptr(table), _dt(table), self._ptr(ids), self._ptr(out),
-                                            rows, hidden, table.shape[0], self._stream()))
+        self._check(self._core.llmlab_embed(self._ptr(table), _dt(table), 1 if packed else 0,
+                                            self._ptr(ids), self._ptr(out), rows, hidden, table.shape[0],
+                                            self._stream()))
 
     def gather_tokens(self, dst, dst_index, src, src_index, n) -> None:
         """dst[dst_index[i]] = src[src_index[i]] for i < n (all int32 on the GPU)."""
@@ -195,7 +274,7 @@ class HipOps:
     # ----------------------------------------------------------------- linear
     def _linear(self, x, w, out, bias, epilogue, n_out) -> None:
         self._need(x, "linear input")
-        self._need(w, "linear weight")
+        w = self._weight(w, "linear weight")
         if x.dtype != w.dtype:
             raise TypeError(f"linear: input is {x.dtype} but the weight is {w.dtype}")
         if out.device != self.device or out.stride(-1) != 1:
@@ -247,9 +326,14 @@ class HipOps:
     fuse_max_rows = 16            # steps up to here take the fused kernels: their rows fit
                                   # the staging buffer; beyond, norm + tiled product is faster
 
-    def can_fuse(self, rows: int, dtype) -> bool:
-        """Whether the fused few-row kernels take this step (bfloat16, few rows)."""
-        return dtype == torch.bfloat16 and 0 < rows <= self.fuse_max_rows
+    STAGE_BYTES = 118 * 1024      # most LDS the staged rows of a fused kernel may take
+
+    def can_fuse(self, rows: int, dtype, inner: int) -> bool:
+        """Whether the fused few-row kernels take this step: bfloat16, few rows, and
+        the rows (``inner`` wide) fit the staging buffer in LDS."""
+        if dtype != torch.bfloat16 or not 0 < rows <= self.fuse_max_rows:
+            return False
+        return rows * ((inner + 31) // 32 * 32 + 8) * 2 <= self.STAGE_BYTES
 
     def _skinny(self, x, norm, x_rows, norm_w, eps, w, bias, epilogue, out, m, n, k, ldo, n_out,
                 qkv=None) -> None:
@@ -267,7 +351,9 @@ class HipOps:
     def _fused_common(self, x, norm_w, w, rows):
         self._need(x, "residual stream", torch.float32)
         self._need(norm_w, "norm weight")
-        self._need(w, "weight", torch.bfloat16)
+        w = self._weight(w, "weight")
+        if w.dtype != torch.bfloat16:
+            raise TypeError("the fused few-row kernels are bfloat16 kernels")
         k = x.shape[1]
         if norm_w.numel() != k or w.shape[1] != k:
             raise ValueError(f"fused norm + product: x {tuple(x.shape)}, norm weight "
@@ -277,14 +363,14 @@ class HipOps:
                 f"bfloat16 matrix products need an inner size that is a multiple of 8, got {k}")
         if not 0 < rows <= self.FUSED_MAX_ROWS:
             raise ValueError(f"the fused kernels take 1..{self.FUSED_MAX_ROWS} rows, got {rows}")
-        return k
+        return w, k
 
     def fused_norm_qkv(self, x, norm_w, eps, w_qkv, b_qkv, num_heads, num_kv_heads, head_dim, inv_freq,
                        positions, row_req, block_table, page_size, k_cache, v_cache, q_out) -> None:
         """q_out = rotate(norm(x) Wq^T + bq); rotated k and v of the new positions go to
         their pages (skipped when no cache is given)."""
         rows = x.shape[0]
-        k = self._fused_common(x, norm_w, w_qkv, rows)
+        w_qkv, k = self._fused_common(x, norm_w, w_qkv, rows)
         n = (num_heads + 2 * num_kv_heads) * head_dim
         if w_qkv.shape[0] != n or tuple(q_out.shape) != (rows, num_heads * head_dim):
             raise ValueError("fused_norm_qkv: weight or output shape does not fit the heads")
@@ -314,7 +400,7 @@ class HipOps:
 
     def fused_norm_swiglu(self, x, norm_w, eps, w_gate_up, out) -> None:
         rows, inter = out.shape
-        k = self._fused_common(x, norm_w, w_gate_up, rows)
+        w_gate_up, k = self._fused_common(x, norm_w, w_gate_up, rows)
         self._need(out, "SwiGLU output", torch.bfloat16)
         if x.shape[0] != rows or w_gate_up.shape[0] != 2 * ((inter + 15) // 16 * 16):
             raise ValueError("fused_norm_swiglu: shapes do not fit")
@@ -324,7 +410,7 @@ class HipOps:
     def fused_norm_logits(self, x, rows_index, norm_w, eps, w, out) -> None:
         """out[i] = norm(x[rows_index[i]]) W^T in float32."""
         rows, vocab = out.shape
-        k = self._fused_common(x, norm_w, w, rows)
+        w, k = self._fused_common(x, norm_w, w, rows)
         self._need(out, "logits", torch.float32)
         if w.shape[0] != vocab:
             raise ValueError("fused_norm_logits: weight rows differ from the vocabulary")

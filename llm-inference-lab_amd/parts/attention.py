@@ -83,13 +83,13 @@ class GQAAttention(Mixer):
         ops.check_product_sizes(self.q_size, dtype, "attention output projection (heads * head size)")
         t = self.tensor_names
         # One projection instead of three: the rows of Wq, Wk, Wv stacked.
-        self.w_qkv = torch.cat([tensors[t["q_weight"]], tensors[t["k_weight"]],
-                                tensors[t["v_weight"]]], dim=0).contiguous()
+        self.w_qkv = ops.prepare_weight(torch.cat([tensors[t["q_weight"]], tensors[t["k_weight"]],
+                                                   tensors[t["v_weight"]]], dim=0).contiguous())
         if self.qkv_bias:
             parts = [tensors[t["q_bias"]], tensors[t["k_bias"]], tensors[t["v_bias"]]]
             kept = parts[0].dtype if all(p.dtype == parts[0].dtype for p in parts) else torch.float32
             self.b_qkv = torch.cat([p.to(kept) for p in parts]).contiguous()
-        self.w_o = tensors[t["o_weight"]].contiguous()
+        self.w_o = ops.prepare_weight(tensors[t["o_weight"]].contiguous())
         self.b_o = tensors[t["o_bias"]].contiguous() if self.out_bias else None
         if self.position is not None:
             self.position.bind(tensors, ops, dtype)
@@ -105,7 +105,7 @@ class GQAAttention(Mixer):
         k_cache = entry.k_cache if entry.writes_cache else None
         v_cache = entry.v_cache if entry.writes_cache else None
         rms = h.rms() if isinstance(h, NormedInput) else None
-        if (rms is not None and ops.can_fuse(rows, self.dtype)
+        if (rms is not None and ops.can_fuse(rows, self.dtype, self.hidden_size)
                 and (self.position is None or table is not None)):
             # few rows: norm, the three projections, bias, rotation and the cache
             # write are one kernel

@@ -69,7 +69,9 @@ class TokenEmbedding(Part):
 
     def bind(self, tensors, ops, dtype):
         super().bind(tensors, ops, dtype)
-        self.table = tensors[self.tensor_names["weight"]]
+        ops.check_product_sizes(self.hidden_size, dtype, "embedding (hidden size)")
+        # in the order the product kernels read, so that a tied output head shares it
+        self.table = ops.prepare_weight(tensors[self.tensor_names["weight"]], shared=True)
 
     def forward(self, ids, out):
         self.ops.embed(self.table, ids, out)
@@ -94,13 +96,13 @@ class LinearHead(Part):
     def bind(self, tensors, ops, dtype):
         super().bind(tensors, ops, dtype)
         ops.check_product_sizes(self.hidden_size, dtype, "output head (hidden size)")
-        self.weight = tensors[self.tensor_names["weight"]]
+        self.weight = ops.prepare_weight(tensors[self.tensor_names["weight"]], shared=True)
 
     takes_normed_input = True
 
     def forward(self, h, out):
         rms = h.rms() if isinstance(h, NormedInput) else None
-        if rms is not None and self.ops.can_fuse(out.shape[0], self.dtype):
+        if rms is not None and self.ops.can_fuse(out.shape[0], self.dtype, self.hidden_size):
             self.ops.fused_norm_logits(rms[0], rms[1], rms[2], rms[3], self.weight, out)
         else:
             if isinstance(h, NormedInput):

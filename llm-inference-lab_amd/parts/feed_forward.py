@@ -60,8 +60,9 @@ class SwiGLU(FeedForward):
         ops.check_product_sizes(self.hidden_size, dtype, "feed-forward (hidden size)")
         ops.check_product_sizes(self.intermediate_size, dtype, "feed-forward (intermediate size)")
         t = self.tensor_names
-        self.w_gate_up = interleave_gate_up(tensors[t["gate_weight"]], tensors[t["up_weight"]])
-        self.w_down = tensors[t["down_weight"]].contiguous()
+        self.w_gate_up = ops.prepare_weight(
+            interleave_gate_up(tensors[t["gate_weight"]], tensors[t["up_weight"]]))
+        self.w_down = ops.prepare_weight(tensors[t["down_weight"]].contiguous())
 
     takes_normed_input = True
 
@@ -69,7 +70,7 @@ class SwiGLU(FeedForward):
         rows = h.shape[0]
         act = ctx.scratch("swiglu.act", (rows, self.intermediate_size), self.dtype)
         rms = h.rms() if isinstance(h, NormedInput) else None
-        if rms is not None and self.ops.can_fuse(rows, self.dtype):
+        if rms is not None and self.ops.can_fuse(rows, self.dtype, self.hidden_size):
             self.ops.fused_norm_swiglu(rms[0], rms[2], rms[3], self.w_gate_up, act)
         else:
             if isinstance(h, NormedInput):

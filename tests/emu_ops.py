@@ -82,8 +82,14 @@ class EmuOps:
     FUSED_MAX_ROWS = 64
     fuse_max_rows = 16
 
-    def can_fuse(self, rows, dtype):
+    def can_fuse(self, rows, dtype, inner):
         return self.fuse and dtype == torch.bfloat16 and 0 < rows <= self.fuse_max_rows
+
+    def prepare_weight(self, w, shared=False):
+        return w
+
+    def release_shared(self):
+        pass
 
     def _normed(self, x, rows_index, norm_w, eps, n):
         v = x.float() if rows_index is None else x.float()[rows_index[:n].long()]

@@ -39,7 +39,7 @@ def close(got, want, dtype, what, scale=1.0):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("rows,hidden,vocab", [(1, 64, 256), (37, 896, 1000), (5, 100, 33)])
+@pytest.mark.parametrize("rows,hidden,vocab", [(1, 64, 256), (37, 896, 1000), (5, 100, 33), (9, 104, 77)])
 def test_embed(ops, emu, dtype, rows, hidden, vocab):
     table = rnd((vocab, hidden), dtype, 1)
     ids = torch.randint(0, vocab, (rows,), generator=torch.Generator().manual_seed(2)).int()
@@ -49,6 +49,10 @@ def test_embed(ops, emu, dtype, rows, hidden, vocab):
     got = torch.empty(rows, hidden, device=DEV)
     ops.embed(table.to(DEV), ids.to(DEV), got)
     assert torch.equal(got.cpu(), want)
+    if dtype == torch.bfloat16 and hidden % 8 == 0:       # the same rows out of the packed order
+        got.zero_()
+        ops.embed(ops.prepare_weight(table.to(DEV)), ids.to(DEV), got)
+        assert torch.equal(got.cpu(), want)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -88,7 +92,7 @@ def test_linear_bias(ops, emu, dtype, m, n, k):
         want = torch.empty(m, n, dtype=dtype)
         emu.linear(x, w, want, bias)
         got = torch.empty(m, n, dtype=dtype, device=DEV)
-        ops.linear(x.to(DEV), w.to(DEV), got, None if bias is None else bias.to(DEV))
+        ops.linear(x.to(DEV), ops.prepare_weight(w.to(DEV)), got, None if bias is None else bias.to(DEV))
         close(got, want, dtype, f"linear {m}x{n}x{k}", want.float().abs().max().item())
 
 
@@ -100,12 +104,12 @@ def test_linear_residual_and_logits(ops, emu, dtype, m, n, k):
     want = resid.clone()
     emu.linear_residual(x, w, want)
     got = resid.clone().to(DEV)
-    ops.linear_residual(x.to(DEV), w.to(DEV), got)
+    ops.linear_residual(x.to(DEV), ops.prepare_weight(w.to(DEV)), got)
     close(got, want, torch.float32, f"linear_residual {m}x{n}x{k}", want.abs().max().item())
     want = torch.empty(m, n)
     emu.linear_logits(x, w, want)
     got = torch.empty(m, n, device=DEV)
-    ops.linear_logits(x.to(DEV), w.to(DEV), got)
+    ops.linear_logits(x.to(DEV), ops.prepare_weight(w.to(DEV)), got)
     close(got, want, torch.float32, f"linear_logits {m}x{n}x{k}", want.abs().max().item())
 
 
@@ -121,11 +125,11 @@ def test_linear_reference_vectors(ops):
         b = (torch.arange(n).float() + 7) / 128
         want = x.double() @ w.double().t() + b.double()
         got = torch.empty(m, n, device=DEV)
-        ops.linear(x.to(DEV), w.to(DEV), got, b.to(DEV))
+        ops.linear(x.to(DEV), ops.prepare_weight(w.to(DEV)), got, b.to(DEV))
         assert (got.cpu().double() - want).abs().max().item() < 1e-4
         # all these values are exact in bfloat16, so that path must agree after one rounding
         gotb = torch.empty(m, n, dtype=torch.bfloat16, device=DEV)
-        ops.linear(x.bfloat16().to(DEV), w.bfloat16().to(DEV), gotb, b.to(DEV))
+        ops.linear(x.bfloat16().to(DEV), ops.prepare_weight(w.bfloat16().to(DEV)), gotb, b.to(DEV))
         assert torch.equal(gotb.cpu(), want.float().bfloat16())
 
 
@@ -144,7 +148,7 @@ def test_linear_swiglu(ops, emu, dtype, m, inter, k):
     direct = g / (1 + torch.exp(-g)) * (x.float() @ up.float().t())
     assert (want.float() - direct).abs().max() < 1e-2 * max(1.0, direct.abs().max().item())
     got = torch.empty(m, inter, dtype=dtype, device=DEV)
-    ops.linear_swiglu(x.to(DEV), w.to(DEV), got)
+    ops.linear_swiglu(x.to(DEV), ops.prepare_weight(w.to(DEV)), got)
     close(got, want, dtype, f"linear_swiglu {m}x{inter}x{k}", want.float().abs().max().item())
 
 
@@ -161,13 +165,13 @@ def test_few_row_products(ops, emu, m, n, k):
     want = torch.empty(m, n, dtype=dtype)
     emu.linear(x, w, want, bias)
     got = torch.empty(m, n, dtype=dtype, device=DEV)
-    ops.linear(x.to(DEV), w.to(DEV), got, bias.to(DEV))
+    ops.linear(x.to(DEV), ops.prepare_weight(w.to(DEV)), got, bias.to(DEV))
     close(got, want, dtype, "few-row linear", want.float().abs().max().item())
     resid = rnd((m, n), torch.float32, 43)
     want = resid.clone()
     emu.linear_residual(x, w, want)
     got = resid.clone().to(DEV)
-    ops.linear_residual(x.to(DEV), w.to(DEV), got)
+    ops.linear_residual(x.to(DEV), ops.prepare_weight(w.to(DEV)), got)
     close(got, want, torch.float32, "few-row residual", want.abs().max().item() * 4)
 
 
@@ -185,7 +189,7 @@ def test_fused_norm_products(ops, emu, wdtype, m, hidden, inter, vocab):
     want = torch.empty(m, inter, dtype=bf)
     emu.fused_norm_swiglu(x[:m], nw, eps, w, want)
     got = torch.empty(m, inter, dtype=bf, device=DEV)
-    ops.fused_norm_swiglu(x[:m].contiguous().to(DEV), nw.to(DEV), eps, w.to(DEV), got)
+    ops.fused_norm_swiglu(x[:m].contiguous().to(DEV), nw.to(DEV), eps, ops.prepare_weight(w.to(DEV)), got)
     close(got, want, bf, "fused norm + swiglu", want.float().abs().max().item())
     # logits of gathered rows
     head = rnd((vocab, hidden), bf, 54, 0.1)
@@ -193,7 +197,7 @@ def test_fused_norm_products(ops, emu, wdtype, m, hidden, inter, vocab):
     want = torch.empty(m, vocab)
     emu.fused_norm_logits(x, idx, nw, eps, head, want)
     got = torch.empty(m, vocab, device=DEV)
-    ops.fused_norm_logits(x.to(DEV), idx.to(DEV), nw.to(DEV), eps, head.to(DEV), got)
+    ops.fused_norm_logits(x.to(DEV), idx.to(DEV), nw.to(DEV), eps, ops.prepare_weight(head.to(DEV)), got)
     close(got, want, torch.float32, "fused norm + logits", want.abs().max().item() * 40)
 
 
@@ -223,7 +227,7 @@ def test_fused_norm_qkv_rope_write(ops, emu, nq, nkv, d, page, hidden, rotate):
     emu.fused_norm_qkv(x, nw, 1e-6, w, b, nq, nkv, d, inv_freq, positions, row_req, table, page,
                        want_k, want_v, want_q)
     got_q, got_k, got_v = torch.empty(rows, nq * d, dtype=bf, device=DEV), kc.to(DEV), vc.to(DEV)
-    ops.fused_norm_qkv(x.to(DEV), nw.to(DEV), 1e-6, w.to(DEV), b.to(DEV), nq, nkv, d,
+    ops.fused_norm_qkv(x.to(DEV), nw.to(DEV), 1e-6, ops.prepare_weight(w.to(DEV)), b.to(DEV), nq, nkv, d,
                        None if inv_freq is None else inv_freq.to(DEV), positions.to(DEV), row_req.to(DEV),
                        table.to(DEV), page, got_k, got_v, got_q)
     scale = want_q.float().abs().max().item()
@@ -418,4 +422,20 @@ def test_refused_sizes(ops):
     x = torch.zeros(2, 100, dtype=torch.bfloat16, device=DEV)
     w = torch.zeros(8, 100, dtype=torch.bfloat16, device=DEV)
     with pytest.raises(UnsupportedSizeError):
-        ops.linear(x, w, torch.zeros(2, 8, dtype=torch.bfloat16, device=DEV))
+        ops.prepare_weight(w)
+    with pytest.raises(TypeError, match="prepare_weight"):      # bfloat16 weights are packed first
+        ops.linear(x[:, :96].contiguous(), w[:, :96].contiguous(),
+                   torch.zeros(2, 8, dtype=torch.bfloat16, device=DEV))
+
+
+@pytest.mark.parametrize("n,k", [(16, 32), (90, 96), (65, 104), (896, 4864), (257, 136)])
+def test_pack_weight_layout(ops, n, k):
+    """Tile t of strip s holds W[16 s + l % 16, 32 t + 8 (l / 16) .. + 7] at 8 l; zeros past n and k."""
+    w = rnd((n, k), torch.bfloat16, 91)
+    packed = ops.prepare_weight(w.to(DEV))
+    assert packed.shape == (n, k)
+    strips, tiles = (n + 15) // 16, (k + 31) // 32
+    padded = torch.zeros(strips * 16, tiles * 32, dtype=torch.bfloat16)
+    padded[:n, :k] = w
+    want = padded.view(strips, 16, tiles, 4, 8).permute(0, 2, 3, 1, 4).contiguous().view(-1)
+    assert torch.equal(packed.data.cpu(), want)

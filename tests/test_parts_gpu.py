@@ -146,7 +146,7 @@ class RunningMean(Mixer):
 
     def bind(self, tensors, ops, dtype):
         super().bind(tensors, ops, dtype)
-        self.weight = tensors[self.tensor_names["weight"]]
+        self.weight = ops.prepare_weight(tensors[self.tensor_names["weight"]])
 
     def state_spec(self):
         return {"sum": ((self.hidden_size,), torch.float32), "count": ((1,), torch.float32)}
