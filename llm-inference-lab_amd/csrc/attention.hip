@@ -76,14 +76,17 @@ struct KeyStep {
 // blocks that split the keys further merge through global memory (see below).
 constexpr int DECODE_WAVES = D <= 64 ? 8 : (D <= 128 ? 4 : 2);
 constexpr int SPLIT_FILL = 1;      // blocks per compute unit a decode step aims at
-constexpr int DECODE_RING = 2;     // key steps in flight per wave (deeper rings measured no faster)
 
-template <int QB, bool DECODE>
+// RING (decode only): key steps a wave keeps in flight; 1 when a wave has one or two
+// steps at all (nothing to run ahead of), 2 for longer shares (deeper rings measured
+// no faster).
+template <int QB, bool DECODE, int RING = 1>
 __global__ __launch_bounds__(DECODE ? 64 * DECODE_WAVES : 256) void attention_bf16_kernel(AttnArgs a) {
   constexpr int DC = (D + 31) / 32;  // 32-wide chunks of d for Q.K
   constexpr int DB = D / 16;         // 16-wide blocks of d for P.V
   constexpr bool PIPE = DECODE;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+  const int lane = threadIdx.x & 63, nw = blockDim.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // the same for all lanes: kept scalar
   const int c = lane & 15, g = lane >> 4;
   const int b = blockIdx.z;
   const int kvh = blockIdx.y / a.splits, split = blockIdx.y % a.splits;
@@ -153,37 +156,6 @@ __global__ __launch_bounds__(DECODE ? 64 * DECODE_WAVES : 256) void attention_bf
 #pragma unroll
     for (int db = 0; db < DB; ++db) o[qb][db] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
-
-  // issue the loads of one step: page numbers first, then key and value fragments
-  auto fetch = [&](int blk, KeyStep<DC, DB>& f) {
-    const int kb = blk << 5;
-#pragma unroll
-    for (int h2 = 0; h2 < 2; ++h2) {
-      const int pos16 = kb + h2 * 16;
-      bool ok = pos16 <= key_hi && pos16 + 15 >= key_lo;
-      int page = -1;
-      if (ok) page = a.table[(size_t)b * a.table_stride + page_index(pos16)];
-      ok = ok && page >= 0;
-      f.ok[h2] = ok;
-      if (ok) {
-        const int off = page_offset(pos16);
-        const bf16_t* kp = kc + (((size_t)page * a.nkv + kvh) * P + off + c) * D;
-        const bf16_t* vp = vc + ((size_t)page * a.nkv + kvh) * D * P + off + g * 4;
-#pragma unroll
-        for (int dc = 0; dc < DC; ++dc) {
-          const int dd = dc * 32 + g * 8;
-          f.k[h2][dc] = (dd < D) ? *(const bf16x8*)(kp + dd) : zero8;
-        }
-#pragma unroll
-        for (int db = 0; db < DB; ++db) f.v[h2][db] = *(const bf16x4*)(vp + (size_t)(db * 16 + c) * P);
-      } else {
-#pragma unroll
-        for (int dc = 0; dc < DC; ++dc) f.k[h2][dc] = zero8;
-#pragma unroll
-        for (int db = 0; db < DB; ++db) f.v[h2][db] = zero4;
-      }
-    }
-  };
 
   auto compute = [&](int blk, const KeyStep<DC, DB>& f) {
     const int kb = blk << 5;
@@ -263,22 +235,58 @@ __global__ __launch_bounds__(DECODE ? 64 * DECODE_WAVES : 256) void attention_bf
   };
 
   if constexpr (PIPE) {
-    // the loads of the next steps are in flight while this one is computed
-    constexpr int RING = DECODE_RING;
+    // The loads of the next steps are in flight while this one is computed.  Every
+    // load in the loop is unconditional (a load under a branch makes the compiler
+    // wait for all loads in flight where the branch ends, and the ring stalls): a
+    // step past the end reads the last step again, a missing page reads page 0, and
+    // the flags keep what was read out of the sums.  The page numbers of up to 32
+    // steps are read ahead of the loop, one 16-key group per lane.
     KeyStep<DC, DB> ring[RING];
+    for (int cb = my_blk0; cb < my_blk1; cb += 32) {
+      const int ce = min(cb + 32, my_blk1);
+      int pages_v;
+      {
+        const int pos16 = (cb * 2 + lane) * 16;
+        const bool in = cb * 2 + lane < ce * 2 && pos16 <= key_hi && pos16 + 15 >= key_lo;
+        const int pg = a.table[(size_t)b * a.table_stride + min(page_index(pos16), a.table_stride - 1)];
+        pages_v = in ? pg : -1;
+      }
+      auto fetch = [&](int blk, KeyStep<DC, DB>& f) {
+        const int bl = min(blk, ce - 1);
 #pragma unroll
-    for (int p = 0; p < RING; ++p)
-      if (my_blk0 + p < my_blk1) fetch(my_blk0 + p, ring[p]);
-    for (int blk0 = my_blk0; blk0 < my_blk1; blk0 += RING) {
+        for (int h2 = 0; h2 < 2; ++h2) {
+          const int page = __builtin_amdgcn_readlane(pages_v, (bl - cb) * 2 + h2);
+          const bool ok = blk < ce && page >= 0;
+          f.ok[h2] = ok;
+          const size_t pg = (size_t)max(page, 0) * a.nkv + kvh;
+          const int off = page_offset(bl * 32 + h2 * 16);
+          const bf16_t* kp = kc + (pg * P + off + c) * D;
+          const bf16_t* vp = vc + pg * D * P + off + g * 4;
 #pragma unroll
-      for (int p = 0; p < RING; ++p) {
-        const int blk = blk0 + p;
-        if (blk < my_blk1) {
+          for (int dc = 0; dc < DC; ++dc)     // a piece past D meets zeros of the query fragment
+            f.k[h2][dc] = *(const bf16x8*)(kp + min(dc * 32 + g * 8, D - 8));
+#pragma unroll
+          for (int db = 0; db < DB; ++db) {
+            const bf16x4 v = *(const bf16x4*)(vp + (size_t)(db * 16 + c) * P);
+            f.v[h2][db] = ok ? v : zero4;
+          }
+        }
+      };
+#pragma unroll
+      for (int p = 0; p < RING; ++p) fetch(cb + p, ring[p]);
+      int blk0 = cb;
+      for (; blk0 + RING < ce; blk0 += RING) {      // rounds that refill the ring
+#pragma unroll
+        for (int p = 0; p < RING; ++p) {
           const KeyStep<DC, DB> cur = ring[p];
-          if (blk + RING < my_blk1) fetch(blk + RING, ring[p]);
-          compute(blk, cur);
+          fetch(blk0 + p + RING, ring[p]);
+          __builtin_amdgcn_sched_barrier(0);
+          compute(blk0 + p, cur);
         }
       }
+#pragma unroll
+      for (int p = 0; p < RING; ++p)               // the last round drains it
+        if (blk0 + p < ce) compute(blk0 + p, ring[p]);
     }
   } else {
     // ---- prefill: tiles of 64 keys go through LDS once per block and serve all its
@@ -295,97 +303,102 @@ __global__ __launch_bounds__(DECODE ? 64 * DECODE_WAVES : 256) void attention_bf
     const int blk_last = min(blk_row0 + nw * 16 * QB, rows_total) - 1;
     const int bkey_hi = sp + blk_last / G;
     const int bkey_lo = a.window > 0 ? max(0, sp + blk_row0 / G - a.window + 1) : 0;
-    // page numbers first, all at once: the tile loop then has one memory round trip
-    // per tile instead of two dependent ones
-    const int page_first = page_index(bkey_lo);
-    const int page_count = min(page_index(bkey_hi) - page_first + 1, PAGE_CAP);
-    for (int i = tid; i < page_count; i += 256)
-      s_pages[i] = a.table[(size_t)b * a.table_stride + page_first + i];
-    __syncthreads();
     // PD tiles are on their way from memory at any time (a ring of register buffers):
-    // one tile's arithmetic is far shorter than the memory latency
+    // one tile's arithmetic is far shorter than the memory latency.  The loads of the
+    // ring are unconditional (see the decode branch): a tile past the end reads the
+    // last tile again, a missing page reads page 0, and the flag zeroes what came.
     constexpr int PD = NCH <= 4 ? 3 : 2;
     bf16x8 regs[PD][NCH];
     bool rok[PD][NCH];
     const int tile_lo = bkey_lo >> 6, tile_hi = bkey_hi >> 6;
-    auto fetch_tile = [&](int slot, int tile) {
+    // The page numbers come from LDS, PAGE_CAP pages at a time (one slice is enough
+    // for any common context), so that a tile costs one memory round trip, not two.
+    const int tiles_per_slice = (PAGE_CAP << pshift) >> 6;
+    for (int ct = tile_lo; ct <= tile_hi; ct += tiles_per_slice) {
+      const int ce = min(ct + tiles_per_slice - 1, tile_hi);
+      const int page_first = page_index(ct * 64);
+      const int page_count = page_index(ce * 64 + 63) - page_first + 1;
+      __syncthreads();
+      for (int i = tid; i < page_count; i += 256) {
+        const int pi = page_first + i;
+        s_pages[i] = pi < a.table_stride ? a.table[(size_t)b * a.table_stride + pi] : -1;
+      }
+      __syncthreads();
+      auto fetch_tile = [&](int slot, int tile) {
+        const int tl = min(tile, ce);
 #pragma unroll
-      for (int n = 0; n < NCH; ++n) {
-        const int i = tid + n * 256;
-        const bool is_v = i >= 8 * D;
-        const int j = is_v ? i - 8 * D : i;
-        const int sub = j / (2 * D), rem = j - sub * (2 * D);
-        const int pos16 = tile * 64 + sub * 16;
-        bool ok = tile <= tile_hi && pos16 <= bkey_hi && pos16 + 15 >= bkey_lo;
-        int page = -1;
-        if (ok) {
-          const int pi = page_index(pos16) - page_first;
-          page = pi < PAGE_CAP ? s_pages[pi] : a.table[(size_t)b * a.table_stride + page_index(pos16)];
-        }
-        ok = ok && page >= 0;
-        rok[slot][n] = ok;
-        regs[slot][n] = zero8;
-        if (ok) {
+        for (int n = 0; n < NCH; ++n) {
+          const int i = tid + n * 256;
+          const bool is_v = i >= 8 * D;
+          const int j = is_v ? i - 8 * D : i;
+          const int sub = j / (2 * D), rem = j - sub * (2 * D);
+          const int pos16 = tl * 64 + sub * 16;
+          const int page = s_pages[page_index(pos16) - page_first];
+          rok[slot][n] = tile <= ce && pos16 <= bkey_hi && pos16 + 15 >= bkey_lo && page >= 0;
+          const size_t pg = (size_t)max(page, 0) * a.nkv + kvh;
           const int off = page_offset(pos16);
+          const int key = rem / (D / 8), ch = rem - key * (D / 8);      // a piece of a key
+          const int drow = rem >> 1, half = rem & 1;                    // or half a row of values
+          const bf16_t* src = is_v ? vc + (pg * D + drow) * P + off + half * 8
+                                   : kc + (pg * P + off + key) * D + ch * 8;
+          regs[slot][n] = *(const bf16x8*)src;
+        }
+      };
+      auto store_tile = [&](int slot) {
+#pragma unroll
+        for (int n = 0; n < NCH; ++n) {
+          const int i = tid + n * 256;
+          const bool is_v = i >= 8 * D;
+          const int j = is_v ? i - 8 * D : i;
+          const int sub = j / (2 * D), rem = j - sub * (2 * D);
+          const bf16x8 v = rok[slot][n] ? regs[slot][n] : zero8;
           if (!is_v) {
             const int key = rem / (D / 8), ch = rem - key * (D / 8);
-            regs[slot][n] = *(const bf16x8*)(kc + (((size_t)page * a.nkv + kvh) * P + off + key) * D + ch * 8);
+            *(bf16x8*)(Ks + (sub * 16 + key) * KS + ch * 8) = v;
+            if (rem == 0) s_ok[sub] = rok[slot][n];
           } else {
             const int drow = rem >> 1, half = rem & 1;
-            regs[slot][n] = *(const bf16x8*)(vc + (((size_t)page * a.nkv + kvh) * D + drow) * P + off + half * 8);
+            *(bf16x8*)(Vs + drow * VS + sub * 16 + half * 8) = v;
           }
         }
-      }
-    };
-    auto store_tile = [&](int slot) {
+      };
 #pragma unroll
-      for (int n = 0; n < NCH; ++n) {
-        const int i = tid + n * 256;
-        const bool is_v = i >= 8 * D;
-        const int j = is_v ? i - 8 * D : i;
-        const int sub = j / (2 * D), rem = j - sub * (2 * D);
-        if (!is_v) {
-          const int key = rem / (D / 8), ch = rem - key * (D / 8);
-          *(bf16x8*)(Ks + (sub * 16 + key) * KS + ch * 8) = regs[slot][n];
-          if (rem == 0) s_ok[sub] = rok[slot][n];
-        } else {
-          const int drow = rem >> 1, half = rem & 1;
-          *(bf16x8*)(Vs + drow * VS + sub * 16 + half * 8) = regs[slot][n];
-        }
-      }
-    };
+      for (int p = 0; p < PD; ++p) fetch_tile(p, ct + p);
+      for (int tile0 = ct; tile0 <= ce; tile0 += PD) {
 #pragma unroll
-    for (int p = 0; p < PD; ++p) fetch_tile(p, tile_lo + p);
-    for (int tile0 = tile_lo; tile0 <= tile_hi; tile0 += PD) {
-#pragma unroll
-      for (int p = 0; p < PD; ++p) {
-        const int tile = tile0 + p;
-        if (tile <= tile_hi) {
-          store_tile(p);
-          __syncthreads();
+        for (int p = 0; p < PD; ++p) {
+          const int tile = tile0 + p;
+          const bool live = tile <= ce;
+          if (live) {
+            store_tile(p);
+            __syncthreads();
+          }
           fetch_tile(p, tile + PD);
+          __builtin_amdgcn_sched_barrier(0);
+          if (live) {
 #pragma unroll
-          for (int st = 0; st < 2; ++st) {
-            const int kb = tile * 64 + st * 32;
-            if (kb <= key_hi && kb + 31 >= key_lo) {        // this wave sees some of these keys
-              KeyStep<DC, DB> f;
+            for (int st = 0; st < 2; ++st) {
+              const int kb = tile * 64 + st * 32;
+              if (kb <= key_hi && kb + 31 >= key_lo) {        // this wave sees some of these keys
+                KeyStep<DC, DB> f;
 #pragma unroll
-              for (int h2 = 0; h2 < 2; ++h2) {
-                const int sub = st * 2 + h2;
-                f.ok[h2] = s_ok[sub] != 0;
+                for (int h2 = 0; h2 < 2; ++h2) {
+                  const int sub = st * 2 + h2;
+                  f.ok[h2] = s_ok[sub] != 0;
 #pragma unroll
-                for (int dc = 0; dc < DC; ++dc) {
-                  const int dd = dc * 32 + g * 8;
-                  f.k[h2][dc] = (dd < D) ? *(const bf16x8*)(Ks + (sub * 16 + c) * KS + dd) : zero8;
+                  for (int dc = 0; dc < DC; ++dc) {
+                    const int dd = dc * 32 + g * 8;
+                    f.k[h2][dc] = *(const bf16x8*)(Ks + (sub * 16 + c) * KS + min(dd, D - 8));
+                  }
+#pragma unroll
+                  for (int db = 0; db < DB; ++db)
+                    f.v[h2][db] = *(const bf16x4*)(Vs + (db * 16 + c) * VS + sub * 16 + g * 4);
                 }
-#pragma unroll
-                for (int db = 0; db < DB; ++db)
-                  f.v[h2][db] = *(const bf16x4*)(Vs + (db * 16 + c) * VS + sub * 16 + g * 4);
+                compute(kb >> 5, f);
               }
-              compute(kb >> 5, f);
             }
+            __syncthreads();
           }
-          __syncthreads();
         }
       }
     }
@@ -613,7 +626,11 @@ extern "C" int llmlab_paged_attention(const void* q, int dtype, int q_stride, in
       a.ml_part = workspace + (size_t)total_rows * nq * splits * D;
     }
     dim3 grid(1, nkv * splits, reqs), block(64 * DECODE_WAVES);
-    hipLaunchKernelGGL((attention_bf16_kernel<1, true>), grid, block, 0, stream, a);
+    const int steps_per_wave = ((steps32 + splits - 1) / splits + DECODE_WAVES - 1) / DECODE_WAVES;
+    if (steps_per_wave > 2)
+      hipLaunchKernelGGL((attention_bf16_kernel<1, true, 2>), grid, block, 0, stream, a);
+    else
+      hipLaunchKernelGGL((attention_bf16_kernel<1, true, 1>), grid, block, 0, stream, a);
     LLMLAB_LAUNCH_CHECK("attention(bfloat16, decode)");
     if (splits > 1) {
       hipLaunchKernelGGL(attention_merge_kernel, dim3(total_rows, nq), dim3(64), 0, stream, a.o_part,
