@@ -44,6 +44,22 @@ constexpr float NEG_INF = -__builtin_huge_valf();
 // which is what a softmax wants of them)
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// Maxima across the four lanes that hold the keys of one row, by the lane-swap
+// instructions of gfx950 instead of LDS permutes.  (No inline assembly for the
+// maxima themselves: the compiler does not see the wait states an MFMA result needs
+// before a hand-written instruction reads it.)
+__device__ __forceinline__ float max_raw(float a, float b) { return fmaxf(a, b); }
+__device__ __forceinline__ float max3_raw(float a, float b, float c) { return fmaxf(fmaxf(a, b), c); }
+__device__ __forceinline__ float max_across_32(float v) {      // with lane l ^ 32
+  const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return max_raw(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ float max_across_16(float v) {      // with lane l ^ 16
+  const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+  return max_raw(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+constexpr float LAZY_MAX = 8.f;    // see compute(): slack of the running maximum, in powers of two
+
 struct AttnArgs {
   const void* q;      // [rows, q_stride], head h at h*D
   const void* kc;     // this layer's key pages
@@ -81,7 +97,7 @@ constexpr int SPLIT_FILL = 1;      // blocks per compute unit a decode step aims
 // steps at all (nothing to run ahead of), 2 for longer shares (deeper rings measured
 // no faster).
 template <int QB, bool DECODE, int RING = 1>
-__global__ __launch_bounds__(DECODE ? 64 * DECODE_WAVES : 256) void attention_bf16_kernel(AttnArgs a) {
+__global__ __launch_bounds__(DECODE ? 64 * DECODE_WAVES : 256, (!DECODE && D <= 64) ? 2 : 1) void attention_bf16_kernel(AttnArgs a) {
   constexpr int DC = (D + 31) / 32;  // 32-wide chunks of d for Q.K
   constexpr int DB = D / 16;         // 16-wide blocks of d for P.V
   constexpr bool PIPE = DECODE;
@@ -93,10 +109,10 @@ __global__ __launch_bounds__(DECODE ? 64 * DECODE_WAVES : 256) void attention_bf
   const int G = a.nq / a.nkv;
   const int r0 = a.q_start[b], qlen = a.q_start[b + 1] - r0, sp = a.start_pos[b];
   const int rows_total = qlen * G;
-  // prefill: the blocks with the longest histories (the last rows) are dispatched first
-  const int xblk = DECODE ? 0 : (int)(gridDim.x - 1 - blockIdx.x);
-  const int row0 = DECODE ? 0 : (xblk * nw + wave) * (16 * QB);
-  if (!DECODE && xblk * nw * (16 * QB) >= rows_total) return;   // the whole block is past the rows
+  // the blocks with the longest histories (the last rows) are dispatched first
+  const int xblk = (int)(gridDim.x - 1 - blockIdx.x);
+  const int row0 = DECODE ? xblk * (16 * QB) : (xblk * nw + wave) * (16 * QB);
+  if ((DECODE ? row0 : xblk * nw * (16 * QB)) >= rows_total) return;   // the whole block is past the rows
   const bool wave_live = row0 < rows_total;      // a wave without rows still helps to stage keys
   const bf16_t* q = (const bf16_t*)a.q;
   const bf16_t* kc = (const bf16_t*)a.kc;
@@ -157,6 +173,11 @@ __global__ __launch_bounds__(DECODE ? 64 * DECODE_WAVES : 256) void attention_bf
     for (int db = 0; db < DB; ++db) o[qb][db] = floatx4{0.f, 0.f, 0.f, 0.f};
   }
 
+  // One step of 32 keys for every row block of the tile.  The running maximum is
+  // kept in the units of the exponent (score * scale * log2 e) and is only raised
+  // when a score exceeds it by more than LAZY_MAX: until then p = 2^(s - m) may be as
+  // large as 2^LAZY_MAX, which float32 sums and bfloat16 probabilities hold without
+  // loss, and the rescaling of the sums (a pass over all of o) becomes rare.
   auto compute = [&](int blk, const KeyStep<DC, DB>& f) {
     const int kb = blk << 5;
     floatx4 s[2][QB];
@@ -173,13 +194,11 @@ __global__ __launch_bounds__(DECODE ? 64 * DECODE_WAVES : 256) void attention_bf
       }
     }
     // all 32 keys visible to every row of the tile (the common case below the diagonal
-    // and inside the window): no comparisons
+    // and inside the window): no comparisons, no infinities
     const bool all_visible = f.ok[0] && f.ok[1] && kb + 31 <= p_first && kb >= full_lo;
     bf16x8 pf[QB];
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
-      // raw scores (masked ones -inf); the running maximum m is kept in raw units too,
-      // the scale goes into the exponent:  p = 2^(s * scale2 - m * scale2)
       float sv[8];
       if (all_visible) {
 #pragma unroll
@@ -193,27 +212,30 @@ __global__ __launch_bounds__(DECODE ? 64 * DECODE_WAVES : 256) void attention_bf
           sv[i] = vis ? s[h2][qb][i & 3] : NEG_INF;
         }
       }
-      float mx = fmaxf(fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3])),
-                       fmaxf(fmaxf(sv[4], sv[5]), fmaxf(sv[6], sv[7])));
-      mx = fmaxf(mx, __shfl_xor(mx, 16, WAVE));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, WAVE));
-      const float m_new = fmaxf(m[qb], mx);
-      if (__any(m_new != m[qb])) {            // some row's maximum grew: rescale what is summed so far
-        const float alpha = m_new == NEG_INF ? 1.f : fast_exp2((m[qb] - m_new) * scale2);
+      // into the units of the exponent (a product is a canonical number, so the maxima
+      // below need no quieting of their inputs)
+#pragma unroll
+      for (int i = 0; i < 8; ++i) sv[i] *= scale2;
+      float mx = max3_raw(max3_raw(sv[0], sv[1], sv[2]), max3_raw(sv[3], sv[4], sv[5]), max_raw(sv[6], sv[7]));
+      mx = max_across_32(mx);
+      mx = max_across_16(mx);
+      const bool grow = mx > m[qb] + LAZY_MAX;
+      if (__any(grow)) {            // some row's maximum grew: rescale what is summed so far
+        const float m_new = grow ? mx : m[qb];
+        const float alpha = grow ? fast_exp2(m[qb] - m_new) : 1.f;     // 2^-inf = 0 the first time
         lsum[qb] *= alpha;
 #pragma unroll
         for (int db = 0; db < DB; ++db) o[qb][db] *= alpha;
         m[qb] = m_new;
       }
-      const float neg_m = m_new == NEG_INF ? 0.f : -m_new * scale2;    // no visible key yet: p = 2^-inf = 0
-      float psum = 0.f;
+      // no visible key yet (masked steps only): every p of the row is 2^-inf = 0
+      const float neg_m = (!all_visible && m[qb] == NEG_INF) ? 0.f : -m[qb];
+      float pv[8];
 #pragma unroll
-      for (int i = 0; i < 8; ++i) {
-        const float p = fast_exp2(__builtin_fmaf(sv[i], scale2, neg_m));
-        psum += p;
-        pf[qb][i] = (bf16_t)p;
-      }
-      lsum[qb] += psum;
+      for (int i = 0; i < 8; ++i) pv[i] = fast_exp2(sv[i] + neg_m);
+      lsum[qb] += ((pv[0] + pv[1]) + (pv[2] + pv[3])) + ((pv[4] + pv[5]) + (pv[6] + pv[7]));
+#pragma unroll
+      for (int i = 0; i < 8; ++i) pf[qb][i] = (bf16_t)pv[i];
     }
     // keys past the last written position hold stale values: keep them out of
     // the product even though their probability is zero
@@ -375,7 +397,87 @@ __global__ __launch_bounds__(DECODE ? 64 * DECODE_WAVES : 256) void attention_bf
           }
           fetch_tile(p, tile + PD);
           __builtin_amdgcn_sched_barrier(0);
-          if (live) {
+          const int kb0 = tile * 64;
+          // a tile below the diagonal of all rows of the wave and inside their windows,
+          // with all its pages there: the whole tile in one piece, without comparisons
+          const bool interior = live && wave_live && kb0 + 63 <= p_first && kb0 >= full_lo &&
+                                (s_ok[0] & s_ok[1] & s_ok[2] & s_ok[3]) != 0;
+          if (interior) {
+            // with one row block the whole tile of 64 keys at once, with two in halves of
+            // 32 (registers): scores of the piece, one maximum, exponentials, products
+            constexpr int SUBS = (QB == 1 && D <= 64) ? 4 : 2;        // 16-key blocks per piece
+#pragma unroll
+            for (int piece = 0; piece < 4 / SUBS; ++piece) {
+              bf16x8 kf[SUBS][DC];
+              bf16x4 vq[SUBS][DB];
+#pragma unroll
+              for (int u = 0; u < SUBS; ++u) {
+                const int sub = piece * SUBS + u;
+#pragma unroll
+                for (int dc = 0; dc < DC; ++dc)
+                  kf[u][dc] = *(const bf16x8*)(Ks + (sub * 16 + c) * KS + min(dc * 32 + g * 8, D - 8));
+#pragma unroll
+                for (int db = 0; db < DB; ++db)
+                  vq[u][db] = *(const bf16x4*)(Vs + (db * 16 + c) * VS + sub * 16 + g * 4);
+              }
+              floatx4 s4[SUBS][QB];
+#pragma unroll
+              for (int u = 0; u < SUBS; ++u)
+#pragma unroll
+                for (int qb = 0; qb < QB; ++qb) {
+                  s4[u][qb] = floatx4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                  for (int dc = 0; dc < DC; ++dc)
+                    s4[u][qb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[u][dc], qf[qb][dc], s4[u][qb], 0, 0, 0);
+                }
+#pragma unroll
+              for (int u = 0; u < SUBS; ++u)       // into the units of the exponent
+#pragma unroll
+                for (int qb = 0; qb < QB; ++qb) s4[u][qb] *= scale2;
+              bf16x8 pf[SUBS / 2][QB];
+#pragma unroll
+              for (int qb = 0; qb < QB; ++qb) {
+                float mx = NEG_INF;
+#pragma unroll
+                for (int u = 0; u < SUBS; ++u)
+                  mx = max3_raw(max3_raw(s4[u][qb][0], s4[u][qb][1], s4[u][qb][2]), s4[u][qb][3], mx);
+                mx = max_across_32(mx);
+                mx = max_across_16(mx);
+                const bool grow = mx > m[qb] + LAZY_MAX;
+                if (__any(grow)) {
+                  const float m_new = grow ? mx : m[qb];
+                  const float alpha = grow ? fast_exp2(m[qb] - m_new) : 1.f;
+                  lsum[qb] *= alpha;
+#pragma unroll
+                  for (int db = 0; db < DB; ++db) o[qb][db] *= alpha;
+                  m[qb] = m_new;
+                }
+                const float neg_m = -m[qb];
+                float psum = 0.f;
+#pragma unroll
+                for (int st = 0; st < SUBS / 2; ++st) {
+                  float pv[8];
+#pragma unroll
+                  for (int i = 0; i < 8; ++i)
+                    pv[i] = fast_exp2(s4[st * 2 + (i >> 2)][qb][i & 3] + neg_m);
+                  psum += ((pv[0] + pv[1]) + (pv[2] + pv[3])) + ((pv[4] + pv[5]) + (pv[6] + pv[7]));
+#pragma unroll
+                  for (int i = 0; i < 8; ++i) pf[st][qb][i] = (bf16_t)pv[i];
+                }
+                lsum[qb] += psum;
+              }
+#pragma unroll
+              for (int st = 0; st < SUBS / 2; ++st)
+#pragma unroll
+                for (int db = 0; db < DB; ++db) {
+                  const bf16x8 vf = __builtin_shufflevector(vq[st * 2][db], vq[st * 2 + 1][db], 0, 1, 2, 3, 4, 5, 6, 7);
+#pragma unroll
+                  for (int qb = 0; qb < QB; ++qb)
+                    o[qb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[st][qb], o[qb][db], 0, 0, 0);
+                }
+            }
+            __syncthreads();
+          } else if (live) {
 #pragma unroll
             for (int st = 0; st < 2; ++st) {
               const int kb = tile * 64 + st * 32;
@@ -423,21 +525,22 @@ __global__ __launch_bounds__(DECODE ? 64 * DECODE_WAVES : 256) void attention_bf
   } else {
     // ---- merge the waves of the block through LDS
     //   acc = sum_w 2^(m_w - m) acc_w,  l = sum_w 2^(m_w - m) l_w,  m = max_w m_w
-    __shared__ float s_m[DECODE_WAVES][16], s_l[DECODE_WAVES][16];
-    __shared__ __attribute__((aligned(16))) float s_o[DECODE_WAVES][16][D];
-    {
-      float l = lsum[0];
+    __shared__ float s_m[DECODE_WAVES][16 * QB], s_l[DECODE_WAVES][16 * QB];
+    __shared__ __attribute__((aligned(16))) float s_o[DECODE_WAVES][16 * QB][D];
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+      float l = lsum[qb];
       l += __shfl_xor(l, 16, WAVE);
       l += __shfl_xor(l, 32, WAVE);
       if (g == 0) {
-        s_m[wave][c] = m[0] * scale2;      // the merges work in the units of the exponent
-        s_l[wave][c] = l;
+        s_m[wave][qb * 16 + c] = m[qb];               // already in the units of the exponent
+        s_l[wave][qb * 16 + c] = l;
       }
 #pragma unroll
-      for (int db = 0; db < DB; ++db) *(floatx4*)(&s_o[wave][c][db * 16 + g * 4]) = o[0][db];
+      for (int db = 0; db < DB; ++db) *(floatx4*)(&s_o[wave][qb * 16 + c][db * 16 + g * 4]) = o[qb][db];
     }
     __syncthreads();
-    const int nrows = rows_total;     // <= 16
+    const int nrows = min(16 * QB, rows_total - row0);
     // sum the `count` entries of s_m / s_l / s_o in their order; write the result
     // (final: normalised, to `out`; else: as this block's partial result)
     auto merge = [&](int count, bool final) {
@@ -451,7 +554,7 @@ __global__ __launch_bounds__(DECODE ? 64 * DECODE_WAVES : 256) void attention_bf
           num += wt * s_o[w][r][dd];
           den += wt * s_l[w][r];
         }
-        const int t = r / G, hh = kvh * G + r % G;
+        const int t = (row0 + r) / G, hh = kvh * G + (row0 + r) % G;
         if (final) {
           ((bf16_t*)a.out)[(size_t)(r0 + t) * a.out_stride + (size_t)hh * D + dd] =
               (bf16_t)(den > 0.f ? num / den : 0.f);
@@ -637,6 +740,22 @@ extern "C" int llmlab_paged_attention(const void* q, int dtype, int q_stride, in
                          a.ml_part, (bf16_t*)out, out_stride, nq, splits);
       LLMLAB_LAUNCH_CHECK("attention merge");
     }
+    return 0;
+  }
+  // Few tiles of rows (a short portion, with or without a long history behind it):
+  // the waves of a block split the keys of one tile of 32 rows and merge in LDS, so
+  // that the work still spreads over the chip.  Else every wave owns its rows and
+  // the block's waves share the keys through LDS.
+  const long blocks16 = ((max_rows + 63) / 64) * nkv * reqs;
+  if (blocks16 < num_cus) {
+    const int steps32 = (max_ctx_len + 31) / 32 + 1;
+    const int steps_per_wave = (steps32 + DECODE_WAVES - 1) / DECODE_WAVES;
+    dim3 grid((unsigned)((max_rows + 31) / 32), nkv, reqs), block(64 * DECODE_WAVES);
+    if (steps_per_wave > 2)
+      hipLaunchKernelGGL((attention_bf16_kernel<2, true, 2>), grid, block, 0, stream, a);
+    else
+      hipLaunchKernelGGL((attention_bf16_kernel<2, true, 1>), grid, block, 0, stream, a);
+    LLMLAB_LAUNCH_CHECK("attention(bfloat16, key split)");
     return 0;
   }
   // rows per wave: 32 when that still gives every compute unit two blocks (or for
