@@ -327,8 +327,10 @@ __global__ __launch_bounds__(MB >= 4 ? 512 : 1024) void skinny_block_kernel(Skin
       float lo = tile[m * cols + il], hi = tile[m * cols + il + half];
       const int pos = s_pos[m];
       if ((is_q || is_k) && a.inv_freq) {
-        float s, co;
-        sincosf((float)pos * s_freq[i], &s, &co);
+        // bfloat16 results: the hardware sine and cosine of r = frac(angle / 2 pi)
+        float r = (float)pos * s_freq[i] * 0.15915494309189535f;
+        r -= floorf(r);
+        const float s = __builtin_amdgcn_sinf(r), co = __builtin_amdgcn_cosf(r);
         const float nlo = lo * co - hi * s, nhi = hi * co + lo * s;
         lo = nlo;
         hi = nhi;

@@ -107,47 +107,68 @@ extern "C" int llmlab_rmsnorm(const float* x, const void* w, int w_dtype, float 
 // key page  K[page][kvh][off][d].  v heads: written to the value page, which is
 // kept transposed,  V[page][kvh][d][off].  page = table[row_req[r]][pos / P],
 // off = pos % P.  Angles, sine and cosine in float32; one rounding to T.
+// Sine and cosine of a float32 angle.  float32 results: the library routine (exact
+// range reduction).  bfloat16 results: the hardware instructions, which take
+// revolutions; the reduction  r = frac(angle / 2 pi)  adds an error of the size the
+// float32 angle itself has (position * frequency rounded to 24 bits).
 template <typename T>
-__global__ void rope_kv_write_kernel(T* __restrict__ qkv, int row_stride, int nq, int nkv, int d,
-                                     const float* __restrict__ inv_freq,
-                                     const int* __restrict__ positions,
-                                     const int* __restrict__ row_req, const int* __restrict__ table,
-                                     int table_stride, int page_size, T* __restrict__ kcache,
-                                     T* __restrict__ vcache) {
-  const int r = blockIdx.x, head = blockIdx.y;
+__device__ __forceinline__ void rope_sincos(float angle, float* s, float* c) {
+  if constexpr (sizeof(T) == 4) {
+    sincosf(angle, s, c);
+  } else {
+    float r = angle * 0.15915494309189535f;
+    r -= floorf(r);
+    *s = __builtin_amdgcn_sinf(r);
+    *c = __builtin_amdgcn_cosf(r);
+  }
+}
+
+// One block per row; a thread keeps its pair index over the heads it visits when
+// the block size is a multiple of d/2, so its sine and cosine are computed once.
+template <typename T>
+__global__ __launch_bounds__(256) void rope_kv_write_kernel(
+    T* __restrict__ qkv, int row_stride, int nq, int nkv, int d, const float* __restrict__ inv_freq,
+    const int* __restrict__ positions, const int* __restrict__ row_req, const int* __restrict__ table,
+    int table_stride, int page_size, T* __restrict__ kcache, T* __restrict__ vcache) {
+  const int r = blockIdx.x;
   const int pos = positions[r];
-  T* base = qkv + (size_t)r * row_stride + (size_t)head * d;
-  const bool is_q = head < nq, is_k = !is_q && head < nq + nkv;
+  T* row = qkv + (size_t)r * row_stride;
   size_t page = 0;
   int off = 0;
-  if (!is_q && kcache) {
+  if (kcache) {
     page = (size_t)table[(size_t)row_req[r] * table_stride + pos / page_size];
     off = pos % page_size;
   }
-  if (is_q || is_k) {
-    const int half = d >> 1;
-    T* kdst = nullptr;
-    if (is_k && kcache)
-      kdst = kcache + ((page * nkv + (head - nq)) * page_size + off) * (size_t)d;
-    for (int i = threadIdx.x; i < half; i += blockDim.x) {
-      float lo = to_float(base[i]), hi = to_float(base[i + half]);
-      if (inv_freq) {
-        float s, c;
-        sincosf((float)pos * inv_freq[i], &s, &c);
-        const float nlo = lo * c - hi * s, nhi = hi * c + lo * s;
-        lo = nlo;
-        hi = nhi;
-        base[i] = from_float<T>(lo);
-        base[i + half] = from_float<T>(hi);
-      }
-      if (kdst) {
-        kdst[i] = from_float<T>(lo);
-        kdst[i + half] = from_float<T>(hi);
-      }
+  const int half = d >> 1;
+  const int qk_heads = (kcache || inv_freq) ? nq + nkv : 0;     // heads rotated (k also written)
+  const bool fixed_pair = (int)blockDim.x % half == 0;
+  float s0 = 0.f, c0 = 1.f;
+  if (inv_freq && fixed_pair) rope_sincos<T>((float)pos * inv_freq[threadIdx.x % half], &s0, &c0);
+  for (int idx = threadIdx.x; idx < qk_heads * half; idx += blockDim.x) {
+    const int head = idx / half, i = idx - head * half;
+    T* base = row + (size_t)head * d;
+    float lo = to_float(base[i]), hi = to_float(base[i + half]);
+    if (inv_freq) {
+      float s = s0, c = c0;
+      if (!fixed_pair) rope_sincos<T>((float)pos * inv_freq[i], &s, &c);
+      const float nlo = lo * c - hi * s, nhi = hi * c + lo * s;
+      lo = nlo;
+      hi = nhi;
+      base[i] = from_float<T>(lo);
+      base[i + half] = from_float<T>(hi);
     }
-  } else if (vcache) {
-    T* vdst = vcache + ((page * nkv + (head - nq - nkv)) * (size_t)d) * page_size + off;
-    for (int i = threadIdx.x; i < d; i += blockDim.x) vdst[(size_t)i * page_size] = base[i];
+    if (head >= nq && kcache) {
+      T* kdst = kcache + ((page * nkv + (head - nq)) * page_size + off) * (size_t)d;
+      kdst[i] = from_float<T>(lo);
+      kdst[i + half] = from_float<T>(hi);
+    }
+  }
+  if (vcache) {
+    const T* vsrc = row + (size_t)(nq + nkv) * d;
+    for (int idx = threadIdx.x; idx < nkv * d; idx += blockDim.x) {
+      const int head = idx / d, i = idx - head * d;
+      vcache[((page * nkv + head) * (size_t)d + i) * page_size + off] = vsrc[idx];
+    }
   }
 }
 
@@ -164,9 +185,8 @@ extern "C" int llmlab_rope_kv_write(void* qkv, int dtype, int rows, int row_stri
                  "rope_kv_write: a cache write needs a block table");
   if (rows == 0) return 0;
   // Without a cache only q and k heads are rotated (k in place) and v is left alone.
-  const int heads = kcache ? nq + 2 * nkv : (inv_freq ? nq + nkv : 0);
-  if (heads == 0) return 0;
-  dim3 grid(rows, heads), block(64);
+  if (!kcache && !inv_freq) return 0;
+  dim3 grid(rows), block(256);
   if (dtype == DT_BF16)
     hipLaunchKernelGGL(rope_kv_write_kernel<bf16_t>, grid, block, 0, stream, (bf16_t*)qkv, row_stride,
                        nq, nkv, d, inv_freq, positions, row_req, table, table_stride, page_size,
@@ -191,7 +211,7 @@ __global__ void rope_inplace_kernel(T* __restrict__ x, long row_stride, long hea
   for (int i = threadIdx.x; i < half; i += blockDim.x) {
     const float lo = to_float(base[i]), hi = to_float(base[i + half]);
     float s, c;
-    sincosf((float)pos * inv_freq[i], &s, &c);
+    rope_sincos<T>((float)pos * inv_freq[i], &s, &c);
     base[i] = from_float<T>(lo * c - hi * s);
     base[i + half] = from_float<T>(hi * c + lo * s);
   }
