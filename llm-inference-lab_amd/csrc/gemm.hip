@@ -48,22 +48,37 @@ __device__ __forceinline__ void epi_store(const EpiArgs& e, int m, int n, float 
 }
 
 // ============================================================ bf16, tiled
-#define LDS_STRIDE 72
-
-template <int BM, int BN, int EPI>
-__global__ __launch_bounds__(256) void gemm_bf16_tiled(const bf16_t* __restrict__ A,
+template <int BM, int BN, int BK, int WM, int WN, int EPI, bool BDIRECT = false>
+__global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __restrict__ A,
                                                         const bf16_t* __restrict__ W, EpiArgs e, int M,
                                                         int N, int K) {
-  constexpr int BK = 64;
-  constexpr int WTM = BM / 2, WTN = BN / 2;  // wave tile
+  constexpr int LDS_STRIDE = BK + 8;         // padded rows: 16-byte reads of 8 lanes cover all banks
+  constexpr int NT = 64 * WM * WN;           // threads: WM x WN waves
+  constexpr int WTM = BM / WM, WTN = BN / WN;  // wave tile
   constexpr int TM = WTM / 16, TN = WTN / 16;
-  constexpr int A_CHUNKS = BM * 8 / 256, B_CHUNKS = BN * 8 / 256;  // 16-byte chunks per thread
+  constexpr int KCH = BK / 8;                // 16-byte chunks in a row of a tile
+  constexpr int A_CHUNKS = BM * KCH / NT, B_CHUNKS = BN * KCH / NT;  // chunks per thread
+  static_assert(A_CHUNKS >= 1 && B_CHUNKS >= 1 && BM * KCH % NT == 0 && BN * KCH % NT == 0, "tile too small");
   __shared__ __attribute__((aligned(16))) bf16_t As[BM * LDS_STRIDE];
-  __shared__ __attribute__((aligned(16))) bf16_t Bs[BN * LDS_STRIDE];
+  __shared__ __attribute__((aligned(16))) bf16_t Bs[BDIRECT ? 8 : BN * LDS_STRIDE];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave >> 1, wn = wave & 1;
-  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  const int wm = wave / WN, wn = wave % WN;
+  // Blocks are handed to the 8 dies (each with an L2 of its own) in turn.  Give
+  // every die a band of neighbouring column tiles, rows running fastest, so that
+  // what its blocks read at one time is a few column tiles of W and the rows of x.
+  int bx = blockIdx.x, by = blockIdx.y;
+#ifndef GEMM_NO_REMAP
+  {
+    const int gx = gridDim.x, gy = gridDim.y, total = gx * gy;
+    const int lin = by * gx + bx;
+    const int whole = total & ~7;            // the last few blocks (total % 8) keep their place
+    const int mapped = lin < whole ? (lin & 7) * (whole >> 3) + (lin >> 3) : lin;
+    bx = mapped / gy;
+    by = mapped - bx * gy;
+  }
+#endif
+  const int m0 = by * BM, n0 = bx * BN;
   const int c = lane & 15, g = lane >> 4;
 
   floatx4 acc[TM][TN];
@@ -76,47 +91,68 @@ __global__ __launch_bounds__(256) void gemm_bf16_tiled(const bf16_t* __restrict_
   // are on their way at any time: a ring of register buffers, refilled as soon as a
   // buffer has been put into LDS.
   constexpr int PD = (A_CHUNKS + B_CHUNKS) <= 4 ? 4 : 3;
-  bf16x8 ra[PD][A_CHUNKS], rb[PD][B_CHUNKS];
+  bf16x8 ra[PD][A_CHUNKS], rb[BDIRECT ? 1 : PD][B_CHUNKS];
+  // BDIRECT: every wave reads the B fragments of its columns straight from the packed
+  // W into registers; only x goes through LDS
+  bf16x8 rbd[BDIRECT ? PD : 1][BK / 32][TN];
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
   // Loads are unconditional (a load under a branch makes the compiler wait for every
   // load in flight where the branch ends).  Rows of x past M and pieces past K read
   // a valid piece instead: they meet zeros of the padded W or land in rows nobody
   // stores.  W is packed in fragment order: the 64 columns of a strip of 16 rows
-  // are 2 KB of consecutive memory, thread p of a strip's 128 reading bytes 16 p...
+  // are consecutive memory (1 KB per 32 columns), a thread reading 16 bytes of it.
   const int T = (K + 31) >> 5, nstrips = (N + 15) >> 4;
   auto fetch = [&](int slot, int k0) {
 #pragma unroll
     for (int i = 0; i < A_CHUNKS; ++i) {
-      const int ch = tid + i * 256, row = ch >> 3, kc = (ch & 7) * 8;
+      const int ch = tid + i * NT, row = ch / KCH, kc = (ch % KCH) * 8;
       const int m = min(m0 + row, M - 1), k = min(k0 + kc, K - 8);
       ra[slot][i] = *(const bf16x8*)(A + (size_t)m * K + k);
     }
+    if constexpr (!BDIRECT) {
 #pragma unroll
-    for (int i = 0; i < B_CHUNKS; ++i) {
-      const int ch = tid + i * 256, sl = ch >> 7, step = (k0 >> 5) + ((ch >> 6) & 1);
-      const int strip = min((n0 >> 4) + sl, nstrips - 1);
-      const bf16x8 v = *(const bf16x8*)(W + ((size_t)strip * T + min(step, T - 1)) * 512 + (ch & 63) * 8);
-      rb[slot][i] = step < T ? v : zero;
+      for (int i = 0; i < B_CHUNKS; ++i) {
+        const int ch = tid + i * NT, sl = ch / (2 * BK), step = (k0 >> 5) + (ch >> 6) % (BK / 32);
+        const int strip = min((n0 >> 4) + sl, nstrips - 1);
+        const bf16x8 v = *(const bf16x8*)(W + ((size_t)strip * T + min(step, T - 1)) * 512 + (ch & 63) * 8);
+        rb[slot][i] = step < T ? v : zero;
+      }
     }
+  };
+  auto fetch_b = [&](int slot, int k0) {
+#pragma unroll
+    for (int ks = 0; ks < BK / 32; ++ks)
+#pragma unroll
+      for (int j = 0; j < TN; ++j) {
+        const int step = (k0 >> 5) + ks;
+        const int strip = min(((n0 + wn * WTN) >> 4) + j, nstrips - 1);
+        const bf16x8 v = *(const bf16x8*)(W + ((size_t)strip * T + min(step, T - 1)) * 512 + lane * 8);
+        rbd[slot][ks][j] = step < T ? v : zero;
+      }
   };
   auto stash = [&](int slot) {
 #pragma unroll
     for (int i = 0; i < A_CHUNKS; ++i) {
-      const int ch = tid + i * 256, row = ch >> 3, kc = (ch & 7) * 8;
+      const int ch = tid + i * NT, row = ch / KCH, kc = (ch % KCH) * 8;
       *(bf16x8*)(As + row * LDS_STRIDE + kc) = ra[slot][i];
     }
+    if constexpr (!BDIRECT) {
 #pragma unroll
-    for (int i = 0; i < B_CHUNKS; ++i) {
-      const int ch = tid + i * 256, l = ch & 63;
-      const int row = (ch >> 7) * 16 + (l & 15), kc = ((ch >> 6) & 1) * 32 + (l >> 4) * 8;
-      *(bf16x8*)(Bs + row * LDS_STRIDE + kc) = rb[slot][i];
+      for (int i = 0; i < B_CHUNKS; ++i) {
+        const int ch = tid + i * NT, l = ch & 63;
+        const int row = ch / (2 * BK) * 16 + (l & 15), kc = (ch >> 6) % (BK / 32) * 32 + (l >> 4) * 8;
+        *(bf16x8*)(Bs + row * LDS_STRIDE + kc) = rb[slot][i];
+      }
     }
   };
 
   const int nk = (K + BK - 1) / BK;
 #pragma unroll
-  for (int p = 0; p < PD; ++p) fetch(p, p * BK);      // past K: zeros for W
+  for (int p = 0; p < PD; ++p) {      // past K: zeros for W
+    fetch(p, p * BK);
+    if constexpr (BDIRECT) fetch_b(p, p * BK);
+  }
   for (int kt = 0; kt < nk; kt += PD) {
 #pragma unroll
     for (int p = 0; p < PD; ++p) {
@@ -128,14 +164,16 @@ __global__ __launch_bounds__(256) void gemm_bf16_tiled(const bf16_t* __restrict_
       fetch(p, (kt + p + PD) * BK);
       if (live) {
 #pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
+        for (int ks = 0; ks < BK / 32; ++ks) {
           bf16x8 a[TM], b[TN];
 #pragma unroll
           for (int i = 0; i < TM; ++i)
             a[i] = *(const bf16x8*)(As + (wm * WTM + i * 16 + c) * LDS_STRIDE + ks * 32 + g * 8);
 #pragma unroll
-          for (int j = 0; j < TN; ++j)
-            b[j] = *(const bf16x8*)(Bs + (wn * WTN + j * 16 + c) * LDS_STRIDE + ks * 32 + g * 8);
+          for (int j = 0; j < TN; ++j) {
+            if constexpr (BDIRECT) b[j] = rbd[p][ks][j];
+            else b[j] = *(const bf16x8*)(Bs + (wn * WTN + j * 16 + c) * LDS_STRIDE + ks * 32 + g * 8);
+          }
 #pragma unroll
           for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -144,6 +182,7 @@ __global__ __launch_bounds__(256) void gemm_bf16_tiled(const bf16_t* __restrict_
         }
         __syncthreads();
       }
+      if constexpr (BDIRECT) fetch_b(p, (kt + p + PD) * BK);
     }
   }
 
@@ -243,10 +282,13 @@ static int launch_bf16(const bf16_t* A, const bf16_t* W, EpiArgs e, int M, int N
   const long big_tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
   if (big_tiles >= num_cus) {
     dim3 grid((N + 127) / 128, (M + 127) / 128);
-    hipLaunchKernelGGL((gemm_bf16_tiled<128, 128, EPI>), grid, dim3(256), 0, stream, A, W, e, M, N, K);
+    hipLaunchKernelGGL((gemm_bf16_tiled<128, 128, 64, 2, 2, EPI, false>), grid, dim3(256), 0, stream, A, W, e, M, N, K);
   } else {
     dim3 grid((N + 63) / 64, (M + 63) / 64);
-    hipLaunchKernelGGL((gemm_bf16_tiled<64, 64, EPI>), grid, dim3(256), 0, stream, A, W, e, M, N, K);
+    // (with the small tile the waves read their B fragments straight from the packed W:
+    // measured faster there, and slower with the large tile, whose waves would read
+    // every fragment twice)
+    hipLaunchKernelGGL((gemm_bf16_tiled<64, 64, 64, 2, 2, EPI, true>), grid, dim3(256), 0, stream, A, W, e, M, N, K);
   }
   return 0;
 }
