@@ -152,6 +152,15 @@ __global__ __launch_bounds__(MB >= 4 ? 512 : 1024) void skinny_block_kernel(Skin
       s_freq[i] = a.inv_freq ? a.inv_freq[i] : 0.f;
   }
 
+  // the residual value this thread will add to (its first one): on its way now, not
+  // after the reduction
+  float resid_old = 0.f;
+  if constexpr (EPI == SK_RESID) {
+    const int idx = threadIdx.x;
+    const int m = idx / cols, nn = n0 + idx - m * cols;
+    if (idx < M * cols && nn < a.N) resid_old = ((const float*)a.out)[(size_t)m * a.ldo + nn];
+  }
+
   floatx4 acc[MB];
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) acc[mb] = fzero;
@@ -299,7 +308,7 @@ __global__ __launch_bounds__(MB >= 4 ? 512 : 1024) void skinny_block_kernel(Skin
     } else if (nn < a.N) {
       const size_t at = (size_t)m * a.ldo + nn;
       if (EPI == SK_STORE) ((bf16_t*)a.out)[at] = (bf16_t)sum;
-      else if (EPI == SK_RESID) ((float*)a.out)[at] += sum;
+      else if (EPI == SK_RESID) ((float*)a.out)[at] = (idx == (int)threadIdx.x ? resid_old : ((float*)a.out)[at]) + sum;
       else ((float*)a.out)[at] = sum;
     }
   }
