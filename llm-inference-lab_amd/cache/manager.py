@@ -5,14 +5,15 @@ per-request state of fixed size.
 Storage of one group (``S`` cache-owning runs of layers, ``N`` pages of ``P``
 tokens, ``G`` kv heads of width ``d``), in the compute dtype::
 
-    keys    [S, N, G, P, d]     a page holds, per kv head, P rows of d
-    values  [S, N, G, d, P]     the same transposed: d rows of P tokens
+    keys    [S, N, G, P, d]     a page holds, per kv head, P keys of d numbers
+    values  [S, N, G, d, P]     and as many values
 
 A page number addresses the same page in every run of the group, so the group
 needs one block table.  Position ``p`` of a request lives in page
-``table[p // P]`` at offset ``p % P``.  The values are kept transposed because
-the matrix cores contract over tokens in the probabilities-times-values product
-and read eight consecutive tokens per lane.
+``table[p // P]`` at offset ``p % P``.  Inside a (page, kv head) pair the
+``P * d`` numbers lie in the order of the attention kernels' matrix-core
+fragments, not row by row (``cache/layout.py`` has the index maps); the manager
+itself never looks inside a page.
 
 The reference's pool has pages of one token, one group, and a slot table
 ``[rows, max_seq_len]`` (rust/engine/src/runner/kv_pool/naive_kvpool.rs:55-81);

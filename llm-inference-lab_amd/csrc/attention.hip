@@ -2,10 +2,11 @@
 // given on the compiler's command line; the library is built once per head size
 // that a model needs).  gfx950 only.
 //
-// Cache of one layer:   keys   K[page][kv_head][P][D]
-//                        values V[page][kv_head][D][P]   (transposed)
-// Position p of the b-th request of the step lives in page table[b][p / P] at
-// offset p % P (P a power of two).  The query at position p sees the keys lo..p, lo = max(0, p -
+// Cache of one layer: per page and kv head P keys of D numbers and as many values,
+// each in the order of this kernel's MFMA fragments (kcache_index / vcache_index in
+// common.h): a 16-key block is 16 D consecutive numbers, and every fragment load of
+// a wave is lane-contiguous.  Position p of the b-th request of the step lives in
+// page table[b][p / P] at offset p % P (P a power of two, at least 16).  The query at position p sees the keys lo..p, lo = max(0, p -
 // window + 1) with a window and 0 without.
 //
 // bfloat16 kernel (matrix cores).  A tile is 16*QB "rows", a row being a (token,
@@ -280,16 +281,18 @@ __global__ __launch_bounds__(DECODE ? 64 * DECODE_WAVES : 256, (!DECODE && D <= 
           const int page = __builtin_amdgcn_readlane(pages_v, (bl - cb) * 2 + h2);
           const bool ok = blk < ce && page >= 0;
           f.ok[h2] = ok;
-          const size_t pg = (size_t)max(page, 0) * a.nkv + kvh;
-          const int off = page_offset(bl * 32 + h2 * 16);
-          const bf16_t* kp = kc + (pg * P + off + c) * D;
-          const bf16_t* vp = vc + pg * D * P + off + g * 4;
+          // the 16-key block of the page: its keys and its values are 16 D numbers each,
+          // in fragment order (see common.h), so every load below is lane-contiguous
+          const size_t blk16 = ((size_t)max(page, 0) * a.nkv + kvh) * P * D +
+                               (size_t)(page_offset(bl * 32 + h2 * 16) >> 4) * (16 * D);
+          const bf16_t* kp = kc + blk16 + c * 8;
+          const bf16_t* vp = vc + blk16 + lane * 4;
 #pragma unroll
           for (int dc = 0; dc < DC; ++dc)     // a piece past D meets zeros of the query fragment
-            f.k[h2][dc] = *(const bf16x8*)(kp + min(dc * 32 + g * 8, D - 8));
+            f.k[h2][dc] = *(const bf16x8*)(kp + min(dc * 4 + g, D / 8 - 1) * 128);
 #pragma unroll
           for (int db = 0; db < DB; ++db) {
-            const bf16x4 v = *(const bf16x4*)(vp + (size_t)(db * 16 + c) * P);
+            const bf16x4 v = *(const bf16x4*)(vp + db * 256);
             f.v[h2][db] = ok ? v : zero4;
           }
         }
@@ -313,10 +316,11 @@ __global__ __launch_bounds__(DECODE ? 64 * DECODE_WAVES : 256, (!DECODE && D <= 
   } else {
     // ---- prefill: tiles of 64 keys go through LDS once per block and serve all its
     // waves; the next tile is fetched into registers while this one is multiplied
-    constexpr int KS = D + 8, VS = 64 + 8;          // padded rows: 16-byte reads of 8 lanes cover all banks
     constexpr int NCH = D / 16;                     // 16-byte pieces per thread and tile (256 threads)
-    __shared__ __attribute__((aligned(16))) bf16_t Ks[64 * KS];   // [key][d]
-    __shared__ __attribute__((aligned(16))) bf16_t Vs[D * VS];    // [d][key]
+    // the tile's four 16-key blocks as they lie in the cache (fragment order): the
+    // copy is straight, and every fragment read below is lane-contiguous
+    __shared__ __attribute__((aligned(16))) bf16_t Ks[64 * D];
+    __shared__ __attribute__((aligned(16))) bf16_t Vs[64 * D];
     __shared__ int s_ok[4];
     constexpr int PAGE_CAP = 2048;
     __shared__ int s_pages[PAGE_CAP];               // the block's slice of its request's block table
@@ -357,13 +361,9 @@ __global__ __launch_bounds__(DECODE ? 64 * DECODE_WAVES : 256, (!DECODE && D <= 
           const int pos16 = tl * 64 + sub * 16;
           const int page = s_pages[page_index(pos16) - page_first];
           rok[slot][n] = tile <= ce && pos16 <= bkey_hi && pos16 + 15 >= bkey_lo && page >= 0;
-          const size_t pg = (size_t)max(page, 0) * a.nkv + kvh;
-          const int off = page_offset(pos16);
-          const int key = rem / (D / 8), ch = rem - key * (D / 8);      // a piece of a key
-          const int drow = rem >> 1, half = rem & 1;                    // or half a row of values
-          const bf16_t* src = is_v ? vc + (pg * D + drow) * P + off + half * 8
-                                   : kc + (pg * P + off + key) * D + ch * 8;
-          regs[slot][n] = *(const bf16x8*)src;
+          const size_t blk16 = ((size_t)max(page, 0) * a.nkv + kvh) * P * D +
+                               (size_t)(page_offset(pos16) >> 4) * (16 * D);
+          regs[slot][n] = *(const bf16x8*)((is_v ? vc : kc) + blk16 + rem * 8);
         }
       };
       auto store_tile = [&](int slot) {
@@ -374,14 +374,8 @@ __global__ __launch_bounds__(DECODE ? 64 * DECODE_WAVES : 256, (!DECODE && D <= 
           const int j = is_v ? i - 8 * D : i;
           const int sub = j / (2 * D), rem = j - sub * (2 * D);
           const bf16x8 v = rok[slot][n] ? regs[slot][n] : zero8;
-          if (!is_v) {
-            const int key = rem / (D / 8), ch = rem - key * (D / 8);
-            *(bf16x8*)(Ks + (sub * 16 + key) * KS + ch * 8) = v;
-            if (rem == 0) s_ok[sub] = rok[slot][n];
-          } else {
-            const int drow = rem >> 1, half = rem & 1;
-            *(bf16x8*)(Vs + drow * VS + sub * 16 + half * 8) = v;
-          }
+          *(bf16x8*)((is_v ? Vs : Ks) + sub * (16 * D) + rem * 8) = v;
+          if (!is_v && rem == 0) s_ok[sub] = rok[slot][n];
         }
       };
 #pragma unroll
@@ -415,10 +409,10 @@ __global__ __launch_bounds__(DECODE ? 64 * DECODE_WAVES : 256, (!DECODE && D <= 
                 const int sub = piece * SUBS + u;
 #pragma unroll
                 for (int dc = 0; dc < DC; ++dc)
-                  kf[u][dc] = *(const bf16x8*)(Ks + (sub * 16 + c) * KS + min(dc * 32 + g * 8, D - 8));
+                  kf[u][dc] = *(const bf16x8*)(Ks + sub * (16 * D) + min(dc * 4 + g, D / 8 - 1) * 128 + c * 8);
 #pragma unroll
                 for (int db = 0; db < DB; ++db)
-                  vq[u][db] = *(const bf16x4*)(Vs + (db * 16 + c) * VS + sub * 16 + g * 4);
+                  vq[u][db] = *(const bf16x4*)(Vs + sub * (16 * D) + db * 256 + lane * 4);
               }
               floatx4 s4[SUBS][QB];
 #pragma unroll
@@ -488,13 +482,11 @@ __global__ __launch_bounds__(DECODE ? 64 * DECODE_WAVES : 256, (!DECODE && D <= 
                   const int sub = st * 2 + h2;
                   f.ok[h2] = s_ok[sub] != 0;
 #pragma unroll
-                  for (int dc = 0; dc < DC; ++dc) {
-                    const int dd = dc * 32 + g * 8;
-                    f.k[h2][dc] = *(const bf16x8*)(Ks + (sub * 16 + c) * KS + min(dd, D - 8));
-                  }
+                  for (int dc = 0; dc < DC; ++dc)
+                    f.k[h2][dc] = *(const bf16x8*)(Ks + sub * (16 * D) + min(dc * 4 + g, D / 8 - 1) * 128 + c * 8);
 #pragma unroll
                   for (int db = 0; db < DB; ++db)
-                    f.v[h2][db] = *(const bf16x4*)(Vs + (db * 16 + c) * VS + sub * 16 + g * 4);
+                    f.v[h2][db] = *(const bf16x4*)(Vs + sub * (16 * D) + db * 256 + lane * 4);
                 }
                 compute(kb >> 5, f);
               }
@@ -637,18 +629,18 @@ __global__ __launch_bounds__(64) void attention_f32_kernel(AttnArgs a) {
   for (int j = lo + lane; j <= p; j += 64) {
     const int page = a.table[(size_t)b * a.table_stride + (j >> a.page_shift)];
     const int off = j & (P - 1);
-    const float* kp = kc + (((size_t)page * a.nkv + kvh) * P + off) * D;
-    const float* vp = vc + ((size_t)page * a.nkv + kvh) * D * P + off;
+    const float* kp = kc + ((size_t)page * a.nkv + kvh) * P * D;
+    const float* vp = vc + ((size_t)page * a.nkv + kvh) * P * D;
     float dot = 0.f;
 #pragma unroll
-    for (int dd = 0; dd < D; ++dd) dot = fmaf(qs[dd], kp[dd], dot);
+    for (int dd = 0; dd < D; ++dd) dot = fmaf(qs[dd], kp[kcache_index(off, dd, D)], dot);
     const float s = dot * a.scale;
     const float m_new = fmaxf(m, s);
     const float alpha = expf(m - m_new);  // m = -inf on the first key: exp(-inf) = 0
     const float pr = expf(s - m_new);
     l = l * alpha + pr;
 #pragma unroll
-    for (int dd = 0; dd < D; ++dd) o[dd] = fmaf(pr, vp[(size_t)dd * P], o[dd] * alpha);
+    for (int dd = 0; dd < D; ++dd) o[dd] = fmaf(pr, vp[vcache_index(off, dd, D)], o[dd] * alpha);
     m = m_new;
   }
   const float mmax = wave_max(m);

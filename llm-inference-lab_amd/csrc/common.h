@@ -90,3 +90,23 @@ __device__ __forceinline__ float block_sum(float v, float* red) {
   __syncthreads();
   return red[16];
 }
+
+// ------------------------------------------------------------------ cache order
+// One page of one kv head holds P keys of d numbers, and as many values.  Both are
+// kept in the order in which the matrix cores read them in the attention products
+// (v_mfma_f32_16x16x32_bf16, lane l = 16 g + c), so that a wave instruction reads
+// consecutive memory:
+//   keys:    [16-key block][octet of d][key in block][8]     (A operand of K . Q^T:
+//            lane (c, g) takes key c, numbers 8 g .. 8 g + 7 of a 32-wide piece of d;
+//            the 1 KB of a (key block, piece) is lane-contiguous)
+//   values:  [16-key block][16-wide block of d][group of 4 keys][number in block][4]
+//            (A operand of V^T . P^T: lane (c, g) takes number c of the block and the
+//            keys 4 g .. 4 g + 3; the 512 bytes of a (key block, d block) are
+//            lane-contiguous)
+// k = key within the page, dd = number within the head, d a multiple of 16.
+__host__ __device__ inline size_t kcache_index(int k, int dd, int d) {
+  return ((size_t)((k >> 4) * (d >> 3) + (dd >> 3)) * 16 + (k & 15)) * 8 + (dd & 7);
+}
+__host__ __device__ inline size_t vcache_index(int k, int dd, int d) {
+  return ((size_t)(((k >> 4) * (d >> 4) + (dd >> 4)) * 4 + ((k & 15) >> 2)) * 16 + (dd & 15)) * 4 + (k & 3);
+}

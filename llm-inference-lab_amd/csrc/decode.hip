@@ -352,13 +352,13 @@ __global__ __launch_bounds__(MB >= 4 ? 512 : 1024) void skinny_block_kernel(Skin
         const size_t page = (size_t)s_page[m];
         const int off = pos % a.page_size;
         if (is_k) {
-          bf16_t* dst = a.kcache + ((page * a.nkv + (head - a.nq)) * a.page_size + off) * (size_t)d;
-          dst[i] = (bf16_t)lo;
-          dst[i + dhalf] = (bf16_t)hi;
+          bf16_t* dst = a.kcache + (page * a.nkv + (head - a.nq)) * (size_t)a.page_size * d;
+          dst[kcache_index(off, i, d)] = (bf16_t)lo;
+          dst[kcache_index(off, i + dhalf, d)] = (bf16_t)hi;
         } else {
-          bf16_t* dst = a.vcache + ((page * a.nkv + (head - a.nq - a.nkv)) * (size_t)d) * a.page_size + off;
-          dst[(size_t)i * a.page_size] = (bf16_t)lo;
-          dst[(size_t)(i + dhalf) * a.page_size] = (bf16_t)hi;
+          bf16_t* dst = a.vcache + (page * a.nkv + (head - a.nq - a.nkv)) * (size_t)a.page_size * d;
+          dst[vcache_index(off, i, d)] = (bf16_t)lo;
+          dst[vcache_index(off, i + dhalf, d)] = (bf16_t)hi;
         }
       }
     }

@@ -105,7 +105,7 @@ extern "C" int llmlab_rmsnorm(const float* x, const void* w, int w_dtype, float 
 //   qkv[r] = [q heads | k heads | v heads], each head `d` wide.
 // q heads: rotated in place.  k heads: rotated, written in place and to the
 // key page  K[page][kvh][off][d].  v heads: written to the value page, which is
-// kept transposed,  V[page][kvh][d][off].  page = table[row_req[r]][pos / P],
+// in the order of the attention kernels' fragments (kcache_index, vcache_index).  page = table[row_req[r]][pos / P],
 // off = pos % P.  Angles, sine and cosine in float32; one rounding to T.
 // Sine and cosine of a float32 angle.  float32 results: the library routine (exact
 // range reduction).  bfloat16 results: the hardware instructions, which take
@@ -158,16 +158,16 @@ __global__ __launch_bounds__(256) void rope_kv_write_kernel(
       base[i + half] = from_float<T>(hi);
     }
     if (head >= nq && kcache) {
-      T* kdst = kcache + ((page * nkv + (head - nq)) * page_size + off) * (size_t)d;
-      kdst[i] = from_float<T>(lo);
-      kdst[i + half] = from_float<T>(hi);
+      T* kdst = kcache + (page * nkv + (head - nq)) * (size_t)page_size * d;
+      kdst[kcache_index(off, i, d)] = from_float<T>(lo);
+      kdst[kcache_index(off, i + half, d)] = from_float<T>(hi);
     }
   }
   if (vcache) {
     const T* vsrc = row + (size_t)(nq + nkv) * d;
     for (int idx = threadIdx.x; idx < nkv * d; idx += blockDim.x) {
       const int head = idx / d, i = idx - head * d;
-      vcache[((page * nkv + head) * (size_t)d + i) * page_size + off] = vsrc[idx];
+      vcache[(page * nkv + head) * (size_t)d * page_size + vcache_index(off, i, d)] = vsrc[idx];
     }
   }
 }

@@ -7,6 +7,7 @@ import pytest
 import torch
 
 from emu_ops import EmuOps
+from llm_inference_lab_amd.cache import layout as cache_layout
 
 pytestmark = pytest.mark.gpu
 
@@ -308,6 +309,8 @@ def run_attention(ops, emu, dtype, nq, nkv, d, page, window, reqs_spec, seed=30,
             pg = int(table[b, end // page])
             kc[pg, :, end % page:, :] = 1e4
             vc[pg, :, :, end % page:] = -1e4
+    # what was set up above by key and number goes into the order the cache keeps
+    kc, vc = cache_layout.keys_to_cache_order(kc), cache_layout.values_to_cache_order(vc)
     q_start_t = torch.tensor(q_start, dtype=torch.int32)
     start_pos_t = torch.tensor(start_pos, dtype=torch.int32)
     scale = scale if scale is not None else 1 / math.sqrt(d)
@@ -439,3 +442,17 @@ def test_pack_weight_layout(ops, n, k):
     padded[:n, :k] = w
     want = padded.view(strips, 16, tiles, 4, 8).permute(0, 2, 3, 1, 4).contiguous().view(-1)
     assert torch.equal(packed.data.cpu(), want)
+
+
+@pytest.mark.parametrize("page,d", [(16, 16), (16, 48), (32, 32), (64, 64), (64, 128), (128, 80)])
+def test_cache_order_round_trip(page, d):
+    """The index maps are permutations of the page, and undo each other."""
+    k = rnd((3, 2, page, d), torch.float32, 71)
+    v = rnd((3, 2, d, page), torch.float32, 72)
+    ki, vi = cache_layout.key_index(page, d), cache_layout.value_index(page, d)
+    assert sorted(ki.reshape(-1).tolist()) == list(range(page * d))
+    assert sorted(vi.reshape(-1).tolist()) == list(range(page * d))
+    assert torch.equal(cache_layout.keys_from_cache_order(cache_layout.keys_to_cache_order(k)), k)
+    assert torch.equal(cache_layout.values_from_cache_order(cache_layout.values_to_cache_order(v)), v)
+    # a 16-key block is 16 * d consecutive numbers, for keys and for values
+    assert int(ki[:16].max()) == 16 * d - 1 and int(vi[:, :16].max()) == 16 * d - 1
