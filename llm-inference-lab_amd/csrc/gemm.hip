@@ -60,7 +60,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __
   constexpr int A_CHUNKS = BM * KCH / NT, B_CHUNKS = BN * KCH / NT;  // chunks per thread
   static_assert(A_CHUNKS >= 1 && B_CHUNKS >= 1 && BM * KCH % NT == 0 && BN * KCH % NT == 0, "tile too small");
   __shared__ __attribute__((aligned(16))) bf16_t As[BM * LDS_STRIDE];
-  __shared__ __attribute__((aligned(16))) bf16_t Bs[BDIRECT ? 8 : BN * LDS_STRIDE];
+  __shared__ __attribute__((aligned(16))) bf16_t Bs[BDIRECT ? 8 : BN * BK];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / WN, wn = wave % WN;
@@ -140,9 +140,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __
     if constexpr (!BDIRECT) {
 #pragma unroll
       for (int i = 0; i < B_CHUNKS; ++i) {
-        const int ch = tid + i * NT, l = ch & 63;
-        const int row = ch / (2 * BK) * 16 + (l & 15), kc = (ch >> 6) % (BK / 32) * 32 + (l >> 4) * 8;
-        *(bf16x8*)(Bs + row * LDS_STRIDE + kc) = rb[slot][i];
+        // as it lies in the packed W: [strip][32-wide step][lane][8], no padding needed
+        *(bf16x8*)(Bs + (tid + i * NT) * 8) = rb[slot][i];
       }
     }
   };
@@ -172,7 +171,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __
 #pragma unroll
           for (int j = 0; j < TN; ++j) {
             if constexpr (BDIRECT) b[j] = rbd[p][ks][j];
-            else b[j] = *(const bf16x8*)(Bs + (wn * WTN + j * 16 + c) * LDS_STRIDE + ks * 32 + g * 8);
+            else b[j] = *(const bf16x8*)(Bs + (((wn * TN + j) * (BK / 32) + ks) * 64 + lane) * 8);
           }
 #pragma unroll
           for (int i = 0; i < TM; ++i)
