@@ -4,9 +4,12 @@
 //
 //   bfloat16:  v_mfma_f32_16x16x32_bf16 everywhere.
 //     * tiled kernel: 256 threads = 4 waves in 2x2, block tile 128x128 or
-//       64x64, K step 64 staged through LDS (rows padded to 72 elements so that the
-//       16-byte fragment reads of 8 lanes cover all banks); three or four tiles are
-//       on their way from memory in a ring of register buffers while one is multiplied.
+//       64x64, K step 64; x staged through two stages of LDS (rows padded to 72
+//       elements so that the 16-byte fragment reads of 8 lanes cover all banks), W
+//       too (in fragment order, as it lies in memory) or read straight into
+//       registers; three or four tiles are on their way from memory in a ring of
+//       register buffers while one is multiplied.  Measured and not adopted: 256x128
+//       tiles with eight 64x64 or four 128x64 wave tiles, K steps of 128.
 //     (products of few rows, as in decode steps, have kernels of their own in decode.hip)
 //   float32: a plain FMA kernel (64x64 tile, 4x4 outputs per thread): true 32-bit
 //     products and sums, no matrix-core shortcut.
@@ -59,8 +62,11 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __
   constexpr int KCH = BK / 8;                // 16-byte chunks in a row of a tile
   constexpr int A_CHUNKS = BM * KCH / NT, B_CHUNKS = BN * KCH / NT;  // chunks per thread
   static_assert(A_CHUNKS >= 1 && B_CHUNKS >= 1 && BM * KCH % NT == 0 && BN * KCH % NT == 0, "tile too small");
-  __shared__ __attribute__((aligned(16))) bf16_t As[BM * LDS_STRIDE];
-  __shared__ __attribute__((aligned(16))) bf16_t Bs[BDIRECT ? 8 : BN * BK];
+  // two stages of LDS: the next tile is put in while this one is multiplied, one
+  // barrier per tile
+  constexpr int A_STAGE = BM * LDS_STRIDE, B_STAGE = BDIRECT ? 8 : BN * BK;
+  __shared__ __attribute__((aligned(16))) bf16_t As2[2 * A_STAGE];
+  __shared__ __attribute__((aligned(16))) bf16_t Bs2[2 * B_STAGE];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / WN, wn = wave % WN;
@@ -131,7 +137,9 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __
         rbd[slot][ks][j] = step < T ? v : zero;
       }
   };
-  auto stash = [&](int slot) {
+  auto stash = [&](int slot, int stage) {
+    bf16_t* As = As2 + stage * A_STAGE;
+    bf16_t* Bs = Bs2 + stage * B_STAGE;
 #pragma unroll
     for (int i = 0; i < A_CHUNKS; ++i) {
       const int ch = tid + i * NT, row = ch / KCH, kc = (ch % KCH) * 8;
@@ -152,16 +160,22 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __
     fetch(p, p * BK);
     if constexpr (BDIRECT) fetch_b(p, p * BK);
   }
+  // tile kt lies in stage kt & 1; it was put there during tile kt - 1 (tile 0: now)
+  stash(0, 0);
+  fetch(0, PD * BK);
+  __syncthreads();
   for (int kt = 0; kt < nk; kt += PD) {
 #pragma unroll
     for (int p = 0; p < PD; ++p) {
-      const bool live = kt + p < nk;
+      const int t = kt + p;
+      const bool live = t < nk;
+      const int stage = t & 1;
+      const int pn = (p + 1) % PD;              // ring slot of tile t + 1 (a constant once unrolled)
+      if (t + 1 < nk) stash(pn, stage ^ 1);
+      fetch(pn, (t + 1 + PD) * BK);
       if (live) {
-        stash(p);
-        __syncthreads();
-      }
-      fetch(p, (kt + p + PD) * BK);
-      if (live) {
+        const bf16_t* As = As2 + stage * A_STAGE;
+        const bf16_t* Bs = Bs2 + stage * B_STAGE;
 #pragma unroll
         for (int ks = 0; ks < BK / 32; ++ks) {
           bf16x8 a[TM], b[TN];
@@ -181,7 +195,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __
         }
         __syncthreads();
       }
-      if constexpr (BDIRECT) fetch_b(p, (kt + p + PD) * BK);
+      if constexpr (BDIRECT) fetch_b(p, (t + PD) * BK);
     }
   }
 
