@@ -707,7 +707,10 @@ extern "C" int llmlab_paged_attention(const void* q, int dtype, int q_stride, in
     // the keys are spread over all of them; but no more blocks than there are steps
     // for their waves
     const long base = (long)reqs * nkv;
-    int splits = (int)((SPLIT_FILL * (long)num_cus + base - 1) / base);
+#ifndef SPLIT_DIV
+#define SPLIT_DIV 1
+#endif
+    int splits = (int)((SPLIT_FILL * (long)num_cus / SPLIT_DIV + base - 1) / base);
     const int most = (steps32 + DECODE_WAVES - 1) / DECODE_WAVES;      // one step per wave at least
     if (splits > most) splits = most;
     if (splits > 16) splits = 16;                               // what the merge kernel takes

@@ -249,3 +249,160 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(dtype):
     finally:
         unregister_part("mixer", "toy_running_mean")
         unregister_architecture("ToyForCausalLM")
+
+
+# ------------------------------------- toy feed-forward with routing, toy position encoding
+from llm_inference_lab_amd.parts import FeedForward, PositionEncoding    # noqa: E402
+
+
+class TopOneExperts(FeedForward):
+    """A feed-forward with routing: router logits in float32, the best of E experts
+    per token, each expert one square matrix; the expert's output is scaled by the
+    router's softmax weight.  Rows are gathered per expert, multiplied by the
+    framework's product kernel, and scattered back into the residual."""
+
+    def __init__(self, hidden_size, num_experts, tensors):
+        super().__init__(tensors)
+        self.hidden_size, self.num_experts = hidden_size, num_experts
+
+    def tensor_specs(self):
+        t, h = self.tensor_names, self.hidden_size
+        specs = {t["router"]: TensorSpec((self.num_experts, h), MATRIX)}
+        for e in range(self.num_experts):
+            specs[f'{t["experts"]}.{e}'] = TensorSpec((h, h), MATRIX)
+        return specs
+
+    def bind(self, tensors, ops, dtype):
+        super().bind(tensors, ops, dtype)
+        t = self.tensor_names
+        self.router = tensors[t["router"]].float()
+        self.experts = [ops.prepare_weight(tensors[f'{t["experts"]}.{e}']) for e in range(self.num_experts)]
+
+    def forward(self, h, residual, ctx):
+        logits = h.float() @ self.router.t()                      # float32 router
+        weight, choice = torch.softmax(logits, dim=-1).max(dim=-1)
+        for e in range(self.num_experts):
+            rows = torch.nonzero(choice == e).flatten()
+            if rows.numel() == 0:
+                continue
+            out = torch.zeros(rows.numel(), self.hidden_size, dtype=torch.float32, device=h.device)
+            self.ops.linear_residual(h[rows].contiguous(), self.experts[e], out)
+            residual.index_add_(0, rows, out * weight[rows, None])
+
+
+class HalfRotary(PositionEncoding):
+    """Another position encoding: only the first half of every head is rotated
+    (pairs (i, i + d/4) of that half), the second half carries no position."""
+
+    def __init__(self, dim, theta, tensors=None):
+        super().__init__(tensors)
+        self.dim, self.theta = dim, theta
+
+    def tensor_specs(self):
+        return {}
+
+    def rotary_table(self):
+        return None                      # not the split-half rotation the fused kernel applies
+
+    def apply(self, q, k, positions):
+        r = self.dim // 2
+        inv = 1.0 / (self.theta ** (torch.arange(0, r, 2, dtype=torch.float64, device=q.device) / r))
+        ang = positions.double()[:, None] * inv[None, :]
+        cos, sin = ang.cos()[:, None, :], ang.sin()[:, None, :]
+        for x in (q, k):
+            lo, hi = x[..., :r // 2].double(), x[..., r // 2:r].double()
+            x[..., :r // 2] = (lo * cos - hi * sin).to(x.dtype)
+            x[..., r // 2:r] = (hi * cos + lo * sin).to(x.dtype)
+
+
+@dataclasses.dataclass(frozen=True)
+class Toy2Config:
+    vocab_size: int
+    hidden_size: int
+    num_experts: int
+    theta: float
+    eps: float
+    architecture: str = "Toy2ForCausalLM"
+
+    @classmethod
+    def from_dict(cls, raw, where="config.json"):
+        return cls(raw["vocab_size"], raw["hidden_size"], raw["num_experts"], raw["theta"], raw["eps"])
+
+    def to_dict(self):
+        return {"architectures": [self.architecture], **dataclasses.asdict(self)}
+
+
+def toy2_spec(cfg):
+    h = cfg.hidden_size
+    norm = lambda n: PartSpec("rmsnorm", dict(size=h, eps=cfg.eps), dict(weight=n))
+    block = BlockSpec(
+        "prenorm",
+        mixer=PartSpec("gqa_attention",
+                       dict(hidden_size=h, num_heads=2, num_kv_heads=2, head_dim=h // 2, qkv_bias=False,
+                            position=PartSpec("toy_half_rotary", dict(dim=h // 2, theta=cfg.theta)), window=None),
+                       dict(q_weight="q", k_weight="k", v_weight="v", o_weight="o")),
+        feed_forward=PartSpec("toy_top_one_experts", dict(hidden_size=h, num_experts=cfg.num_experts),
+                              dict(router="router", experts="expert")),
+        norm1=norm("n1"), norm2=norm("n2"), params=dict(hidden_size=h))
+    sizes = dict(vocab_size=cfg.vocab_size, hidden_size=h)
+    return ModelSpec("Toy2ForCausalLM", cfg.vocab_size, h, 4096,
+                     PartSpec("token_embedding", sizes, dict(weight="embed")), (block,),
+                     (ScheduleEntry(0),), norm("final"), PartSpec("linear_head", sizes, dict(weight="head")))
+
+
+def toy2_plain(ids, w, cfg):
+    h, t = cfg.hidden_size, len(ids)
+    d, r = h // 2, h // 4
+    x = w["embed"][torch.tensor(ids)]
+    n = P.rms_norm(x, w["n1"], cfg.eps)
+    q, k, v = (P.linear(n, w[s]).view(t, 2, d) for s in "qkv")
+    inv = 1.0 / (cfg.theta ** (torch.arange(0, r, 2, dtype=torch.float64) / r))
+    ang = torch.arange(t, dtype=torch.float64)[:, None] * inv[None, :]
+    cos, sin = ang.cos()[:, None, :], ang.sin()[:, None, :]
+    def rot(y):
+        y = y.clone()
+        lo, hi = y[..., :r // 2].clone(), y[..., r // 2:r].clone()
+        y[..., :r // 2], y[..., r // 2:r] = lo * cos - hi * sin, hi * cos + lo * sin
+        return y
+    a = P.causal_attention_dense(rot(q), rot(k), v, torch.arange(t)).reshape(t, h)
+    x = x + P.linear(a, w["o"])
+    n = P.rms_norm(x, w["n2"], cfg.eps)
+    probs = torch.softmax(P.linear(n, w["router"]), dim=-1)
+    weight, choice = probs.max(dim=-1)
+    y = torch.stack([P.linear(n[i:i + 1], w[f"expert.{int(choice[i])}"])[0] * weight[i] for i in range(t)])
+    x = x + y
+    return P.linear(P.rms_norm(x, w["final"], cfg.eps), w["head"])
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_toy_routed_feed_forward_and_other_position_encoding(dtype):
+    """A feed-forward with routing and a position encoding of another kind, both
+    defined here, are registered, built into an architecture and stepped in every
+    cut without a change to the framework's files."""
+    register_part("feed_forward", "toy_top_one_experts", TopOneExperts, replace=True)
+    register_part("position", "toy_half_rotary", HalfRotary, replace=True)
+    register_architecture("Toy2ForCausalLM", Toy2Config, toy2_spec, replace=True)
+    try:
+        cfg = Toy2Config(vocab_size=61, hidden_size=64, num_experts=3, theta=100.0, eps=1e-6)
+        from llm_inference_lab_amd.engine.model import CausalLM
+        from llm_inference_lab_amd.weights import random_tensors
+        tensors = dict(random_tensors(CausalLM(toy2_spec(cfg)).tensor_specs(), 5, torch.bfloat16,
+                                      is_norm=lambda n: n in ("n1", "n2", "final")))
+        for n in ("embed", "q", "k"):
+            tensors[n] = (tensors[n].float() * 8).to(torch.bfloat16)
+        # a decisive router: the best expert wins by a margin that bfloat16 rounding cannot turn
+        tensors["router"] = (tensors["router"].float() * 40).to(torch.bfloat16)
+        engine = H.lab.Engine(config=cfg, tensors=tensors.items(), dtype=dtype, page_size=16, num_pages=16,
+                              max_requests=3, max_batch_tokens=128, max_seq_len=256)
+        g = torch.Generator().manual_seed(1)
+        seqs = {f"r{i}": torch.randint(0, 61, (n,), generator=g).tolist() for i, n in enumerate([40, 70, 19])}
+        w64 = {k: v.double() for k, v in tensors.items()}
+        want = {rid: toy2_plain(ids, w64, cfg) for rid, ids in seqs.items()}
+        for steps in (H.steps_whole(seqs), H.steps_portions(seqs), H.steps_mixed(seqs, seed=3, max_live=3)):
+            got = H.run_trace(engine, seqs, steps)
+            bad = H.first_wrong(got, want, H.TOL[dtype])
+            assert bad is None, f"first wrong logits at (request, position, error) = {bad}"
+    finally:
+        unregister_part("feed_forward", "toy_top_one_experts")
+        unregister_part("position", "toy_half_rotary")
+        unregister_architecture("Toy2ForCausalLM")
