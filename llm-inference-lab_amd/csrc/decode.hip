@@ -37,7 +37,7 @@
 
 #include "common.h"
 
-enum { SK_STORE = 0, SK_RESID = 1, SK_F32 = 2, SK_SWIGLU = 3, SK_QKV = 4 };
+enum { SK_STORE = 0, SK_RESID = 1, SK_F32 = 2, SK_SWIGLU = 3, SK_QKV = 4, SK_PART = 5 };
 
 struct SkinnyArgs {
   const void* x;        // NORM: float32 rows of the residual stream; else bfloat16 [M, K]
@@ -59,6 +59,16 @@ struct SkinnyArgs {
   int qsplit;   // QKV: blocks per head (1, or d/32: a block then owns the strips p and p + d/32)
   int nq, nkv, d, table_stride, page_size;
   float eps;
+  // Sums that a former product left in pieces (SK_PART) and that still belong to the
+  // float32 rows this kernel reads (NORM) or adds into (RESID): pend[s][row][pend_ld],
+  // s < pend_splits, added in the order of s.
+  const float* pend;
+  int pend_splits, pend_ld;
+  size_t pend_stride;
+  // SK_PART: K is split over `ksplit` groups of blocks as well; group s leaves its sums
+  // (no residual, bias in group 0) in out[s][M][ldo], part_stride numbers apart.
+  int ksplit;
+  size_t part_stride;
 };
 
 __device__ __forceinline__ float sk_silu(float z) { return z / (1.f + __expf(-z)); }
@@ -99,7 +109,11 @@ __global__ __launch_bounds__(MB >= 4 ? 512 : 1024) void skinny_block_kernel(Skin
   const int strip = wave % nsb, ks = wave / nsb;
   const int c = lane & 15, g = lane >> 4;
   const int cols = 16 * nsb;
-  const int n0 = blockIdx.x * cols;
+  // SK_PART: the blocks of one K group follow each other
+  const int nblk = (EPI == SK_PART) ? (int)gridDim.x / a.ksplit : (int)gridDim.x;
+  const int ksp = (EPI == SK_PART) ? (int)blockIdx.x / nblk : 0;
+  const int bidx = (EPI == SK_PART) ? (int)blockIdx.x - ksp * nblk : (int)blockIdx.x;
+  const int n0 = bidx * cols;
   const int K = a.K, M = a.M;
   const int steps = (K + 31) >> 5;      // K steps of 32; W is packed and zero-padded to this
 
@@ -117,8 +131,8 @@ __global__ __launch_bounds__(MB >= 4 ? 512 : 1024) void skinny_block_kernel(Skin
   // d/2 + p*16.. of the head, i.e. both halves of the rotary pairs
   int qhead = 0, qp = 0;
   if constexpr (EPI == SK_QKV) {
-    qhead = blockIdx.x / a.qsplit;
-    qp = blockIdx.x - qhead * a.qsplit;
+    qhead = bidx / a.qsplit;
+    qp = bidx - qhead * a.qsplit;
   }
   auto head_col = [&](int col) {   // column of the block -> column of the head
     if (a.qsplit == 1) return col;
@@ -126,19 +140,22 @@ __global__ __launch_bounds__(MB >= 4 ? 512 : 1024) void skinny_block_kernel(Skin
   };
   // the strip of 16 weight rows this wave multiplies (past the last one: the last
   // one again, and what comes of it is dropped by the epilogue)
-  int wstrip = (EPI == SK_QKV) ? (qhead * a.d + head_col(strip * 16)) >> 4 : blockIdx.x * nsb + strip;
+  int wstrip = (EPI == SK_QKV) ? (qhead * a.d + head_col(strip * 16)) >> 4 : bidx * nsb + strip;
   wstrip = min(wstrip, ((a.N + 15) >> 4) - 1);
   const bf16_t* wp = a.W + (size_t)wstrip * steps * 512 + lane * 8;
-  const int per = (steps + kw - 1) / kw;
-  const int s_begin = ks * per;
-  const int s_end = min(steps, s_begin + per);
+  // this block's K steps (all of them, or its group's share), split over its waves
+  const int gsteps = (EPI == SK_PART) ? (steps + a.ksplit - 1) / a.ksplit : steps;
+  const int g_begin = ksp * gsteps, g_end = min(steps, g_begin + gsteps);
+  const int per = (max(g_end - g_begin, 0) + kw - 1) / kw;
+  const int s_begin = g_begin + ks * per;
+  const int s_end = min(g_end, s_begin + per);
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
   const floatx4 fzero = {0.f, 0.f, 0.f, 0.f};
 
   // ---- what the epilogue needs from global memory, fetched now
   for (int i = threadIdx.x; i < cols; i += blockDim.x) {
     const int nn = (EPI == SK_QKV) ? qhead * a.d + head_col(i) : n0 + i;
-    s_bias[i] = (a.bias && nn < a.N) ? load_vec(a.bias, a.bias_bf16, nn) : 0.f;
+    s_bias[i] = (a.bias && nn < a.N && ksp == 0) ? load_vec(a.bias, a.bias_bf16, nn) : 0.f;
   }
   if constexpr (EPI == SK_QKV) {
     const int head = qhead;
@@ -158,7 +175,11 @@ __global__ __launch_bounds__(MB >= 4 ? 512 : 1024) void skinny_block_kernel(Skin
   if constexpr (EPI == SK_RESID) {
     const int idx = threadIdx.x;
     const int m = idx / cols, nn = n0 + idx - m * cols;
-    if (idx < M * cols && nn < a.N) resid_old = ((const float*)a.out)[(size_t)m * a.ldo + nn];
+    if (idx < M * cols && nn < a.N) {
+      resid_old = ((const float*)a.out)[(size_t)m * a.ldo + nn];
+      for (int sp = 0; sp < a.pend_splits; ++sp)
+        resid_old += a.pend[sp * a.pend_stride + (size_t)m * a.pend_ld + nn];
+    }
   }
 
   floatx4 acc[MB];
@@ -181,8 +202,14 @@ __global__ __launch_bounds__(MB >= 4 ? 512 : 1024) void skinny_block_kernel(Skin
       if constexpr (NORM) {
         const float* src = (const float*)a.x + (size_t)(a.x_rows ? a.x_rows[r] : r) * K;
         float ssq = 0.f;
+        const size_t prow = (size_t)(a.x_rows ? a.x_rows[r] : r) * a.pend_ld;
         for (int ch = lane; ch < chunks; ch += 64) {
-          const floatx4 p = *(const floatx4*)(src + ch * 8), q = *(const floatx4*)(src + ch * 8 + 4);
+          floatx4 p = *(const floatx4*)(src + ch * 8), q = *(const floatx4*)(src + ch * 8 + 4);
+          for (int sp = 0; sp < a.pend_splits; ++sp) {       // sums still owed to these rows
+            const float* pp = a.pend + sp * a.pend_stride + prow + ch * 8;
+            p += *(const floatx4*)pp;
+            q += *(const floatx4*)(pp + 4);
+          }
           float wv[8];
           if (a.norm_w_bf16) {
             const bf16x8 w8 = *(const bf16x8*)((const bf16_t*)a.norm_w + ch * 8);
@@ -308,8 +335,18 @@ __global__ __launch_bounds__(MB >= 4 ? 512 : 1024) void skinny_block_kernel(Skin
     } else if (nn < a.N) {
       const size_t at = (size_t)m * a.ldo + nn;
       if (EPI == SK_STORE) ((bf16_t*)a.out)[at] = (bf16_t)sum;
-      else if (EPI == SK_RESID) ((float*)a.out)[at] = (idx == (int)threadIdx.x ? resid_old : ((float*)a.out)[at]) + sum;
-      else ((float*)a.out)[at] = sum;
+      else if (EPI == SK_RESID) {
+        float old = resid_old;
+        if (idx != (int)threadIdx.x) {
+          old = ((float*)a.out)[at];
+          for (int sp = 0; sp < a.pend_splits; ++sp) old += a.pend[sp * a.pend_stride + (size_t)m * a.pend_ld + nn];
+        }
+        ((float*)a.out)[at] = old + sum;
+      } else if (EPI == SK_PART) {
+        ((float*)a.out)[ksp * a.part_stride + at] = sum;
+      } else {
+        ((float*)a.out)[at] = sum;
+      }
     }
   }
   if constexpr (EPI == SK_SWIGLU) {
@@ -430,8 +467,9 @@ struct SkinnyShape {
 // its share of W and of x (a unit sustains far less than 1/256 of the chip's
 // bandwidth would suggest, so spreading the matrix over all units matters most),
 // or the memory round trips of a wave if those take longer.
-static SkinnyShape skinny_choose(int epilogue, bool norm, int mb, int M, int N, int K, int d, int num_cus) {
-  const int steps = (K + 31) / 32;
+static SkinnyShape skinny_choose(int epilogue, bool norm, int mb, int M, int N, int K, int d, int num_cus,
+                                 int ksplit = 1) {
+  const int steps = ((K + 31) / 32 + ksplit - 1) / ksplit;     // per K group of blocks
   const int strips = (N + 15) / 16;
   const int max_waves = mb >= 4 ? 8 : 16;
   SkinnyShape best{0, 0, false, 1};
@@ -447,11 +485,11 @@ static SkinnyShape skinny_choose(int epilogue, bool norm, int mb, int M, int N, 
     const int nsb = cand[ci];
     if (nsb > max_waves) continue;
     for (int kw = 1; kw * nsb <= max_waves && kw <= steps; ++kw) {
-      for (int st = norm ? 1 : 0; st < 2; ++st) {
+      for (int st = norm ? 1 : 0; st < (epilogue == SK_PART ? 1 : 2); ++st) {     // pieces of K: no staging
         const bool stage = st == 1;
         const size_t lds = skinny_lds_bytes(nsb, kw, mb, M, K, epilogue, stage);
         if (lds > SK_LDS_LIMIT) continue;
-        const int blocks = (strips + nsb - 1) / nsb;     // (for QKV: heads, or heads * d/32)
+        const int blocks = (strips + nsb - 1) / nsb * ksplit;     // (for QKV: heads, or heads * d/32)
         const int per_cu = (blocks + num_cus - 1) / num_cus;       // blocks the busiest unit runs
         int resident = 16 / (nsb * kw);                             // of which so many at a time
         if (resident > per_cu) resident = per_cu;
@@ -488,16 +526,31 @@ static SkinnyShape skinny_choose(int epilogue, bool norm, int mb, int M, int N, 
 // One entry point for the whole family.
 //   norm != 0: x is the float32 residual stream (rows x_rows[m] or m), norm_w/eps its RMSNorm
 //   epilogue SK_QKV: N = (nq + 2 nkv) * d, one block per head, `out` is q [M, ldo]
+//   epilogue SK_PART: K is split over `ksplit` groups of blocks, `out` is float32
+//     [ksplit][M][ldo] (part_stride numbers from one piece to the next); nothing is added up
+//   pend / pend_splits / pend_ld / pend_stride: pieces that a former SK_PART call left and
+//     that belong to the rows of x (norm != 0: added while the rows are read) or to the
+//     rows of out (SK_RESID: added with the product, which folds them into the stream)
 extern "C" int llmlab_skinny_linear(const void* x, int norm, const int* x_rows, const void* norm_w,
                                     int norm_w_dtype, float eps, const void* w, const void* bias,
                                     int bias_dtype, int epilogue, void* out, int M, int N, int K,
                                     int ldo, int n_out, const float* inv_freq, const int* positions,
                                     const int* row_req, const int* table, int table_stride,
                                     int page_size, void* kcache, void* vcache, int nq, int nkv, int d,
-                                    int num_cus, hipStream_t stream) {
+                                    int num_cus, const float* pend, int pend_splits, int pend_ld,
+                                    size_t pend_stride, int ksplit, size_t part_stride,
+                                    hipStream_t stream) {
   LLMLAB_REQUIRE(M >= 0 && M <= 64, "skinny_linear: takes at most 64 rows, got %d", M);
   LLMLAB_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "skinny_linear: bad sizes N=%d K=%d (K must be a multiple of 8)", N, K);
-  LLMLAB_REQUIRE(epilogue >= 0 && epilogue <= 4, "skinny_linear: unknown epilogue %d", epilogue);
+  LLMLAB_REQUIRE(epilogue >= 0 && epilogue <= 5, "skinny_linear: unknown epilogue %d", epilogue);
+  LLMLAB_REQUIRE(pend_splits >= 0 && (pend_splits == 0 || (pend != nullptr && (norm || epilogue == SK_RESID))),
+                 "skinny_linear: pending sums go with a norm or into the residual");
+  LLMLAB_REQUIRE(pend_splits == 0 || !norm ||
+                 (pend_ld % 4 == 0 && (uintptr_t)pend % 16 == 0 && pend_stride % 4 == 0),
+                 "skinny_linear: pending sums under a norm are read 16 bytes at a time: not aligned");
+  if (epilogue != SK_PART) ksplit = 1;
+  LLMLAB_REQUIRE(ksplit >= 1 && ksplit <= 16 && (epilogue != SK_PART || (!norm && part_stride >= (size_t)M * ldo)),
+                 "skinny_linear(pieces): bad split %d", ksplit);
   LLMLAB_REQUIRE(((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0) &&
                  (norm_w == nullptr || (uintptr_t)norm_w % 16 == 0),
                  "skinny_linear: operands must be 16-byte aligned");
@@ -520,22 +573,24 @@ extern "C" int llmlab_skinny_linear(const void* x, int norm, const int* x_rows, 
     LLMLAB_REQUIRE(n_out == N, "skinny_linear: n_out %d != N %d", n_out, N);
   }
   LLMLAB_REQUIRE(ldo >= (epilogue == SK_QKV ? nq * d : n_out), "skinny_linear: output stride too small");
-  SkinnyShape shape = skinny_choose(epilogue, norm != 0, mb, M, N, K, d, num_cus);
+  SkinnyShape shape = skinny_choose(epilogue, norm != 0, mb, M, N, K, d, num_cus, ksplit);
   if (g_force_nsb > 0 && epilogue != SK_QKV) shape.nsb = g_force_nsb;
   if (g_force_nsb > 0 && epilogue == SK_QKV && d % 32 == 0 && d > 32) {
     shape.nsb = g_force_nsb == 2 ? 2 : d / 16;
     shape.qsplit = g_force_nsb == 2 ? d / 32 : 1;
   }
   if (g_force_kw > 0) shape.kw = g_force_kw;
-  if (g_force_stage >= 0) shape.stage = norm || g_force_stage != 0;
+  if (g_force_stage >= 0) shape.stage = norm || (g_force_stage != 0 && epilogue != SK_PART);
   LLMLAB_REQUIRE(shape.nsb > 0 && shape.kw > 0,
                  "skinny_linear: no block shape fits N=%d K=%d M=%d (rows of x to stage: %zu bytes of LDS)",
                  N, K, M, (size_t)M * ((K + 31) / 32 * 32 + SK_APAD) * sizeof(bf16_t));
   const size_t lds = skinny_lds_bytes(shape.nsb, shape.kw, mb, M, K, epilogue, shape.stage);
   LLMLAB_REQUIRE(lds <= SK_LDS_LIMIT && shape.nsb * shape.kw <= (mb >= 4 ? 8 : 16),
                  "skinny_linear: block shape %dx%d does not fit", shape.nsb, shape.kw);
-  const int blocks = (N + 16 * shape.nsb - 1) / (16 * shape.nsb);
+  const int blocks = (N + 16 * shape.nsb - 1) / (16 * shape.nsb) * ksplit;
   SkinnyArgs a;
+  a.pend = pend; a.pend_splits = pend_splits; a.pend_ld = pend_ld; a.pend_stride = pend_stride;
+  a.ksplit = ksplit; a.part_stride = part_stride;
   a.qsplit = shape.qsplit;
   a.x = x; a.x_rows = x_rows; a.norm_w = norm_w; a.W = (const bf16_t*)w; a.bias = bias; a.out = out;
   a.inv_freq = inv_freq; a.positions = positions; a.row_req = row_req; a.table = table;
@@ -558,6 +613,7 @@ extern "C" int llmlab_skinny_linear(const void* x, int norm, const int* x_rows, 
       case SK_RESID: rc = skinny_launch_stage<SK_RESID, false>(a, shape.stage, mb, blocks, lds, stream); break;
       case SK_F32: rc = skinny_launch_stage<SK_F32, false>(a, shape.stage, mb, blocks, lds, stream); break;
       case SK_SWIGLU: rc = skinny_launch_stage<SK_SWIGLU, false>(a, shape.stage, mb, blocks, lds, stream); break;
+      case SK_PART: rc = skinny_launch_stage<SK_PART, false>(a, false, mb, blocks, lds, stream); break;
       default: LLMLAB_REQUIRE(false, "skinny_linear: epilogue %d needs the norm", epilogue);
     }
   }

@@ -4,7 +4,7 @@
 
 extern "C" const char* llmlab_last_error() { return g_llmlab_error; }
 
-extern "C" int llmlab_abi_version() { return 2; }
+extern "C" int llmlab_abi_version() { return 3; }
 
 // --------------------------------------------------------------- embedding
 // out[r, :] = float(table[ids[r], :]); an id outside [0, vocab) is clamped (the
@@ -285,5 +285,29 @@ extern "C" int llmlab_pack_weight(const void* src, void* dst, int N, int K, hipS
   hipLaunchKernelGGL(pack_weight_kernel, dim3((unsigned)((chunks + 255) / 256)), dim3(256), 0, stream,
                      (const bf16_t*)src, (bf16_t*)dst, N, K, tiles, chunks);
   LLMLAB_LAUNCH_CHECK("pack_weight");
+  return 0;
+}
+
+// ------------------------------------------------------------ pending sums
+// x[r, :] += sum_s pend[s][r, :], s in order: folds what a product left in pieces
+// into the float32 residual stream (for consumers that cannot add it on the fly).
+__global__ __launch_bounds__(256) void add_pending_kernel(float* __restrict__ x, const float* __restrict__ pend,
+                                                           int splits, size_t stride, long count) {
+  const long i = (long)blockIdx.x * 256 + threadIdx.x;
+  if (i >= count) return;
+  float v = x[i];
+  for (int s = 0; s < splits; ++s) v += pend[s * stride + i];
+  x[i] = v;
+}
+
+extern "C" int llmlab_add_pending(float* x, const float* pend, int splits, size_t stride, int rows,
+                                  int width, hipStream_t stream) {
+  LLMLAB_REQUIRE(rows >= 0 && width > 0 && splits >= 0 && stride >= (size_t)rows * width,
+                 "add_pending: bad sizes rows=%d width=%d splits=%d", rows, width, splits);
+  if (rows == 0 || splits == 0) return 0;
+  const long count = (long)rows * width;
+  hipLaunchKernelGGL(add_pending_kernel, dim3((unsigned)((count + 255) / 256)), dim3(256), 0, stream, x, pend,
+                     splits, stride, count);
+  LLMLAB_LAUNCH_CHECK("add_pending");
   return 0;
 }

@@ -128,10 +128,12 @@ class CausalLM:
         logits ``[wanted, vocab]`` for ``ctx.want_rows`` (None if none wanted)."""
         rows, hidden = ctx.n_rows, self.spec.hidden_size
         x = ctx.scratch("model.residual", (rows, hidden), torch.float32)
+        ctx.pending = None         # sums a product leaves in pieces for the next reader of x
         self.embedding.forward(ctx.token_ids, x)
         for view in self.entries:
             self.blocks[view.block].forward(x, ctx, view)
         if ctx.n_want == 0:
+            ctx.pending = None
             return None
         h = NormedInput(self.final_norm, x, ctx, "model.final_normed", self.dtype,
                         rows=ctx.want_rows, n_rows=ctx.n_want)

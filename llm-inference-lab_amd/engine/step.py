@@ -90,6 +90,7 @@ class StepContext:
         self.scratch_version = 0
         self.n_rows = self.n_reqs = self.n_want = 0
         self.max_q_len = self.max_ctx_len = 0
+        self.pending = None            # PendingSums owed to the residual stream, within a forward
         self.host_q_start: List[int] = []
         self.host_start_pos: List[int] = []
         self.host_req_rows: List[int] = []

@@ -15,10 +15,11 @@ from typing import Dict, Optional
 import torch
 
 from ..config.errors import UnsupportedSizeError
+from ..parts.base import PendingSums
 from . import build
 
 DT_F32, DT_BF16 = 0, 1
-EPI_STORE, EPI_RESID, EPI_F32, EPI_SWIGLU, EPI_QKV = 0, 1, 2, 3, 4
+EPI_STORE, EPI_RESID, EPI_F32, EPI_SWIGLU, EPI_QKV, EPI_PART = 0, 1, 2, 3, 4, 5
 
 _c_int, _c_long, _c_float, _c_size, _c_ptr = (ctypes.c_int, ctypes.c_long, ctypes.c_float,
                                               ctypes.c_size_t, ctypes.c_void_p)
@@ -77,7 +78,7 @@ class HipOps:
         torch.cuda.set_device(self.device)
         self._core = self._load(build.core_library())
         self._declare_core()
-        if self._core.llmlab_abi_version() != 2:
+        if self._core.llmlab_abi_version() != 3:
             raise RuntimeError("kernel library and Python bindings disagree on the interface")
         self._attn: Dict[int, ctypes.CDLL] = {}
         self._shared: Dict[int, tuple] = {}
@@ -119,7 +120,10 @@ class HipOps:
         c.llmlab_skinny_linear.argtypes = [
             _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_float, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr,
             _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
-            _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr]
+            _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int,
+            _c_ptr, _c_int, _c_int, _c_size, _c_int, _c_size, _c_ptr]
+        c.llmlab_add_pending.argtypes = [_c_ptr, _c_ptr, _c_int, _c_size, _c_int, _c_int, _c_ptr]
+        c.llmlab_add_pending.restype = _c_int
         for fn in (c.llmlab_embed, c.llmlab_rmsnorm, c.llmlab_rope_kv_write, c.llmlab_rope_inplace,
                    c.llmlab_linear, c.llmlab_sample, c.llmlab_skinny_linear):
             fn.restype = _c_int
@@ -272,7 +276,7 @@ class HipOps:
                                               self._stream()))
 
     # ----------------------------------------------------------------- linear
-    def _linear(self, x, w, out, bias, epilogue, n_out) -> None:
+    def _linear(self, x, w, out, bias, epilogue, n_out, pending: Optional[PendingSums] = None) -> None:
         self._need(x, "linear input")
         w = self._weight(w, "linear weight")
         if x.dtype != w.dtype:
@@ -298,8 +302,11 @@ class HipOps:
         # few rows: the block kernel that splits K inside a block; from 17 rows on only
         # for narrow outputs (the tiled kernel has too few tiles there), measured
         if x.dtype == torch.bfloat16 and (m <= 16 or (m <= self.skinny_max_rows and n < 8192)):
-            self._skinny(x, False, None, None, 0.0, w, bias, epilogue, out, m, n, k, ldo, n_out)
+            self._skinny(x, False, None, None, 0.0, w, bias, epilogue, out, m, n, k, ldo, n_out,
+                         pending=pending)
             return
+        if pending is not None:
+            self.add_pending(out, pending)
         self._check(self._core.llmlab_linear(
             self._ptr(x), self._ptr(w), _dt(x), epilogue, self._ptr(out), self._ptr(bias),
             _dt(bias) if bias is not None else 0, m, n, k, ldo, n_out, self.num_cus, self._stream()))
@@ -307,8 +314,9 @@ class HipOps:
     def linear(self, x, w, out, bias=None) -> None:
         self._linear(x, w, out, bias, EPI_STORE, w.shape[0])
 
-    def linear_residual(self, x, w, resid, bias=None) -> None:
-        self._linear(x, w, resid, bias, EPI_RESID, w.shape[0])
+    def linear_residual(self, x, w, resid, bias=None, pending: Optional[PendingSums] = None) -> None:
+        """``resid += x w^T (+ bias)``, and the pending pieces of ``resid`` with it."""
+        self._linear(x, w, resid, bias, EPI_RESID, w.shape[0], pending)
 
     def linear_logits(self, x, w, out) -> None:
         self._linear(x, w, out, None, EPI_F32, w.shape[0])
@@ -336,9 +344,21 @@ class HipOps:
         return rows * ((inner + 31) // 32 * 32 + 8) * 2 <= self.STAGE_BYTES
 
     def _skinny(self, x, norm, x_rows, norm_w, eps, w, bias, epilogue, out, m, n, k, ldo, n_out,
-                qkv=None) -> None:
+                qkv=None, pending: Optional[PendingSums] = None, ksplit: int = 1,
+                part_stride: int = 0) -> None:
         q = qkv or {}
         table = q.get("table")
+        if pending is not None:
+            p = pending.parts
+            if (p.dtype != torch.float32 or p.dim() != 3 or p.stride(2) != 1 or p.device != self.device
+                    or pending.splits > p.shape[0]):
+                raise ValueError("pending sums: float32 [splits, rows, width] on the GPU expected")
+            width = x.shape[1] if norm else n
+            if p.shape[2] != width:
+                raise ValueError(f"pending sums are {p.shape[2]} wide, the rows they belong to {width}")
+            pend = (self._ptr(p), pending.splits, p.stride(1), p.stride(0))
+        else:
+            pend = (_c_ptr(0), 0, 0, 0)
         self._check(self._core.llmlab_skinny_linear(
             self._ptr(x), 1 if norm else 0, self._ptr(x_rows), self._ptr(norm_w),
             _dt(norm_w) if norm_w is not None else 0, float(eps), self._ptr(w), self._ptr(bias),
@@ -346,7 +366,51 @@ class HipOps:
             self._ptr(q.get("inv_freq")), self._ptr(q.get("positions")), self._ptr(q.get("row_req")),
             self._ptr(table), table.stride(0) if table is not None else 0, q.get("page_size", 0),
             self._ptr(q.get("k_cache")), self._ptr(q.get("v_cache")), q.get("nq", 0), q.get("nkv", 0),
-            q.get("d", 0), self.num_cus, self._stream()))
+            q.get("d", 0), self.num_cus, pend[0], pend[1], pend[2], pend[3], int(ksplit),
+            int(part_stride), self._stream()))
+
+    # --------------------------------------------- sums left in pieces (deferred)
+    MAX_SPLITS = 8
+    min_steps_per_split = 8       # K steps of 32 a piece should have at least (tests lower it)
+
+    def split_count(self, rows: int, dtype, n: int, k: int) -> int:
+        """Into how many pieces along the inner size a few-row product ``[rows, k] x
+        [n, k]^T`` should be cut so that it spreads over the chip: a narrow output
+        gives too few blocks otherwise, and a compute unit draws only so much from
+        memory.  1: do not cut."""
+        if dtype != torch.bfloat16 or not 0 < rows <= self.fuse_max_rows:
+            return 1
+        strips, steps = (n + 15) // 16, (k + 31) // 32
+        want = self.num_cus // max(strips, 1)
+        return max(1, min(want, steps // self.min_steps_per_split, self.MAX_SPLITS))
+
+    def linear_partials(self, x, w, parts: torch.Tensor, splits: int, bias=None) -> PendingSums:
+        """``parts[s] = x[:, K_s] w[:, K_s]^T`` for the ``splits`` pieces ``K_s`` of the inner
+        size (bias in piece 0): the product without the final sum."""
+        self._need(x, "linear input", torch.bfloat16)
+        w = self._weight(w, "linear weight")
+        m, k = x.shape
+        n = w.shape[0]
+        if (w.shape[1] != k or parts.dtype != torch.float32 or parts.dim() != 3 or parts.shape[0] < splits
+                or parts.shape[1] != m or parts.shape[2] != n or parts.stride(2) != 1
+                or parts.device != self.device):
+            raise ValueError(f"linear_partials: x {tuple(x.shape)}, w {tuple(w.shape)}, "
+                             f"parts {tuple(parts.shape)} for {splits} pieces do not fit")
+        if not 1 <= splits <= self.MAX_SPLITS or m > self.fuse_max_rows:
+            raise ValueError(f"linear_partials: {splits} pieces of {m} rows")
+        self._skinny(x, False, None, None, 0.0, w, bias, EPI_PART, parts, m, n, k, parts.stride(1), n,
+                     ksplit=splits, part_stride=parts.stride(0))
+        return PendingSums(parts, splits)
+
+    def add_pending(self, x: torch.Tensor, pending: PendingSums) -> None:
+        """``x += sum_s parts[s]``: fold the pieces into the float32 stream."""
+        self._need(x, "residual stream", torch.float32)
+        p = pending.parts
+        rows, width = x.shape
+        if p.shape[1] != rows or p.shape[2] != width or not p[0].is_contiguous():
+            raise ValueError("add_pending: pieces and stream differ in shape")
+        self._check(self._core.llmlab_add_pending(self._ptr(x), self._ptr(p), pending.splits, p.stride(0),
+                                                  rows, width, self._stream()))
 
     def _fused_common(self, x, norm_w, w, rows):
         self._need(x, "residual stream", torch.float32)
@@ -366,9 +430,11 @@ class HipOps:
         return w, k
 
     def fused_norm_qkv(self, x, norm_w, eps, w_qkv, b_qkv, num_heads, num_kv_heads, head_dim, inv_freq,
-                       positions, row_req, block_table, page_size, k_cache, v_cache, q_out) -> None:
+                       positions, row_req, block_table, page_size, k_cache, v_cache, q_out,
+                       pending: Optional[PendingSums] = None) -> None:
         """q_out = rotate(norm(x) Wq^T + bq); rotated k and v of the new positions go to
-        their pages (skipped when no cache is given)."""
+        their pages (skipped when no cache is given).  ``pending``: pieces still owed to
+        the rows of x, added while they are read (x itself is left as it is)."""
         rows = x.shape[0]
         w_qkv, k = self._fused_common(x, norm_w, w_qkv, rows)
         n = (num_heads + 2 * num_kv_heads) * head_dim
@@ -396,18 +462,18 @@ class HipOps:
                      q_out.shape[1], n,
                      dict(inv_freq=inv_freq, positions=positions, row_req=row_req, table=block_table,
                           page_size=page_size, k_cache=k_cache, v_cache=v_cache, nq=num_heads,
-                          nkv=num_kv_heads, d=head_dim))
+                          nkv=num_kv_heads, d=head_dim), pending=pending)
 
-    def fused_norm_swiglu(self, x, norm_w, eps, w_gate_up, out) -> None:
+    def fused_norm_swiglu(self, x, norm_w, eps, w_gate_up, out, pending: Optional[PendingSums] = None) -> None:
         rows, inter = out.shape
         w_gate_up, k = self._fused_common(x, norm_w, w_gate_up, rows)
         self._need(out, "SwiGLU output", torch.bfloat16)
         if x.shape[0] != rows or w_gate_up.shape[0] != 2 * ((inter + 15) // 16 * 16):
             raise ValueError("fused_norm_swiglu: shapes do not fit")
         self._skinny(x, True, None, norm_w, eps, w_gate_up, None, EPI_SWIGLU, out, rows,
-                     w_gate_up.shape[0], k, out.shape[1], inter)
+                     w_gate_up.shape[0], k, out.shape[1], inter, pending=pending)
 
-    def fused_norm_logits(self, x, rows_index, norm_w, eps, w, out) -> None:
+    def fused_norm_logits(self, x, rows_index, norm_w, eps, w, out, pending: Optional[PendingSums] = None) -> None:
         """out[i] = norm(x[rows_index[i]]) W^T in float32."""
         rows, vocab = out.shape
         w, k = self._fused_common(x, norm_w, w, rows)
@@ -421,7 +487,7 @@ class HipOps:
         elif x.shape[0] != rows:
             raise ValueError("fused_norm_logits: rows differ")
         self._skinny(x, True, rows_index, norm_w, eps, w, None, EPI_F32, out, rows, vocab, k,
-                     out.shape[1], vocab)
+                     out.shape[1], vocab, pending=pending)
 
     # ------------------------------------------------------------------- rope
     def rope_inplace(self, x, positions, inv_freq) -> None:

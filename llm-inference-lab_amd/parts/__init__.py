@@ -1,5 +1,5 @@
 from .registry import register_part, unregister_part, part_class, build_part, FAMILIES
-from .base import (Part, Norm, NormedInput, PositionEncoding, Mixer, FeedForward, Block,
+from .base import (Part, Norm, NormedInput, PendingSums, PositionEncoding, Mixer, FeedForward, Block,
                    KVCacheSpec)
 from .norms import RMSNorm
 from .positions import RotaryEmbedding, NoPosition

@@ -104,15 +104,20 @@ class GQAAttention(Mixer):
         group = ctx.group(entry.group)
         k_cache = entry.k_cache if entry.writes_cache else None
         v_cache = entry.v_cache if entry.writes_cache else None
-        rms = h.rms() if isinstance(h, NormedInput) else None
-        if (rms is not None and ops.can_fuse(rows, self.dtype, self.hidden_size)
-                and (self.position is None or table is not None)):
+        fuse = (isinstance(h, NormedInput) and ops.can_fuse(rows, self.dtype, self.hidden_size)
+                and (self.position is None or table is not None))
+        rms = h.rms(accept_pending=True) if fuse else None
+        pending = None
+        if rms is not None:
             # few rows: norm, the three projections, bias, rotation and the cache
             # write are one kernel
             q = ctx.scratch("attention.q", (rows, self.q_size), self.dtype)
+            # pieces still owed to the stream are added as its rows are read, and folded
+            # in by the output projection below
+            pending = getattr(ctx, "pending", None)
             ops.fused_norm_qkv(rms[0], rms[2], rms[3], self.w_qkv, self.b_qkv, self.num_heads,
                                self.num_kv_heads, self.head_dim, table, ctx.positions, ctx.row_req,
-                               group.block_table, group.page_size, k_cache, v_cache, q)
+                               group.block_table, group.page_size, k_cache, v_cache, q, pending=pending)
         else:
             if isinstance(h, NormedInput):
                 h = h.tensor()
@@ -132,7 +137,11 @@ class GQAAttention(Mixer):
             entry.k_cache, entry.v_cache, group.block_table, group.page_size,
             ctx.q_start, ctx.start_pos, ctx.n_reqs, ctx.max_q_len, ctx.max_ctx_len,
             self.window, self.scale, out, ctx)
-        ops.linear_residual(out, self.w_o, residual, self.b_o)
+        if pending is not None:
+            ops.linear_residual(out, self.w_o, residual, self.b_o, pending=pending)
+            ctx.pending = None
+        else:
+            ops.linear_residual(out, self.w_o, residual, self.b_o)
 
     def weight_bytes(self):
         total = 0

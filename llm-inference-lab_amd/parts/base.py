@@ -66,6 +66,18 @@ class Norm(Part):
         return None
 
 
+class PendingSums:
+    """Sums that a product left in pieces instead of adding them into the float32
+    residual stream: ``parts[s, r, :]`` for ``s < splits`` belongs to row ``r``.
+    Whoever reads the stream next adds them on the fly, whoever adds into it next
+    folds them in (``HipOps.add_pending`` does it on its own)."""
+
+    __slots__ = ("parts", "splits")
+
+    def __init__(self, parts: torch.Tensor, splits: int):
+        self.parts, self.splits = parts, int(splits)
+
+
 class NormedInput:
     """The input of a mixer, feed-forward or head whose norm has not run yet.
 
@@ -85,15 +97,30 @@ class NormedInput:
     def shape(self):
         return (self.n_rows, self.x.shape[1])
 
-    def rms(self):
-        """``(x, rows, weight, eps)`` for a fused kernel, or None."""
+    def rms(self, accept_pending: bool = False):
+        """``(x, rows, weight, eps)`` for a fused kernel, or None.
+
+        The stream ``x`` may still be owed sums that a former product left in pieces
+        (``ctx.pending``).  A caller that passes ``accept_pending=True`` takes that on:
+        it hands ``ctx.pending`` to its kernels (which add the pieces while they read
+        ``x``, and fold them in where they add into ``x``) and clears it once they
+        are folded.  For every other caller the pieces are folded in here."""
         params = self.norm.rms_params()
         if params is None:
             return None
+        if not accept_pending:
+            self._fold_pending()
         return self.x, self.rows, params[0], params[1]
+
+    def _fold_pending(self) -> None:
+        pending = getattr(self.ctx, "pending", None)
+        if pending is not None:
+            self.norm.ops.add_pending(self.x, pending)
+            self.ctx.pending = None
 
     def tensor(self) -> torch.Tensor:
         if self._tensor is None:
+            self._fold_pending()
             out = self.ctx.scratch(self.name, (self.n_rows, self.x.shape[1]), self.dtype)
             self.norm.forward(self.x, out, self.rows)
             self._tensor = out

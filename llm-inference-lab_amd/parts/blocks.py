@@ -101,9 +101,13 @@ class LinearHead(Part):
     takes_normed_input = True
 
     def forward(self, h, out):
-        rms = h.rms() if isinstance(h, NormedInput) else None
-        if rms is not None and self.ops.can_fuse(out.shape[0], self.dtype, self.hidden_size):
-            self.ops.fused_norm_logits(rms[0], rms[1], rms[2], rms[3], self.weight, out)
+        fuse = isinstance(h, NormedInput) and self.ops.can_fuse(out.shape[0], self.dtype, self.hidden_size)
+        rms = h.rms(accept_pending=True) if fuse else None
+        if rms is not None:
+            # the last reader of the stream: pieces still owed to it are added on the fly
+            pending = getattr(h.ctx, "pending", None)
+            self.ops.fused_norm_logits(rms[0], rms[1], rms[2], rms[3], self.weight, out, pending=pending)
+            h.ctx.pending = None
         else:
             if isinstance(h, NormedInput):
                 h = h.tensor()

@@ -76,7 +76,14 @@ class SwiGLU(FeedForward):
             if isinstance(h, NormedInput):
                 h = h.tensor()
             self.ops.linear_swiglu(h, self.w_gate_up, act)
-        self.ops.linear_residual(act, self.w_down, residual, None)
+        splits = self.ops.split_count(rows, self.dtype, self.hidden_size, self.intermediate_size)
+        if splits > 1 and hasattr(ctx, "pending") and ctx.pending is None:
+            # a narrow output: the product is cut along the inner size so that it spreads
+            # over the chip, and its pieces are left for the next reader of the stream
+            parts = ctx.scratch("swiglu.pieces", (splits, rows, self.hidden_size), torch.float32)
+            ctx.pending = self.ops.linear_partials(act, self.w_down, parts, splits)
+        else:
+            self.ops.linear_residual(act, self.w_down, residual, None)
 
     def weight_bytes(self):
         return sum(w.numel() * w.element_size() for w in (self.w_gate_up, self.w_down))

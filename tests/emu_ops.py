@@ -14,6 +14,7 @@ import math
 import torch
 
 from llm_inference_lab_amd.cache import layout as cache_layout
+from llm_inference_lab_amd.parts import PendingSums
 
 
 class EmuOps:
@@ -58,12 +59,46 @@ class EmuOps:
             y = y + bias.float()
         out.copy_(y.to(out.dtype))
 
-    def linear_residual(self, x, w, resid, bias=None):
+    def linear_residual(self, x, w, resid, bias=None, pending=None):
         self._count("linear_residual")
         y = x.float() @ w.float().t()
         if bias is not None:
             y = y + bias.float()
+        if pending is not None:
+            resid.add_(self._owed(pending))
         resid.add_(y)
+
+    # ---------------------------------------------------- sums left in pieces
+    MAX_SPLITS = 8
+    num_cus = 256
+    min_steps_per_split = 8
+
+    @staticmethod
+    def _owed(pending):
+        return pending.parts[:pending.splits].sum(0) if pending is not None else 0.0
+
+    def split_count(self, rows, dtype, n, k):
+        if not self.fuse or dtype != torch.bfloat16 or not 0 < rows <= self.fuse_max_rows:
+            return 1
+        strips, steps = (n + 15) // 16, (k + 31) // 32
+        return max(1, min(self.num_cus // max(strips, 1), steps // self.min_steps_per_split, self.MAX_SPLITS))
+
+    def linear_partials(self, x, w, parts, splits, bias=None):
+        """Piece s covers the K steps of 32 from s * ceil(steps / splits) on."""
+        self._count("linear_partials")
+        k = x.shape[1]
+        steps = (k + 31) // 32
+        per = (steps + splits - 1) // splits
+        for s in range(splits):
+            lo, hi = min(k, s * per * 32), min(k, (s + 1) * per * 32)
+            parts[s] = x[:, lo:hi].float() @ w[:, lo:hi].float().t()
+        if bias is not None:
+            parts[0] += bias.float()
+        return PendingSums(parts, splits)
+
+    def add_pending(self, x, pending):
+        self._count("add_pending")
+        x.add_(self._owed(pending))
 
     def linear_logits(self, x, w, out):
         self._count("linear_logits")
@@ -93,17 +128,18 @@ class EmuOps:
     def release_shared(self):
         pass
 
-    def _normed(self, x, rows_index, norm_w, eps, n):
-        v = x.float() if rows_index is None else x.float()[rows_index[:n].long()]
+    def _normed(self, x, rows_index, norm_w, eps, n, pending=None):
+        v = x.float() + self._owed(pending)
+        v = v if rows_index is None else v[rows_index[:n].long()]
         inv = torch.rsqrt((v * v).sum(-1, keepdim=True) / v.shape[-1] + eps)
         # the kernel rounds x * w to bfloat16 and scales by inv_rms afterwards
         return (v * norm_w.float()).to(torch.bfloat16).float() * inv
 
     def fused_norm_qkv(self, x, norm_w, eps, w_qkv, b_qkv, num_heads, num_kv_heads, head_dim, inv_freq,
-                       positions, row_req, block_table, page_size, k_cache, v_cache, q_out):
+                       positions, row_req, block_table, page_size, k_cache, v_cache, q_out, pending=None):
         self._count("fused_norm_qkv")
         rows = x.shape[0]
-        y = self._normed(x, None, norm_w, eps, rows) @ w_qkv.float().t()
+        y = self._normed(x, None, norm_w, eps, rows, pending) @ w_qkv.float().t()
         if b_qkv is not None:
             y = y + b_qkv.float()
         qkv = y.clone()                      # float32: the kernel rotates before it rounds
@@ -111,14 +147,14 @@ class EmuOps:
                            block_table, page_size, k_cache, v_cache)
         q_out.copy_(qkv[:, :num_heads * head_dim].to(q_out.dtype))
 
-    def fused_norm_swiglu(self, x, norm_w, eps, w_gate_up, out):
+    def fused_norm_swiglu(self, x, norm_w, eps, w_gate_up, out, pending=None):
         self._count("fused_norm_swiglu")
-        h = self._normed(x, None, norm_w, eps, x.shape[0])
+        h = self._normed(x, None, norm_w, eps, x.shape[0], pending)
         self.linear_swiglu(h, w_gate_up, out)
 
-    def fused_norm_logits(self, x, rows_index, norm_w, eps, w, out):
+    def fused_norm_logits(self, x, rows_index, norm_w, eps, w, out, pending=None):
         self._count("fused_norm_logits")
-        out.copy_(self._normed(x, rows_index, norm_w, eps, out.shape[0]) @ w.float().t())
+        out.copy_(self._normed(x, rows_index, norm_w, eps, out.shape[0], pending) @ w.float().t())
 
     # ------------------------------------------------------------------- rope
     @staticmethod

@@ -58,6 +58,47 @@ def test_few_row_steps_take_the_fused_operations(name, cut):
         assert calls.get("linear_swiglu", 0) > 0    # the long first portions take the general path
 
 
+@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("cut", ["decode", "mixed"])
+def test_sums_left_in_pieces_reach_every_reader(name, cut):
+    """The feed-forward leaves its last product in pieces (threshold lowered so that
+    the tiny models do it); the next reader of the stream adds them, the next product
+    into the stream folds them in, and a step of many rows folds them on its own."""
+    seqs = sequences_of(name)
+    want = {rid: H.plain_logits(name, 1, ids) for rid, ids in seqs.items()}
+    engine = engine_of(name, "bf16", page_size=16, num_pages=14, max_requests=4)
+    engine.ops.min_steps_per_split = 1
+    steps = {"decode": H.steps_prefill_then_decode, "mixed": H.steps_mixed}[cut](seqs)
+    got = H.run_trace(engine, seqs, steps)
+    bad = H.first_wrong(got, want, H.TOL["bf16"])
+    assert bad is None, f"first wrong logits at (request, position, error) = {bad}"
+    calls = engine.ops.calls
+    assert calls["linear_partials"] > 0
+
+
+def test_a_reader_that_cannot_add_pieces_gets_them_folded_in():
+    """``NormedInput.tensor()`` (and ``rms()`` without ``accept_pending``) fold pending
+    sums into the stream before the norm runs, and clear them."""
+    from llm_inference_lab_amd.parts import NormedInput, PendingSums
+    engine = engine_of("A", "bf16", page_size=16, num_pages=4, max_requests=1)
+    norm = engine.model.final_norm
+    ctx = engine.step_fn.ctx
+    x = torch.randn(3, engine.model.spec.hidden_size)
+    parts = torch.randn(2, 3, x.shape[1])
+    for use in ("tensor", "rms"):
+        stream = x.clone()
+        ctx.pending = PendingSums(parts.clone(), 2)
+        h = NormedInput(norm, stream, ctx, "t", torch.bfloat16)
+        getattr(h, use)()
+        assert ctx.pending is None
+        assert torch.allclose(stream, x + parts.sum(0))
+    stream = x.clone()
+    ctx.pending = PendingSums(parts.clone(), 2)
+    NormedInput(norm, stream, ctx, "t", torch.bfloat16).rms(accept_pending=True)
+    assert ctx.pending is not None and torch.equal(stream, x)      # the caller took it on
+    ctx.pending = None
+
+
 def test_pages_are_reused_in_mixed():
     seqs = sequences_of("B", seed=3)
     engine = engine_of("B", "f32", page_size=16, num_pages=10)

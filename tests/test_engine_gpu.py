@@ -46,6 +46,25 @@ def test_every_cut_matches_plain(dtype, name, cut, page_size):
     assert m["rows_used"] == 0 and all(g["pages_used"] == 0 for g in m["groups"])
 
 
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("cut", ["decode", "portions", "mixed"])
+def test_sums_left_in_pieces_reach_every_reader(name, cut):
+    """With the threshold lowered so that the tiny models take that path too, the
+    feed-forward's last product is left in pieces along its inner size, the next
+    layer's q/k/v projection (or the output head) adds them as it reads the stream, and
+    the attention output projection folds them in; steps of more rows fold them with the
+    stand-alone kernel.  Same logits."""
+    seqs = sequences_of(name)
+    want = {rid: H.plain_logits(name, 1, ids) for rid, ids in seqs.items()}
+    engine = H.make_engine(name, 1, "bf16", page_size=16, num_pages=40, max_requests=4)
+    engine.ops.min_steps_per_split = 1
+    cfg = H.config_of(name)
+    assert engine.ops.split_count(4, torch.bfloat16, cfg.hidden_size, cfg.intermediate_size) > 1
+    got = H.run_trace(engine, seqs, CUTS[cut](seqs))
+    bad = H.first_wrong(got, want, H.TOL["bf16"])
+    assert bad is None, f"first wrong logits at (request, position, error) = {bad}"
+
+
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 def test_cuts_agree_with_each_other_more_closely_than_with_plain(dtype):
     """The logits at a position do not depend on how the tokens were cut, beyond rounding."""

@@ -456,3 +456,41 @@ def test_cache_order_round_trip(page, d):
     assert torch.equal(cache_layout.values_from_cache_order(cache_layout.values_to_cache_order(v)), v)
     # a 16-key block is 16 * d consecutive numbers, for keys and for values
     assert int(ki[:16].max()) == 16 * d - 1 and int(vi[:, :16].max()) == 16 * d - 1
+
+
+@pytest.mark.parametrize("m,n,k,splits", [(8, 896, 4864, 4), (1, 896, 896, 3), (16, 90, 512, 2), (5, 130, 264, 1)])
+def test_linear_partials_and_pending(ops, emu, m, n, k, splits):
+    """A product left in pieces along K; the pieces added on the fly where the rows are
+    read (fused norm + product), folded in where a product adds into them, or folded
+    by the stand-alone kernel: each against the same sum done at once."""
+    bf = torch.bfloat16
+    x, w = rnd((m, k), bf, 81), rnd((n, k), bf, 82, 0.1)
+    parts = torch.zeros(ops.MAX_SPLITS, m, n, device=DEV)
+    pending = ops.linear_partials(x.to(DEV), ops.prepare_weight(w.to(DEV)), parts, splits)
+    want_parts = torch.zeros(ops.MAX_SPLITS, m, n)
+    emu.linear_partials(x, w, want_parts, splits)
+    close(parts[:splits], want_parts[:splits], torch.float32, "pieces", want_parts.abs().max().item())
+    whole = x.float() @ w.float().t()
+    close(parts[:splits].sum(0), whole, torch.float32, "sum of pieces", whole.abs().max().item())
+    # stand-alone fold
+    resid = rnd((m, n), torch.float32, 83)
+    got = resid.clone().to(DEV)
+    ops.add_pending(got, pending)
+    close(got, resid + want_parts[:splits].sum(0), torch.float32, "fold", 4.0)
+    # fold with the next product into the same rows
+    x2, w2 = rnd((m, 96), bf, 84), rnd((n, 96), bf, 85, 0.1)
+    got = resid.clone().to(DEV)
+    ops.linear_residual(x2.to(DEV), ops.prepare_weight(w2.to(DEV)), got, pending=pending)
+    want = resid + want_parts[:splits].sum(0) + x2.float() @ w2.float().t()
+    close(got, want, torch.float32, "fold with a product", want.abs().max().item())
+    # added on the fly by a fused norm + product that reads the rows (n must fit the norm: use n wide rows)
+    if n % 8 == 0:
+        nw = (1 + 0.1 * rnd((n,), torch.float32, 86)).to(bf)
+        w3 = rnd((48, n), bf, 87, 0.1)
+        logits = torch.zeros(m, 48, device=DEV)
+        ops.fused_norm_logits(resid.to(DEV), None, nw.to(DEV), 1e-6, ops.prepare_weight(w3.to(DEV)), logits,
+                              pending=pending)
+        want_l = torch.zeros(m, 48)
+        emu.fused_norm_logits(resid, None, nw, 1e-6, w3, want_l,
+                              pending=type(pending)(want_parts, splits))
+        close(logits, want_l, torch.float32, "pending under a fused norm", want_l.abs().max().item() * 4)
