@@ -177,8 +177,14 @@ __global__ __launch_bounds__(MB >= 4 ? 512 : 1024) void skinny_block_kernel(Skin
     const int m = idx / cols, nn = n0 + idx - m * cols;
     if (idx < M * cols && nn < a.N) {
       resid_old = ((const float*)a.out)[(size_t)m * a.ldo + nn];
-      for (int sp = 0; sp < a.pend_splits; ++sp)
-        resid_old += a.pend[sp * a.pend_stride + (size_t)m * a.pend_ld + nn];
+      for (int sp0 = 0; sp0 < a.pend_splits; sp0 += 4) {      // four pieces at a time, as above
+        float pp[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          pp[j] = a.pend[min(sp0 + j, a.pend_splits - 1) * a.pend_stride + (size_t)m * a.pend_ld + nn];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) resid_old += sp0 + j < a.pend_splits ? pp[j] : 0.f;
+      }
     }
   }
 
@@ -205,10 +211,22 @@ __global__ __launch_bounds__(MB >= 4 ? 512 : 1024) void skinny_block_kernel(Skin
         const size_t prow = (size_t)(a.x_rows ? a.x_rows[r] : r) * a.pend_ld;
         for (int ch = lane; ch < chunks; ch += 64) {
           floatx4 p = *(const floatx4*)(src + ch * 8), q = *(const floatx4*)(src + ch * 8 + 4);
-          for (int sp = 0; sp < a.pend_splits; ++sp) {       // sums still owed to these rows
-            const float* pp = a.pend + sp * a.pend_stride + prow + ch * 8;
-            p += *(const floatx4*)pp;
-            q += *(const floatx4*)(pp + 4);
+          // sums still owed to these rows: four pieces at a time, loads unconditional
+          // (past the last piece: the last one again, not added) so that they travel together
+          for (int sp0 = 0; sp0 < a.pend_splits; sp0 += 4) {
+            floatx4 pp[4], qq[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              const float* src2 = a.pend + min(sp0 + j, a.pend_splits - 1) * a.pend_stride + prow + ch * 8;
+              pp[j] = *(const floatx4*)src2;
+              qq[j] = *(const floatx4*)(src2 + 4);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+              const float on = sp0 + j < a.pend_splits ? 1.f : 0.f;
+              p += pp[j] * on;
+              q += qq[j] * on;
+            }
           }
           float wv[8];
           if (a.norm_w_bf16) {
