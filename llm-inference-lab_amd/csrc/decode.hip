@@ -28,8 +28,17 @@
 // of the same read, and inv_rms[m] scales the reduced sums in the epilogue.
 //
 // What the epilogue needs from global memory (bias, positions, page numbers,
-// rotary frequencies) is fetched into LDS at the start of the kernel, so those
-// latencies overlap the weight stream instead of following it.
+// rotary frequencies, the residual value it adds to) is fetched at the start of the
+// kernel, so those latencies overlap the weight stream instead of following it.
+//
+// A compute unit draws only about 50 GB/s from HBM, so a product with a narrow
+// output (few strips, hence few blocks) is bound by the units it uses, not by the
+// chip.  Epilogue SK_PART cuts such a product along K over `ksplit` groups of blocks
+// as well and leaves one piece of the result per group, unsummed: no second kernel
+// and no atomics.  The pieces are owed to the float32 rows they would have been
+// added to; the next kernel that reads those rows (under a fused norm) adds them on
+// the fly in their order, and the next SK_RESID product into those rows folds them
+// in for good (`pend` below).
 //
 // Fragment layout of v_mfma_f32_16x16x32_bf16 (lane l): A row l%16, B column l%16,
 // k = 8*(l/16)..+7; result element i: row 4*(l/16)+i, column l%16.
