@@ -74,6 +74,7 @@ struct AttnArgs {
   int q_stride, out_stride, table_stride, page_size;
   int nq, nkv, window, splits;
   int page_shift;     // log2(page_size); page sizes are powers of two
+  int tiles;          // paired kernel: tiles of rows per request (blocks take two each)
   float scale;
 };
 
@@ -97,8 +98,8 @@ constexpr int SPLIT_FILL = 1;      // blocks per compute unit a decode step aims
 // RING (decode only): key steps a wave keeps in flight; 1 when a wave has one or two
 // steps at all (nothing to run ahead of), 2 for longer shares (deeper rings measured
 // no faster).
-template <int QB, bool DECODE, int RING = 1>
-__global__ __launch_bounds__(DECODE ? 64 * DECODE_WAVES : 256, (!DECODE && D <= 64) ? 2 : 1) void attention_bf16_kernel(AttnArgs a) {
+template <int QB, bool DECODE, int RING>
+__device__ __forceinline__ void attention_tile(const AttnArgs& a, const int xblk) {
   constexpr int DC = (D + 31) / 32;  // 32-wide chunks of d for Q.K
   constexpr int DB = D / 16;         // 16-wide blocks of d for P.V
   constexpr bool PIPE = DECODE;
@@ -110,8 +111,6 @@ __global__ __launch_bounds__(DECODE ? 64 * DECODE_WAVES : 256, (!DECODE && D <= 
   const int G = a.nq / a.nkv;
   const int r0 = a.q_start[b], qlen = a.q_start[b + 1] - r0, sp = a.start_pos[b];
   const int rows_total = qlen * G;
-  // the blocks with the longest histories (the last rows) are dispatched first
-  const int xblk = (int)(gridDim.x - 1 - blockIdx.x);
   const int row0 = DECODE ? xblk * (16 * QB) : (xblk * nw + wave) * (16 * QB);
   if ((DECODE ? row0 : xblk * nw * (16 * QB)) >= rows_total) return;   // the whole block is past the rows
   const bool wave_live = row0 < rows_total;      // a wave without rows still helps to stage keys
@@ -564,6 +563,27 @@ __global__ __launch_bounds__(DECODE ? 64 * DECODE_WAVES : 256, (!DECODE && D <= 
   }
 }
 
+// One tile of rows per block; the blocks with the longest histories (the last rows)
+// are dispatched first.
+template <int QB, bool DECODE, int RING = 1>
+__global__ __launch_bounds__(DECODE ? 64 * DECODE_WAVES : 256, (!DECODE && D <= 64) ? 2 : 1) void attention_bf16_kernel(AttnArgs a) {
+  attention_tile<QB, DECODE, RING>(a, (int)(gridDim.x - 1 - blockIdx.x));
+}
+
+// Two tiles of rows per block, one after the other: tile t from the end and tile t
+// from the start.  Under a causal mask their histories add up to the same length for
+// every t, so all blocks of a prompt carry the same load; with one tile per block the
+// last tiles' blocks run on while the units of the first ones idle.
+template <int QB>
+__global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void attention_bf16_paired_kernel(AttnArgs a) {
+  const int late = a.tiles - 1 - (int)blockIdx.x, early = (int)blockIdx.x;
+  for (int pass = 0; pass < 2; ++pass) {
+    if (pass == 1 && early >= late) break;
+    attention_tile<QB, false, 1>(a, pass == 0 ? late : early);
+    __syncthreads();
+  }
+}
+
 // Merge of the key splits of a decode step, one block per (row, head):
 //   out = sum_s w_s acc_s / sum_s w_s l_s,  w_s = 2^(m_s - max m), in the order of s.
 // A kernel of its own: within one kernel, results of blocks on other dies would
@@ -685,6 +705,7 @@ extern "C" int llmlab_paged_attention(const void* q, int dtype, int q_stride, in
   a.q_stride = q_stride; a.out_stride = out_stride; a.table_stride = table_stride; a.page_size = page_size;
   a.nq = nq; a.nkv = nkv; a.window = window; a.splits = 1; a.scale = scale;
   a.page_shift = 0;
+  a.tiles = 0;
   while ((1 << a.page_shift) < page_size) ++a.page_shift;
   if (dtype == DT_F32) {
     dim3 grid(max_q_len, nq, reqs), block(64);
@@ -759,6 +780,12 @@ extern "C" int llmlab_paged_attention(const void* q, int dtype, int q_stride, in
   if (D <= 128 && blocks32 >= 2L * num_cus) {
     dim3 grid((unsigned)((max_rows + 127) / 128), nkv, reqs), block(256);
     hipLaunchKernelGGL((attention_bf16_kernel<2, false>), grid, block, 0, stream, a);
+  } else if (window <= 0 && blocks16 >= (3L * num_cus) / 2) {
+    // not enough tiles to keep every unit busy with what the longest ones leave over:
+    // pair late and early tiles (no window: then the loads add up evenly)
+    a.tiles = (int)((max_rows + 63) / 64);
+    dim3 grid((unsigned)((a.tiles + 1) / 2), nkv, reqs), block(256);
+    hipLaunchKernelGGL((attention_bf16_paired_kernel<1>), grid, block, 0, stream, a);
   } else {
     dim3 grid((unsigned)((max_rows + 63) / 64), nkv, reqs), block(256);
     hipLaunchKernelGGL((attention_bf16_kernel<1, false>), grid, block, 0, stream, a);
