@@ -371,6 +371,7 @@ class HipOps:
 
     # --------------------------------------------- sums left in pieces (deferred)
     MAX_SPLITS = 8
+    split_max_rows = 64           # most rows of a product that is left in pieces
     min_steps_per_split = 8       # K steps of 32 a piece should have at least (tests lower it)
 
     def split_count(self, rows: int, dtype, n: int, k: int) -> int:
@@ -378,7 +379,7 @@ class HipOps:
         [n, k]^T`` should be cut so that it spreads over the chip: a narrow output
         gives too few blocks otherwise, and a compute unit draws only so much from
         memory.  1: do not cut."""
-        if dtype != torch.bfloat16 or not 0 < rows <= self.fuse_max_rows:
+        if dtype != torch.bfloat16 or not 0 < rows <= self.split_max_rows:
             return 1
         strips, steps = (n + 15) // 16, (k + 31) // 32
         want = self.num_cus // max(strips, 1)
@@ -396,7 +397,7 @@ class HipOps:
                 or parts.device != self.device):
             raise ValueError(f"linear_partials: x {tuple(x.shape)}, w {tuple(w.shape)}, "
                              f"parts {tuple(parts.shape)} for {splits} pieces do not fit")
-        if not 1 <= splits <= self.MAX_SPLITS or m > self.fuse_max_rows:
+        if not 1 <= splits <= self.MAX_SPLITS or m > self.split_max_rows:
             raise ValueError(f"linear_partials: {splits} pieces of {m} rows")
         self._skinny(x, False, None, None, 0.0, w, bias, EPI_PART, parts, m, n, k, parts.stride(1), n,
                      ksplit=splits, part_stride=parts.stride(0))

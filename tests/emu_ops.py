@@ -78,7 +78,7 @@ class EmuOps:
         return pending.parts[:pending.splits].sum(0) if pending is not None else 0.0
 
     def split_count(self, rows, dtype, n, k):
-        if not self.fuse or dtype != torch.bfloat16 or not 0 < rows <= self.fuse_max_rows:
+        if not self.fuse or dtype != torch.bfloat16 or not 0 < rows <= 64:
             return 1
         strips, steps = (n + 15) // 16, (k + 31) // 32
         return max(1, min(self.num_cus // max(strips, 1), steps // self.min_steps_per_split, self.MAX_SPLITS))
