@@ -28,7 +28,22 @@ __device__ __forceinline__ Best better(Best a, Best b) {
 
 __device__ Best block_argmax(const float* __restrict__ row, int vocab, float inv_t, Best* red) {
   Best best{0.f, -1};
-  for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
+  int i0 = 0;
+  if (((uintptr_t)row & 15) == 0) {
+    // four at a time where the row allows it; a thread's candidates come in rising
+    // index order, so "larger wins, equal keeps the earlier" is the tie rule here too
+    const int quads = vocab >> 2;
+    for (int q = threadIdx.x; q < quads; q += blockDim.x) {
+      const floatx4 v4 = *(const floatx4*)(row + 4 * q);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float v = v4[j] * inv_t;
+        if (v == v && (best.i < 0 || v > best.v)) best = Best{v, 4 * q + j};
+      }
+    }
+    i0 = quads << 2;
+  }
+  for (int i = i0 + threadIdx.x; i < vocab; i += blockDim.x) {
     const float v = row[i] * inv_t;
     if (v != v) continue;  // NaN
     best = better(best, Best{v, i});
