@@ -524,11 +524,16 @@ static SkinnyShape skinny_choose(int epilogue, bool norm, int mb, int M, int N, 
         if (resident > by_lds) resident = by_lds;
         if (resident < 1) resident = 1;
         const int rounds = (per_cu + resident - 1) / resident;
-        // a compute unit streams about 25 GB/s from HBM (3.5 GB/s per resident wave until
-        // that limit) and about 50 GB/s from L2; rows of x read by every wave on its own
+        // a compute unit streams about 50 GB/s from HBM (a good 3 GB/s per resident wave
+        // until that limit) and more from the caches; rows of x read by every wave on its own
         // (not staged) come in short strided pieces and cost about twice that
-        double rate = 3.5e3 * resident * nsb * kw;
-        if (rate > 25.0e3) rate = 25.0e3;
+        // (fitted twice: a large matrix is bound by what the waves of a unit keep in
+        // flight, up to about 50 GB/s; a small one by latencies, which the lower figures
+        // stand for)
+        const bool large = (double)N * K * 2.0 >= 64e6;
+        double rate = (large ? 3.2e3 : 3.5e3) * resident * nsb * kw;
+        const double cap = large ? 50.0e3 : 25.0e3;
+        if (rate > cap) rate = cap;
         const double t_stream = per_cu * (16.0 * nsb * K * 2.0) / rate;
         const double x_bytes = (double)(stage ? 1 : 2 * nsb) * M * K * (norm ? 4.0 : 2.0);
         const double t_x = per_cu * x_bytes / 50.0e3;
@@ -548,6 +553,14 @@ static SkinnyShape skinny_choose(int epilogue, bool norm, int mb, int M, int N, 
     }
   }
   return best;
+}
+
+// The shape the chooser takes for a product (for tests and tuning): out = {nsb, kw, stage, qsplit}.
+extern "C" void llmlab_skinny_shape(int epilogue, int norm, int M, int N, int K, int d, int num_cus, int ksplit,
+                                    int* out) {
+  const int mb = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
+  const SkinnyShape s = skinny_choose(epilogue, norm != 0, mb, M, N, K, d, num_cus, ksplit < 1 ? 1 : ksplit);
+  out[0] = s.nsb; out[1] = s.kw; out[2] = s.stage; out[3] = s.qsplit;
 }
 
 // One entry point for the whole family.
