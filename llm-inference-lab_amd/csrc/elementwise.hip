@@ -4,7 +4,7 @@
 
 extern "C" const char* llmlab_last_error() { return g_llmlab_error; }
 
-extern "C" int llmlab_abi_version() { return 3; }
+extern "C" int llmlab_abi_version() { return 4; }
 
 // --------------------------------------------------------------- embedding
 // out[r, :] = float(table[ids[r], :]); an id outside [0, vocab) is clamped (the
@@ -64,38 +64,94 @@ extern "C" int llmlab_embed(const void* table, int dtype, int packed, const int*
 // out[i, :] = x[row_i, :] * rsqrt(mean(x[row_i]^2) + eps) * w, row_i = rows[i] or
 // i.  The square, the mean, the rsqrt and both products are float32; one
 // rounding to T at the end.
-template <typename T>
-__global__ void rmsnorm_kernel(const float* __restrict__ x, const void* __restrict__ w, int w_bf16,
+// With pieces that a product left for the stream (pend[s][row, :], s < splits), the
+// row is first made whole, x[r] += sum_s pend[s][r] (written back: every element
+// belongs to one thread), and then normed; rows must not be gathered then.
+// A thread keeps its first KEEP groups of W elements (and their weights) in
+// registers, so a row of up to KEEP * W * blockDim.x elements costs one trip to
+// memory; what lies beyond is read again after the reduction.  VEC: groups of four
+// (hidden % 4 == 0 and 16-byte aligned rows).
+template <typename T, bool VEC>
+__global__ void rmsnorm_kernel(float* __restrict__ x, const void* __restrict__ w, int w_bf16,
                                float eps, T* __restrict__ out, const int* __restrict__ rows,
-                               int hidden) {
+                               int hidden, const float* __restrict__ pend, int splits, size_t pend_stride) {
+  constexpr int KEEP = 4, W = VEC ? 4 : 1;
   __shared__ float red[17];
   const int i = blockIdx.x;
   const int r = rows ? rows[i] : i;
-  const float* src = x + (size_t)r * hidden;
+  float* src = x + (size_t)r * hidden;
+  const float* prow = pend + (size_t)r * hidden;
+  const int stride = blockDim.x * W;
+  float keep[KEEP][W], wk[KEEP][W];
   float ss = 0.f;
-  for (int c = threadIdx.x; c < hidden; c += blockDim.x) {
-    const float v = src[c];
-    ss += v * v;
+  auto fetch = [&](int c, float* v) {       // the whole values of elements c .. c+W-1, written back if pieces came in
+    if constexpr (VEC) {
+      floatx4 t = *(const floatx4*)(src + c);
+      for (int s = 0; s < splits; ++s) t += *(const floatx4*)(prow + s * pend_stride + c);
+      if (splits > 0) *(floatx4*)(src + c) = t;
+#pragma unroll
+      for (int e = 0; e < W; ++e) v[e] = t[e];
+    } else {
+      float t = src[c];
+      for (int s = 0; s < splits; ++s) t += prow[s * pend_stride + c];
+      if (splits > 0) src[c] = t;
+      v[0] = t;
+    }
+  };
+#pragma unroll
+  for (int j = 0; j < KEEP; ++j) {
+    const int c = threadIdx.x * W + j * stride;
+    if (c < hidden) {
+      fetch(c, keep[j]);
+#pragma unroll
+      for (int e = 0; e < W; ++e) { wk[j][e] = load_vec(w, w_bf16, c + e); ss += keep[j][e] * keep[j][e]; }
+    }
   }
-  ss = block_sum(ss, red);
+  for (int c = threadIdx.x * W + KEEP * stride; c < hidden; c += stride) {
+    float v[W];
+    fetch(c, v);
+#pragma unroll
+    for (int e = 0; e < W; ++e) ss += v[e] * v[e];
+  }
+  ss = block_sum(ss, red);      // (a barrier; below a thread reads back only what it wrote itself)
   const float inv = rsqrtf(ss / (float)hidden + eps);
   T* dst = out + (size_t)i * hidden;
-  for (int c = threadIdx.x; c < hidden; c += blockDim.x)
-    dst[c] = from_float<T>(src[c] * inv * load_vec(w, w_bf16, c));
+#pragma unroll
+  for (int j = 0; j < KEEP; ++j) {
+    const int c = threadIdx.x * W + j * stride;
+    if (c < hidden) {
+      if constexpr (VEC) {
+        typedef T outx4 __attribute__((ext_vector_type(4)));
+        outx4 o;
+#pragma unroll
+        for (int e = 0; e < W; ++e) o[e] = from_float<T>(keep[j][e] * inv * wk[j][e]);
+        *(outx4*)(dst + c) = o;
+      } else {
+        dst[c] = from_float<T>(keep[j][0] * inv * wk[j][0]);
+      }
+    }
+  }
+  for (int c = threadIdx.x * W + KEEP * stride; c < hidden; c += stride)
+#pragma unroll
+    for (int e = 0; e < W; ++e) dst[c + e] = from_float<T>(src[c + e] * inv * load_vec(w, w_bf16, c + e));
 }
 
-extern "C" int llmlab_rmsnorm(const float* x, const void* w, int w_dtype, float eps, void* out,
+extern "C" int llmlab_rmsnorm(float* x, const void* w, int w_dtype, float eps, void* out,
                               int out_dtype, const int* rows, int n_out, int hidden,
-                              hipStream_t stream) {
+                              const float* pend, int splits, size_t pend_stride, hipStream_t stream) {
   LLMLAB_REQUIRE(n_out >= 0 && hidden > 0, "rmsnorm: bad sizes n=%d hidden=%d", n_out, hidden);
+  LLMLAB_REQUIRE(splits == 0 || (pend != nullptr && rows == nullptr && pend_stride >= (size_t)n_out * hidden),
+                 "rmsnorm: pending sums go with all rows in order");
   if (n_out == 0) return 0;
-  dim3 grid(n_out), block(hidden >= 2048 ? 512 : 256);
-  if (out_dtype == DT_BF16)
-    hipLaunchKernelGGL(rmsnorm_kernel<bf16_t>, grid, block, 0, stream, x, w, w_dtype == DT_BF16, eps,
-                       (bf16_t*)out, rows, hidden);
-  else
-    hipLaunchKernelGGL(rmsnorm_kernel<float>, grid, block, 0, stream, x, w, w_dtype == DT_BF16, eps,
-                       (float*)out, rows, hidden);
+  const bool vec = hidden % 4 == 0 && pend_stride % 4 == 0 &&
+                   (((uintptr_t)x | (uintptr_t)pend | (uintptr_t)out) & 15) == 0;
+  dim3 grid(n_out), block(hidden >= 8192 ? 512 : 256);
+#define LLMLAB_RMSNORM(T, VEC)                                                                      \
+  hipLaunchKernelGGL((rmsnorm_kernel<T, VEC>), grid, block, 0, stream, x, w, w_dtype == DT_BF16, eps, \
+                     (T*)out, rows, hidden, pend, splits, pend_stride)
+  if (out_dtype == DT_BF16) { if (vec) LLMLAB_RMSNORM(bf16_t, true); else LLMLAB_RMSNORM(bf16_t, false); }
+  else                      { if (vec) LLMLAB_RMSNORM(float, true);  else LLMLAB_RMSNORM(float, false); }
+#undef LLMLAB_RMSNORM
   LLMLAB_LAUNCH_CHECK("rmsnorm");
   return 0;
 }

@@ -78,7 +78,7 @@ class HipOps:
         torch.cuda.set_device(self.device)
         self._core = self._load(build.core_library())
         self._declare_core()
-        if self._core.llmlab_abi_version() != 3:
+        if self._core.llmlab_abi_version() != 4:
             raise RuntimeError("kernel library and Python bindings disagree on the interface")
         self._attn: Dict[int, ctypes.CDLL] = {}
         self._shared: Dict[int, tuple] = {}
@@ -100,7 +100,7 @@ class HipOps:
         c.llmlab_abi_version.restype = _c_int
         c.llmlab_embed.argtypes = [_c_ptr, _c_int, _c_int, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_ptr]
         c.llmlab_rmsnorm.argtypes = [_c_ptr, _c_ptr, _c_int, _c_float, _c_ptr, _c_int, _c_ptr, _c_int,
-                                     _c_int, _c_ptr]
+                                     _c_int, _c_ptr, _c_int, _c_size, _c_ptr]
         c.llmlab_rope_kv_write.argtypes = [_c_ptr, _c_int, _c_int, _c_int, _c_int, _c_int, _c_int,
                                            _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr,
                                            _c_ptr, _c_ptr]
@@ -255,7 +255,9 @@ class HipOps:
         self._check(self._core.llmlab_gather_tokens(self._ptr(dst), self._ptr(dst_index), self._ptr(src),
                                                     self._ptr(src_index), int(n), self._stream()))
 
-    def rmsnorm(self, x, weight, eps, out, rows=None) -> None:
+    def rmsnorm(self, x, weight, eps, out, rows=None, pending=None) -> None:
+        """``out[i] = norm(x[rows[i]])``.  ``pending`` (all rows in order only): the pieces are
+        folded into ``x`` on the way, ``x += sum_s parts[s]``, and the whole rows are normed."""
         self._need(x, "norm input", torch.float32)
         self._need(weight, "norm weight")
         self._need(out, "norm output")
@@ -271,9 +273,15 @@ class HipOps:
             self._need(rows, "norm row indices", torch.int32)
             if rows.numel() != n_out:
                 raise ValueError("rmsnorm: one row index per output row")
+        pend = (_c_ptr(0), 0, 0)
+        if pending is not None:
+            p = pending.parts
+            if rows is not None or p.shape[1] != n_out or p.shape[2] != hidden or not p[0].is_contiguous():
+                raise ValueError("rmsnorm: pending sums go with all rows in order and the same shape")
+            pend = (self._ptr(p), pending.splits, p.stride(0))
         self._check(self._core.llmlab_rmsnorm(self._ptr(x), self._ptr(weight), _dt(weight), float(eps),
                                               self._ptr(out), _dt(out), self._ptr(rows), n_out, hidden,
-                                              self._stream()))
+                                              pend[0], pend[1], pend[2], self._stream()))
 
     # ----------------------------------------------------------------- linear
     def _linear(self, x, w, out, bias, epilogue, n_out, pending: Optional[PendingSums] = None) -> None:

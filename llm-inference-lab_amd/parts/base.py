@@ -55,6 +55,10 @@ class Part:
 
 
 class Norm(Part):
+    # True: ``forward(x, out, None, pending=p)`` first makes the stream whole,
+    # ``x += sum_s p.parts[s]``, in the same pass (all rows in order only).
+    folds_pending = False
+
     def forward(self, x: torch.Tensor, out: torch.Tensor, rows: Optional[torch.Tensor] = None) -> None:
         """``out[i] = norm(x[rows[i]])`` (all rows in order when ``rows`` is None).
         ``x`` float32, ``out`` compute dtype."""
@@ -120,9 +124,14 @@ class NormedInput:
 
     def tensor(self) -> torch.Tensor:
         if self._tensor is None:
-            self._fold_pending()
             out = self.ctx.scratch(self.name, (self.n_rows, self.x.shape[1]), self.dtype)
-            self.norm.forward(self.x, out, self.rows)
+            pending = getattr(self.ctx, "pending", None)
+            if pending is not None and self.rows is None and self.norm.folds_pending:
+                self.norm.forward(self.x, out, None, pending=pending)     # folded in by the norm itself
+                self.ctx.pending = None
+            else:
+                self._fold_pending()
+                self.norm.forward(self.x, out, self.rows)
             self._tensor = out
         return self._tensor
 

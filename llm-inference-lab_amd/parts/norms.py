@@ -18,6 +18,8 @@ class RMSNorm(Norm):
     reference rounds once more, before the weight product; in float32 the two
     are the same).  ``size`` and ``eps`` come from the caller."""
 
+    folds_pending = True
+
     def __init__(self, size: int, eps: float, tensors: Dict[str, str]):
         super().__init__(tensors)
         self.size = int(size)
@@ -31,8 +33,11 @@ class RMSNorm(Norm):
         super().bind(tensors, ops, dtype)
         self.weight = tensors[self.tensor_names["weight"]].contiguous()
 
-    def forward(self, x, out, rows=None):
-        self.ops.rmsnorm(x, self.weight, self.eps, out, rows)
+    def forward(self, x, out, rows=None, pending=None):
+        if pending is None:
+            self.ops.rmsnorm(x, self.weight, self.eps, out, rows)
+        else:
+            self.ops.rmsnorm(x, self.weight, self.eps, out, rows, pending=pending)
 
     def rms_params(self):
         return self.weight, self.eps

@@ -45,8 +45,11 @@ class EmuOps:
         for i in range(n):
             dst[int(dst_index[i])] = src[int(src_index[i])]
 
-    def rmsnorm(self, x, weight, eps, out, rows=None):
+    def rmsnorm(self, x, weight, eps, out, rows=None, pending=None):
         self._count("rmsnorm")
+        if pending is not None:
+            assert rows is None and pending.parts.shape[1:] == x.shape
+            x += pending.parts[:pending.splits].float().sum(0)
         v = x.float() if rows is None else x.float()[rows.long()]
         inv = torch.rsqrt((v * v).sum(-1, keepdim=True) / v.shape[-1] + eps)
         out.copy_((v * inv * weight.float()).to(out.dtype))

@@ -58,7 +58,8 @@ def test_embed(ops, emu, dtype, rows, hidden, vocab):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("wdtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("rows,hidden,eps", [(1, 64, 1e-6), (19, 896, 1e-5), (7, 3584, 1e-6), (3, 100, 1e-3)])
+@pytest.mark.parametrize("rows,hidden,eps", [(1, 64, 1e-6), (19, 896, 1e-5), (7, 3584, 1e-6), (3, 100, 1e-3),
+                                           (4, 1130, 1e-6), (3, 5120, 1e-6), (2, 8192, 1e-5)])
 def test_rmsnorm(ops, emu, dtype, wdtype, rows, hidden, eps):
     x = rnd((rows, hidden), torch.float32, 3, 3.0)
     w = (1 + 0.1 * torch.randn(hidden, generator=torch.Generator().manual_seed(4))).to(wdtype)
@@ -75,6 +76,16 @@ def test_rmsnorm(ops, emu, dtype, wdtype, rows, hidden, eps):
         got = torch.empty(3, hidden, dtype=dtype, device=DEV)
         ops.rmsnorm(x.to(DEV), w.to(DEV), eps, got, idx.to(DEV))
         close(got, want, dtype, "rmsnorm gather", 4.0)
+    # sums left in pieces: folded into the stream and normed in one pass
+    from llm_inference_lab_amd.parts.base import PendingSums
+    pieces = rnd((4, rows, hidden), torch.float32, 9, 2.0)
+    whole = x + pieces[:3].sum(0)
+    want = torch.empty(rows, hidden, dtype=dtype)
+    emu.rmsnorm(whole, w, eps, want)
+    xs, got = x.to(DEV), torch.empty(rows, hidden, dtype=dtype, device=DEV)
+    ops.rmsnorm(xs, w.to(DEV), eps, got, pending=PendingSums(pieces.to(DEV), 3))
+    close(got, want, dtype, "rmsnorm with pieces", 4.0)
+    assert torch.allclose(xs.cpu(), whole, rtol=1e-6, atol=1e-6)
 
 
 LINEAR_SHAPES = [
