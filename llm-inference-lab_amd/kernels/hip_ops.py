@@ -339,17 +339,21 @@ class HipOps:
     # ----------------------------------------------- few rows: fused kernels
     FUSED_MAX_ROWS = 64           # most rows the few-row kernels take at all
     skinny_max_rows = 64          # plain products up to here may take the few-row kernel
-    fuse_max_rows = 16            # steps up to here take the fused kernels: their rows fit
-                                  # the staging buffer; beyond, norm + tiled product is faster
-
+    fuse_max_rows = 64            # steps up to here may take the fused kernels
+    FUSE_TILE_ROWS = 16           # the few-row kernels cut the rows into tiles of so many
+    FUSE_WIDE_BYTES = 64e6        # beyond 16 rows: only for matrices smaller than this (a larger
+                                  # one is read once per tile of rows, and norm + tiled product wins)
     STAGE_BYTES = 118 * 1024      # most LDS the staged rows of a fused kernel may take
 
-    def can_fuse(self, rows: int, dtype, inner: int) -> bool:
-        """Whether the fused few-row kernels take this step: bfloat16, few rows, and
-        the rows (``inner`` wide) fit the staging buffer in LDS."""
+    def can_fuse(self, rows: int, dtype, inner: int, outer: Optional[int] = None) -> bool:
+        """Whether the fused few-row kernels take this step: bfloat16, few rows, a tile
+        of rows (``inner`` wide) fits the staging buffer in LDS, and beyond one tile the
+        matrix (``outer`` rows) is a small one."""
         if dtype != torch.bfloat16 or not 0 < rows <= self.fuse_max_rows:
             return False
-        return rows * ((inner + 31) // 32 * 32 + 8) * 2 <= self.STAGE_BYTES
+        if rows > self.FUSE_TILE_ROWS and (outer is None or outer * inner * 2 >= self.FUSE_WIDE_BYTES):
+            return False
+        return min(rows, self.FUSE_TILE_ROWS) * ((inner + 31) // 32 * 32 + 8) * 2 <= self.STAGE_BYTES
 
     def _skinny(self, x, norm, x_rows, norm_w, eps, w, bias, epilogue, out, m, n, k, ldo, n_out,
                 qkv=None, pending: Optional[PendingSums] = None, ksplit: int = 1,
@@ -379,7 +383,7 @@ class HipOps:
 
     # --------------------------------------------- sums left in pieces (deferred)
     MAX_SPLITS = 8
-    split_max_rows = 64           # most rows of a product that is left in pieces
+    split_max_rows = 32           # most rows of a product that is left in pieces
     min_steps_per_split = 8       # K steps of 32 a piece should have at least (tests lower it)
 
     def split_count(self, rows: int, dtype, n: int, k: int) -> int:
@@ -405,7 +409,7 @@ class HipOps:
                 or parts.device != self.device):
             raise ValueError(f"linear_partials: x {tuple(x.shape)}, w {tuple(w.shape)}, "
                              f"parts {tuple(parts.shape)} for {splits} pieces do not fit")
-        if not 1 <= splits <= self.MAX_SPLITS or m > self.split_max_rows:
+        if not 1 <= splits <= self.MAX_SPLITS or m > self.FUSED_MAX_ROWS:
             raise ValueError(f"linear_partials: {splits} pieces of {m} rows")
         self._skinny(x, False, None, None, 0.0, w, bias, EPI_PART, parts, m, n, k, parts.stride(1), n,
                      ksplit=splits, part_stride=parts.stride(0))
@@ -438,25 +442,19 @@ class HipOps:
             raise ValueError(f"the fused kernels take 1..{self.FUSED_MAX_ROWS} rows, got {rows}")
         return w, k
 
-    def fused_norm_qkv(self, x, norm_w, eps, w_qkv, b_qkv, num_heads, num_kv_heads, head_dim, inv_freq,
-                       positions, row_req, block_table, page_size, k_cache, v_cache, q_out,
-                       pending: Optional[PendingSums] = None) -> None:
-        """q_out = rotate(norm(x) Wq^T + bq); rotated k and v of the new positions go to
-        their pages (skipped when no cache is given).  ``pending``: pieces still owed to
-        the rows of x, added while they are read (x itself is left as it is)."""
-        rows = x.shape[0]
-        w_qkv, k = self._fused_common(x, norm_w, w_qkv, rows)
+    def _qkv_checks(self, what, rows, w_qkv, b_qkv, num_heads, num_kv_heads, head_dim, inv_freq, positions,
+                    row_req, block_table, page_size, k_cache, v_cache, q_out) -> int:
         n = (num_heads + 2 * num_kv_heads) * head_dim
         if w_qkv.shape[0] != n or tuple(q_out.shape) != (rows, num_heads * head_dim):
-            raise ValueError("fused_norm_qkv: weight or output shape does not fit the heads")
+            raise ValueError(f"{what}: weight or output shape does not fit the heads")
         self._need(q_out, "q output", torch.bfloat16)
         self._need(positions, "positions", torch.int32)
         if positions.numel() < rows:
-            raise ValueError("fused_norm_qkv: one position per row")
+            raise ValueError(f"{what}: one position per row")
         if b_qkv is not None and b_qkv.numel() != n:
-            raise ValueError("fused_norm_qkv: bias length")
+            raise ValueError(f"{what}: bias length")
         if inv_freq is not None and (inv_freq.dtype != torch.float32 or inv_freq.numel() != head_dim // 2):
-            raise ValueError("fused_norm_qkv: the frequency table must hold head_dim/2 float32 entries")
+            raise ValueError(f"{what}: the frequency table must hold head_dim/2 float32 entries")
         if k_cache is not None:
             self._need(row_req, "row -> request map", torch.int32)
             self._need(block_table, "block table", torch.int32)
@@ -466,12 +464,50 @@ class HipOps:
                     or not k_cache.is_contiguous() or not v_cache.is_contiguous()
                     or k_cache.dtype != torch.bfloat16 or v_cache.dtype != torch.bfloat16
                     or row_req.numel() < rows):
-                raise ValueError("fused_norm_qkv: cache tensors do not have the paged layout")
+                raise ValueError(f"{what}: cache tensors do not have the paged layout")
+        return n
+
+    def fused_norm_qkv(self, x, norm_w, eps, w_qkv, b_qkv, num_heads, num_kv_heads, head_dim, inv_freq,
+                       positions, row_req, block_table, page_size, k_cache, v_cache, q_out,
+                       pending: Optional[PendingSums] = None) -> None:
+        """q_out = rotate(norm(x) Wq^T + bq); rotated k and v of the new positions go to
+        their pages (skipped when no cache is given).  ``pending``: pieces still owed to
+        the rows of x, added while they are read (x itself is left as it is)."""
+        rows = x.shape[0]
+        w_qkv, k = self._fused_common(x, norm_w, w_qkv, rows)
+        n = self._qkv_checks("fused_norm_qkv", rows, w_qkv, b_qkv, num_heads, num_kv_heads, head_dim,
+                             inv_freq, positions, row_req, block_table, page_size, k_cache, v_cache, q_out)
         self._skinny(x, True, None, norm_w, eps, w_qkv, b_qkv, EPI_QKV, q_out, rows, n, k,
                      q_out.shape[1], n,
                      dict(inv_freq=inv_freq, positions=positions, row_req=row_req, table=block_table,
                           page_size=page_size, k_cache=k_cache, v_cache=v_cache, nq=num_heads,
                           nkv=num_kv_heads, d=head_dim), pending=pending)
+
+    QKV_ROPE_MAX_ROWS = 64
+
+    def can_fuse_qkv_rope(self, rows: int, dtype, head_dim: int) -> bool:
+        """Whether ``qkv_rope_cache`` takes this step: bfloat16, at most 64 rows, and a
+        head that one block of the few-row kernel holds."""
+        if dtype != torch.bfloat16 or not 0 < rows <= self.QKV_ROPE_MAX_ROWS:
+            return False
+        return head_dim % 16 == 0 and 16 <= head_dim <= (128 if rows > 32 else 256)
+
+    def qkv_rope_cache(self, h, w_qkv, b_qkv, num_heads, num_kv_heads, head_dim, inv_freq, positions,
+                       row_req, block_table, page_size, k_cache, v_cache, q_out) -> None:
+        """The same for activations ``h`` (bfloat16, already normed) of up to 64 rows:
+        product, bias, rotation and cache write in one kernel."""
+        rows, k = h.shape
+        self._need(h, "activations", torch.bfloat16)
+        w_qkv = self._weight(w_qkv, "weight")
+        if w_qkv.shape[1] != k or k % 8 != 0 or not self.can_fuse_qkv_rope(rows, h.dtype, head_dim):
+            raise ValueError(f"qkv_rope_cache: {rows} rows of {k}, heads of {head_dim} do not fit")
+        n = self._qkv_checks("qkv_rope_cache", rows, w_qkv, b_qkv, num_heads, num_kv_heads, head_dim,
+                             inv_freq, positions, row_req, block_table, page_size, k_cache, v_cache, q_out)
+        self._skinny(h, False, None, None, 0.0, w_qkv, b_qkv, EPI_QKV, q_out, rows, n, k,
+                     q_out.shape[1], n,
+                     dict(inv_freq=inv_freq, positions=positions, row_req=row_req, table=block_table,
+                          page_size=page_size, k_cache=k_cache, v_cache=v_cache, nq=num_heads,
+                          nkv=num_kv_heads, d=head_dim))
 
     def fused_norm_swiglu(self, x, norm_w, eps, w_gate_up, out, pending: Optional[PendingSums] = None) -> None:
         rows, inter = out.shape

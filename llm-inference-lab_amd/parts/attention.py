@@ -104,7 +104,7 @@ class GQAAttention(Mixer):
         group = ctx.group(entry.group)
         k_cache = entry.k_cache if entry.writes_cache else None
         v_cache = entry.v_cache if entry.writes_cache else None
-        fuse = (isinstance(h, NormedInput) and ops.can_fuse(rows, self.dtype, self.hidden_size)
+        fuse = (isinstance(h, NormedInput) and ops.can_fuse(rows, self.dtype, self.hidden_size, self.q_size + 2 * self.kv_size)
                 and (self.position is None or table is not None))
         rms = h.rms(accept_pending=True) if fuse else None
         pending = None
@@ -118,6 +118,15 @@ class GQAAttention(Mixer):
             ops.fused_norm_qkv(rms[0], rms[2], rms[3], self.w_qkv, self.b_qkv, self.num_heads,
                                self.num_kv_heads, self.head_dim, table, ctx.positions, ctx.row_req,
                                group.block_table, group.page_size, k_cache, v_cache, q, pending=pending)
+        elif (ops.can_fuse_qkv_rope(rows, self.dtype, self.head_dim)
+              and (self.position is None or table is not None)):
+            # some more rows: the norm on its own, then one kernel for the rest
+            if isinstance(h, NormedInput):
+                h = h.tensor()
+            q = ctx.scratch("attention.q", (rows, self.q_size), self.dtype)
+            ops.qkv_rope_cache(h, self.w_qkv, self.b_qkv, self.num_heads, self.num_kv_heads,
+                               self.head_dim, table, ctx.positions, ctx.row_req, group.block_table,
+                               group.page_size, k_cache, v_cache, q)
         else:
             if isinstance(h, NormedInput):
                 h = h.tensor()

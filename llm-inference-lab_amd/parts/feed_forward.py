@@ -70,7 +70,7 @@ class SwiGLU(FeedForward):
         rows = h.shape[0]
         act = ctx.scratch("swiglu.act", (rows, self.intermediate_size), self.dtype)
         rms = h.rms() if isinstance(h, NormedInput) else None
-        if rms is not None and self.ops.can_fuse(rows, self.dtype, self.hidden_size):
+        if rms is not None and self.ops.can_fuse(rows, self.dtype, self.hidden_size, self.w_gate_up.shape[0]):
             self.ops.fused_norm_swiglu(rms[0], rms[2], rms[3], self.w_gate_up, act)
         else:
             if isinstance(h, NormedInput):

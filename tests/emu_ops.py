@@ -122,7 +122,7 @@ class EmuOps:
     FUSED_MAX_ROWS = 64
     fuse_max_rows = 16
 
-    def can_fuse(self, rows, dtype, inner):
+    def can_fuse(self, rows, dtype, inner, outer=None):
         return self.fuse and dtype == torch.bfloat16 and 0 < rows <= self.fuse_max_rows
 
     def prepare_weight(self, w, shared=False):
@@ -143,6 +143,20 @@ class EmuOps:
         self._count("fused_norm_qkv")
         rows = x.shape[0]
         y = self._normed(x, None, norm_w, eps, rows, pending) @ w_qkv.float().t()
+        if b_qkv is not None:
+            y = y + b_qkv.float()
+        qkv = y.clone()                      # float32: the kernel rotates before it rounds
+        self.rope_kv_write(qkv, num_heads, num_kv_heads, head_dim, inv_freq, positions, row_req,
+                           block_table, page_size, k_cache, v_cache)
+        q_out.copy_(qkv[:, :num_heads * head_dim].to(q_out.dtype))
+
+    def can_fuse_qkv_rope(self, rows, dtype, head_dim):
+        return self.fuse and dtype == torch.bfloat16 and 0 < rows <= 64 and head_dim % 16 == 0
+
+    def qkv_rope_cache(self, h, w_qkv, b_qkv, num_heads, num_kv_heads, head_dim, inv_freq, positions,
+                       row_req, block_table, page_size, k_cache, v_cache, q_out):
+        self._count("qkv_rope_cache")
+        y = h.float() @ w_qkv.float().t()
         if b_qkv is not None:
             y = y + b_qkv.float()
         qkv = y.clone()                      # float32: the kernel rotates before it rounds

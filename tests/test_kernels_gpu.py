@@ -215,10 +215,10 @@ def test_fused_norm_products(ops, emu, wdtype, m, hidden, inter, vocab):
 
 @pytest.mark.parametrize("nq,nkv,d,page,hidden", [(4, 2, 16, 16, 64), (3, 1, 32, 32, 96), (14, 2, 64, 64, 896),
                                                  (6, 3, 48, 16, 72), (8, 8, 128, 64, 256), (2, 1, 256, 16, 64)])
-@pytest.mark.parametrize("rotate", [True, False])
-def test_fused_norm_qkv_rope_write(ops, emu, nq, nkv, d, page, hidden, rotate):
+@pytest.mark.parametrize("rotate,rows_per", [(True, [5, 1, 9]), (False, [5, 1, 9]), (True, [17, 30, 16])])
+def test_fused_norm_qkv_rope_write(ops, emu, nq, nkv, d, page, hidden, rotate, rows_per):
     bf = torch.bfloat16
-    rows_per, starts, reqs, num_pages = [5, 1, 9], [3, 40, 0], 3, 12
+    starts, reqs, num_pages = [3, 40, 0], 3, 16
     rows = sum(rows_per)
     x = rnd((rows, hidden), torch.float32, 60, 2.0)
     nw = (1 + 0.1 * rnd((hidden,), torch.float32, 61)).to(bf)
@@ -246,6 +246,48 @@ def test_fused_norm_qkv_rope_write(ops, emu, nq, nkv, d, page, hidden, rotate):
     close(got_q, want_q, bf, "fused q", scale)
     close(got_k, want_k, bf, "fused key cache", scale)
     close(got_v, want_v, bf, "fused value cache", scale)
+    untouched = (want_k == kc)
+    assert torch.equal(got_k.cpu()[untouched], kc[untouched])
+
+
+@pytest.mark.parametrize("nq,nkv,d,page,hidden", [(4, 2, 16, 16, 64), (14, 2, 64, 64, 896), (6, 3, 48, 16, 72),
+                                                 (8, 8, 128, 64, 256), (2, 1, 256, 16, 64)])
+@pytest.mark.parametrize("rows_per", [[5, 1, 9], [20, 1, 1, 3], [17, 30, 16]])
+def test_qkv_rope_cache_of_normed_rows(ops, emu, nq, nkv, d, page, hidden, rows_per):
+    bf = torch.bfloat16
+    rows, reqs, num_pages = sum(rows_per), len(rows_per), 16
+    if not ops.can_fuse_qkv_rope(rows, bf, d):
+        with pytest.raises(ValueError):
+            ops.qkv_rope_cache(torch.zeros(rows, hidden, dtype=bf, device=DEV),
+                               ops.prepare_weight(torch.zeros((nq + 2 * nkv) * d, hidden, dtype=bf, device=DEV)),
+                               None, nq, nkv, d, None, torch.zeros(rows, dtype=torch.int32, device=DEV), None,
+                               None, page, None, None, torch.empty(rows, nq * d, dtype=bf, device=DEV))
+        return
+    starts = [3, 40, 0, 7][:reqs]
+    h = rnd((rows, hidden), bf, 70)
+    n = (nq + 2 * nkv) * d
+    w, b = rnd((n, hidden), bf, 72, 0.2), rnd((n,), bf, 73)
+    positions = torch.cat([torch.arange(s, s + c) for s, c in zip(starts, rows_per)]).int()
+    row_req = torch.cat([torch.full((c,), i) for i, c in enumerate(rows_per)]).int()
+    table = torch.full((reqs, 8), -1, dtype=torch.int32)
+    perm = torch.randperm(num_pages, generator=torch.Generator().manual_seed(74)).int()
+    at = 0
+    for i in range(reqs):
+        need = (starts[i] + rows_per[i] + page - 1) // page
+        table[i, :need] = perm[at:at + need]
+        at += need
+    assert at <= num_pages
+    inv_freq = (1.0 / (1e4 ** (torch.arange(0, d, 2, dtype=torch.float64) / d))).float()
+    kc, vc = make_cache(num_pages, nkv, page, d, bf, 75)
+    want_q, want_k, want_v = torch.empty(rows, nq * d, dtype=bf), kc.clone(), vc.clone()
+    emu.qkv_rope_cache(h, w, b, nq, nkv, d, inv_freq, positions, row_req, table, page, want_k, want_v, want_q)
+    got_q, got_k, got_v = torch.empty(rows, nq * d, dtype=bf, device=DEV), kc.to(DEV), vc.to(DEV)
+    ops.qkv_rope_cache(h.to(DEV), ops.prepare_weight(w.to(DEV)), b.to(DEV), nq, nkv, d, inv_freq.to(DEV),
+                       positions.to(DEV), row_req.to(DEV), table.to(DEV), page, got_k, got_v, got_q)
+    scale = want_q.float().abs().max().item()
+    close(got_q, want_q, bf, "q", scale)
+    close(got_k, want_k, bf, "key cache", scale)
+    close(got_v, want_v, bf, "value cache", scale)
     untouched = (want_k == kc)
     assert torch.equal(got_k.cpu()[untouched], kc[untouched])
 
@@ -469,7 +511,8 @@ def test_cache_order_round_trip(page, d):
     assert int(ki[:16].max()) == 16 * d - 1 and int(vi[:, :16].max()) == 16 * d - 1
 
 
-@pytest.mark.parametrize("m,n,k,splits", [(8, 896, 4864, 4), (1, 896, 896, 3), (16, 90, 512, 2), (5, 130, 264, 1)])
+@pytest.mark.parametrize("m,n,k,splits", [(8, 896, 4864, 4), (1, 896, 896, 3), (16, 90, 512, 2), (5, 130, 264, 1),
+                                          (40, 896, 512, 2), (64, 130, 264, 3)])
 def test_linear_partials_and_pending(ops, emu, m, n, k, splits):
     """A product left in pieces along K; the pieces added on the fly where the rows are
     read (fused norm + product), folded in where a product adds into them, or folded
