@@ -2,6 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch B] [--context S]
                     [--shape 0.5b|7b|32b] [--layers L]
+    python bench.py --mixed [--shape 7b] [--requests 64] [--chunk 512] [--outputs 64]
 
 Default: the layer sizes of the Qwen2.5-0.5B shape with seeded random weights,
 batch 8, context 4096, bfloat16.  A "step" is one decode step of the whole
@@ -9,6 +10,11 @@ batch through the scheduler's own path (step function + sampling, tokens fed
 back).  One JSON line is printed: decoded tokens a second as ``value``, plus
 ``prefill`` (one 2,048-token prompt), ``roofline`` (bytes the decode step has to
 read over its time against 8 TB/s) and ``points`` (decode at batch 1 and 64).
+
+``--mixed``: many requests with prompts of different lengths go through the
+scheduler with a small token budget, so that portions of prompts run beside the
+decode tokens of the requests that are already in; one JSON line with all tokens
+(prompt and generated) a second.
 """
 import argparse
 import json
@@ -46,6 +52,66 @@ def prefill_flops(cfg, tokens):
     return cfg.num_hidden_layers * (tokens * per_token_layer + attention_layer) + 2 * h * v
 
 
+def mixed_run(args, cfg, layers, full_layers):
+    """Requests with prompts of 128..2048 tokens, all admitted at once; the scheduler cuts
+    the prompts into portions under a budget of ``--chunk`` tokens a step, beside one
+    token for every request that is decoding.  Timed from the first step to the last."""
+    import torch
+    import llm_inference_lab_amd as lab
+    from llm_inference_lab_amd.sampling import SamplingConfig
+
+    page = 64
+    gen = torch.Generator().manual_seed(4321)
+    lengths = torch.randint(128, 2049, (args.requests,), generator=gen).tolist()
+    longest = max(lengths) + args.outputs
+    engine = lab.Engine(config=cfg, seed=0, dtype=args.dtype, device="cuda:0", page_size=page,
+                        max_cache_tokens=sum(n + args.outputs + page for n in lengths),
+                        max_requests=args.requests, max_batch_tokens=args.chunk + args.requests,
+                        max_seq_len=longest + page, graph=not args.no_graph)
+
+    def one_run():
+        sched = engine.scheduler(max_batch_tokens=args.chunk + args.requests)
+        for n in lengths:
+            ids = torch.randint(0, cfg.vocab_size, (n,), generator=gen).tolist()
+            sched.add_request(ids, SamplingConfig(max_new_tokens=args.outputs, eos_token_id=[]))
+        steps = 0
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        while sched.active or sched.waiting:
+            sched.step()
+            steps += 1
+        torch.cuda.synchronize()
+        seconds = time.perf_counter() - t0
+        assert engine.cache.live_requests == 0
+        return seconds, steps
+
+    one_run()                                   # warm-up: scratch buffers, graphs, kernel loading
+    seconds, steps = one_run()
+    prompt_tokens, new_tokens = sum(lengths), args.requests * args.outputs
+    # every prompt token and every generated token but a request's last goes through the model once
+    flops = sum(prefill_flops(cfg, n + args.outputs - 1) - 2 * cfg.hidden_size * cfg.vocab_size for n in lengths)
+    flops += new_tokens * 2 * cfg.hidden_size * cfg.vocab_size
+    print(json.dumps({
+        "metric": "mixed_tokens_per_second", "value": round((prompt_tokens + new_tokens) / seconds, 1),
+        "unit": "tokens/s", "n_gpus": 1, "steps": steps, "warmup": steps,
+        "ms_per_step": round(seconds / steps * 1e3, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": args.dtype, "data": "synthetic",
+        "config": {
+            "model": f"Qwen2.5-{args.shape.upper()} shape, random weights", "global_batch": args.requests,
+            "seq_len": longest, "parallelism": "single GPU", "layers": layers,
+            "layers_of_full_model": full_layers, "hidden_size": cfg.hidden_size,
+            "num_attention_heads": cfg.num_attention_heads,
+            "num_key_value_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
+            "intermediate_size": cfg.intermediate_size, "vocab_size": cfg.vocab_size,
+            "prompt_lengths": "uniform 128..2048", "prompt_tokens": prompt_tokens,
+            "outputs_per_request": args.outputs, "token_budget": args.chunk + args.requests,
+            "page_size": page, "weights_seed": 0,
+        },
+        "seconds": round(seconds, 4), "generated_tokens_per_second": round(new_tokens / seconds, 1),
+        "flops_frac": round(flops / seconds / PEAK_FLOPS[args.dtype], 4),
+    }))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -60,6 +126,12 @@ def main():
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "f32"])
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 / 64 and the prefill")
+    ap.add_argument("--mixed", action="store_true",
+                    help="mixed run: --requests prompts of 128..2048 tokens, portions of --chunk tokens "
+                         "beside decode tokens, --outputs tokens each")
+    ap.add_argument("--requests", type=int, default=64)
+    ap.add_argument("--chunk", type=int, default=512)
+    ap.add_argument("--outputs", type=int, default=64)
     ap.add_argument("--only-prefill", action="store_true",
                     help="run nothing but the 2,048-token prefill (for profiling); prints its numbers")
     args = ap.parse_args()
@@ -76,6 +148,9 @@ def main():
     layers = args.layers or full_layers
     raw = dict(SHAPES[args.shape], num_hidden_layers=layers)
     cfg = lab.Qwen2Config.from_dict(raw)
+    if args.mixed:
+        mixed_run(args, cfg, layers, full_layers)
+        return
     batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
     max_batch = max(batches)
     page = 64

@@ -75,6 +75,8 @@ struct AttnArgs {
   int nq, nkv, window, splits;
   int page_shift;     // log2(page_size); page sizes are powers of two
   int tiles;          // paired kernel: tiles of rows per request (blocks take two each)
+  int qlen_lo, qlen_hi;  // only requests that bring so many tokens are worked on (a step may be
+                         // served by two launches: its short requests by one, its long ones by the other)
   float scale;
 };
 
@@ -113,6 +115,7 @@ __device__ __forceinline__ void attention_tile(const AttnArgs& a, const int xblk
   const int rows_total = qlen * G;
   const int row0 = DECODE ? xblk * (16 * QB) : (xblk * nw + wave) * (16 * QB);
   if ((DECODE ? row0 : xblk * nw * (16 * QB)) >= rows_total) return;   // the whole block is past the rows
+  if (qlen < a.qlen_lo || qlen > a.qlen_hi) return;                     // another launch's request
   const bool wave_live = row0 < rows_total;      // a wave without rows still helps to stage keys
   const bf16_t* q = (const bf16_t*)a.q;
   const bf16_t* kc = (const bf16_t*)a.kc;
@@ -591,8 +594,14 @@ __global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void attention_bf16_paired_ke
 __global__ __launch_bounds__(64) void attention_merge_kernel(const float* __restrict__ o_part,
                                                              const float* __restrict__ ml_part,
                                                              bf16_t* __restrict__ out, int out_stride,
-                                                             int nq, int splits) {
+                                                             int nq, int splits,
+                                                             const int* __restrict__ row_req,
+                                                             const int* __restrict__ q_start, int qlen_hi) {
   const int row = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+  if (row_req) {      // rows of requests that another launch serves have no partial results
+    const int b = row_req[row];
+    if (q_start[b + 1] - q_start[b] > qlen_hi) return;
+  }
   const size_t at0 = ((size_t)row * nq + head) * splits;
   float ms = NEG_INF, ls = 0.f;
   if (lane < splits) {
@@ -680,16 +689,67 @@ extern "C" const char* llmlab_last_error() { return g_llmlab_error; }
 
 extern "C" int llmlab_attention_head_dim() { return D; }
 
+// The decode-like launch: a block of DECODE_WAVES waves per (request, kv head, split); a
+// wave gets about two steps of 32 keys, a block's waves merge in LDS, and only what is
+// left is split over blocks; the merge kernel follows.  `live` requests (of `reqs`) pass
+// the filter of `a`, `ctx_len` is their longest context.
+static int launch_key_split_decode(AttnArgs a, int reqs, int live, int ctx_len, int window, int total_rows,
+                                   int nq, int nkv, float* workspace, size_t workspace_floats, int num_cus,
+                                   const int* row_req, void* out, int out_stride, hipStream_t stream) {
+  const int visible = window > 0 ? min(window, ctx_len) : ctx_len;
+  const int steps32 = (visible + 31) / 32 + 1;
+  // about SPLIT_FILL blocks per compute unit: a unit's memory rate is the limit, so
+  // the keys are spread over all of them; but no more blocks than there are steps
+  // for their waves
+  const long base = (long)live * nkv;
+#ifndef SPLIT_DIV
+#define SPLIT_DIV 1
+#endif
+  int splits = (int)((SPLIT_FILL * (long)num_cus / SPLIT_DIV + base - 1) / base);
+  const int most = (steps32 + DECODE_WAVES - 1) / DECODE_WAVES;      // one step per wave at least
+  if (splits > most) splits = most;
+  if (splits > 16) splits = 16;                               // what the merge kernel takes
+  if (splits < 1) splits = 1;
+  const size_t per_split = (size_t)total_rows * nq * (D + 2);
+  while (splits > 1 && per_split * splits > workspace_floats) --splits;
+  if (splits < 1) splits = 1;
+  a.splits = splits;
+  if (splits > 1) {
+    a.o_part = workspace;
+    a.ml_part = workspace + (size_t)total_rows * nq * splits * D;
+  }
+  dim3 grid(1, nkv * splits, reqs), block(64 * DECODE_WAVES);
+  const int steps_per_wave = ((steps32 + splits - 1) / splits + DECODE_WAVES - 1) / DECODE_WAVES;
+  if (steps_per_wave > 2)
+    hipLaunchKernelGGL((attention_bf16_kernel<1, true, 2>), grid, block, 0, stream, a);
+  else
+    hipLaunchKernelGGL((attention_bf16_kernel<1, true, 1>), grid, block, 0, stream, a);
+  LLMLAB_LAUNCH_CHECK("attention(bfloat16, decode)");
+  if (splits > 1) {
+    hipLaunchKernelGGL(attention_merge_kernel, dim3(total_rows, nq), dim3(64), 0, stream, a.o_part,
+                       a.ml_part, (bf16_t*)out, out_stride, nq, splits, row_req, a.q_start, a.qlen_hi);
+    LLMLAB_LAUNCH_CHECK("attention merge");
+  }
+  return 0;
+}
+
 // q rows are the step's packed rows; reqs requests; max_q_len / max_ctx_len are
 // the largest portion and the longest context in the step (they size the grid
 // and choose the key splits).  workspace: float32 scratch for split partials.
+// A mixed step (portions of prompts beside single decoded tokens) may say so:
+// n_short of its requests bring at most short_len tokens each, the longest context
+// among those is short_ctx, and row_req[row] is the request of a row.  Its short
+// requests are then served by the decode-like launch and the others by the tiled one;
+// in one launch the few rows of a decoding request would walk its whole history in
+// one wave while the rest of the chip waits.
 extern "C" int llmlab_paged_attention(const void* q, int dtype, int q_stride, int nq, int nkv,
                                       const void* kcache, const void* vcache, const int* table,
                                       int table_stride, int page_size, const int* q_start,
                                       const int* start_pos, int reqs, int max_q_len, int max_ctx_len,
                                       int window, float scale, void* out, int out_stride,
                                       float* workspace, size_t workspace_floats, int total_rows,
-                                      int num_cus, hipStream_t stream) {
+                                      int num_cus, const int* row_req, int short_len, int n_short,
+                                      int short_ctx, hipStream_t stream) {
   LLMLAB_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0, "attention: %d heads, %d kv heads", nq, nkv);
   LLMLAB_REQUIRE(page_size >= 16 && (page_size & (page_size - 1)) == 0,
                  "attention: page size %d is not a power of two >= 16", page_size);
@@ -697,6 +757,8 @@ extern "C" int llmlab_paged_attention(const void* q, int dtype, int q_stride, in
   LLMLAB_REQUIRE(reqs >= 0 && reqs <= 65535 && nq <= 65535, "attention: grid too large");
   LLMLAB_REQUIRE(window >= 0, "attention: negative window");
   LLMLAB_REQUIRE(scale > 0.f, "attention: the score scale must be positive, got %g", (double)scale);
+  LLMLAB_REQUIRE(n_short >= 0 && n_short <= reqs && short_len >= 0 && short_ctx >= 0 && short_ctx <= max_ctx_len,
+                 "attention: bad description of the short requests");
   if (reqs == 0 || max_q_len <= 0) return 0;
   if (num_cus <= 0) num_cus = 256;
   AttnArgs a;
@@ -706,6 +768,7 @@ extern "C" int llmlab_paged_attention(const void* q, int dtype, int q_stride, in
   a.nq = nq; a.nkv = nkv; a.window = window; a.splits = 1; a.scale = scale;
   a.page_shift = 0;
   a.tiles = 0;
+  a.qlen_lo = 0; a.qlen_hi = 0x7fffffff;
   while ((1 << a.page_shift) < page_size) ++a.page_shift;
   if (dtype == DT_F32) {
     dim3 grid(max_q_len, nq, reqs), block(64);
@@ -718,51 +781,25 @@ extern "C" int llmlab_paged_attention(const void* q, int dtype, int q_stride, in
                  "attention(bfloat16): operands are not aligned for vector loads");
   const int G = nq / nkv;
   const long max_rows = (long)max_q_len * G;
-  if (max_rows <= 16) {
-    // decode-like step: a block of DECODE_WAVES waves per (request, kv head, split);
-    // a wave gets about two steps of 32 keys, a block's waves merge in LDS, and only
-    // what is left is split over blocks
-    const int visible = window > 0 ? min(window, max_ctx_len) : max_ctx_len;
-    const int steps32 = (visible + 31) / 32 + 1;
-    // about SPLIT_FILL blocks per compute unit: a unit's memory rate is the limit, so
-    // the keys are spread over all of them; but no more blocks than there are steps
-    // for their waves
-    const long base = (long)reqs * nkv;
-#ifndef SPLIT_DIV
-#define SPLIT_DIV 1
-#endif
-    int splits = (int)((SPLIT_FILL * (long)num_cus / SPLIT_DIV + base - 1) / base);
-    const int most = (steps32 + DECODE_WAVES - 1) / DECODE_WAVES;      // one step per wave at least
-    if (splits > most) splits = most;
-    if (splits > 16) splits = 16;                               // what the merge kernel takes
-    if (splits < 1) splits = 1;
-    const size_t per_split = (size_t)total_rows * nq * (D + 2);
-    while (splits > 1 && per_split * splits > workspace_floats) --splits;
-    if (splits < 1) splits = 1;
-    a.splits = splits;
-    if (splits > 1) {
-      a.o_part = workspace;
-      a.ml_part = workspace + (size_t)total_rows * nq * splits * D;
-    }
-    dim3 grid(1, nkv * splits, reqs), block(64 * DECODE_WAVES);
-    const int steps_per_wave = ((steps32 + splits - 1) / splits + DECODE_WAVES - 1) / DECODE_WAVES;
-    if (steps_per_wave > 2)
-      hipLaunchKernelGGL((attention_bf16_kernel<1, true, 2>), grid, block, 0, stream, a);
-    else
-      hipLaunchKernelGGL((attention_bf16_kernel<1, true, 1>), grid, block, 0, stream, a);
-    LLMLAB_LAUNCH_CHECK("attention(bfloat16, decode)");
-    if (splits > 1) {
-      hipLaunchKernelGGL(attention_merge_kernel, dim3(total_rows, nq), dim3(64), 0, stream, a.o_part,
-                         a.ml_part, (bf16_t*)out, out_stride, nq, splits);
-      LLMLAB_LAUNCH_CHECK("attention merge");
-    }
-    return 0;
+  if (max_rows <= 16)
+    return launch_key_split_decode(a, reqs, reqs, max_ctx_len, window, total_rows, nq, nkv, workspace,
+                                   workspace_floats, num_cus, nullptr, out, out_stride, stream);
+  int live = reqs;
+  if (row_req != nullptr && n_short > 0 && n_short < reqs && (long)short_len * G <= 16) {
+    AttnArgs s = a;
+    s.qlen_hi = short_len;
+    const int rc = launch_key_split_decode(s, reqs, n_short, short_ctx, window, total_rows, nq, nkv,
+                                           workspace, workspace_floats, num_cus, row_req, out, out_stride,
+                                           stream);
+    if (rc) return rc;
+    a.qlen_lo = short_len + 1;
+    live = reqs - n_short;
   }
   // Few tiles of rows (a short portion, with or without a long history behind it):
   // the waves of a block split the keys of one tile of 32 rows and merge in LDS, so
   // that the work still spreads over the chip.  Else every wave owns its rows and
   // the block's waves share the keys through LDS.
-  const long blocks16 = ((max_rows + 63) / 64) * nkv * reqs;
+  const long blocks16 = ((max_rows + 63) / 64) * nkv * live;
   if (blocks16 < num_cus) {
     const int steps32 = (max_ctx_len + 31) / 32 + 1;
     const int steps_per_wave = (steps32 + DECODE_WAVES - 1) / DECODE_WAVES;
@@ -776,7 +813,7 @@ extern "C" int llmlab_paged_attention(const void* q, int dtype, int q_stride, in
   }
   // rows per wave: 32 when that still gives every compute unit two blocks (or for
   // nothing smaller), else 16; always 16 for the largest heads (registers)
-  const long blocks32 = ((max_rows + 127) / 128) * nkv * reqs;
+  const long blocks32 = ((max_rows + 127) / 128) * nkv * live;
   if (D <= 128 && blocks32 >= 2L * num_cus) {
     dim3 grid((unsigned)((max_rows + 127) / 128), nkv, reqs), block(256);
     hipLaunchKernelGGL((attention_bf16_kernel<2, false>), grid, block, 0, stream, a);

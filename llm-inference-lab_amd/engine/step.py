@@ -90,6 +90,7 @@ class StepContext:
         self.scratch_version = 0
         self.n_rows = self.n_reqs = self.n_want = 0
         self.max_q_len = self.max_ctx_len = 0
+        self._short = {}
         self.pending = None            # PendingSums owed to the residual stream, within a forward
         self.host_q_start: List[int] = []
         self.host_start_pos: List[int] = []
@@ -126,6 +127,20 @@ class StepContext:
             self.scratch_version += 1
         return buf[:count].view(shape)
 
+    def short_requests(self, limit: int) -> Tuple[int, int]:
+        """How many of this step's requests bring at most ``limit`` tokens, and the
+        longest context among those (0 if none)."""
+        hit = self._short.get(limit)
+        if hit is None:
+            count = longest = 0
+            for b in range(self.n_reqs):
+                n = self.host_q_start[b + 1] - self.host_q_start[b]
+                if n <= limit:
+                    count += 1
+                    longest = max(longest, self.host_start_pos[b] + n)
+            hit = self._short[limit] = (count, longest)
+        return hit
+
     # ------------------------------------------------------------------ fill
     def fill(self, entries: Sequence[StepEntry], cache: CacheManager) -> None:
         n_rows = sum(len(e.tokens) for e in entries)
@@ -143,6 +158,7 @@ class StepContext:
         feeds: List[Tuple[int, int]] = []
         feed_tensor = None
         self.host_q_start, self.host_start_pos, self.host_req_rows = [], [], []
+        self._short = {}
         max_q = max_ctx = 0
         for b, e in enumerate(entries):
             n = len(e.tokens)

@@ -76,6 +76,8 @@ class HipOps:
         if self.device.type != "cuda":
             raise RuntimeError(f"the kernels need a GPU device, got '{device}'")
         torch.cuda.set_device(self.device)
+        if self.device.index is None:
+            self.device = torch.device("cuda", torch.cuda.current_device())
         self._core = self._load(build.core_library())
         self._declare_core()
         if self._core.llmlab_abi_version() != 4:
@@ -140,7 +142,7 @@ class HipOps:
             lib.llmlab_paged_attention.argtypes = [
                 _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr,
                 _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_float, _c_ptr, _c_int, _c_ptr, _c_size,
-                _c_int, _c_int, _c_ptr]
+                _c_int, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_ptr]
             lib.llmlab_paged_attention.restype = _c_int
             self._attn[head_dim] = lib
             self.loaded_libraries.append(lib._name)
@@ -207,6 +209,11 @@ class HipOps:
 
     # ---------------------------------------------------------------- helpers
     def _stream(self):
+        # the raw handle of the current stream (under graph capture: the capturing one);
+        # asked for at every launch, so by the short way where torch has one
+        raw = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+        if raw is not None:
+            return _c_ptr(raw(self.device.index))
         return _c_ptr(torch.cuda.current_stream(self.device).cuda_stream)
 
     def _check(self, code: int, lib=None) -> None:
@@ -609,13 +616,25 @@ class HipOps:
         if page_size < 16 or page_size & (page_size - 1):
             raise UnsupportedSizeError(f"page size {page_size} is not a power of two >= 16")
         q_stride = qkv.stride(0) if rows > 1 else qkv.shape[1]
+        # a mixed step: its requests of a few tokens (decoding ones) go to the launch that
+        # splits their keys over the chip, the portions of prompts to the tiled one
+        row_req, short_len, n_short, short_ctx = None, 0, 0, 0
+        group = num_heads // num_kv_heads
+        if (ctx is not None and qkv.dtype == torch.bfloat16 and group <= 16 < max_q_len * group
+                and hasattr(ctx, "short_requests")):
+            n_short, short_ctx = ctx.short_requests(16 // group)
+            if 0 < n_short < n_reqs:
+                row_req, short_len = ctx.row_req, 16 // group
+                self._need(row_req, "row -> request map", torch.int32)
+            else:
+                n_short = short_ctx = 0
         self._check(lib.llmlab_paged_attention(
             self._ptr(qkv), _dt(qkv), q_stride, num_heads, num_kv_heads, self._ptr(k_cache),
             self._ptr(v_cache), self._ptr(block_table), block_table.stride(0), page_size,
             self._ptr(q_start), self._ptr(start_pos), n_reqs, max_q_len, max_ctx_len,
             int(window) if window else 0, float(scale), self._ptr(out), out.stride(0) if rows > 1 else
             out.shape[1], self._ptr(self.workspace), self.workspace.numel(), rows, self.num_cus,
-            self._stream()), lib)
+            self._ptr(row_req), short_len, n_short, short_ctx, self._stream()), lib)
 
     # --------------------------------------------------------------- sampling
     def argmax(self, logits, out) -> None:

@@ -292,6 +292,16 @@ def test_qkv_rope_cache_of_normed_rows(ops, emu, nq, nkv, d, page, hidden, rows_
     assert torch.equal(got_k.cpu()[untouched], kc[untouched])
 
 
+@pytest.mark.parametrize("window", [None, 40])
+def test_attention_of_a_mixed_step(ops, emu, window):
+    """Portions of prompts beside decoding requests with long histories, one of which has a
+    key that stands out far back."""
+    spec = [(700, 1), (64, 300), (1500, 1), (0, 1), (31, 2), (200, 90), (999, 1)]
+    run_attention(ops, emu, torch.bfloat16, 14, 2, 64, 64, window, spec, seed=90, amplify=(2, 100 if window is None else 1480, 30.0))
+    run_attention(ops, emu, torch.bfloat16, 6, 3, 48, 16, window, spec[:5], seed=91)
+    run_attention(ops, emu, torch.bfloat16, 8, 1, 128, 32, window, spec[:4], seed=92)
+
+
 def make_cache(num_pages, nkv, page, d, dtype, seed):
     k = rnd((num_pages, nkv, page, d), dtype, seed)
     v = rnd((num_pages, nkv, d, page), dtype, seed + 1)
@@ -377,6 +387,23 @@ def run_attention(ops, emu, dtype, nq, nkv, d, page, window, reqs_spec, seed=30,
     tol = 2e-5 if dtype == torch.float32 else 2e-2
     err = (got.float().cpu() - want.float()).abs().max().item()
     assert err <= tol * max(1.0, want.float().abs().max().item()), f"attention error {err}"
+
+    # the same step described as the engine describes it (which requests are short): a
+    # mixed step is then served by two launches
+    class Described:
+        row_req = torch.cat([torch.full((n,), b) for b, (_, n) in enumerate(reqs_spec)]).int().to(DEV)
+
+        @staticmethod
+        def short_requests(limit):
+            short = [(s, n) for s, n in reqs_spec if n <= limit]
+            return len(short), max((s + n for s, n in short), default=0)
+
+    got2 = torch.zeros(rows, nq * d, dtype=dtype, device=DEV)
+    ops.paged_attention(qkv.to(DEV), nq, nkv, d, kc.to(DEV), vc.to(DEV), table.to(DEV), page,
+                        q_start_t.to(DEV), start_pos_t.to(DEV), reqs, max(n for _, n in reqs_spec),
+                        max_ctx, window, scale, got2, Described())
+    err = (got2.float().cpu() - want.float()).abs().max().item()
+    assert err <= tol * max(1.0, want.float().abs().max().item()), f"attention error {err} (described step)"
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
