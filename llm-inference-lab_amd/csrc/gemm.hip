@@ -20,12 +20,13 @@
 //
 // Epilogues: STORE  out[M,N] (T) = acc (+bias)            RESID  out[M,N] (f32) += acc (+bias)
 //            F32    out[M,N] (f32) = acc                   SWIGLU out[M,N/2] (T) = silu(g)*u
+//            PART   out[z][M,N] (f32) = acc over the K range of group z
 // For SWIGLU the rows of W alternate in runs of 16: gate rows of 16 outputs, then
 // the up rows of the same 16 outputs, so fragments j and j+1 hold gate and up of
 // the same outputs in the same lanes.
 #include "common.h"
 
-enum { EPI_STORE = 0, EPI_RESID = 1, EPI_F32 = 2, EPI_SWIGLU = 3 };
+enum { EPI_STORE = 0, EPI_RESID = 1, EPI_F32 = 2, EPI_SWIGLU = 3, EPI_PART = 5 };
 
 struct EpiArgs {
   void* out;         // T or float, see above
@@ -33,6 +34,11 @@ struct EpiArgs {
   int bias_bf16;
   int ldo;    // row stride of out in elements
   int n_out;  // logical output columns (SWIGLU: intermediate size; else N)
+  // PART: the inner size is cut over the blocks of grid z, kt_per_split K tiles each; group z
+  // leaves its sums (float32, bias in group 0) in out + z * part_stride: the product without
+  // the final sum, which the next reader of those rows does
+  int kt_per_split;
+  size_t part_stride;
 };
 
 __device__ __forceinline__ float silu_f(float z) { return z / (1.f + __expf(-z)); }
@@ -154,15 +160,24 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __
     }
   };
 
-  const int nk = (K + BK - 1) / BK;
+  // this block's K tiles: all of them, or (PART) its group's share starting at tile kt0
+  // (tiles past the share are fetched like any other and never multiplied)
+  int nk = (K + BK - 1) / BK, kt0 = 0;
+  if constexpr (EPI == EPI_PART) {
+    kt0 = (int)blockIdx.z * e.kt_per_split;
+    nk = max(0, min(nk - kt0, e.kt_per_split));
+    e.out = (float*)e.out + (size_t)blockIdx.z * e.part_stride;
+    if (blockIdx.z > 0) e.bias = nullptr;
+  }
+  const int kbase = kt0 * BK;
 #pragma unroll
   for (int p = 0; p < PD; ++p) {      // past K: zeros for W
-    fetch(p, p * BK);
-    if constexpr (BDIRECT) fetch_b(p, p * BK);
+    fetch(p, kbase + p * BK);
+    if constexpr (BDIRECT) fetch_b(p, kbase + p * BK);
   }
   // tile kt lies in stage kt & 1; it was put there during tile kt - 1 (tile 0: now)
   stash(0, 0);
-  fetch(0, PD * BK);
+  fetch(0, kbase + PD * BK);
   __syncthreads();
   for (int kt = 0; kt < nk; kt += PD) {
 #pragma unroll
@@ -172,7 +187,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __
       const int stage = t & 1;
       const int pn = (p + 1) % PD;              // ring slot of tile t + 1 (a constant once unrolled)
       if (t + 1 < nk) stash(pn, stage ^ 1);
-      fetch(pn, (t + 1 + PD) * BK);
+      fetch(pn, kbase + (t + 1 + PD) * BK);
       if (live) {
         const bf16_t* As = As2 + stage * A_STAGE;
         const bf16_t* Bs = Bs2 + stage * B_STAGE;
@@ -195,7 +210,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __
         }
         __syncthreads();
       }
-      if constexpr (BDIRECT) fetch_b(p, (t + PD) * BK);
+      if constexpr (BDIRECT) fetch_b(p, kbase + (t + PD) * BK);
     }
   }
 
@@ -306,6 +321,27 @@ static int launch_bf16(const bf16_t* A, const bf16_t* W, EpiArgs e, int M, int N
   return 0;
 }
 
+// parts[z] = x[:, K_z] . W[:, K_z]^T for `ksplit` ranges K_z of the inner size (whole K
+// tiles of 64 each); bias in parts[0].  bfloat16 only; for products whose output gives
+// the large tile too few blocks to fill the chip.
+extern "C" int llmlab_linear_partials(const void* x, const void* w, float* parts, const void* bias,
+                                      int bias_dtype, int M, int N, int K, int ldo, int ksplit,
+                                      size_t part_stride, hipStream_t stream) {
+  LLMLAB_REQUIRE(M >= 0 && N > 0 && K > 0 && K % 8 == 0, "linear_partials: bad sizes M=%d N=%d K=%d", M, N, K);
+  LLMLAB_REQUIRE(ksplit >= 1 && ksplit <= 16 && ldo >= N && part_stride >= (size_t)M * ldo,
+                 "linear_partials: %d pieces, row stride %d", ksplit, ldo);
+  LLMLAB_REQUIRE(((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0),
+                 "linear_partials: operands must be 16-byte aligned");
+  if (M == 0) return 0;
+  const int nk = (K + 63) / 64;
+  EpiArgs e{parts, bias, bias_dtype == DT_BF16, ldo, N, (nk + ksplit - 1) / ksplit, part_stride};
+  dim3 grid((N + 127) / 128, (M + 127) / 128, ksplit);
+  hipLaunchKernelGGL((gemm_bf16_tiled<128, 128, 64, 2, 2, EPI_PART, false>), grid, dim3(256), 0, stream,
+                     (const bf16_t*)x, (const bf16_t*)w, e, M, N, K);
+  LLMLAB_LAUNCH_CHECK("linear_partials");
+  return 0;
+}
+
 // x [M,K] (dtype), w [N,K] (float32: row-major; bfloat16: packed); epilogue selects what `out` is.  For SWIGLU N
 // is the number of interleaved weight rows (2 * ceil16(n_out)).
 extern "C" int llmlab_linear(const void* x, const void* w, int dtype, int epilogue, void* out,
@@ -322,7 +358,7 @@ extern "C" int llmlab_linear(const void* x, const void* w, int dtype, int epilog
   }
   LLMLAB_REQUIRE(ldo >= n_out, "linear: output row stride %d < %d columns", ldo, n_out);
   if (M == 0) return 0;
-  EpiArgs e{out, bias, bias_dtype == DT_BF16, ldo, n_out};
+  EpiArgs e{out, bias, bias_dtype == DT_BF16, ldo, n_out, 0, 0};
   if (num_cus <= 0) num_cus = 256;
   if (dtype == DT_BF16) {
     LLMLAB_REQUIRE(K % 8 == 0, "linear(bfloat16): inner size %d must be a multiple of 8", K);

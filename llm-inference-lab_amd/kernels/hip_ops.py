@@ -119,6 +119,8 @@ class HipOps:
         c.llmlab_pack_weight.restype = _c_int
         c.llmlab_argmax.argtypes = [_c_ptr, _c_long, _c_int, _c_int, _c_ptr, _c_ptr, _c_size, _c_ptr]
         c.llmlab_argmax.restype = _c_int
+        c.llmlab_linear_partials.argtypes = [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int,
+                                             _c_int, _c_int, _c_size, _c_ptr]
         c.llmlab_skinny_linear.argtypes = [
             _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_float, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr,
             _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
@@ -127,7 +129,8 @@ class HipOps:
         c.llmlab_add_pending.argtypes = [_c_ptr, _c_ptr, _c_int, _c_size, _c_int, _c_int, _c_ptr]
         c.llmlab_add_pending.restype = _c_int
         for fn in (c.llmlab_embed, c.llmlab_rmsnorm, c.llmlab_rope_kv_write, c.llmlab_rope_inplace,
-                   c.llmlab_linear, c.llmlab_sample, c.llmlab_skinny_linear):
+                   c.llmlab_linear, c.llmlab_sample, c.llmlab_skinny_linear,
+                   c.llmlab_linear_partials):
             fn.restype = _c_int
 
     def _attention_lib(self, head_dim: int) -> ctypes.CDLL:
@@ -392,13 +395,39 @@ class HipOps:
     MAX_SPLITS = 8
     split_max_rows = 32           # most rows of a product that is left in pieces
     min_steps_per_split = 8       # K steps of 32 a piece should have at least (tests lower it)
+    min_tiles_per_split = 8       # many rows: K tiles of 64 a piece should have at least (tests lower it)
 
     def split_count(self, rows: int, dtype, n: int, k: int) -> int:
         """Into how many pieces along the inner size a few-row product ``[rows, k] x
         [n, k]^T`` should be cut so that it spreads over the chip: a narrow output
         gives too few blocks otherwise, and a compute unit draws only so much from
         memory.  1: do not cut."""
-        if dtype != torch.bfloat16 or not 0 < rows <= self.split_max_rows:
+        if dtype != torch.bfloat16 or rows <= 0:
+            return 1
+        if rows > self.FUSED_MAX_ROWS:
+            # many rows, tiled kernel.  Time is rounds of 128 x 128 blocks over the chip times
+            # the K tiles of a block; every piece costs a write and a read of the result.
+            # Fitted to sweeps of the down products of two model shapes (128 to 4096 rows),
+            # where it picks the measured best or its neighbour.  Where the large tile has
+            # too few blocks the small one would run instead, which moves every operand
+            # twice as often: pieces win there whenever K is long enough to cut.
+            if k % 8:
+                return 1
+            tiles = ((rows + 127) // 128) * ((n + 127) // 128)
+            nk = (k + 63) // 64
+            piece = rows * n * 2.2e-6 + 0.3
+            best, best_cost = 1, None
+            if tiles >= self.num_cus:
+                best_cost = -(-tiles // self.num_cus) * nk * 0.65
+            for s in range(2, self.MAX_SPLITS + 1):
+                per = -(-nk // s)
+                if per < self.min_tiles_per_split:
+                    break
+                cost = -(-tiles * s // self.num_cus) * per * 0.65 + s * piece
+                if best_cost is None or cost < best_cost:
+                    best, best_cost = s, cost
+            return best
+        if rows > self.split_max_rows:
             return 1
         strips, steps = (n + 15) // 16, (k + 31) // 32
         want = self.num_cus // max(strips, 1)
@@ -416,10 +445,18 @@ class HipOps:
                 or parts.device != self.device):
             raise ValueError(f"linear_partials: x {tuple(x.shape)}, w {tuple(w.shape)}, "
                              f"parts {tuple(parts.shape)} for {splits} pieces do not fit")
-        if not 1 <= splits <= self.MAX_SPLITS or m > self.FUSED_MAX_ROWS:
-            raise ValueError(f"linear_partials: {splits} pieces of {m} rows")
-        self._skinny(x, False, None, None, 0.0, w, bias, EPI_PART, parts, m, n, k, parts.stride(1), n,
-                     ksplit=splits, part_stride=parts.stride(0))
+        if not 1 <= splits <= self.MAX_SPLITS:
+            raise ValueError(f"linear_partials: {splits} pieces")
+        if m <= self.FUSED_MAX_ROWS:
+            self._skinny(x, False, None, None, 0.0, w, bias, EPI_PART, parts, m, n, k, parts.stride(1), n,
+                         ksplit=splits, part_stride=parts.stride(0))
+        else:
+            if bias is not None:
+                self._need(bias, "bias")
+            self._check(self._core.llmlab_linear_partials(
+                self._ptr(x), self._ptr(w), self._ptr(parts), self._ptr(bias),
+                _dt(bias) if bias is not None else 0, m, n, k, parts.stride(1), splits, parts.stride(0),
+                self._stream()))
         return PendingSums(parts, splits)
 
     def add_pending(self, x: torch.Tensor, pending: PendingSums) -> None:

@@ -87,13 +87,15 @@ class EmuOps:
         return max(1, min(self.num_cus // max(strips, 1), steps // self.min_steps_per_split, self.MAX_SPLITS))
 
     def linear_partials(self, x, w, parts, splits, bias=None):
-        """Piece s covers the K steps of 32 from s * ceil(steps / splits) on."""
+        """Piece s covers the K steps from s * ceil(steps / splits) on; a step is 32 wide
+        for up to 64 rows and 64 wide for more (the two kernels' K tiles)."""
         self._count("linear_partials")
         k = x.shape[1]
-        steps = (k + 31) // 32
+        width = 32 if x.shape[0] <= 64 else 64
+        steps = (k + width - 1) // width
         per = (steps + splits - 1) // splits
         for s in range(splits):
-            lo, hi = min(k, s * per * 32), min(k, (s + 1) * per * 32)
+            lo, hi = min(k, s * per * width), min(k, (s + 1) * per * width)
             parts[s] = x[:, lo:hi].float() @ w[:, lo:hi].float().t()
         if bias is not None:
             parts[0] += bias.float()

@@ -65,6 +65,23 @@ def test_sums_left_in_pieces_reach_every_reader(name, cut):
     assert bad is None, f"first wrong logits at (request, position, error) = {bad}"
 
 
+@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("cut", ["whole", "decode"])
+def test_sums_of_many_rows_left_in_pieces(name, cut):
+    """The same for steps of many rows (tiled product cut along its inner size): the next
+    layer's norm folds the pieces into the stream as it reads it, the final norm of
+    gathered rows has them folded first."""
+    seqs = sequences_of(name)
+    want = {rid: H.plain_logits(name, 1, ids) for rid, ids in seqs.items()}
+    engine = H.make_engine(name, 1, "bf16", page_size=16, num_pages=40, max_requests=4)
+    engine.ops.min_tiles_per_split = 1
+    cfg = H.config_of(name)
+    assert engine.ops.split_count(130, torch.bfloat16, cfg.hidden_size, cfg.intermediate_size) > 1
+    got = H.run_trace(engine, seqs, CUTS[cut](seqs))
+    bad = H.first_wrong(got, want, H.TOL["bf16"])
+    assert bad is None, f"first wrong logits at (request, position, error) = {bad}"
+
+
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 def test_cuts_agree_with_each_other_more_closely_than_with_plain(dtype):
     """The logits at a position do not depend on how the tokens were cut, beyond rounding."""

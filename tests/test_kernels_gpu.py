@@ -539,7 +539,8 @@ def test_cache_order_round_trip(page, d):
 
 
 @pytest.mark.parametrize("m,n,k,splits", [(8, 896, 4864, 4), (1, 896, 896, 3), (16, 90, 512, 2), (5, 130, 264, 1),
-                                          (40, 896, 512, 2), (64, 130, 264, 3)])
+                                          (40, 896, 512, 2), (64, 130, 264, 3), (200, 896, 4864, 4),
+                                          (577, 300, 1160, 3), (130, 64, 72, 2)])
 def test_linear_partials_and_pending(ops, emu, m, n, k, splits):
     """A product left in pieces along K; the pieces added on the fly where the rows are
     read (fused norm + product), folded in where a product adds into them, or folded
@@ -564,8 +565,17 @@ def test_linear_partials_and_pending(ops, emu, m, n, k, splits):
     ops.linear_residual(x2.to(DEV), ops.prepare_weight(w2.to(DEV)), got, pending=pending)
     want = resid + want_parts[:splits].sum(0) + x2.float() @ w2.float().t()
     close(got, want, torch.float32, "fold with a product", want.abs().max().item())
+    # folded in by a stand-alone norm of the rows
+    nw32 = 1 + 0.1 * rnd((n,), torch.float32, 88)
+    got, normed = resid.clone().to(DEV), torch.empty(m, n, dtype=bf, device=DEV)
+    ops.rmsnorm(got, nw32.to(DEV), 1e-6, normed, pending=pending)
+    whole_rows = resid + want_parts[:splits].sum(0)
+    close(got, whole_rows, torch.float32, "fold under a norm", 4.0)
+    want_n = torch.empty(m, n, dtype=bf)
+    emu.rmsnorm(whole_rows, nw32, 1e-6, want_n)
+    close(normed, want_n, bf, "norm of the folded rows", 4.0)
     # added on the fly by a fused norm + product that reads the rows (n must fit the norm: use n wide rows)
-    if n % 8 == 0:
+    if n % 8 == 0 and m <= 64:
         nw = (1 + 0.1 * rnd((n,), torch.float32, 86)).to(bf)
         w3 = rnd((48, n), bf, 87, 0.1)
         logits = torch.zeros(m, 48, device=DEV)
