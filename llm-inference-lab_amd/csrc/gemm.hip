@@ -9,7 +9,9 @@
 //       too (in fragment order, as it lies in memory) or read straight into
 //       registers; three or four tiles are on their way from memory in a ring of
 //       register buffers while one is multiplied.  Measured and not adopted: 256x128
-//       tiles with eight 64x64 or four 128x64 wave tiles, K steps of 128.
+//       tiles with eight 64x64 or four 128x64 wave tiles, K steps of 128, and 256x256
+//       tiles with four 128x128 wave tiles (half the LDS traffic per product, one wave
+//       per SIMD: 833 against 793 TF/s on the largest product tried, slower on the rest).
 //     (products of few rows, as in decode steps, have kernels of their own in decode.hip)
 //   float32: a plain FMA kernel (64x64 tile, 4x4 outputs per thread): true 32-bit
 //     products and sums, no matrix-core shortcut.
@@ -303,12 +305,16 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__
 }
 
 // ================================================================ dispatch
+// A tile can be forced for measurements (0 = choose; 64, 128).
+static int g_force_tile = 0;
+extern "C" void llmlab_gemm_force(int tile) { g_force_tile = tile; }
+
 template <int EPI>
 static int launch_bf16(const bf16_t* A, const bf16_t* W, EpiArgs e, int M, int N, int K, int num_cus,
                        hipStream_t stream) {
   // the large tile when it still fills the chip, else the small one
   const long big_tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
-  if (big_tiles >= num_cus) {
+  if (g_force_tile != 64 && (big_tiles >= num_cus || g_force_tile == 128)) {
     dim3 grid((N + 127) / 128, (M + 127) / 128);
     hipLaunchKernelGGL((gemm_bf16_tiled<128, 128, 64, 2, 2, EPI, false>), grid, dim3(256), 0, stream, A, W, e, M, N, K);
   } else {
