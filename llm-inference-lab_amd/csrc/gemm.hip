@@ -73,8 +73,13 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __
   // two stages of LDS: the next tile is put in while this one is multiplied, one
   // barrier per tile
   constexpr int A_STAGE = BM * LDS_STRIDE, B_STAGE = BDIRECT ? 8 : BN * BK;
-  __shared__ __attribute__((aligned(16))) bf16_t As2[2 * A_STAGE];
-  __shared__ __attribute__((aligned(16))) bf16_t Bs2[2 * B_STAGE];
+  // (one array: after the last tile it holds the block's results for the epilogue)
+  constexpr int C_STRIDE = BN + 4;           // floats per row of the result tile in LDS
+  constexpr size_t STAGE_BYTES = (size_t)(2 * A_STAGE + 2 * B_STAGE) * sizeof(bf16_t);
+  constexpr size_t C_BYTES = (size_t)BM * C_STRIDE * sizeof(float);
+  __shared__ __attribute__((aligned(16))) char smem[STAGE_BYTES > C_BYTES ? STAGE_BYTES : C_BYTES];
+  bf16_t* As2 = (bf16_t*)smem;
+  bf16_t* Bs2 = As2 + 2 * A_STAGE;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / WN, wn = wave % WN;
@@ -216,24 +221,77 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __
     }
   }
 
+  // ---- epilogue.  The results go through LDS so that global memory is written (and the
+  // residual read) in pieces of 16 bytes, consecutive lanes next to each other: straight
+  // from the MFMA layout a wave instruction would touch 32 bytes in each of four rows.
+  // (Every live tile ended with a barrier, so the stages are free.)
+  float* Cs = (float*)smem;
 #pragma unroll
-  for (int i = 0; i < TM; ++i) {
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < TN; ++j) {
-      const int nb = n0 + wn * WTN + j * 16;
+    for (int j = 0; j < TN; ++j)
 #pragma unroll
-      for (int x = 0; x < 4; ++x) {
-        const int m = m0 + wm * WTM + i * 16 + g * 4 + x;
-        if (m >= M) continue;
-        if constexpr (EPI == EPI_SWIGLU) {
-          if (j & 1) continue;
-          const int o = (nb >> 5) * 16 + c;
-          if (o < e.n_out)
-            ((bf16_t*)e.out)[(size_t)m * e.ldo + o] =
-                (bf16_t)(silu_f(acc[i][j][x]) * acc[i][j | 1][x]);
+      for (int x = 0; x < 4; ++x)
+        Cs[(wm * WTM + i * 16 + g * 4 + x) * C_STRIDE + wn * WTN + j * 16 + c] = acc[i][j][x];
+  __syncthreads();
+  if constexpr (EPI == EPI_SWIGLU) {
+    // columns of the tile alternate in runs of 16: gate, up of the same 16 outputs
+    constexpr int OUTS = BN / 2, CH = OUTS / 8;      // outputs per row of the tile, chunks of 8 of them
+    bf16_t* out = (bf16_t*)e.out;
+    const int o0 = n0 >> 1;
+    const bool vec = (e.ldo & 7) == 0 && ((uintptr_t)out & 15) == 0;
+    for (int ch = tid; ch < BM * CH; ch += NT) {
+      const int row = ch / CH, oc = (ch % CH) * 8;      // 8 outputs within one run of 16
+      const int m = m0 + row;
+      if (m >= M) continue;
+      const float* gp = Cs + row * C_STRIDE + (oc >> 4) * 32 + (oc & 15);
+      const floatx4 g0 = *(const floatx4*)gp, g1 = *(const floatx4*)(gp + 4);
+      const floatx4 u0 = *(const floatx4*)(gp + 16), u1 = *(const floatx4*)(gp + 20);
+      bf16x8 v;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        v[q] = (bf16_t)(silu_f(g0[q]) * u0[q]);
+        v[4 + q] = (bf16_t)(silu_f(g1[q]) * u1[q]);
+      }
+      bf16_t* dst = out + (size_t)m * e.ldo + o0 + oc;
+      if (vec && o0 + oc + 8 <= e.n_out) *(bf16x8*)dst = v;
+      else
+        for (int q = 0; q < 8; ++q)
+          if (o0 + oc + q < e.n_out) dst[q] = v[q];
+    }
+  } else {
+    constexpr int CH = BN / 4;                         // chunks of 4 columns per row of the tile
+    constexpr bool OUT32 = EPI != EPI_STORE;
+    const bool vec = (e.ldo & 3) == 0 && ((uintptr_t)e.out & 15) == 0 && (OUT32 || (e.ldo & 7) == 0);
+    for (int ch = tid; ch < BM * CH; ch += NT) {
+      const int row = ch / CH, col = (ch % CH) * 4;
+      const int m = m0 + row, n = n0 + col;
+      if (m >= M || n >= N) continue;
+      floatx4 v = *(const floatx4*)(Cs + row * C_STRIDE + col);
+      if (e.bias)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) v[q] += load_vec(e.bias, e.bias_bf16, min(n + q, N - 1));
+      const size_t at = (size_t)m * e.ldo + n;
+      const bool whole = vec && n + 4 <= N;
+      if constexpr (EPI == EPI_STORE) {
+        bf16_t* dst = (bf16_t*)e.out + at;
+        if (whole) {
+          bf16x4 o;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) o[q] = (bf16_t)v[q];
+          *(bf16x4*)dst = o;
         } else {
-          const int n = nb + c;
-          if (n < N) epi_store<bf16_t, EPI>(e, m, n, acc[i][j][x]);
+          for (int q = 0; q < 4; ++q)
+            if (n + q < N) dst[q] = (bf16_t)v[q];
+        }
+      } else {
+        float* dst = (float*)e.out + at;
+        if (whole) {
+          if constexpr (EPI == EPI_RESID) v += *(const floatx4*)dst;
+          *(floatx4*)dst = v;
+        } else {
+          for (int q = 0; q < 4; ++q)
+            if (n + q < N) dst[q] = (EPI == EPI_RESID ? dst[q] : 0.f) + v[q];
         }
       }
     }
