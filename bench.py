@@ -9,7 +9,9 @@ batch 8, context 4096, bfloat16.  A "step" is one decode step of the whole
 batch through the scheduler's own path (step function + sampling, tokens fed
 back).  One JSON line is printed: decoded tokens a second as ``value``, plus
 ``prefill`` (one 2,048-token prompt), ``roofline`` (bytes the decode step has to
-read over its time against 8 TB/s) and ``points`` (decode at batch 1 and 64).
+read over its time against 8 TB/s), ``points`` (decode at batch 1 and 64), ``step_ms`` (median
+and 95th percentile of single steps timed through GPU completion) and ``eager`` (the
+same decode steps without the HIP graph).
 
 ``--mixed``: many requests with prompts of different lengths go through the
 scheduler with a small token budget, so that portions of prompts run beside the
@@ -201,6 +203,27 @@ def main():
         assert engine.cache.live_requests == 0
         return seconds, live_tokens
 
+    def step_latencies(batch, steps=32):
+        """Single decode steps, each timed through GPU completion: (p50, p95) in ms."""
+        outputs = batch * context // FILL_TOKENS + 2 + 4 + steps + 1
+        sched = engine.scheduler(max_batch_tokens=FILL_TOKENS)
+        for b in range(batch):
+            sched.add_request(random_ids(context - outputs), SamplingConfig(max_new_tokens=outputs, eos_token_id=[]))
+        while any(not r.decoding for r in sched.active) or sched.waiting:
+            sched.step()
+        for _ in range(4):
+            sched.step()
+        times = []
+        for _ in range(steps):
+            sync()
+            t0 = time.perf_counter()
+            sched.step()
+            sync()
+            times.append((time.perf_counter() - t0) * 1e3)
+        sched.run()
+        times.sort()
+        return round(times[len(times) // 2], 4), round(times[min(len(times) - 1, int(len(times) * 0.95))], 4)
+
     def prefill_run(tokens=2048, repeats=4):
         times = []
         for _ in range(repeats):
@@ -255,6 +278,14 @@ def main():
             s, _ = decode_run(b, max(8, args.steps // 2), max(2, args.warmup // 2))
             points[f"decode_b{b}"] = round(b * max(8, args.steps // 2) / s, 1)
         result["points"] = points
+        p50, p95 = step_latencies(args.batch)
+        result["step_ms"] = {"p50": p50, "p95": p95}
+        if engine.step_fn.use_graph:      # the same steps launched kernel by kernel
+            engine.step_fn.use_graph = False
+            s, _ = decode_run(args.batch, max(8, args.steps // 2), max(2, args.warmup // 2))
+            engine.step_fn.use_graph = True
+            result["eager"] = {"value": round(args.batch * max(8, args.steps // 2) / s, 1),
+                               "ms_per_step": round(s / max(8, args.steps // 2) * 1e3, 4)}
     print(json.dumps(result))
 
 
