@@ -216,8 +216,8 @@ class HipOps:
         # asked for at every launch, so by the short way where torch has one
         raw = getattr(torch._C, "_cuda_getCurrentRawStream", None)
         if raw is not None:
-            return _c_ptr(raw(self.device.index))
-        return _c_ptr(torch.cuda.current_stream(self.device).cuda_stream)
+            return raw(self.device.index)
+        return torch.cuda.current_stream(self.device).cuda_stream
 
     def _check(self, code: int, lib=None) -> None:
         if code != 0:
@@ -235,7 +235,8 @@ class HipOps:
 
     @staticmethod
     def _ptr(t: Optional[torch.Tensor]):
-        return _c_ptr(t.data_ptr()) if t is not None else _c_ptr(0)
+        # (a plain integer: ctypes makes the pointer argument of it, None is the null pointer)
+        return t.data_ptr() if t is not None else None
 
     def synchronize(self) -> None:
         torch.cuda.synchronize(self.device)
