@@ -23,12 +23,13 @@
 // Epilogues: STORE  out[M,N] (T) = acc (+bias)            RESID  out[M,N] (f32) += acc (+bias)
 //            F32    out[M,N] (f32) = acc                   SWIGLU out[M,N/2] (T) = silu(g)*u
 //            PART   out[z][M,N] (f32) = acc over the K range of group z
+//            QKV    q (T) = rotate(acc + bias); rotated k and v of the rows go to their cache pages
 // For SWIGLU the rows of W alternate in runs of 16: gate rows of 16 outputs, then
 // the up rows of the same 16 outputs, so fragments j and j+1 hold gate and up of
 // the same outputs in the same lanes.
 #include "common.h"
 
-enum { EPI_STORE = 0, EPI_RESID = 1, EPI_F32 = 2, EPI_SWIGLU = 3, EPI_PART = 5 };
+enum { EPI_STORE = 0, EPI_RESID = 1, EPI_F32 = 2, EPI_SWIGLU = 3, EPI_QKV = 4, EPI_PART = 5 };
 
 struct EpiArgs {
   void* out;         // T or float, see above
@@ -41,6 +42,16 @@ struct EpiArgs {
   // the final sum, which the next reader of those rows does
   int kt_per_split;
   size_t part_stride;
+  // QKV: the columns are [q heads | k heads | v heads] of size d; q and k are rotated by
+  // their row's position, q goes to out [M, ldo], k and v into the cache pages of the row's
+  // request (skipped when no cache is given).  A head must lie within one tile (BN % d == 0).
+  const float* inv_freq;   // [d/2] or null (no rotation)
+  const int* positions;    // [M]
+  const int* row_req;      // [M]
+  const int* table;        // block table
+  bf16_t* kcache;
+  bf16_t* vcache;
+  int table_stride, page_size, nq, nkv, d;
 };
 
 __device__ __forceinline__ float silu_f(float z) { return z / (1.f + __expf(-z)); }
@@ -234,7 +245,73 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __
       for (int x = 0; x < 4; ++x)
         Cs[(wm * WTM + i * 16 + g * 4 + x) * C_STRIDE + wn * WTN + j * 16 + c] = acc[i][j][x];
   __syncthreads();
-  if constexpr (EPI == EPI_SWIGLU) {
+  if constexpr (EPI == EPI_QKV) {
+    // a unit of work: four pairs (i .. i+3, and those + d/2) of one head of one row
+    const int d = e.d, dh = d >> 1, heads = BN / d, cpl = dh >> 2;
+    const int units = BM * heads * cpl;
+    const bool vec = (e.ldo & 3) == 0 && ((uintptr_t)e.out & 7) == 0;
+    for (int u = tid; u < units; u += NT) {
+      const int jc = u % cpl, t = u / cpl, hh = t % heads, row = t / heads;
+      const int m = m0 + row, head = n0 / d + hh, i = jc * 4;
+      if (m >= M || head >= e.nq + 2 * e.nkv) continue;
+      const float* src = Cs + row * C_STRIDE + hh * d + i;
+      floatx4 lo = *(const floatx4*)src, hi = *(const floatx4*)(src + dh);
+      if (e.bias)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          lo[q] += load_vec(e.bias, e.bias_bf16, head * d + i + q);
+          hi[q] += load_vec(e.bias, e.bias_bf16, head * d + dh + i + q);
+        }
+      const bool is_q = head < e.nq, is_k = !is_q && head < e.nq + e.nkv;
+      const int pos = e.positions[m];
+      if ((is_q || is_k) && e.inv_freq) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          // the hardware sine and cosine of r = frac(angle / 2 pi)
+          float r = (float)pos * e.inv_freq[i + q] * 0.15915494309189535f;
+          r -= floorf(r);
+          const float sn = __builtin_amdgcn_sinf(r), cs = __builtin_amdgcn_cosf(r);
+          const float nlo = lo[q] * cs - hi[q] * sn, nhi = hi[q] * cs + lo[q] * sn;
+          lo[q] = nlo;
+          hi[q] = nhi;
+        }
+      }
+      bf16x4 blo, bhi;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        blo[q] = (bf16_t)lo[q];
+        bhi[q] = (bf16_t)hi[q];
+      }
+      if (is_q) {
+        bf16_t* dst = (bf16_t*)e.out + (size_t)m * e.ldo + (size_t)head * d + i;
+        if (vec) {
+          *(bf16x4*)dst = blo;
+          *(bf16x4*)(dst + dh) = bhi;
+        } else {
+          for (int q = 0; q < 4; ++q) {
+            dst[q] = blo[q];
+            dst[dh + q] = bhi[q];
+          }
+        }
+      } else if (e.kcache) {
+        const size_t page = (size_t)e.table[(size_t)e.row_req[m] * e.table_stride + pos / e.page_size];
+        const int off = pos % e.page_size;
+        if (is_k) {
+          // four neighbours of one octet of d lie next to each other in the key order
+          bf16_t* dst = e.kcache + (page * e.nkv + (head - e.nq)) * (size_t)e.page_size * d;
+          *(bf16x4*)(dst + kcache_index(off, i, d)) = blo;
+          *(bf16x4*)(dst + kcache_index(off, i + dh, d)) = bhi;
+        } else {
+          bf16_t* dst = e.vcache + (page * e.nkv + (head - e.nq - e.nkv)) * (size_t)e.page_size * d;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            dst[vcache_index(off, i + q, d)] = blo[q];
+            dst[vcache_index(off, i + dh + q, d)] = bhi[q];
+          }
+        }
+      }
+    }
+  } else if constexpr (EPI == EPI_SWIGLU) {
     // columns of the tile alternate in runs of 16: gate, up of the same 16 outputs
     constexpr int OUTS = BN / 2, CH = OUTS / 8;      // outputs per row of the tile, chunks of 8 of them
     bf16_t* out = (bf16_t*)e.out;
@@ -385,6 +462,50 @@ static int launch_bf16(const bf16_t* A, const bf16_t* W, EpiArgs e, int M, int N
   return 0;
 }
 
+// q/k/v projection of many rows with bias, rotation and cache write in the epilogue
+// (bfloat16).  The tile is chosen as for any product; the head size must divide it.
+extern "C" int llmlab_linear_qkv(const void* x, const void* w, const void* bias, int bias_dtype, void* q_out,
+                                 int M, int N, int K, int ldo, const float* inv_freq, const int* positions,
+                                 const int* row_req, const int* table, int table_stride, int page_size,
+                                 void* kcache, void* vcache, int nq, int nkv, int d, int num_cus,
+                                 hipStream_t stream) {
+  LLMLAB_REQUIRE(M >= 0 && N > 0 && K > 0 && K % 8 == 0, "linear_qkv: bad sizes M=%d N=%d K=%d", M, N, K);
+  LLMLAB_REQUIRE(d >= 16 && d % 16 == 0 && nq > 0 && nkv > 0 && N == (nq + 2 * nkv) * d && ldo >= nq * d,
+                 "linear_qkv: %d + 2 x %d heads of %d do not make %d columns (row stride %d)", nq, nkv, d, N, ldo);
+  LLMLAB_REQUIRE((kcache == nullptr) == (vcache == nullptr), "linear_qkv: both caches or none");
+  LLMLAB_REQUIRE(positions != nullptr && (kcache == nullptr || (table && row_req && page_size > 0)),
+                 "linear_qkv: positions and block table are needed");
+  LLMLAB_REQUIRE(((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0) &&
+                 ((uintptr_t)kcache % 8 == 0) && ((uintptr_t)vcache % 8 == 0),
+                 "linear_qkv: operands must be 16-byte aligned");
+  if (M == 0) return 0;
+  if (num_cus <= 0) num_cus = 256;
+  EpiArgs e{q_out, bias, bias_dtype == DT_BF16, ldo, N, 0, 0, inv_freq, positions, row_req, table,
+            (bf16_t*)kcache, (bf16_t*)vcache, table_stride, page_size, nq, nkv, d};
+  const long big_tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
+  const int tile = (g_force_tile != 64 && (big_tiles >= num_cus || g_force_tile == 128)) ? 128 : 64;
+  LLMLAB_REQUIRE(tile % d == 0, "linear_qkv: heads of %d do not divide the tile of %d columns", d, tile);
+  if (tile == 128) {
+    dim3 grid((N + 127) / 128, (M + 127) / 128);
+    hipLaunchKernelGGL((gemm_bf16_tiled<128, 128, 64, 2, 2, EPI_QKV, false>), grid, dim3(256), 0, stream,
+                       (const bf16_t*)x, (const bf16_t*)w, e, M, N, K);
+  } else {
+    dim3 grid((N + 63) / 64, (M + 63) / 64);
+    hipLaunchKernelGGL((gemm_bf16_tiled<64, 64, 64, 2, 2, EPI_QKV, true>), grid, dim3(256), 0, stream,
+                       (const bf16_t*)x, (const bf16_t*)w, e, M, N, K);
+  }
+  LLMLAB_LAUNCH_CHECK("linear_qkv");
+  return 0;
+}
+
+// The tile that a product of these sizes gets (64 or 128): for callers that must know
+// whether a head fits it.
+extern "C" int llmlab_linear_tile(int M, int N, int num_cus) {
+  if (num_cus <= 0) num_cus = 256;
+  const long big_tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
+  return (g_force_tile != 64 && (big_tiles >= num_cus || g_force_tile == 128)) ? 128 : 64;
+}
+
 // parts[z] = x[:, K_z] . W[:, K_z]^T for `ksplit` ranges K_z of the inner size (whole K
 // tiles of 64 each); bias in parts[0].  bfloat16 only; for products whose output gives
 // the large tile too few blocks to fill the chip.
@@ -398,7 +519,8 @@ extern "C" int llmlab_linear_partials(const void* x, const void* w, float* parts
                  "linear_partials: operands must be 16-byte aligned");
   if (M == 0) return 0;
   const int nk = (K + 63) / 64;
-  EpiArgs e{parts, bias, bias_dtype == DT_BF16, ldo, N, (nk + ksplit - 1) / ksplit, part_stride};
+  EpiArgs e{parts, bias, bias_dtype == DT_BF16, ldo, N, (nk + ksplit - 1) / ksplit, part_stride,
+            nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 0, 0, 0};
   dim3 grid((N + 127) / 128, (M + 127) / 128, ksplit);
   hipLaunchKernelGGL((gemm_bf16_tiled<128, 128, 64, 2, 2, EPI_PART, false>), grid, dim3(256), 0, stream,
                      (const bf16_t*)x, (const bf16_t*)w, e, M, N, K);
@@ -422,7 +544,8 @@ extern "C" int llmlab_linear(const void* x, const void* w, int dtype, int epilog
   }
   LLMLAB_REQUIRE(ldo >= n_out, "linear: output row stride %d < %d columns", ldo, n_out);
   if (M == 0) return 0;
-  EpiArgs e{out, bias, bias_dtype == DT_BF16, ldo, n_out, 0, 0};
+  EpiArgs e{out, bias, bias_dtype == DT_BF16, ldo, n_out, 0, 0,
+            nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 0, 0, 0};
   if (num_cus <= 0) num_cus = 256;
   if (dtype == DT_BF16) {
     LLMLAB_REQUIRE(K % 8 == 0, "linear(bfloat16): inner size %d must be a multiple of 8", K);

@@ -119,6 +119,11 @@ class HipOps:
         c.llmlab_pack_weight.restype = _c_int
         c.llmlab_argmax.argtypes = [_c_ptr, _c_long, _c_int, _c_int, _c_ptr, _c_ptr, _c_size, _c_ptr]
         c.llmlab_argmax.restype = _c_int
+        c.llmlab_linear_qkv.argtypes = [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_int,
+                                        _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr,
+                                        _c_int, _c_int, _c_int, _c_int, _c_ptr]
+        c.llmlab_linear_tile.argtypes = [_c_int, _c_int, _c_int]
+        c.llmlab_linear_tile.restype = _c_int
         c.llmlab_linear_partials.argtypes = [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int,
                                              _c_int, _c_int, _c_size, _c_ptr]
         c.llmlab_skinny_linear.argtypes = [
@@ -130,7 +135,7 @@ class HipOps:
         c.llmlab_add_pending.restype = _c_int
         for fn in (c.llmlab_embed, c.llmlab_rmsnorm, c.llmlab_rope_kv_write, c.llmlab_rope_inplace,
                    c.llmlab_linear, c.llmlab_sample, c.llmlab_skinny_linear,
-                   c.llmlab_linear_partials):
+                   c.llmlab_linear_partials, c.llmlab_linear_qkv):
             fn.restype = _c_int
 
     def _attention_lib(self, head_dim: int) -> ctypes.CDLL:
@@ -528,31 +533,45 @@ class HipOps:
                           page_size=page_size, k_cache=k_cache, v_cache=v_cache, nq=num_heads,
                           nkv=num_kv_heads, d=head_dim), pending=pending)
 
-    QKV_ROPE_MAX_ROWS = 64
+    QKV_ROPE_MAX_ROWS = 64        # up to here the few-row kernel, beyond it the tiled one
 
-    def can_fuse_qkv_rope(self, rows: int, dtype, head_dim: int) -> bool:
-        """Whether ``qkv_rope_cache`` takes this step: bfloat16, at most 64 rows, and a
-        head that one block of the few-row kernel holds."""
-        if dtype != torch.bfloat16 or not 0 < rows <= self.QKV_ROPE_MAX_ROWS:
+    def can_fuse_qkv_rope(self, rows: int, dtype, head_dim: int, n: Optional[int] = None) -> bool:
+        """Whether ``qkv_rope_cache`` takes this step: bfloat16, and a head that one block
+        holds (few rows: the few-row kernel's block; more: the tile that a product of ``rows``
+        x ``n`` gets, which a head must divide)."""
+        if dtype != torch.bfloat16 or rows <= 0 or head_dim % 16 or head_dim < 16:
             return False
-        return head_dim % 16 == 0 and 16 <= head_dim <= (128 if rows > 32 else 256)
+        if rows <= self.QKV_ROPE_MAX_ROWS:
+            return head_dim <= (128 if rows > 32 else 256)
+        return n is not None and self._core.llmlab_linear_tile(rows, n, self.num_cus) % head_dim == 0
 
     def qkv_rope_cache(self, h, w_qkv, b_qkv, num_heads, num_kv_heads, head_dim, inv_freq, positions,
                        row_req, block_table, page_size, k_cache, v_cache, q_out) -> None:
-        """The same for activations ``h`` (bfloat16, already normed) of up to 64 rows:
-        product, bias, rotation and cache write in one kernel."""
+        """The same for activations ``h`` (bfloat16, already normed): product, bias, rotation
+        and cache write in one kernel."""
         rows, k = h.shape
         self._need(h, "activations", torch.bfloat16)
         w_qkv = self._weight(w_qkv, "weight")
-        if w_qkv.shape[1] != k or k % 8 != 0 or not self.can_fuse_qkv_rope(rows, h.dtype, head_dim):
+        n = w_qkv.shape[0]
+        if w_qkv.shape[1] != k or k % 8 != 0 or not self.can_fuse_qkv_rope(rows, h.dtype, head_dim, n):
             raise ValueError(f"qkv_rope_cache: {rows} rows of {k}, heads of {head_dim} do not fit")
-        n = self._qkv_checks("qkv_rope_cache", rows, w_qkv, b_qkv, num_heads, num_kv_heads, head_dim,
-                             inv_freq, positions, row_req, block_table, page_size, k_cache, v_cache, q_out)
-        self._skinny(h, False, None, None, 0.0, w_qkv, b_qkv, EPI_QKV, q_out, rows, n, k,
-                     q_out.shape[1], n,
-                     dict(inv_freq=inv_freq, positions=positions, row_req=row_req, table=block_table,
-                          page_size=page_size, k_cache=k_cache, v_cache=v_cache, nq=num_heads,
-                          nkv=num_kv_heads, d=head_dim))
+        self._qkv_checks("qkv_rope_cache", rows, w_qkv, b_qkv, num_heads, num_kv_heads, head_dim,
+                         inv_freq, positions, row_req, block_table, page_size, k_cache, v_cache, q_out)
+        if rows <= self.QKV_ROPE_MAX_ROWS:
+            self._skinny(h, False, None, None, 0.0, w_qkv, b_qkv, EPI_QKV, q_out, rows, n, k,
+                         q_out.shape[1], n,
+                         dict(inv_freq=inv_freq, positions=positions, row_req=row_req, table=block_table,
+                              page_size=page_size, k_cache=k_cache, v_cache=v_cache, nq=num_heads,
+                              nkv=num_kv_heads, d=head_dim))
+            return
+        if b_qkv is not None:
+            self._need(b_qkv, "bias")
+        self._check(self._core.llmlab_linear_qkv(
+            self._ptr(h), self._ptr(w_qkv), self._ptr(b_qkv), _dt(b_qkv) if b_qkv is not None else 0,
+            self._ptr(q_out), rows, n, k, q_out.stride(0), self._ptr(inv_freq), self._ptr(positions),
+            self._ptr(row_req), self._ptr(block_table), block_table.stride(0) if block_table is not None else 0,
+            int(page_size), self._ptr(k_cache), self._ptr(v_cache), num_heads, num_kv_heads, head_dim,
+            self.num_cus, self._stream()))
 
     def fused_norm_swiglu(self, x, norm_w, eps, w_gate_up, out, pending: Optional[PendingSums] = None) -> None:
         rows, inter = out.shape

@@ -152,8 +152,9 @@ class EmuOps:
                            block_table, page_size, k_cache, v_cache)
         q_out.copy_(qkv[:, :num_heads * head_dim].to(q_out.dtype))
 
-    def can_fuse_qkv_rope(self, rows, dtype, head_dim):
-        return self.fuse and dtype == torch.bfloat16 and 0 < rows <= 64 and head_dim % 16 == 0
+    def can_fuse_qkv_rope(self, rows, dtype, head_dim, n=None):
+        return self.fuse and dtype == torch.bfloat16 and rows > 0 and head_dim % 16 == 0 and (
+            rows <= 64 or (n is not None and 64 % head_dim == 0))
 
     def qkv_rope_cache(self, h, w_qkv, b_qkv, num_heads, num_kv_heads, head_dim, inv_freq, positions,
                        row_req, block_table, page_size, k_cache, v_cache, q_out):

@@ -252,11 +252,21 @@ def test_fused_norm_qkv_rope_write(ops, emu, nq, nkv, d, page, hidden, rotate, r
 
 @pytest.mark.parametrize("nq,nkv,d,page,hidden", [(4, 2, 16, 16, 64), (14, 2, 64, 64, 896), (6, 3, 48, 16, 72),
                                                  (8, 8, 128, 64, 256), (2, 1, 256, 16, 64)])
-@pytest.mark.parametrize("rows_per", [[5, 1, 9], [20, 1, 1, 3], [17, 30, 16]])
+@pytest.mark.parametrize("rows_per", [[5, 1, 9], [20, 1, 1, 3], [17, 30, 16], [70, 1, 130], [300, 2, 2, 90]])
 def test_qkv_rope_cache_of_normed_rows(ops, emu, nq, nkv, d, page, hidden, rows_per):
+    if d == 128 and sum(rows_per) > 64:
+        ops._core.llmlab_gemm_force(128)      # the large tile, which this few rows would not get
+    try:
+        check_qkv_rope_cache(ops, emu, nq, nkv, d, page, hidden, rows_per)
+    finally:
+        ops._core.llmlab_gemm_force(0)
+
+
+def check_qkv_rope_cache(ops, emu, nq, nkv, d, page, hidden, rows_per):
     bf = torch.bfloat16
-    rows, reqs, num_pages = sum(rows_per), len(rows_per), 16
-    if not ops.can_fuse_qkv_rope(rows, bf, d):
+    rows, reqs = sum(rows_per), len(rows_per)
+    num_pages = 16 + sum((40 + c + page - 1) // page for c in rows_per)
+    if not ops.can_fuse_qkv_rope(rows, bf, d, (nq + 2 * nkv) * d):
         with pytest.raises(ValueError):
             ops.qkv_rope_cache(torch.zeros(rows, hidden, dtype=bf, device=DEV),
                                ops.prepare_weight(torch.zeros((nq + 2 * nkv) * d, hidden, dtype=bf, device=DEV)),
@@ -269,7 +279,8 @@ def test_qkv_rope_cache_of_normed_rows(ops, emu, nq, nkv, d, page, hidden, rows_
     w, b = rnd((n, hidden), bf, 72, 0.2), rnd((n,), bf, 73)
     positions = torch.cat([torch.arange(s, s + c) for s, c in zip(starts, rows_per)]).int()
     row_req = torch.cat([torch.full((c,), i) for i, c in enumerate(rows_per)]).int()
-    table = torch.full((reqs, 8), -1, dtype=torch.int32)
+    table = torch.full((reqs, max((s0 + c + page - 1) // page for s0, c in zip(starts, rows_per))), -1,
+                       dtype=torch.int32)
     perm = torch.randperm(num_pages, generator=torch.Generator().manual_seed(74)).int()
     at = 0
     for i in range(reqs):
