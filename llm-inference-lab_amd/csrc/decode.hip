@@ -513,13 +513,15 @@ static int skinny_launch_stage(const SkinnyArgs& a, bool stage, int mb, int bloc
 }
 
 // A choice of block shape can be forced for measurements (0 = choose).
-static int g_force_nsb = 0, g_force_kw = 0, g_force_stage = -1, g_force_mb = 0;
+static int g_force_nsb = 0, g_force_kw = 0, g_force_stage = -1, g_force_mb = 0, g_force_epi = -1;
 extern "C" void llmlab_skinny_force(int nsb, int kw, int stage, int mb) {
   g_force_nsb = nsb;
   g_force_kw = kw;
   g_force_stage = stage;
   g_force_mb = mb;
 }
+// ... for one epilogue only (-1: for all)
+extern "C" void llmlab_skinny_force_epilogue(int epilogue) { g_force_epi = epilogue; }
 
 struct SkinnyShape {
   int nsb, kw;
@@ -606,7 +608,9 @@ static SkinnyShape skinny_choose(int epilogue, bool norm, int M, int N, int K, i
   double best_cost = 1e30;
   const int mb_max = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
   for (int mb = mb_max; mb >= 1; mb >>= 1) {
-    if (g_force_mb > 0 && mb != g_force_mb && !(g_force_mb > mb_max && mb == mb_max)) continue;
+    if (g_force_mb > 0 && (g_force_epi < 0 || g_force_epi == epilogue) && mb != g_force_mb &&
+        !(g_force_mb > mb_max && mb == mb_max))
+      continue;
     const int tiles = sk_tiles(M, mb);
     double cost;
     const SkinnyShape s = skinny_choose_tile(epilogue, norm, mb, M < 16 * mb ? M : 16 * mb, tiles, N, K, d,
@@ -675,13 +679,14 @@ extern "C" int llmlab_skinny_linear(const void* x, int norm, const int* x_rows, 
   LLMLAB_REQUIRE(ldo >= (epilogue == SK_QKV ? nq * d : n_out), "skinny_linear: output stride too small");
   SkinnyShape shape = skinny_choose(epilogue, norm != 0, M, N, K, d, num_cus, ksplit);
   const int mb = shape.mb, tiles = sk_tiles(M, mb), tile_rows = M < 16 * mb ? M : 16 * mb;
-  if (g_force_nsb > 0 && epilogue != SK_QKV) shape.nsb = g_force_nsb;
-  if (g_force_nsb > 0 && epilogue == SK_QKV && d % 32 == 0 && d > 32) {
+  const bool forced = g_force_epi < 0 || g_force_epi == epilogue;
+  if (forced && g_force_nsb > 0 && epilogue != SK_QKV) shape.nsb = g_force_nsb;
+  if (forced && g_force_nsb > 0 && epilogue == SK_QKV && d % 32 == 0 && d > 32) {
     shape.nsb = g_force_nsb == 2 ? 2 : d / 16;
     shape.qsplit = g_force_nsb == 2 ? d / 32 : 1;
   }
-  if (g_force_kw > 0) shape.kw = g_force_kw;
-  if (g_force_stage >= 0) shape.stage = norm || (g_force_stage != 0 && epilogue != SK_PART);
+  if (forced && g_force_kw > 0) shape.kw = g_force_kw;
+  if (forced && g_force_stage >= 0) shape.stage = norm || (g_force_stage != 0 && epilogue != SK_PART);
   LLMLAB_REQUIRE(shape.nsb > 0 && shape.kw > 0,
                  "skinny_linear: no block shape fits N=%d K=%d M=%d (16 rows of x to stage: %zu bytes of LDS)",
                  N, K, M, (size_t)(M < 16 ? M : 16) * ((K + 31) / 32 * 32 + SK_APAD) * sizeof(bf16_t));
