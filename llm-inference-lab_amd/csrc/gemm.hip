@@ -3,15 +3,19 @@
 // for gfx950, with the epilogues the model needs fused in.
 //
 //   bfloat16:  v_mfma_f32_16x16x32_bf16 everywhere.
-//     * tiled kernel: 256 threads = 4 waves in 2x2, block tile 128x128 or
-//       64x64, K step 64; x staged through two stages of LDS (rows padded to 72
-//       elements so that the 16-byte fragment reads of 8 lanes cover all banks), W
-//       too (in fragment order, as it lies in memory) or read straight into
-//       registers; three or four tiles are on their way from memory in a ring of
-//       register buffers while one is multiplied.  Measured and not adopted: 256x128
-//       tiles with eight 64x64 or four 128x64 wave tiles, K steps of 128, and 256x256
-//       tiles with four 128x128 wave tiles (half the LDS traffic per product, one wave
-//       per SIMD: 833 against 793 TF/s on the largest product tried, slower on the rest).
+//     * tiled kernel: 256 threads = 4 waves, block tile 64x64 (waves 2x2), 64x128 or
+//       128x128 (waves 1x4, side by side along the columns), K step 64; x staged through
+//       two stages of LDS (rows padded to 72 elements so that the 16-byte fragment reads
+//       of 8 lanes cover all banks), the fragments of W read straight from the packed
+//       matrix into registers; three or four tiles are on their way from memory in a
+//       ring of register buffers while one is multiplied.  With the waves 1x4 every
+//       fragment of W is read by one wave only and all four share the rows of x in LDS:
+//       5 to 35 % faster than 2x2 waves with W staged through LDS too (which was the
+//       large tile before).  Also measured and not adopted: 256x128 tiles with eight
+//       64x64 or four 128x64 wave tiles, K steps of 128, 128x256 and 128x64 tiles with
+//       1x4 waves, and 256x256 tiles with four 128x128 wave tiles (half the LDS traffic
+//       per product, one wave per SIMD: 833 against 793 TF/s on the largest product
+//       tried, slower on the rest).
 //     (products of few rows, as in decode steps, have kernels of their own in decode.hip)
 //   float32: a plain FMA kernel (64x64 tile, 4x4 outputs per thread): true 32-bit
 //     products and sums, no matrix-core shortcut.
@@ -70,7 +74,7 @@ __device__ __forceinline__ void epi_store(const EpiArgs& e, int m, int n, float 
 }
 
 // ============================================================ bf16, tiled
-template <int BM, int BN, int BK, int WM, int WN, int EPI, bool BDIRECT = false>
+template <int BM, int BN, int BK, int WM, int WN, int EPI>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __restrict__ A,
                                                         const bf16_t* __restrict__ W, EpiArgs e, int M,
                                                         int N, int K) {
@@ -79,18 +83,17 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __
   constexpr int WTM = BM / WM, WTN = BN / WN;  // wave tile
   constexpr int TM = WTM / 16, TN = WTN / 16;
   constexpr int KCH = BK / 8;                // 16-byte chunks in a row of a tile
-  constexpr int A_CHUNKS = BM * KCH / NT, B_CHUNKS = BN * KCH / NT;  // chunks per thread
-  static_assert(A_CHUNKS >= 1 && B_CHUNKS >= 1 && BM * KCH % NT == 0 && BN * KCH % NT == 0, "tile too small");
-  // two stages of LDS: the next tile is put in while this one is multiplied, one
+  constexpr int A_CHUNKS = BM * KCH / NT;    // chunks of x per thread
+  static_assert(A_CHUNKS >= 1 && BM * KCH % NT == 0, "tile too small");
+  // two stages of LDS for x: the next tile is put in while this one is multiplied, one
   // barrier per tile
-  constexpr int A_STAGE = BM * LDS_STRIDE, B_STAGE = BDIRECT ? 8 : BN * BK;
+  constexpr int A_STAGE = BM * LDS_STRIDE;
   // (one array: after the last tile it holds the block's results for the epilogue)
   constexpr int C_STRIDE = BN + 4;           // floats per row of the result tile in LDS
-  constexpr size_t STAGE_BYTES = (size_t)(2 * A_STAGE + 2 * B_STAGE) * sizeof(bf16_t);
+  constexpr size_t STAGE_BYTES = (size_t)(2 * A_STAGE) * sizeof(bf16_t);
   constexpr size_t C_BYTES = (size_t)BM * C_STRIDE * sizeof(float);
   __shared__ __attribute__((aligned(16))) char smem[STAGE_BYTES > C_BYTES ? STAGE_BYTES : C_BYTES];
   bf16_t* As2 = (bf16_t*)smem;
-  bf16_t* Bs2 = As2 + 2 * A_STAGE;
 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / WN, wn = wave % WN;
@@ -120,11 +123,11 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __
   // Memory latency is several times the time a tile takes to multiply, so PD tiles
   // are on their way at any time: a ring of register buffers, refilled as soon as a
   // buffer has been put into LDS.
-  constexpr int PD = (A_CHUNKS + B_CHUNKS) <= 4 ? 4 : 3;
-  bf16x8 ra[PD][A_CHUNKS], rb[BDIRECT ? 1 : PD][B_CHUNKS];
-  // BDIRECT: every wave reads the B fragments of its columns straight from the packed
-  // W into registers; only x goes through LDS
-  bf16x8 rbd[BDIRECT ? PD : 1][BK / 32][TN];
+  constexpr int PD = (A_CHUNKS + BN * KCH / NT) <= 4 ? 4 : 3;
+  bf16x8 ra[PD][A_CHUNKS];
+  // every wave reads the B fragments of its columns straight from the packed W into
+  // registers; only x goes through LDS
+  bf16x8 rbd[PD][BK / 32][TN];
   const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
 
   // Loads are unconditional (a load under a branch makes the compiler wait for every
@@ -140,15 +143,6 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __
       const int m = min(m0 + row, M - 1), k = min(k0 + kc, K - 8);
       ra[slot][i] = *(const bf16x8*)(A + (size_t)m * K + k);
     }
-    if constexpr (!BDIRECT) {
-#pragma unroll
-      for (int i = 0; i < B_CHUNKS; ++i) {
-        const int ch = tid + i * NT, sl = ch / (2 * BK), step = (k0 >> 5) + (ch >> 6) % (BK / 32);
-        const int strip = min((n0 >> 4) + sl, nstrips - 1);
-        const bf16x8 v = *(const bf16x8*)(W + ((size_t)strip * T + min(step, T - 1)) * 512 + (ch & 63) * 8);
-        rb[slot][i] = step < T ? v : zero;
-      }
-    }
   };
   auto fetch_b = [&](int slot, int k0) {
 #pragma unroll
@@ -163,18 +157,10 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __
   };
   auto stash = [&](int slot, int stage) {
     bf16_t* As = As2 + stage * A_STAGE;
-    bf16_t* Bs = Bs2 + stage * B_STAGE;
 #pragma unroll
     for (int i = 0; i < A_CHUNKS; ++i) {
       const int ch = tid + i * NT, row = ch / KCH, kc = (ch % KCH) * 8;
       *(bf16x8*)(As + row * LDS_STRIDE + kc) = ra[slot][i];
-    }
-    if constexpr (!BDIRECT) {
-#pragma unroll
-      for (int i = 0; i < B_CHUNKS; ++i) {
-        // as it lies in the packed W: [strip][32-wide step][lane][8], no padding needed
-        *(bf16x8*)(Bs + (tid + i * NT) * 8) = rb[slot][i];
-      }
     }
   };
 
@@ -191,7 +177,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __
 #pragma unroll
   for (int p = 0; p < PD; ++p) {      // past K: zeros for W
     fetch(p, kbase + p * BK);
-    if constexpr (BDIRECT) fetch_b(p, kbase + p * BK);
+    fetch_b(p, kbase + p * BK);
   }
   // tile kt lies in stage kt & 1; it was put there during tile kt - 1 (tile 0: now)
   stash(0, 0);
@@ -208,7 +194,6 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __
       fetch(pn, kbase + (t + 1 + PD) * BK);
       if (live) {
         const bf16_t* As = As2 + stage * A_STAGE;
-        const bf16_t* Bs = Bs2 + stage * B_STAGE;
 #pragma unroll
         for (int ks = 0; ks < BK / 32; ++ks) {
           bf16x8 a[TM], b[TN];
@@ -216,10 +201,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __
           for (int i = 0; i < TM; ++i)
             a[i] = *(const bf16x8*)(As + (wm * WTM + i * 16 + c) * LDS_STRIDE + ks * 32 + g * 8);
 #pragma unroll
-          for (int j = 0; j < TN; ++j) {
-            if constexpr (BDIRECT) b[j] = rbd[p][ks][j];
-            else b[j] = *(const bf16x8*)(Bs + (((wn * TN + j) * (BK / 32) + ks) * 64 + lane) * 8);
-          }
+          for (int j = 0; j < TN; ++j) b[j] = rbd[p][ks][j];
 #pragma unroll
           for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -228,7 +210,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __
         }
         __syncthreads();
       }
-      if constexpr (BDIRECT) fetch_b(p, kbase + (t + PD) * BK);
+      fetch_b(p, kbase + (t + PD) * BK);
     }
   }
 
@@ -440,26 +422,86 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__
 }
 
 // ================================================================ dispatch
-// A tile can be forced for measurements (0 = choose; 64, 128).
+// Three tile shapes, all with four waves, x through LDS and W straight from the packed
+// matrix: 64 x 64 (waves 2 x 2) for small products, 64 x 128 and 128 x 128 with the waves
+// side by side along the columns (1 x 4), so that every fragment of W is read by one wave
+// only and the rows of x in LDS are shared by all four.  The shape is picked by an
+// estimate of the time, fitted to sweeps of the three products of a layer at two model
+// shapes and 576 to 4096 rows (its picks cost 1.4 % over the best shape there):
+//   time = L + rounds * (f + K tiles * tk),  rounds = max(1, blocks / (units * resident)).
+enum { TILE_64 = 0, TILE_64x128 = 1, TILE_128 = 2 };
+struct TileModel {
+  int bm, bn;
+  double L, f, tk, resident;
+};
+static const TileModel TILE_MODELS[3] = {
+    {64, 64, 6.39, 0.79, 0.289, 1.0}, {64, 128, 6.54, 0.71, 0.552, 1.5}, {128, 128, 9.78, 0.48, 0.704, 1.0}};
+
+static double tile_cost(int kind, int M, int N, int K, int num_cus, int pieces) {
+  const TileModel& t = TILE_MODELS[kind];
+  const double blocks = (double)((M + t.bm - 1) / t.bm) * ((N + t.bn - 1) / t.bn) * pieces;
+  const double rounds = blocks / (num_cus * t.resident);
+  const int nk = ((K + 63) / 64 + pieces - 1) / pieces;
+  return t.L + (rounds > 1.0 ? rounds : 1.0) * (t.f + nk * t.tk);
+}
+
+// A tile can be forced for measurements (0 = choose; 64, 130 = 64 x 128, 129 = 128 x 128).
 static int g_force_tile = 0;
 extern "C" void llmlab_gemm_force(int tile) { g_force_tile = tile; }
 
-template <int EPI>
-static int launch_bf16(const bf16_t* A, const bf16_t* W, EpiArgs e, int M, int N, int K, int num_cus,
-                       hipStream_t stream) {
-  // the large tile when it still fills the chip, else the small one
-  const long big_tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
-  if (g_force_tile != 64 && (big_tiles >= num_cus || g_force_tile == 128)) {
-    dim3 grid((N + 127) / 128, (M + 127) / 128);
-    hipLaunchKernelGGL((gemm_bf16_tiled<128, 128, 64, 2, 2, EPI, false>), grid, dim3(256), 0, stream, A, W, e, M, N, K);
-  } else {
-    dim3 grid((N + 63) / 64, (M + 63) / 64);
-    // (with the small tile the waves read their B fragments straight from the packed W:
-    // measured faster there, and slower with the large tile, whose waves would read
-    // every fragment twice)
-    hipLaunchKernelGGL((gemm_bf16_tiled<64, 64, 64, 2, 2, EPI, true>), grid, dim3(256), 0, stream, A, W, e, M, N, K);
+static int choose_tile(int M, int N, int K, int num_cus) {
+  if (g_force_tile == 64) return TILE_64;
+  if (g_force_tile == 130) return TILE_64x128;
+  if (g_force_tile == 129 || g_force_tile == 128) return TILE_128;
+  int best = 0;
+  double best_cost = 1e30;
+  for (int kind = 0; kind < 3; ++kind) {
+    const double c = tile_cost(kind, M, N, K, num_cus, 1);
+    if (c < best_cost) {
+      best_cost = c;
+      best = kind;
+    }
   }
-  return 0;
+  return best;
+}
+
+template <int EPI>
+static void launch_tile(int kind, const bf16_t* A, const bf16_t* W, const EpiArgs& e, int M, int N, int K,
+                        int pieces, hipStream_t stream) {
+  const TileModel& t = TILE_MODELS[kind];
+  dim3 grid((N + t.bn - 1) / t.bn, (M + t.bm - 1) / t.bm, pieces);
+  if (kind == TILE_64)
+    hipLaunchKernelGGL((gemm_bf16_tiled<64, 64, 64, 2, 2, EPI>), grid, dim3(256), 0, stream, A, W, e, M, N, K);
+  else if (kind == TILE_64x128)
+    hipLaunchKernelGGL((gemm_bf16_tiled<64, 128, 64, 1, 4, EPI>), grid, dim3(256), 0, stream, A, W, e, M, N, K);
+  else
+    hipLaunchKernelGGL((gemm_bf16_tiled<128, 128, 64, 1, 4, EPI>), grid, dim3(256), 0, stream, A, W, e, M, N, K);
+}
+
+// Whether (and into how many pieces along K) a product that adds into float32 rows should
+// be left unsummed, and with which tile: out = {pieces (1: no), tile kind}.  A piece costs
+// a write and a read of the result by whoever sums it up later.
+extern "C" void llmlab_linear_plan(int M, int N, int K, int num_cus, int max_pieces, int min_tiles_per_piece,
+                                   int* out) {
+  if (num_cus <= 0) num_cus = 256;
+  const int nk = (K + 63) / 64;
+  const double piece = (double)M * N * 2.2e-6 + 0.3;
+  int best_kind = choose_tile(M, N, K, num_cus), best_pieces = 1;
+  double best_cost = tile_cost(best_kind, M, N, K, num_cus, 1);
+  for (int kind = TILE_64x128; kind <= TILE_128; ++kind) {
+    if (g_force_tile != 0 && kind != choose_tile(M, N, K, num_cus)) continue;
+    for (int s = 2; s <= max_pieces; ++s) {
+      if ((nk + s - 1) / s < min_tiles_per_piece) break;
+      const double c = tile_cost(kind, M, N, K, num_cus, s) + s * piece;
+      if (c < best_cost) {
+        best_cost = c;
+        best_kind = kind;
+        best_pieces = s;
+      }
+    }
+  }
+  out[0] = best_pieces;
+  out[1] = best_kind;
 }
 
 // q/k/v projection of many rows with bias, rotation and cache write in the epilogue
@@ -482,48 +524,37 @@ extern "C" int llmlab_linear_qkv(const void* x, const void* w, const void* bias,
   if (num_cus <= 0) num_cus = 256;
   EpiArgs e{q_out, bias, bias_dtype == DT_BF16, ldo, N, 0, 0, inv_freq, positions, row_req, table,
             (bf16_t*)kcache, (bf16_t*)vcache, table_stride, page_size, nq, nkv, d};
-  const long big_tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
-  const int tile = (g_force_tile != 64 && (big_tiles >= num_cus || g_force_tile == 128)) ? 128 : 64;
-  LLMLAB_REQUIRE(tile % d == 0, "linear_qkv: heads of %d do not divide the tile of %d columns", d, tile);
-  if (tile == 128) {
-    dim3 grid((N + 127) / 128, (M + 127) / 128);
-    hipLaunchKernelGGL((gemm_bf16_tiled<128, 128, 64, 2, 2, EPI_QKV, false>), grid, dim3(256), 0, stream,
-                       (const bf16_t*)x, (const bf16_t*)w, e, M, N, K);
-  } else {
-    dim3 grid((N + 63) / 64, (M + 63) / 64);
-    hipLaunchKernelGGL((gemm_bf16_tiled<64, 64, 64, 2, 2, EPI_QKV, true>), grid, dim3(256), 0, stream,
-                       (const bf16_t*)x, (const bf16_t*)w, e, M, N, K);
-  }
+  const int kind = choose_tile(M, N, K, num_cus);
+  LLMLAB_REQUIRE(TILE_MODELS[kind].bn % d == 0, "linear_qkv: heads of %d do not divide the tile of %d columns", d,
+                 TILE_MODELS[kind].bn);
+  launch_tile<EPI_QKV>(kind, (const bf16_t*)x, (const bf16_t*)w, e, M, N, K, 1, stream);
   LLMLAB_LAUNCH_CHECK("linear_qkv");
   return 0;
 }
 
-// The tile that a product of these sizes gets (64 or 128): for callers that must know
-// whether a head fits it.
-extern "C" int llmlab_linear_tile(int M, int N, int num_cus) {
+// The width of the tile (64 or 128 columns) that a product of these sizes gets: for
+// callers that must know whether a head fits it.
+extern "C" int llmlab_linear_tile(int M, int N, int K, int num_cus) {
   if (num_cus <= 0) num_cus = 256;
-  const long big_tiles = (long)((M + 127) / 128) * ((N + 127) / 128);
-  return (g_force_tile != 64 && (big_tiles >= num_cus || g_force_tile == 128)) ? 128 : 64;
+  return TILE_MODELS[choose_tile(M, N, K, num_cus)].bn;
 }
 
 // parts[z] = x[:, K_z] . W[:, K_z]^T for `ksplit` ranges K_z of the inner size (whole K
-// tiles of 64 each); bias in parts[0].  bfloat16 only; for products whose output gives
-// the large tile too few blocks to fill the chip.
+// tiles of 64 each); bias in parts[0].  bfloat16 only; `tile` as llmlab_linear_plan gives it.
 extern "C" int llmlab_linear_partials(const void* x, const void* w, float* parts, const void* bias,
                                       int bias_dtype, int M, int N, int K, int ldo, int ksplit,
-                                      size_t part_stride, hipStream_t stream) {
+                                      size_t part_stride, int tile, hipStream_t stream) {
   LLMLAB_REQUIRE(M >= 0 && N > 0 && K > 0 && K % 8 == 0, "linear_partials: bad sizes M=%d N=%d K=%d", M, N, K);
   LLMLAB_REQUIRE(ksplit >= 1 && ksplit <= 16 && ldo >= N && part_stride >= (size_t)M * ldo,
                  "linear_partials: %d pieces, row stride %d", ksplit, ldo);
+  LLMLAB_REQUIRE(tile >= TILE_64 && tile <= TILE_128, "linear_partials: unknown tile %d", tile);
   LLMLAB_REQUIRE(((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0),
                  "linear_partials: operands must be 16-byte aligned");
   if (M == 0) return 0;
   const int nk = (K + 63) / 64;
   EpiArgs e{parts, bias, bias_dtype == DT_BF16, ldo, N, (nk + ksplit - 1) / ksplit, part_stride,
             nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, 0, 0, 0, 0, 0};
-  dim3 grid((N + 127) / 128, (M + 127) / 128, ksplit);
-  hipLaunchKernelGGL((gemm_bf16_tiled<128, 128, 64, 2, 2, EPI_PART, false>), grid, dim3(256), 0, stream,
-                     (const bf16_t*)x, (const bf16_t*)w, e, M, N, K);
+  launch_tile<EPI_PART>(tile, (const bf16_t*)x, (const bf16_t*)w, e, M, N, K, ksplit, stream);
   LLMLAB_LAUNCH_CHECK("linear_partials");
   return 0;
 }
@@ -553,11 +584,12 @@ extern "C" int llmlab_linear(const void* x, const void* w, int dtype, int epilog
                    "linear(bfloat16): operands must be 16-byte aligned");
     const bf16_t* A = (const bf16_t*)x;
     const bf16_t* W = (const bf16_t*)w;
+    const int kind = choose_tile(M, N, K, num_cus);
     switch (epilogue) {
-      case EPI_STORE: launch_bf16<EPI_STORE>(A, W, e, M, N, K, num_cus, stream); break;
-      case EPI_RESID: launch_bf16<EPI_RESID>(A, W, e, M, N, K, num_cus, stream); break;
-      case EPI_F32: launch_bf16<EPI_F32>(A, W, e, M, N, K, num_cus, stream); break;
-      default: launch_bf16<EPI_SWIGLU>(A, W, e, M, N, K, num_cus, stream); break;
+      case EPI_STORE: launch_tile<EPI_STORE>(kind, A, W, e, M, N, K, 1, stream); break;
+      case EPI_RESID: launch_tile<EPI_RESID>(kind, A, W, e, M, N, K, 1, stream); break;
+      case EPI_F32: launch_tile<EPI_F32>(kind, A, W, e, M, N, K, 1, stream); break;
+      default: launch_tile<EPI_SWIGLU>(kind, A, W, e, M, N, K, 1, stream); break;
     }
   } else {
     dim3 grid((N + 63) / 64, (M + 63) / 64), block(256);

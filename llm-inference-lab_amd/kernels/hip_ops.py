@@ -122,10 +122,12 @@ class HipOps:
         c.llmlab_linear_qkv.argtypes = [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_int,
                                         _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr,
                                         _c_int, _c_int, _c_int, _c_int, _c_ptr]
-        c.llmlab_linear_tile.argtypes = [_c_int, _c_int, _c_int]
+        c.llmlab_linear_tile.argtypes = [_c_int, _c_int, _c_int, _c_int]
         c.llmlab_linear_tile.restype = _c_int
         c.llmlab_linear_partials.argtypes = [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int,
-                                             _c_int, _c_int, _c_size, _c_ptr]
+                                             _c_int, _c_int, _c_size, _c_int, _c_ptr]
+        c.llmlab_linear_plan.argtypes = [_c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr]
+        c.llmlab_linear_plan.restype = None
         c.llmlab_skinny_linear.argtypes = [
             _c_ptr, _c_int, _c_ptr, _c_ptr, _c_int, _c_float, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr,
             _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
@@ -401,7 +403,8 @@ class HipOps:
     MAX_SPLITS = 8
     split_max_rows = 32           # most rows of a product that is left in pieces
     min_steps_per_split = 8       # K steps of 32 a piece should have at least (tests lower it)
-    min_tiles_per_split = 8       # many rows: K tiles of 64 a piece should have at least (tests lower it)
+    min_tiles_per_split = 8       # many rows: K tiles of 64 a piece should have at least
+    force_tiled_pieces = 0        # many rows: this many pieces whatever the estimate says (tests)
 
     def split_count(self, rows: int, dtype, n: int, k: int) -> int:
         """Into how many pieces along the inner size a few-row product ``[rows, k] x
@@ -411,33 +414,24 @@ class HipOps:
         if dtype != torch.bfloat16 or rows <= 0:
             return 1
         if rows > self.FUSED_MAX_ROWS:
-            # many rows, tiled kernel.  Time is rounds of 128 x 128 blocks over the chip times
-            # the K tiles of a block; every piece costs a write and a read of the result.
-            # Fitted to sweeps of the down products of two model shapes (128 to 4096 rows),
-            # where it picks the measured best or its neighbour.  Where the large tile has
-            # too few blocks the small one would run instead, which moves every operand
-            # twice as often: pieces win there whenever K is long enough to cut.
+            # many rows, tiled kernel: its own estimate (rounds of blocks over the chip times
+            # the K tiles of a block, plus a write and a read of the result for every piece)
             if k % 8:
                 return 1
-            tiles = ((rows + 127) // 128) * ((n + 127) // 128)
-            nk = (k + 63) // 64
-            piece = rows * n * 2.2e-6 + 0.3
-            best, best_cost = 1, None
-            if tiles >= self.num_cus:
-                best_cost = -(-tiles // self.num_cus) * nk * 0.65
-            for s in range(2, self.MAX_SPLITS + 1):
-                per = -(-nk // s)
-                if per < self.min_tiles_per_split:
-                    break
-                cost = -(-tiles * s // self.num_cus) * per * 0.65 + s * piece
-                if best_cost is None or cost < best_cost:
-                    best, best_cost = s, cost
-            return best
+            if self.force_tiled_pieces:         # (tests: tiny products would never be cut)
+                return max(1, min(self.force_tiled_pieces, (k + 63) // 64, self.MAX_SPLITS))
+            return self._linear_plan(rows, n, k)[0]
         if rows > self.split_max_rows:
             return 1
         strips, steps = (n + 15) // 16, (k + 31) // 32
         want = self.num_cus // max(strips, 1)
         return max(1, min(want, steps // self.min_steps_per_split, self.MAX_SPLITS))
+
+    def _linear_plan(self, rows: int, n: int, k: int):
+        """(pieces, tile) for a many-row product that adds into float32 rows."""
+        out = (_c_int * 2)()
+        self._core.llmlab_linear_plan(rows, n, k, self.num_cus, self.MAX_SPLITS, self.min_tiles_per_split, out)
+        return out[0], out[1]
 
     def linear_partials(self, x, w, parts: torch.Tensor, splits: int, bias=None) -> PendingSums:
         """``parts[s] = x[:, K_s] w[:, K_s]^T`` for the ``splits`` pieces ``K_s`` of the inner
@@ -462,7 +456,7 @@ class HipOps:
             self._check(self._core.llmlab_linear_partials(
                 self._ptr(x), self._ptr(w), self._ptr(parts), self._ptr(bias),
                 _dt(bias) if bias is not None else 0, m, n, k, parts.stride(1), splits, parts.stride(0),
-                self._stream()))
+                self._linear_plan(m, n, k)[1], self._stream()))
         return PendingSums(parts, splits)
 
     def add_pending(self, x: torch.Tensor, pending: PendingSums) -> None:
@@ -535,15 +529,17 @@ class HipOps:
 
     QKV_ROPE_MAX_ROWS = 64        # up to here the few-row kernel, beyond it the tiled one
 
-    def can_fuse_qkv_rope(self, rows: int, dtype, head_dim: int, n: Optional[int] = None) -> bool:
+    def can_fuse_qkv_rope(self, rows: int, dtype, head_dim: int, n: Optional[int] = None,
+                          k: Optional[int] = None) -> bool:
         """Whether ``qkv_rope_cache`` takes this step: bfloat16, and a head that one block
-        holds (few rows: the few-row kernel's block; more: the tile that a product of ``rows``
-        x ``n`` gets, which a head must divide)."""
+        holds (few rows: the few-row kernel's block; more: the tile that a product ``[rows, k]
+        x [n, k]^T`` gets, which a head must divide)."""
         if dtype != torch.bfloat16 or rows <= 0 or head_dim % 16 or head_dim < 16:
             return False
         if rows <= self.QKV_ROPE_MAX_ROWS:
             return head_dim <= (128 if rows > 32 else 256)
-        return n is not None and self._core.llmlab_linear_tile(rows, n, self.num_cus) % head_dim == 0
+        return (n is not None and k is not None
+                and self._core.llmlab_linear_tile(rows, n, k, self.num_cus) % head_dim == 0)
 
     def qkv_rope_cache(self, h, w_qkv, b_qkv, num_heads, num_kv_heads, head_dim, inv_freq, positions,
                        row_req, block_table, page_size, k_cache, v_cache, q_out) -> None:
@@ -553,7 +549,7 @@ class HipOps:
         self._need(h, "activations", torch.bfloat16)
         w_qkv = self._weight(w_qkv, "weight")
         n = w_qkv.shape[0]
-        if w_qkv.shape[1] != k or k % 8 != 0 or not self.can_fuse_qkv_rope(rows, h.dtype, head_dim, n):
+        if w_qkv.shape[1] != k or k % 8 != 0 or not self.can_fuse_qkv_rope(rows, h.dtype, head_dim, n, k):
             raise ValueError(f"qkv_rope_cache: {rows} rows of {k}, heads of {head_dim} do not fit")
         self._qkv_checks("qkv_rope_cache", rows, w_qkv, b_qkv, num_heads, num_kv_heads, head_dim,
                          inv_freq, positions, row_req, block_table, page_size, k_cache, v_cache, q_out)

@@ -118,7 +118,8 @@ class GQAAttention(Mixer):
             ops.fused_norm_qkv(rms[0], rms[2], rms[3], self.w_qkv, self.b_qkv, self.num_heads,
                                self.num_kv_heads, self.head_dim, table, ctx.positions, ctx.row_req,
                                group.block_table, group.page_size, k_cache, v_cache, q, pending=pending)
-        elif (ops.can_fuse_qkv_rope(rows, self.dtype, self.head_dim, self.q_size + 2 * self.kv_size)
+        elif (ops.can_fuse_qkv_rope(rows, self.dtype, self.head_dim, self.q_size + 2 * self.kv_size,
+                                    self.hidden_size)
               and (self.position is None or table is not None)):
             # more rows: the norm on its own, then one kernel for the rest
             if isinstance(h, NormedInput):

@@ -152,7 +152,7 @@ class EmuOps:
                            block_table, page_size, k_cache, v_cache)
         q_out.copy_(qkv[:, :num_heads * head_dim].to(q_out.dtype))
 
-    def can_fuse_qkv_rope(self, rows, dtype, head_dim, n=None):
+    def can_fuse_qkv_rope(self, rows, dtype, head_dim, n=None, k=None):
         return self.fuse and dtype == torch.bfloat16 and rows > 0 and head_dim % 16 == 0 and (
             rows <= 64 or (n is not None and 64 % head_dim == 0))
 

@@ -74,7 +74,7 @@ def test_sums_of_many_rows_left_in_pieces(name, cut):
     seqs = sequences_of(name)
     want = {rid: H.plain_logits(name, 1, ids) for rid, ids in seqs.items()}
     engine = H.make_engine(name, 1, "bf16", page_size=16, num_pages=40, max_requests=4)
-    engine.ops.min_tiles_per_split = 1
+    engine.ops.force_tiled_pieces = 2
     cfg = H.config_of(name)
     assert engine.ops.split_count(130, torch.bfloat16, cfg.hidden_size, cfg.intermediate_size) > 1
     got = H.run_trace(engine, seqs, CUTS[cut](seqs))

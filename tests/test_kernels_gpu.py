@@ -266,7 +266,7 @@ def check_qkv_rope_cache(ops, emu, nq, nkv, d, page, hidden, rows_per):
     bf = torch.bfloat16
     rows, reqs = sum(rows_per), len(rows_per)
     num_pages = 16 + sum((40 + c + page - 1) // page for c in rows_per)
-    if not ops.can_fuse_qkv_rope(rows, bf, d, (nq + 2 * nkv) * d):
+    if not ops.can_fuse_qkv_rope(rows, bf, d, (nq + 2 * nkv) * d, hidden):
         with pytest.raises(ValueError):
             ops.qkv_rope_cache(torch.zeros(rows, hidden, dtype=bf, device=DEV),
                                ops.prepare_weight(torch.zeros((nq + 2 * nkv) * d, hidden, dtype=bf, device=DEV)),
