@@ -12,8 +12,9 @@
 //       fragment of W is read by one wave only and all four share the rows of x in LDS:
 //       5 to 35 % faster than 2x2 waves with W staged through LDS too (which was the
 //       large tile before).  Also measured and not adopted: 256x128 tiles with eight
-//       64x64 or four 128x64 wave tiles, K steps of 128, 128x256 and 128x64 tiles with
-//       1x4 waves, and 256x256 tiles with four 128x128 wave tiles (half the LDS traffic
+//       64x64 or four 128x64 wave tiles, K steps of 128, 128x256, 64x256, 128x64 and
+//       32x128 tiles with 1x4 waves (the second as good as 128x128, no better), eight
+//       waves 2x4 on 128x128 and 64x128, and 256x256 tiles with four 128x128 wave tiles (half the LDS traffic
 //       per product, one wave per SIMD: 833 against 793 TF/s on the largest product
 //       tried, slower on the rest).
 //     (products of few rows, as in decode steps, have kernels of their own in decode.hip)

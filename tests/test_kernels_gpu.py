@@ -125,6 +125,48 @@ def test_linear_residual_and_logits(ops, emu, dtype, m, n, k):
     close(got, want, torch.float32, f"linear_logits {m}x{n}x{k}", want.abs().max().item())
 
 
+@pytest.mark.parametrize("tile", [64, 130, 129])
+@pytest.mark.parametrize("m,n,k", [(65, 130, 72), (200, 1152, 896), (300, 257, 136), (513, 384, 264), (129, 64, 1160)])
+def test_every_tile_shape_of_the_tiled_products(ops, emu, tile, m, n, k):
+    """Every epilogue with each of the three tile shapes forced, on sizes with ragged edges
+    in all three dimensions (the chooser would pick only one of them per size)."""
+    from llm_inference_lab_amd.parts.feed_forward import interleave_gate_up
+    bf = torch.bfloat16
+    ops._core.llmlab_gemm_force(tile)
+    try:
+        x, w, bias = rnd((m, k), bf, 5), rnd((n, k), bf, 6, 0.1), rnd((n,), torch.float32, 7)
+        pw = ops.prepare_weight(w.to(DEV))
+        want = torch.empty(m, n, dtype=bf)
+        emu.linear(x, w, want, bias)
+        got = torch.empty(m, n, dtype=bf, device=DEV)
+        ops.linear(x.to(DEV), pw, got, bias.to(DEV))
+        close(got, want, bf, "store", want.float().abs().max().item())
+        resid = rnd((m, n), torch.float32, 11)
+        want = resid.clone()
+        emu.linear_residual(x, w, want)
+        got = resid.clone().to(DEV)
+        ops.linear_residual(x.to(DEV), pw, got)
+        close(got, want, torch.float32, "residual", want.abs().max().item())
+        want = torch.empty(m, n)
+        emu.linear_logits(x, w, want)
+        got = torch.empty(m, n, device=DEV)
+        ops.linear_logits(x.to(DEV), pw, got)
+        close(got, want, torch.float32, "logits", want.abs().max().item())
+        inter = n // 2 + 3
+        gu = interleave_gate_up(rnd((inter, k), bf, 12, 0.1), rnd((inter, k), bf, 13, 0.1))
+        want = torch.empty(m, inter, dtype=bf)
+        emu.linear_swiglu(x, gu, want)
+        got = torch.empty(m, inter, dtype=bf, device=DEV)
+        ops.linear_swiglu(x.to(DEV), ops.prepare_weight(gu.to(DEV)), got)
+        close(got, want, bf, "swiglu", want.float().abs().max().item())
+        parts = torch.zeros(3, m, n, device=DEV)
+        ops.linear_partials(x.to(DEV), pw, parts, 3)
+        whole = x.float() @ w.float().t()
+        close(parts.sum(0), whole, torch.float32, "pieces", whole.abs().max().item())
+    finally:
+        ops._core.llmlab_gemm_force(0)
+
+
 def test_linear_reference_vectors(ops):
     """The closed-form vectors of the reference's own linear tests
     (rust/engine/src/runner/model/qwen2/engine.rs:3574-3612): x = ((i*17 % 31) - 15)/32,
