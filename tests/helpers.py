@@ -33,7 +33,13 @@ TINY_C = dict(architectures=["Qwen2ForCausalLM"], model_type="qwen2", vocab_size
               num_key_value_heads=3, head_dim=48, rms_norm_eps=1e-6, rope_theta=50000.0,
               max_position_embeddings=512, tie_word_embeddings=False, use_sliding_window=True,
               sliding_window=40, max_window_layers=0)
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
+# The layer sizes of Qwen2.5-0.5B (two layers, a small odd vocabulary): the kernels'
+# choices of block shape at real sizes, end to end.
+REAL_LAYER = dict(architectures=["Qwen2ForCausalLM"], model_type="qwen2", vocab_size=4099, hidden_size=896,
+                  intermediate_size=4864, num_hidden_layers=2, num_attention_heads=14,
+                  num_key_value_heads=2, head_dim=64, rms_norm_eps=1e-6, rope_theta=1000000.0,
+                  max_position_embeddings=4096, tie_word_embeddings=True, use_sliding_window=False)
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "R": REAL_LAYER}
 
 # Decided before the first run and not widened since.  Logits of these models are
 # of order 1.  float32: sums in another order than the float64 reference.
@@ -54,11 +60,15 @@ def make_tensors(cfg, seed, sharp=8.0):
     attention is peaked: with the plain N(0, 0.02) scores are nearly uniform and a
     wrong key, mask or page would change the logits by less than the tolerance."""
     tensors = dict(random_tensors(expected_tensors(cfg), seed, torch.bfloat16))
+    if cfg.hidden_size > 128:       # (queries and keys grow with the root of the width as well)
+        sharp *= (64.0 / cfg.hidden_size) ** 0.5
     for name in tensors:
         if name.endswith("q_proj.weight") or name.endswith("k_proj.weight"):
             tensors[name] = (tensors[name].float() * sharp).to(torch.bfloat16)
         if name.endswith("embed_tokens.weight"):
-            tensors[name] = (tensors[name].float() * 10).to(torch.bfloat16)
+            # (a wide model's logits would grow with the root of its width: keep them of order 1)
+            scale = 10.0 if cfg.hidden_size <= 128 else 10.0 * (64.0 / cfg.hidden_size) ** 0.5
+            tensors[name] = (tensors[name].float() * scale).to(torch.bfloat16)
     return tensors
 
 

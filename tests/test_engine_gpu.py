@@ -22,6 +22,15 @@ CUTS = {"whole": H.steps_whole, "decode": H.steps_prefill_then_decode, "portions
         "mixed": H.steps_mixed}
 
 
+# Layers 896 wide: float32 within 1e-3 of the float64 plain implementation (sums of 896
+# to 4864 terms).  For bfloat16 the floor is what rounding the activations to 8 bits of
+# mantissa at the engine's rounding points costs at this width: the emulation of the
+# kernels on the CPU (tests/emu_ops.py, float32 arithmetic, the same roundings) is off
+# the plain implementation by 0.09 to 0.10 at most and 0.016 to 0.017 in the root mean
+# square over the logits of these sequences; the GPU may be off by half as much again.
+TOL_REAL = {"f32": (1e-3, 1e-3), "bf16": (0.15, 0.025)}     # (max, root mean square)
+
+
 def sequences_of(name, seed=0):
     cfg = H.config_of(name)
     return {f"r{i}": H.random_ids(cfg, n, 100 * seed + i) for i, n in enumerate(LENGTHS[name])}
@@ -44,6 +53,22 @@ def test_every_cut_matches_plain(dtype, name, cut, page_size):
     engine.cache.check()
     m = engine.cache.metrics()
     assert m["rows_used"] == 0 and all(g["pages_used"] == 0 for g in m["groups"])
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("cut", list(CUTS))
+def test_layers_of_real_size(dtype, cut):
+    """Two layers with the sizes of Qwen2.5-0.5B: what the kernels choose at real sizes
+    (block shapes, tiles, pieces, fused paths) against the plain implementation."""
+    cfg = H.config_of("R")
+    seqs = {f"r{i}": H.random_ids(cfg, n, 700 + i) for i, n in enumerate([3, 75, 140, 330])}
+    want = {rid: H.plain_logits("R", 1, ids) for rid, ids in seqs.items()}
+    engine = H.make_engine("R", 1, dtype, page_size=64, num_pages=12, max_requests=4, max_batch_tokens=512)
+    got = H.run_trace(engine, seqs, CUTS[cut](seqs))
+    bad = H.first_wrong(got, want, TOL_REAL[dtype][0])
+    assert bad is None, f"first wrong logits at (request, position, error) = {bad}"
+    err = torch.cat([(got[r].double() - want[r])[~torch.isnan(got[r]).any(1)].flatten() for r in seqs])
+    assert float((err ** 2).mean().sqrt()) <= TOL_REAL[dtype][1]
 
 
 @pytest.mark.parametrize("name", ["A", "B", "C"])
