@@ -352,8 +352,27 @@ __device__ __forceinline__ void attention_tile(const AttnArgs& a, const int xblk
         s_pages[i] = pi < a.table_stride ? a.table[(size_t)b * a.table_stride + pi] : -1;
       }
       __syncthreads();
+      // (a block of 4 waves and head sizes in steps of 32: a 16-key block is 2 D pieces
+      // of 16 bytes, a whole number of pieces per lane)
+      constexpr bool FAST_PIECES = D % 32 == 0;
       auto fetch_tile = [&](int slot, int tile) {
         const int tl = min(tile, ce);
+        if constexpr (FAST_PIECES) {
+          // wave w copies the w-th 16-key block of the tile, keys and values: one page
+          // lookup and one address for all pieces of a thread
+          const int pos16 = tl * 64 + wave * 16;
+          const int page = s_pages[page_index(pos16) - page_first];
+          const bool ok = tile <= ce && pos16 <= bkey_hi && pos16 + 15 >= bkey_lo && page >= 0;
+          const size_t at = ((size_t)max(page, 0) * a.nkv + kvh) * P * D +
+                            (size_t)(page_offset(pos16) >> 4) * (16 * D) + lane * 8;
+#pragma unroll
+          for (int n = 0; n < NCH / 2; ++n) {
+            rok[slot][n] = rok[slot][n + NCH / 2] = ok;
+            regs[slot][n] = *(const bf16x8*)(kc + at + n * 512);
+            regs[slot][n + NCH / 2] = *(const bf16x8*)(vc + at + n * 512);
+          }
+          return;
+        }
 #pragma unroll
         for (int n = 0; n < NCH; ++n) {
           const int i = tid + n * 256;
@@ -369,6 +388,16 @@ __device__ __forceinline__ void attention_tile(const AttnArgs& a, const int xblk
         }
       };
       auto store_tile = [&](int slot) {
+        if constexpr (FAST_PIECES) {
+#pragma unroll
+          for (int n = 0; n < NCH / 2; ++n) {
+            const bool ok = rok[slot][n];
+            *(bf16x8*)(Ks + wave * (16 * D) + (lane + n * 64) * 8) = ok ? regs[slot][n] : zero8;
+            *(bf16x8*)(Vs + wave * (16 * D) + (lane + n * 64) * 8) = ok ? regs[slot][n + NCH / 2] : zero8;
+          }
+          if (lane == 0) s_ok[wave] = rok[slot][0];
+          return;
+        }
 #pragma unroll
         for (int n = 0; n < NCH; ++n) {
           const int i = tid + n * 256;
