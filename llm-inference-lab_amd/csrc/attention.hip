@@ -323,6 +323,16 @@ __device__ __forceinline__ void attention_tile(const AttnArgs& a, const int xblk
     // copy is straight, and every fragment read below is lane-contiguous
     __shared__ __attribute__((aligned(16))) bf16_t Ks[64 * D];
     __shared__ __attribute__((aligned(16))) bf16_t Vs[64 * D];
+    // The values lie in LDS so that one 16-byte read gives a lane its MFMA operand of a
+    // step of 32 keys: [pair of 16-key blocks][16-wide block of d][lane][even block's 4 |
+    // odd block's 4].  A 16-byte piece as it comes from the cache (two lanes' values of
+    // one 16-key block) goes there in two halves.
+    auto vs_at = [&](int sub, int db, int ln) { return (((sub >> 1) * DB + db) * 64 + ln) * 8 + (sub & 1) * 4; };
+    auto vs_store = [&](int sub, int rem, const bf16x8& v) {     // piece `rem` of 16-key block `sub`
+      bf16_t* dst = Vs + vs_at(sub, rem >> 5, (rem & 31) * 2);
+      *(bf16x4*)dst = __builtin_shufflevector(v, v, 0, 1, 2, 3);
+      *(bf16x4*)(dst + 8) = __builtin_shufflevector(v, v, 4, 5, 6, 7);
+    };
     __shared__ int s_ok[4];
     constexpr int PAGE_CAP = 2048;
     __shared__ int s_pages[PAGE_CAP];               // the block's slice of its request's block table
@@ -391,9 +401,10 @@ __device__ __forceinline__ void attention_tile(const AttnArgs& a, const int xblk
         if constexpr (FAST_PIECES) {
 #pragma unroll
           for (int n = 0; n < NCH / 2; ++n) {
-            const bool ok = rok[slot][n];
-            *(bf16x8*)(Ks + wave * (16 * D) + (lane + n * 64) * 8) = ok ? regs[slot][n] : zero8;
-            *(bf16x8*)(Vs + wave * (16 * D) + (lane + n * 64) * 8) = ok ? regs[slot][n + NCH / 2] : zero8;
+            // (what came for a 16-key block that is not there goes in as it is: s_ok keeps
+            // the keys out of the scores, and the values are zeroed where they are read)
+            *(bf16x8*)(Ks + wave * (16 * D) + (lane + n * 64) * 8) = regs[slot][n];
+            vs_store(wave, lane + n * 64, regs[slot][n + NCH / 2]);
           }
           if (lane == 0) s_ok[wave] = rok[slot][0];
           return;
@@ -405,7 +416,8 @@ __device__ __forceinline__ void attention_tile(const AttnArgs& a, const int xblk
           const int j = is_v ? i - 8 * D : i;
           const int sub = j / (2 * D), rem = j - sub * (2 * D);
           const bf16x8 v = rok[slot][n] ? regs[slot][n] : zero8;
-          *(bf16x8*)((is_v ? Vs : Ks) + sub * (16 * D) + rem * 8) = v;
+          if (is_v) vs_store(sub, rem, v);
+          else *(bf16x8*)(Ks + sub * (16 * D) + rem * 8) = v;
           if (!is_v && rem == 0) s_ok[sub] = rok[slot][n];
         }
       };
@@ -434,17 +446,20 @@ __device__ __forceinline__ void attention_tile(const AttnArgs& a, const int xblk
 #pragma unroll
             for (int piece = 0; piece < 4 / SUBS; ++piece) {
               bf16x8 kf[SUBS][DC];
-              bf16x4 vq[SUBS][DB];
+              bf16x8 vf[SUBS / 2][DB];
 #pragma unroll
               for (int u = 0; u < SUBS; ++u) {
                 const int sub = piece * SUBS + u;
 #pragma unroll
                 for (int dc = 0; dc < DC; ++dc)
                   kf[u][dc] = *(const bf16x8*)(Ks + sub * (16 * D) + min(dc * 4 + g, D / 8 - 1) * 128 + c * 8);
+              }
+              // the values of a step of 32 keys (two 16-key blocks): one read per operand
+#pragma unroll
+              for (int st = 0; st < SUBS / 2; ++st)
 #pragma unroll
                 for (int db = 0; db < DB; ++db)
-                  vq[u][db] = *(const bf16x4*)(Vs + sub * (16 * D) + db * 256 + lane * 4);
-              }
+                  vf[st][db] = *(const bf16x8*)(Vs + vs_at(piece * SUBS + st * 2, db, lane));
               floatx4 s4[SUBS][QB];
 #pragma unroll
               for (int u = 0; u < SUBS; ++u)
@@ -455,19 +470,18 @@ __device__ __forceinline__ void attention_tile(const AttnArgs& a, const int xblk
                   for (int dc = 0; dc < DC; ++dc)
                     s4[u][qb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[u][dc], qf[qb][dc], s4[u][qb], 0, 0, 0);
                 }
-#pragma unroll
-              for (int u = 0; u < SUBS; ++u)       // into the units of the exponent
-#pragma unroll
-                for (int qb = 0; qb < QB; ++qb) s4[u][qb] *= scale2;
               bf16x8 pf[SUBS / 2][QB];
 #pragma unroll
               for (int qb = 0; qb < QB; ++qb) {
+                // the maximum of the raw scores, then into the units of the exponent (the
+                // scale is positive); the scores themselves are scaled inside the FMA below
                 float mx = NEG_INF;
 #pragma unroll
                 for (int u = 0; u < SUBS; ++u)
                   mx = max3_raw(max3_raw(s4[u][qb][0], s4[u][qb][1], s4[u][qb][2]), s4[u][qb][3], mx);
                 mx = max_across_32(mx);
                 mx = max_across_16(mx);
+                mx *= scale2;
                 const bool grow = mx > m[qb] + LAZY_MAX;
                 if (__any(grow)) {
                   const float m_new = grow ? mx : m[qb];
@@ -484,7 +498,7 @@ __device__ __forceinline__ void attention_tile(const AttnArgs& a, const int xblk
                   float pv[8];
 #pragma unroll
                   for (int i = 0; i < 8; ++i)
-                    pv[i] = fast_exp2(s4[st * 2 + (i >> 2)][qb][i & 3] + neg_m);
+                    pv[i] = fast_exp2(fmaf(s4[st * 2 + (i >> 2)][qb][i & 3], scale2, neg_m));
                   psum += ((pv[0] + pv[1]) + (pv[2] + pv[3])) + ((pv[4] + pv[5]) + (pv[6] + pv[7]));
 #pragma unroll
                   for (int i = 0; i < 8; ++i) pf[st][qb][i] = (bf16_t)pv[i];
@@ -495,10 +509,9 @@ __device__ __forceinline__ void attention_tile(const AttnArgs& a, const int xblk
               for (int st = 0; st < SUBS / 2; ++st)
 #pragma unroll
                 for (int db = 0; db < DB; ++db) {
-                  const bf16x8 vf = __builtin_shufflevector(vq[st * 2][db], vq[st * 2 + 1][db], 0, 1, 2, 3, 4, 5, 6, 7);
 #pragma unroll
                   for (int qb = 0; qb < QB; ++qb)
-                    o[qb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pf[st][qb], o[qb][db], 0, 0, 0);
+                    o[qb][db] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[st][db], pf[st][qb], o[qb][db], 0, 0, 0);
                 }
             }
             __syncthreads();
@@ -517,7 +530,7 @@ __device__ __forceinline__ void attention_tile(const AttnArgs& a, const int xblk
                     f.k[h2][dc] = *(const bf16x8*)(Ks + sub * (16 * D) + min(dc * 4 + g, D / 8 - 1) * 128 + c * 8);
 #pragma unroll
                   for (int db = 0; db < DB; ++db)
-                    f.v[h2][db] = *(const bf16x4*)(Vs + sub * (16 * D) + db * 256 + lane * 4);
+                    f.v[h2][db] = f.ok[h2] ? *(const bf16x4*)(Vs + vs_at(sub, db, lane)) : zero4;
                 }
                 compute(kb >> 5, f);
               }
