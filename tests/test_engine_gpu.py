@@ -167,6 +167,29 @@ def test_greedy_generation_through_the_entry_point(name):
     assert agree >= 0.8 * 16 * len(prompts), (got, want)
 
 
+@pytest.mark.parametrize("name,graph", [("A", False), ("B", True)])
+def test_many_requests_through_a_small_pool(name, graph):
+    """Fourteen requests of random lengths, a token budget of 24 a step and pages for about
+    three of them: requests wait for pages, prompts are cut into portions beside decodes,
+    pages are handed on many times.  Every request's greedy tokens equal the plain
+    implementation's (float32), and everything is given back at the end."""
+    import random
+    cfg = H.config_of(name)
+    tensors = H.make_tensors(cfg, 1)
+    rnd = random.Random(5)
+    prompts = [H.random_ids(cfg, rnd.choice([1, 2, 5, 17, 33, 60, 90]), 500 + i) for i in range(14)]
+    news = [rnd.choice([1, 3, 9, 20]) for _ in prompts]
+    want = [plain_qwen2.greedy_generate(p, n, tensors, cfg.to_dict()) for p, n in zip(prompts, news)]
+    engine = H.make_engine(name, 1, "f32", graph=graph, page_size=16, num_pages=21, max_requests=4,
+                           max_batch_tokens=24)
+    from llm_inference_lab_amd.sampling import SamplingConfig
+    got = engine.generate(prompts, sampling=[SamplingConfig(max_new_tokens=n, eos_token_id=[]) for n in news])
+    assert got == want
+    engine.cache.check()
+    m = engine.cache.metrics()
+    assert m["rows_used"] == 0 and all(g["pages_used"] == 0 for g in m["groups"])
+
+
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 def test_decode_graph_replays_equal_eager(dtype):
     """Several replays with eager work and synchronisation between them, each checked."""
