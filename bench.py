@@ -9,7 +9,8 @@ batch 8, context 4096, bfloat16.  A "step" is one decode step of the whole
 batch through the scheduler's own path (step function + sampling, tokens fed
 back).  One JSON line is printed: decoded tokens a second as ``value``, plus
 ``prefill`` (one 2,048-token prompt), ``roofline`` (bytes the decode step has to
-read over its time against 8 TB/s), ``points`` (decode at batch 1 and 64), ``step_ms`` (median
+read over its time against 8 TB/s), ``points`` (decode at batch 1 and 64; the ``--mixed``
+run at the 7B shape, all tokens a second), ``step_ms`` (median
 and 95th percentile of single steps timed through GPU completion) and ``eager`` (the
 same decode steps without the HIP graph).
 
@@ -114,6 +115,18 @@ def mixed_run(args, cfg, layers, full_layers):
     }))
 
 
+def mixed_point(timeout=420):
+    """`bench.py --mixed --shape 7b` in a child process: all tokens a second, or None."""
+    import subprocess
+    try:
+        out = subprocess.run([sys.executable, os.path.abspath(__file__), "--mixed", "--shape", "7b"],
+                             capture_output=True, text=True, timeout=timeout)
+        lines = [ln for ln in out.stdout.splitlines() if ln.startswith("{")]
+        return json.loads(lines[-1])["value"] if out.returncode == 0 and lines else None
+    except Exception:
+        return None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -140,6 +153,12 @@ def main():
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         sys.exit(2)
+
+    # The mixed run at the 7B shape is a point of the default line: it runs as a child
+    # process of its own, before this process touches the GPU.
+    mixed_7b = None
+    if not (args.mixed or args.no_points or args.only_prefill) and args.shape == "0.5b":
+        mixed_7b = mixed_point()
 
     import torch
     import llm_inference_lab_amd as lab
@@ -277,6 +296,8 @@ def main():
                 continue
             s, _ = decode_run(b, max(8, args.steps // 2), max(2, args.warmup // 2))
             points[f"decode_b{b}"] = round(b * max(8, args.steps // 2) / s, 1)
+        if mixed_7b is not None:
+            points["mixed_7b_tokens_per_second"] = mixed_7b
         result["points"] = points
         p50, p95 = step_latencies(args.batch)
         result["step_ms"] = {"p50": p50, "p95": p95}
