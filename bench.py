@@ -11,8 +11,9 @@ back).  One JSON line is printed: decoded tokens a second as ``value``, plus
 ``prefill`` (one 2,048-token prompt), ``roofline`` (bytes the decode step has to
 read over its time against 8 TB/s), ``points`` (decode at batch 1 and 64; the ``--mixed``
 run at the 7B shape, all tokens a second), ``step_ms`` (median
-and 95th percentile of single steps timed through GPU completion) and ``eager`` (the
-same decode steps without the HIP graph).
+and 95th percentile of single steps timed through GPU completion) and ``eager`` or ``graph``
+(the same decode steps the other way: launched kernel by kernel, or replayed from a HIP
+graph; ``--graph auto``, the default, lets the engine choose).
 
 ``--mixed``: many requests with prompts of different lengths go through the
 scheduler with a small token budget, so that portions of prompts run beside the
@@ -70,7 +71,7 @@ def mixed_run(args, cfg, layers, full_layers):
     engine = lab.Engine(config=cfg, seed=0, dtype=args.dtype, device="cuda:0", page_size=page,
                         max_cache_tokens=sum(n + args.outputs + page for n in lengths),
                         max_requests=args.requests, max_batch_tokens=args.chunk + args.requests,
-                        max_seq_len=longest + page, graph=not args.no_graph)
+                        max_seq_len=longest + page, graph=False if args.no_graph else args.graph)
 
     def one_run():
         sched = engine.scheduler(max_batch_tokens=args.chunk + args.requests)
@@ -140,6 +141,8 @@ def main():
                     help="run fewer layers than the shape has (both numbers are reported)")
     ap.add_argument("--dtype", default="bf16", choices=["bf16", "f32"])
     ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--graph", default="auto", choices=["auto", "on"],
+                    help="decode from a HIP graph: always, or where the engine expects it to pay")
     ap.add_argument("--no-points", action="store_true", help="skip batch 1 / 64 and the prefill")
     ap.add_argument("--mixed", action="store_true",
                     help="mixed run: --requests prompts of 128..2048 tokens, portions of --chunk tokens "
@@ -178,7 +181,8 @@ def main():
     context = args.context
     engine = lab.Engine(config=cfg, seed=0, dtype=args.dtype, device="cuda:0", page_size=page,
                         max_cache_tokens=max_batch * (context + page), max_requests=max_batch,
-                        max_batch_tokens=FILL_TOKENS, max_seq_len=context + page, graph=not args.no_graph)
+                        max_batch_tokens=FILL_TOKENS, max_seq_len=context + page,
+                        graph=False if args.no_graph else args.graph)
     gen = torch.Generator().manual_seed(1234)
 
     def random_ids(n):
@@ -281,7 +285,7 @@ def main():
             "num_key_value_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
             "intermediate_size": cfg.intermediate_size, "vocab_size": cfg.vocab_size,
             "tie_word_embeddings": cfg.tie_word_embeddings, "page_size": page,
-            "hip_graph_decode": not args.no_graph, "weights_seed": 0,
+            "hip_graph_decode": bool(engine.step_fn.use_graph), "weights_seed": 0,
         },
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
                      "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4)},
@@ -301,12 +305,14 @@ def main():
         result["points"] = points
         p50, p95 = step_latencies(args.batch)
         result["step_ms"] = {"p50": p50, "p95": p95}
-        if engine.step_fn.use_graph:      # the same steps launched kernel by kernel
-            engine.step_fn.use_graph = False
+        if not args.no_graph:             # the same steps the other way: kernel by kernel, or from a graph
+            chosen = engine.step_fn.use_graph
+            engine.step_fn.use_graph = not chosen
             s, _ = decode_run(args.batch, max(8, args.steps // 2), max(2, args.warmup // 2))
-            engine.step_fn.use_graph = True
-            result["eager"] = {"value": round(args.batch * max(8, args.steps // 2) / s, 1),
-                               "ms_per_step": round(s / max(8, args.steps // 2) * 1e3, 4)}
+            engine.step_fn.use_graph = chosen
+            result["eager" if chosen else "graph"] = {
+                "value": round(args.batch * max(8, args.steps // 2) / s, 1),
+                "ms_per_step": round(s / max(8, args.steps // 2) * 1e3, 4)}
     print(json.dumps(result))
 
 

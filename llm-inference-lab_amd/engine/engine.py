@@ -55,7 +55,7 @@ class Engine:
                  dtype="bf16", device: str = "cuda:0", ops=None, page_size: int = 64,
                  max_cache_tokens: Optional[int] = None, num_pages: Optional[int] = None,
                  max_requests: int = 64, max_batch_tokens: int = 512,
-                 max_seq_len: Optional[int] = None, tensors=None, graph: bool = False,
+                 max_seq_len: Optional[int] = None, tensors=None, graph=False,
                  progress: Optional[Callable[[str], None]] = None):
         self.dtype = parse_dtype(dtype)
         if model_dir is not None:
@@ -103,9 +103,26 @@ class Engine:
                                   state_specs, self.dtype, self.device)
         self.model.attach_cache(self.cache)
         self.step_fn = StepFunction(self.model, self.cache, self.ops, self.max_batch_tokens,
-                                    graph=graph)
+                                    graph=self._graph_choice(graph))
         self._sampler = None
         self.last_scheduler = None
+
+    # A decode step replayed from a HIP graph costs the host nothing, but the GPU about a
+    # microsecond more at every kernel boundary than kernels launched one by one by a host
+    # that runs ahead (measured: 4.05 against 3.90 ms a step at the 7B shape, 17.3 against
+    # 16.9 at the 32B shape; 0.97 against 1.7 at the 0.5B shape, where the host cannot keep
+    # up).  ``graph="auto"`` takes the graph unless the step's reading of the weights
+    # clearly outlasts the host's launching of its kernels.
+    HOST_SECONDS_PER_KERNEL = 12e-6
+    STREAMED_BYTES_PER_SECOND = 4.2e12
+
+    def _graph_choice(self, graph) -> bool:
+        if graph != "auto":
+            return bool(graph)
+        kernels = 6 * len(self.spec.schedule) + 6
+        host = kernels * self.HOST_SECONDS_PER_KERNEL
+        gpu = self.model.weight_bytes_per_step() / self.STREAMED_BYTES_PER_SECOND
+        return gpu < 1.25 * host
 
     # ------------------------------------------------------------- requests
     def open(self, request_id) -> RequestCache:
