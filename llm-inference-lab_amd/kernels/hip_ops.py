@@ -202,7 +202,7 @@ class HipOps:
         n, k = w.shape
         self.check_product_sizes(k, w.dtype, "weight matrix")
         data = torch.empty(self._core.llmlab_packed_elements(n, k), dtype=torch.bfloat16, device=self.device)
-        self._check(self._core.llmlab_pack_weight(self._ptr(w), self._ptr(data), n, k, self._stream()))
+        self._call(self._core.llmlab_pack_weight, self._ptr(w), self._ptr(data), n, k, self._stream())
         return PackedWeight(data, n, k)
 
     def _weight(self, w, name: str):
@@ -225,6 +225,12 @@ class HipOps:
         if raw is not None:
             return raw(self.device.index)
         return torch.cuda.current_stream(self.device).cuda_stream
+
+    def _call(self, fn, *args, lib=None) -> None:
+        """One call into the kernel libraries; a failure raises with the library's message."""
+        code = fn(*args)
+        if code != 0:
+            self._check(code, lib)
 
     def _check(self, code: int, lib=None) -> None:
         if code != 0:
@@ -260,9 +266,9 @@ class HipOps:
         if ids.numel() != rows or table.shape[1] != hidden:
             raise ValueError(f"embed: ids {tuple(ids.shape)}, table {tuple(table.shape)}, "
                              f"out {tuple(out.shape)} do not fit")
-        self._check(self._core.llmlab_embed(self._ptr(table), _dt(table), 1 if packed else 0,
+        self._call(self._core.llmlab_embed, self._ptr(table), _dt(table), 1 if packed else 0,
                                             self._ptr(ids), self._ptr(out), rows, hidden, table.shape[0],
-                                            self._stream()))
+                                            self._stream())
 
     def gather_tokens(self, dst, dst_index, src, src_index, n) -> None:
         """dst[dst_index[i]] = src[src_index[i]] for i < n (all int32 on the GPU)."""
@@ -270,8 +276,8 @@ class HipOps:
             self._need(t, f"gather_tokens {name}", torch.int32)
         if dst_index.numel() < n or src_index.numel() < n:
             raise ValueError("gather_tokens: index arrays are shorter than the count")
-        self._check(self._core.llmlab_gather_tokens(self._ptr(dst), self._ptr(dst_index), self._ptr(src),
-                                                    self._ptr(src_index), int(n), self._stream()))
+        self._call(self._core.llmlab_gather_tokens, self._ptr(dst), self._ptr(dst_index), self._ptr(src),
+                                                    self._ptr(src_index), int(n), self._stream())
 
     def rmsnorm(self, x, weight, eps, out, rows=None, pending=None) -> None:
         """``out[i] = norm(x[rows[i]])``.  ``pending`` (all rows in order only): the pieces are
@@ -297,9 +303,9 @@ class HipOps:
             if rows is not None or p.shape[1] != n_out or p.shape[2] != hidden or not p[0].is_contiguous():
                 raise ValueError("rmsnorm: pending sums go with all rows in order and the same shape")
             pend = (self._ptr(p), pending.splits, p.stride(0))
-        self._check(self._core.llmlab_rmsnorm(self._ptr(x), self._ptr(weight), _dt(weight), float(eps),
+        self._call(self._core.llmlab_rmsnorm, self._ptr(x), self._ptr(weight), _dt(weight), float(eps),
                                               self._ptr(out), _dt(out), self._ptr(rows), n_out, hidden,
-                                              pend[0], pend[1], pend[2], self._stream()))
+                                              pend[0], pend[1], pend[2], self._stream())
 
     # ----------------------------------------------------------------- linear
     def _linear(self, x, w, out, bias, epilogue, n_out, pending: Optional[PendingSums] = None) -> None:
@@ -333,9 +339,9 @@ class HipOps:
             return
         if pending is not None:
             self.add_pending(out, pending)
-        self._check(self._core.llmlab_linear(
+        self._call(self._core.llmlab_linear,
             self._ptr(x), self._ptr(w), _dt(x), epilogue, self._ptr(out), self._ptr(bias),
-            _dt(bias) if bias is not None else 0, m, n, k, ldo, n_out, self.num_cus, self._stream()))
+            _dt(bias) if bias is not None else 0, m, n, k, ldo, n_out, self.num_cus, self._stream())
 
     def linear(self, x, w, out, bias=None) -> None:
         self._linear(x, w, out, bias, EPI_STORE, w.shape[0])
@@ -389,7 +395,7 @@ class HipOps:
             pend = (self._ptr(p), pending.splits, p.stride(1), p.stride(0))
         else:
             pend = (_c_ptr(0), 0, 0, 0)
-        self._check(self._core.llmlab_skinny_linear(
+        self._call(self._core.llmlab_skinny_linear,
             self._ptr(x), 1 if norm else 0, self._ptr(x_rows), self._ptr(norm_w),
             _dt(norm_w) if norm_w is not None else 0, float(eps), self._ptr(w), self._ptr(bias),
             _dt(bias) if bias is not None else 0, epilogue, self._ptr(out), m, n, k, ldo, n_out,
@@ -397,7 +403,7 @@ class HipOps:
             self._ptr(table), table.stride(0) if table is not None else 0, q.get("page_size", 0),
             self._ptr(q.get("k_cache")), self._ptr(q.get("v_cache")), q.get("nq", 0), q.get("nkv", 0),
             q.get("d", 0), self.num_cus, pend[0], pend[1], pend[2], pend[3], int(ksplit),
-            int(part_stride), self._stream()))
+            int(part_stride), self._stream())
 
     # --------------------------------------------- sums left in pieces (deferred)
     MAX_SPLITS = 8
@@ -453,10 +459,10 @@ class HipOps:
         else:
             if bias is not None:
                 self._need(bias, "bias")
-            self._check(self._core.llmlab_linear_partials(
+            self._call(self._core.llmlab_linear_partials,
                 self._ptr(x), self._ptr(w), self._ptr(parts), self._ptr(bias),
                 _dt(bias) if bias is not None else 0, m, n, k, parts.stride(1), splits, parts.stride(0),
-                self._linear_plan(m, n, k)[1], self._stream()))
+                self._linear_plan(m, n, k)[1], self._stream())
         return PendingSums(parts, splits)
 
     def add_pending(self, x: torch.Tensor, pending: PendingSums) -> None:
@@ -466,8 +472,8 @@ class HipOps:
         rows, width = x.shape
         if p.shape[1] != rows or p.shape[2] != width or not p[0].is_contiguous():
             raise ValueError("add_pending: pieces and stream differ in shape")
-        self._check(self._core.llmlab_add_pending(self._ptr(x), self._ptr(p), pending.splits, p.stride(0),
-                                                  rows, width, self._stream()))
+        self._call(self._core.llmlab_add_pending, self._ptr(x), self._ptr(p), pending.splits, p.stride(0),
+                                                  rows, width, self._stream())
 
     def _fused_common(self, x, norm_w, w, rows):
         self._need(x, "residual stream", torch.float32)
@@ -562,12 +568,12 @@ class HipOps:
             return
         if b_qkv is not None:
             self._need(b_qkv, "bias")
-        self._check(self._core.llmlab_linear_qkv(
+        self._call(self._core.llmlab_linear_qkv,
             self._ptr(h), self._ptr(w_qkv), self._ptr(b_qkv), _dt(b_qkv) if b_qkv is not None else 0,
             self._ptr(q_out), rows, n, k, q_out.stride(0), self._ptr(inv_freq), self._ptr(positions),
             self._ptr(row_req), self._ptr(block_table), block_table.stride(0) if block_table is not None else 0,
             int(page_size), self._ptr(k_cache), self._ptr(v_cache), num_heads, num_kv_heads, head_dim,
-            self.num_cus, self._stream()))
+            self.num_cus, self._stream())
 
     def fused_norm_swiglu(self, x, norm_w, eps, w_gate_up, out, pending: Optional[PendingSums] = None) -> None:
         rows, inter = out.shape
@@ -603,9 +609,9 @@ class HipOps:
         self._need(inv_freq, "rotary frequencies", torch.float32)
         if inv_freq.numel() != d // 2 or positions.numel() < rows:
             raise ValueError("rope: frequency table or positions do not fit")
-        self._check(self._core.llmlab_rope_inplace(
+        self._call(self._core.llmlab_rope_inplace,
             self._ptr(x), _dt(x), rows, heads, d, x.stride(0), x.stride(1), self._ptr(inv_freq),
-            self._ptr(positions), self._stream()))
+            self._ptr(positions), self._stream())
 
     def rope_kv_write(self, qkv, num_heads, num_kv_heads, head_dim, inv_freq, positions, row_req,
                       block_table, page_size, k_cache, v_cache) -> None:
@@ -634,11 +640,11 @@ class HipOps:
                     or k_cache.dtype != qkv.dtype or v_cache.dtype != qkv.dtype):
                 raise ValueError("rope_kv_write: cache tensors do not have the paged layout")
             table_stride = block_table.stride(0)
-        self._check(self._core.llmlab_rope_kv_write(
+        self._call(self._core.llmlab_rope_kv_write,
             self._ptr(qkv), _dt(qkv), rows, qkv.stride(0) if rows > 1 else qkv.shape[1], num_heads,
             num_kv_heads, head_dim, self._ptr(inv_freq), self._ptr(positions), self._ptr(row_req),
             self._ptr(block_table), table_stride, page_size, self._ptr(k_cache), self._ptr(v_cache),
-            self._stream()))
+            self._stream())
 
     # -------------------------------------------------------------- attention
     def paged_attention(self, qkv, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_table,
@@ -681,13 +687,13 @@ class HipOps:
                 self._need(row_req, "row -> request map", torch.int32)
             else:
                 n_short = short_ctx = 0
-        self._check(lib.llmlab_paged_attention(
+        self._call(lib.llmlab_paged_attention,
             self._ptr(qkv), _dt(qkv), q_stride, num_heads, num_kv_heads, self._ptr(k_cache),
             self._ptr(v_cache), self._ptr(block_table), block_table.stride(0), page_size,
             self._ptr(q_start), self._ptr(start_pos), n_reqs, max_q_len, max_ctx_len,
             int(window) if window else 0, float(scale), self._ptr(out), out.stride(0) if rows > 1 else
             out.shape[1], self._ptr(self.workspace), self.workspace.numel(), rows, self.num_cus,
-            self._ptr(row_req), short_len, n_short, short_ctx, self._stream()), lib)
+            self._ptr(row_req), short_len, n_short, short_ctx, self._stream(), lib=lib)
 
     # --------------------------------------------------------------- sampling
     def argmax(self, logits, out) -> None:
@@ -696,9 +702,9 @@ class HipOps:
         rows, vocab = logits.shape
         if logits.stride(1) != 1 or out.numel() < rows:
             raise ValueError("argmax: logits rows must be contiguous and out must hold one token per row")
-        self._check(self._core.llmlab_argmax(
+        self._call(self._core.llmlab_argmax,
             self._ptr(logits), logits.stride(0) if rows > 1 else vocab, rows, vocab, self._ptr(out),
-            self._ptr(self.workspace), self.workspace.numel(), self._stream()))
+            self._ptr(self.workspace), self.workspace.numel(), self._stream())
 
     def sample(self, logits, temperatures, uniforms, out) -> None:
         self._need(logits, "logits", torch.float32, contiguous=False)
@@ -711,6 +717,6 @@ class HipOps:
             self._need(uniforms, "uniform numbers", torch.float32)
             if temperatures.numel() < rows or uniforms.numel() < rows:
                 raise ValueError("sample: one temperature and one uniform number per row")
-        self._check(self._core.llmlab_sample(
+        self._call(self._core.llmlab_sample,
             self._ptr(logits), logits.stride(0) if rows > 1 else vocab, rows, vocab,
-            self._ptr(temperatures), self._ptr(uniforms), self._ptr(out), self._stream()))
+            self._ptr(temperatures), self._ptr(uniforms), self._ptr(out), self._stream())
