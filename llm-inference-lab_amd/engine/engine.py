@@ -97,6 +97,10 @@ class Engine:
             tokens = max_cache_tokens if max_cache_tokens is not None else \
                 self.max_requests * self.max_seq_len
             num_pages = pages_for_tokens(int(tokens), self.page_size)
+            if max_cache_tokens is None:
+                # nobody asked for a size: every request at full length, or what the
+                # memory that the weights left free can hold, whichever is less
+                num_pages = min(num_pages, self._pages_that_fit(groups))
         for g in groups:
             g.num_pages = int(num_pages)
         self.cache = CacheManager(groups, self.page_size, self.max_requests, self.max_seq_len,
@@ -106,6 +110,20 @@ class Engine:
                                     graph=self._graph_choice(graph))
         self._sampler = None
         self.last_scheduler = None
+
+    CACHE_SHARE_OF_FREE_MEMORY = 0.9
+
+    def _pages_that_fit(self, groups) -> int:
+        """Pages (per group) that fit the GPU memory that is free now, leaving a tenth of
+        it for scratch buffers; at least one request of full length."""
+        if self.device.type != "cuda":
+            return 1 << 40
+        width = torch.empty((), dtype=self.dtype).element_size()
+        page_bytes = sum(2 * len(g.entries) * g.spec.num_kv_heads * g.spec.head_dim * width
+                         for g in groups) * self.page_size
+        free, _ = torch.cuda.mem_get_info(self.device)
+        fit = int(free * self.CACHE_SHARE_OF_FREE_MEMORY) // max(page_bytes, 1)
+        return max(fit, pages_for_tokens(self.max_seq_len, self.page_size))
 
     # A decode step replayed from a HIP graph costs the host nothing, but the GPU about a
     # microsecond more at every kernel boundary than kernels launched one by one by a host
