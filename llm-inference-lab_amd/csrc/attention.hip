@@ -96,6 +96,9 @@ struct KeyStep {
 // blocks that split the keys further merge through global memory (see below).
 constexpr int DECODE_WAVES = D <= 64 ? 8 : (D <= 128 ? 4 : 2);
 constexpr int SPLIT_FILL = 1;      // blocks per compute unit a decode step aims at
+#ifndef MAX_KEY_SPLITS
+#define MAX_KEY_SPLITS 128
+#endif
 
 // RING (decode only): key steps a wave keeps in flight; 1 when a wave has one or two
 // steps at all (nothing to run ahead of), 2 for longer shares (deeper rings measured
@@ -629,50 +632,73 @@ __global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void attention_bf16_paired_ke
   }
 }
 
-// Merge of the key splits of a decode step, one block per (row, head):
-//   out = sum_s w_s acc_s / sum_s w_s l_s,  w_s = 2^(m_s - max m), in the order of s.
+// Merge of the key splits of a decode step, one block of four waves per (row, head):
+//   out = sum_s w_s acc_s / sum_s w_s l_s,  w_s = 2^(m_s - max m).
+// Every wave takes a quarter of the splits (lane = element of the head), has all of
+// its partial sums on their way before the first is used (sixteen at a time: up to 64
+// splits cost one trip to memory), and the quarters meet in LDS in their order.
 // A kernel of its own: within one kernel, results of blocks on other dies would
 // need device-wide fences, which cost far more than a launch.
-__global__ __launch_bounds__(64) void attention_merge_kernel(const float* __restrict__ o_part,
-                                                             const float* __restrict__ ml_part,
-                                                             bf16_t* __restrict__ out, int out_stride,
-                                                             int nq, int splits,
-                                                             const int* __restrict__ row_req,
-                                                             const int* __restrict__ q_start, int qlen_hi) {
-  const int row = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
+constexpr int MERGE_WAVES = 4;
+__global__ __launch_bounds__(64 * MERGE_WAVES) void attention_merge_kernel(
+    const float* __restrict__ o_part, const float* __restrict__ ml_part, bf16_t* __restrict__ out,
+    int out_stride, int nq, int splits, const int* __restrict__ row_req, const int* __restrict__ q_start,
+    int qlen_hi) {
+  constexpr int PER = (D + 63) / 64;
+  __shared__ float s_num[MERGE_WAVES][PER * 64];
+  const int row = blockIdx.x, head = blockIdx.y, lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   if (row_req) {      // rows of requests that another launch serves have no partial results
     const int b = row_req[row];
     if (q_start[b + 1] - q_start[b] > qlen_hi) return;
   }
   const size_t at0 = ((size_t)row * nq + head) * splits;
-  float ms = NEG_INF, ls = 0.f;
-  if (lane < splits) {
-    ms = ml_part[(at0 + lane) * 2];
-    ls = ml_part[(at0 + lane) * 2 + 1];
-  }
-  // every partial sum on its way before the first is used
-  constexpr int PER = (D + 63) / 64;
-  float v[PER][16];
+  // in every wave, lane l holds the maxima and sums of the splits l and l + 64
+  float ms[2] = {NEG_INF, NEG_INF}, ls[2] = {0.f, 0.f};
 #pragma unroll
-  for (int p = 0; p < PER; ++p)
-#pragma unroll
-    for (int u = 0; u < 16; ++u) {
-      const int dd = p * 64 + lane;
-      v[p][u] = (u < splits && dd < D) ? o_part[(at0 + u) * D + dd] : 0.f;
+  for (int h = 0; h < 2; ++h)
+    if (h * 64 + lane < splits) {
+      ms[h] = ml_part[(at0 + h * 64 + lane) * 2];
+      ls[h] = ml_part[(at0 + h * 64 + lane) * 2 + 1];
     }
-  const float mmax = wave_max(ms);
-  const float w = ms == NEG_INF ? 0.f : exp2f(ms - mmax);
-  const float wl = w * ls;
-  float den = 0.f;
-  for (int s2 = 0; s2 < splits; ++s2) den += __shfl(wl, s2, WAVE);
+  const int quarter = (splits + MERGE_WAVES - 1) / MERGE_WAVES;
+  const int u_lo = wave * quarter, u_hi = min(u_lo + quarter, splits);
+  float num[PER];
+#pragma unroll
+  for (int p = 0; p < PER; ++p) num[p] = 0.f;
+  float mmax = NEG_INF, w[2] = {0.f, 0.f};
+  for (int u0 = u_lo; u0 < u_hi; u0 += 16) {
+    float v[PER][16];
+#pragma unroll
+    for (int p = 0; p < PER; ++p)
+#pragma unroll
+      for (int u = 0; u < 16; ++u) {
+        const int dd = p * 64 + lane;
+        v[p][u] = (u0 + u < u_hi && dd < D) ? o_part[(at0 + u0 + u) * D + dd] : 0.f;
+      }
+    if (u0 == u_lo) {     // the weights, while the first loads are under way
+      mmax = wave_max(fmaxf(ms[0], ms[1]));
+#pragma unroll
+      for (int h = 0; h < 2; ++h) w[h] = ms[h] == NEG_INF ? 0.f : exp2f(ms[h] - mmax);
+    }
+#pragma unroll
+    for (int p = 0; p < PER; ++p)
+#pragma unroll
+      for (int u = 0; u < 16; ++u) num[p] += __shfl(u0 + u < 64 ? w[0] : w[1], (u0 + u) & 63, WAVE) * v[p][u];
+  }
+#pragma unroll
+  for (int p = 0; p < PER; ++p) s_num[wave][p * 64 + lane] = num[p];
+  __syncthreads();
+  if (wave != 0) return;
+  const float den = wave_sum(w[0] * ls[0] + w[1] * ls[1]);
   const float inv = den > 0.f ? 1.f / den : 0.f;
 #pragma unroll
   for (int p = 0; p < PER; ++p) {
-    float num = 0.f;
-#pragma unroll
-    for (int u = 0; u < 16; ++u) num += __shfl(w, u, WAVE) * v[p][u];
     const int dd = p * 64 + lane;
-    if (dd < D) out[(size_t)row * out_stride + (size_t)head * D + dd] = (bf16_t)(num * inv);
+    float total = 0.f;
+#pragma unroll
+    for (int q = 0; q < MERGE_WAVES; ++q) total += s_num[q][dd];
+    if (dd < D) out[(size_t)row * out_stride + (size_t)head * D + dd] = (bf16_t)(total * inv);
   }
 }
 
@@ -731,6 +757,10 @@ extern "C" const char* llmlab_last_error() { return g_llmlab_error; }
 
 extern "C" int llmlab_attention_head_dim() { return D; }
 
+// Tests and tuning runs may fix the number of key splits (0: chosen here).
+static int g_force_splits = 0;
+extern "C" void llmlab_attention_force_splits(int splits) { g_force_splits = splits; }
+
 // The decode-like launch: a block of DECODE_WAVES waves per (request, kv head, split); a
 // wave gets about two steps of 32 keys, a block's waves merge in LDS, and only what is
 // left is split over blocks; the merge kernel follows.  `live` requests (of `reqs`) pass
@@ -750,7 +780,8 @@ static int launch_key_split_decode(AttnArgs a, int reqs, int live, int ctx_len, 
   int splits = (int)((SPLIT_FILL * (long)num_cus / SPLIT_DIV + base - 1) / base);
   const int most = (steps32 + DECODE_WAVES - 1) / DECODE_WAVES;      // one step per wave at least
   if (splits > most) splits = most;
-  if (splits > 16) splits = 16;                               // what the merge kernel takes
+  if (splits > MAX_KEY_SPLITS) splits = MAX_KEY_SPLITS;       // what the merge kernel takes: two per lane
+  if (g_force_splits > 0) splits = min(g_force_splits, MAX_KEY_SPLITS);
   if (splits < 1) splits = 1;
   const size_t per_split = (size_t)total_rows * nq * (D + 2);
   while (splits > 1 && per_split * splits > workspace_floats) --splits;
@@ -768,7 +799,7 @@ static int launch_key_split_decode(AttnArgs a, int reqs, int live, int ctx_len, 
     hipLaunchKernelGGL((attention_bf16_kernel<1, true, 1>), grid, block, 0, stream, a);
   LLMLAB_LAUNCH_CHECK("attention(bfloat16, decode)");
   if (splits > 1) {
-    hipLaunchKernelGGL(attention_merge_kernel, dim3(total_rows, nq), dim3(64), 0, stream, a.o_part,
+    hipLaunchKernelGGL(attention_merge_kernel, dim3(total_rows, nq), dim3(64 * MERGE_WAVES), 0, stream, a.o_part,
                        a.ml_part, (bf16_t*)out, out_stride, nq, splits, row_req, a.q_start, a.qlen_hi);
     LLMLAB_LAUNCH_CHECK("attention merge");
   }

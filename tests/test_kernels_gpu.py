@@ -496,6 +496,14 @@ def test_attention_far_key_among_hundreds(ops, emu, dtype):
     run_attention(ops, emu, dtype, 14, 2, 64, 64, None, [(4000, 1), (2000, 1)], amplify=(1, 1999, 30.0))
 
 
+@pytest.mark.parametrize("d,length,key", [(64, 9000, 8000), (128, 5000, 70), (64, 20001, 11), (64, 40000, 33000)])
+def test_attention_one_request_over_a_long_history(ops, emu, d, length, key):
+    """One decoded token of a single request: its keys are split over as many blocks
+    as the merge takes (from 35 to the limit of 128 here), and one key far from both ends
+    carries the answer."""
+    run_attention(ops, emu, torch.bfloat16, 4, 1, d, 64, None, [(length - 1, 1)], amplify=(0, key, 30.0))
+
+
 @pytest.mark.parametrize("vocab", [1, 255, 256, 257, 4095, 4097, 151936])
 def test_argmax(ops, emu, vocab):
     """Vocabulary sizes and special rows of the reference's argmax tests
