@@ -130,6 +130,48 @@ def test_block_alone(dtype, name, layer):
     engine.close(req)
 
 
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("name,layer,cuts", [("A", 1, (0, 40, 41, 42, 50)), ("B", 2, (0, 2, 35, 50)),
+                                             ("C", 0, (0, 50))])
+def test_attention_part_alone(dtype, name, layer, cuts):
+    """The attention mixer alone, handed activations that are normed already (so its
+    fused-norm kernel is not the one that runs): projections with bias, rotation,
+    cache, attention (with the layer's window, if it has one), output projection
+    and the sum into the residual rows, over portions and single tokens."""
+    cfg = H.config_of(name)
+    conf = cfg.to_dict()
+    engine = H.make_engine(name, 2, dtype, page_size=16, num_pages=8)
+    w = {k: v.double() for k, v in H.make_tensors(cfg, 2).items()}
+    nq, nkv = cfg.num_attention_heads, cfg.num_key_value_heads
+    d = conf.get("head_dim") or cfg.hidden_size // nq
+    t = cuts[-1]
+    h = rnd((t, cfg.hidden_size), 12).to(torch.bfloat16)          # what a norm would have left
+    resid = rnd((t, cfg.hidden_size), 13, 2.0)
+    p = f"model.layers.{layer}.self_attn."
+    hd, pos = h.double(), torch.arange(t)
+    q = P.rope(P.linear(hd, w[p + "q_proj.weight"], w[p + "q_proj.bias"]).view(t, nq, d), pos, conf["rope_theta"])
+    k = P.rope(P.linear(hd, w[p + "k_proj.weight"], w[p + "k_proj.bias"]).view(t, nkv, d), pos, conf["rope_theta"])
+    v = P.linear(hd, w[p + "v_proj.weight"], w[p + "v_proj.bias"]).view(t, nkv, d)
+    a = P.causal_attention_dense(q, k, v, pos, P.layer_window(conf, layer)).reshape(t, nq * d)
+    want = resid.double() + P.linear(a, w[p + "o_proj.weight"])
+
+    req = engine.open("x")
+    view = engine.model.entries[layer]
+    mixer = engine.model.blocks[view.block].mixer
+    outs = []
+    for lo, hi in zip(cuts, cuts[1:]):
+        engine.cache.reserve(req, hi - lo)
+        engine.step_fn.ctx.fill([H.lab.StepEntry(req, [0] * (hi - lo), [])], engine.cache)
+        rows = resid[lo:hi].clone().to(DEV)
+        mixer.forward(h[lo:hi].to(mixer.dtype).to(DEV), rows, engine.step_fn.ctx, view)
+        engine.cache.commit(req)
+        outs.append(rows.cpu())
+    got = torch.cat(outs)
+    tol = 2e-4 if dtype == "f32" else 5e-2
+    assert (got.double() - want).abs().max() < tol * max(1.0, want.abs().max().item() / 4)
+    engine.close(req)
+
+
 # ---------------------------------------------------------------- toy mixer
 class RunningMean(Mixer):
     """A mixer with state of fixed size and no cache: the output at a token is a
