@@ -890,9 +890,12 @@ extern "C" int llmlab_paged_attention(const void* q, int dtype, int q_stride, in
   if (D <= 128 && blocks32 >= 2L * num_cus) {
     dim3 grid((unsigned)((max_rows + 127) / 128), nkv, reqs), block(256);
     hipLaunchKernelGGL((attention_bf16_kernel<2, false>), grid, block, 0, stream, a);
-  } else if (window <= 0 && blocks16 >= (3L * num_cus) / 2) {
+  } else if (window <= 0 && blocks16 >= (3L * num_cus) / 2 && 16L * (max_ctx_len - max_q_len) <= max_q_len) {
     // not enough tiles to keep every unit busy with what the longest ones leave over:
-    // pair late and early tiles (no window: then the loads add up evenly)
+    // pair late and early tiles (no window: then the loads add up evenly).  Only at the
+    // start of a prompt: behind a history all tiles carry about the same load, and the
+    // pairs only halve the blocks (2,048 tokens behind 8,192, head size 64: 246 us in
+    // pairs, 172 without)
     a.tiles = (int)((max_rows + 63) / 64);
     dim3 grid((unsigned)((a.tiles + 1) / 2), nkv, reqs), block(256);
     hipLaunchKernelGGL((attention_bf16_paired_kernel<1>), grid, block, 0, stream, a);

@@ -355,6 +355,33 @@ def test_attention_of_a_mixed_step(ops, emu, window):
     run_attention(ops, emu, torch.bfloat16, 8, 1, 128, 32, window, spec[:4], seed=92)
 
 
+@pytest.mark.parametrize("window", [None, 40])
+@pytest.mark.parametrize("cus", [8, 16, 30, 60, 80, 100, 1000])
+@pytest.mark.parametrize("nq,nkv,d,page", [(14, 2, 64, 64), (6, 3, 48, 16), (8, 1, 128, 32), (2, 1, 256, 16)])
+def test_attention_tilings_of_many_rows(ops, emu, window, cus, nq, nkv, d, page):
+    """The kernel variants for many tiles of rows (tiles of 128 rows, of 64, of 64 in
+    pairs, keys split over the waves of a block) are chosen by the tiles per compute
+    unit: told of fewer units than the chip has, a step of a few hundred rows takes
+    each of them."""
+    real = ops.num_cus
+    ops.num_cus = cus
+    try:
+        run_attention(ops, emu, torch.bfloat16, nq, nkv, d, page, window, [(0, 300), (0, 200)], seed=93,
+                      amplify=(0, 70, 30.0))
+        # behind a history (never in pairs), and one request decoding beside
+        run_attention(ops, emu, torch.bfloat16, nq, nkv, d, page, window, [(500, 300), (64, 200), (900, 1)], seed=94,
+                      amplify=(0, 130 if window is None else 770, 30.0))
+    finally:
+        ops.num_cus = real
+
+
+@pytest.mark.parametrize("start", [0, 3000])
+def test_attention_of_a_long_portion(ops, emu, start):
+    """2,048 tokens of a prompt at the 0.5B head counts, at its start and behind a
+    history: enough tiles for the whole chip, as in a prefill step of the engine."""
+    run_attention(ops, emu, torch.bfloat16, 14, 2, 64, 64, None, [(start, 2048)], seed=95, amplify=(0, 1033, 30.0))
+
+
 def make_cache(num_pages, nkv, page, d, dtype, seed):
     k = rnd((num_pages, nkv, page, d), dtype, seed)
     v = rnd((num_pages, nkv, d, page), dtype, seed + 1)
