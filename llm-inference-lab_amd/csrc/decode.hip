@@ -693,6 +693,11 @@ extern "C" int llmlab_skinny_linear(const void* x, int norm, const int* x_rows, 
   const size_t lds = skinny_lds_bytes(shape.nsb, shape.kw, mb, tile_rows, K, epilogue, shape.stage);
   LLMLAB_REQUIRE(lds <= SK_LDS_LIMIT && shape.nsb * shape.kw <= (mb >= 4 ? 8 : 16),
                  "skinny_linear: block shape %dx%d does not fit", shape.nsb, shape.kw);
+  // (only a forced shape can fail these: a gate strip and its up strip share a block, and
+  // every K slice has a step)
+  LLMLAB_REQUIRE(!(epilogue == SK_SWIGLU && shape.nsb % 2 != 0) &&
+                     shape.kw <= ((K + 31) / 32 + ksplit - 1) / ksplit,
+                 "skinny_linear: block shape %dx%d does not fit this product", shape.nsb, shape.kw);
   const int blocks = (N + 16 * shape.nsb - 1) / (16 * shape.nsb) * ksplit;
   SkinnyArgs a;
   a.pend = pend; a.pend_splits = pend_splits; a.pend_ld = pend_ld; a.pend_stride = pend_stride;

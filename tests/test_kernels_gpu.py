@@ -229,6 +229,55 @@ def test_few_row_products(ops, emu, m, n, k):
     close(got, want, torch.float32, "few-row residual", want.abs().max().item() * 4)
 
 
+@pytest.mark.parametrize("mb", [1, 2, 4])
+@pytest.mark.parametrize("stage", [0, 1])
+@pytest.mark.parametrize("nsb,kw", [(1, 1), (1, 4), (1, 16), (2, 2), (2, 8), (4, 1), (4, 4), (8, 2), (16, 1)])
+def test_few_row_products_in_every_block_shape(ops, emu, nsb, kw, stage, mb):
+    """The block shape (strips per block, K slices per strip, staged rows or not, rows
+    per tile) is chosen by a cost estimate, so most shapes never run at a given size:
+    each is forced here.  A shape that does not fit says so and computes nothing."""
+    from llm_inference_lab_amd.kernels.hip_ops import KernelError
+    from llm_inference_lab_amd.parts.feed_forward import interleave_gate_up
+    dtype = torch.bfloat16
+    ran = 0
+    for m, n, k in ((5, 130, 264), (40, 896, 1160), (64, 320, 96)):
+        x, w = rnd((m, k), dtype, 44), rnd((n, k), dtype, 45, 0.1)
+        bias, resid = rnd((n,), torch.float32, 46), rnd((m, n), torch.float32, 47)
+        gate_up = interleave_gate_up(w, rnd((n, k), dtype, 48, 0.1))
+        want = torch.empty(m, n, dtype=dtype)
+        emu.linear(x, w, want, bias)
+        want_resid = resid.clone()
+        emu.linear_residual(x, w, want_resid)
+        want_act = torch.empty(m, n, dtype=dtype)
+        emu.linear_swiglu(x, gate_up, want_act)
+        xd, wd, gd = x.to(DEV), ops.prepare_weight(w.to(DEV)), ops.prepare_weight(gate_up.to(DEV))
+        def forced(fn):
+            """Runs fn under the forced shape; False if the kernel refused the shape."""
+            ops._core.llmlab_skinny_force(nsb, kw, stage, mb)
+            try:
+                fn()
+                return True
+            except KernelError as err:
+                assert "does not fit" in str(err) or "no block shape" in str(err), err
+                return False
+            finally:
+                ops._core.llmlab_skinny_force(0, 0, -1, 0)
+
+        got = torch.full((m, n), float("nan"), dtype=dtype, device=DEV)
+        if forced(lambda: ops.linear(xd, wd, got, bias.to(DEV))):
+            ran += 1
+            close(got, want, dtype, f"forced {nsb}x{kw} linear", want.float().abs().max().item())
+        got_resid = resid.clone().to(DEV)
+        if forced(lambda: ops.linear_residual(xd, wd, got_resid)):
+            ran += 1
+            close(got_resid, want_resid, torch.float32, f"forced {nsb}x{kw} residual", want_resid.abs().max().item() * 4)
+        got_act = torch.full((m, n), float("nan"), dtype=dtype, device=DEV)
+        if forced(lambda: ops.linear_swiglu(xd, gd, got_act)):
+            ran += 1
+            close(got_act, want_act, dtype, f"forced {nsb}x{kw} swiglu", want_act.float().abs().max().item())
+    assert ran > 0 or nsb * kw > 8, "no size ran this shape"
+
+
 @pytest.mark.parametrize("wdtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("m", [1, 8, 17, 33, 64])
 @pytest.mark.parametrize("hidden,inter,vocab", [(64, 128, 256), (96, 320, 515), (896, 4864, 3001), (72, 200, 301)])
