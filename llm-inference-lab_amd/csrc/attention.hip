@@ -95,7 +95,6 @@ struct KeyStep {
 // block share one tile and split the block's keys; they merge through LDS, and
 // blocks that split the keys further merge through global memory (see below).
 constexpr int DECODE_WAVES = D <= 64 ? 8 : (D <= 128 ? 4 : 2);
-constexpr int SPLIT_FILL = 1;      // blocks per compute unit a decode step aims at
 #ifndef MAX_KEY_SPLITS
 #define MAX_KEY_SPLITS 128
 #endif
@@ -770,14 +769,13 @@ static int launch_key_split_decode(AttnArgs a, int reqs, int live, int ctx_len, 
                                    const int* row_req, void* out, int out_stride, hipStream_t stream) {
   const int visible = window > 0 ? min(window, ctx_len) : ctx_len;
   const int steps32 = (visible + 31) / 32 + 1;
-  // about SPLIT_FILL blocks per compute unit: a unit's memory rate is the limit, so
-  // the keys are spread over all of them; but no more blocks than there are steps
-  // for their waves
+  // A unit's memory rate is the limit, so the keys are spread over the units: as many
+  // splits as still give every block a unit of its own.  One block more than units
+  // would double the load of the busiest one (24 requests of 4 kv heads over 4,096
+  // keys: 2 splits 44 us, 3 splits 59 us); and once there are more blocks than units
+  // anyway, splitting only adds work.
   const long base = (long)live * nkv;
-#ifndef SPLIT_DIV
-#define SPLIT_DIV 1
-#endif
-  int splits = (int)((SPLIT_FILL * (long)num_cus / SPLIT_DIV + base - 1) / base);
+  int splits = (int)(num_cus / base);
   const int most = (steps32 + DECODE_WAVES - 1) / DECODE_WAVES;      // one step per wave at least
   if (splits > most) splits = most;
   if (splits > MAX_KEY_SPLITS) splits = MAX_KEY_SPLITS;       // what the merge kernel takes: two per lane

@@ -112,7 +112,7 @@ constexpr int SK_APAD = 8;   // padding of a staged row, in elements: 16-byte re
 // floats of LDS before the staged rows (host and device must agree)
 __host__ __device__ inline size_t sk_float_words(int nsb, int kw, int mb, int M, int epi) {
   size_t f = (size_t)kw * nsb * mb * 256;        // partial sums
-  f += (size_t)mb * 16;                           // inverse rms
+  f += (size_t)mb * 16 + 16;                      // inverse rms; sums of squares of the parts of a row
   f += (size_t)16 * nsb;                          // bias
   f += (size_t)mb * 16 * 2 + 128;                 // positions, pages, frequencies
   if (epi == SK_SWIGLU || epi == SK_QKV) f += (size_t)M * 16 * nsb;
@@ -164,7 +164,8 @@ __global__ __launch_bounds__(MB >= 4 ? 512 : 1024) void skinny_block_kernel(Skin
 
   float* part = smem;                                   // [kw*nsb][MB][64][4]
   float* inv = part + (size_t)kw * nsb * MB * 256;      // [MB*16]
-  float* s_bias = inv + MB * 16;                        // [cols]
+  float* s_ssq = inv + MB * 16;                         // [16]: a row's sum of squares, by the waves that share it
+  float* s_bias = s_ssq + 16;                           // [cols]
   int* s_pos = (int*)(s_bias + cols);                   // [MB*16]
   int* s_page = s_pos + MB * 16;                        // [MB*16]
   float* s_freq = (float*)(s_page + MB * 16);           // [128]
@@ -247,14 +248,19 @@ __global__ __launch_bounds__(MB >= 4 ? 512 : 1024) void skinny_block_kernel(Skin
 #pragma unroll
     for (int u = 0; u < R; ++u) b[u] = wload(min(s_begin + u, s_end - 1));
     // ---- the first weight tiles are on their way; stage the rows of x
+    // Fewer rows than waves: `wpr` waves share a row, each taking every wpr-th run of 64
+    // chunks (one wave alone would walk a long row in many trips while the others wait)
     const int chunks = K >> 3, chunks_pad = steps * 4;
-    for (int r = wave; r < M; r += nwaves) {
+    int wpr = 1;
+    while (2 * wpr * M <= nwaves) wpr *= 2;
+    for (int unit = wave; unit < M * wpr; unit += nwaves) {
+      const int r = unit / wpr, sub = unit - r * wpr;
       bf16_t* dst = As + (size_t)r * lda;
       if constexpr (NORM) {
         const float* src = (const float*)a.x + (size_t)(a.x_rows ? a.x_rows[r] : r) * K;
         float ssq = 0.f;
         const size_t prow = (size_t)(a.x_rows ? a.x_rows[r] : r) * a.pend_ld;
-        for (int ch = lane; ch < chunks; ch += 64) {
+        for (int ch = sub * 64 + lane; ch < chunks; ch += 64 * wpr) {
           floatx4 p = *(const floatx4*)(src + ch * 8), q = *(const floatx4*)(src + ch * 8 + 4);
           // sums still owed to these rows: four pieces at a time, loads unconditional
           // (past the last piece: the last one again, not added) so that they travel together
@@ -297,14 +303,27 @@ __global__ __launch_bounds__(MB >= 4 ? 512 : 1024) void skinny_block_kernel(Skin
           *(bf16x8*)(dst + ch * 8) = av;
         }
         ssq = wave_sum(ssq);
-        if (lane == 0) inv[r] = rsqrtf(ssq / (float)K + a.eps);
+        if (lane == 0) {
+          if (wpr == 1) inv[r] = rsqrtf(ssq / (float)K + a.eps);
+          else s_ssq[unit] = ssq;       // (M * wpr <= 16 waves)
+        }
       } else {
         const bf16_t* src = (const bf16_t*)a.x + (size_t)r * K;
-        for (int ch = lane; ch < chunks; ch += 64) *(bf16x8*)(dst + ch * 8) = *(const bf16x8*)(src + ch * 8);
+        for (int ch = sub * 64 + lane; ch < chunks; ch += 64 * wpr)
+          *(bf16x8*)(dst + ch * 8) = *(const bf16x8*)(src + ch * 8);
       }
-      for (int ch = chunks + lane; ch < chunks_pad; ch += 64) *(bf16x8*)(dst + ch * 8) = zero;
+      if (sub == 0)
+        for (int ch = chunks + lane; ch < chunks_pad; ch += 64) *(bf16x8*)(dst + ch * 8) = zero;
     }
     __syncthreads();
+    if constexpr (NORM) {
+      // the parts of a row in their order (read by the epilogue, behind the next barrier)
+      if (wpr > 1 && (int)threadIdx.x < M) {
+        float total = 0.f;
+        for (int sub = 0; sub < wpr; ++sub) total += s_ssq[threadIdx.x * wpr + sub];
+        inv[threadIdx.x] = rsqrtf(total / (float)K + a.eps);
+      }
+    }
     // rows past M are not staged: their lanes read the last row, and what they
     // compute lands in rows of the result that nobody reads
     const bf16_t* arow[MB];

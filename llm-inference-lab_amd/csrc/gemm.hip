@@ -430,20 +430,29 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__
 // estimate of the time, fitted to sweeps of the three products of a layer at two model
 // shapes and 576 to 4096 rows (its picks cost 1.4 % over the best shape there):
 //   time = L + rounds * (f + K tiles * tk),  rounds = max(1, blocks / (units * resident)).
+// With few rows the product is bound by the read of W instead: a block draws `stream`
+// bytes a microsecond, the chip 5.3e6 at most (one tile of rows, 17 to 64 of them, of
+// matrices from 9 to 283 MB, in 4 or 8 pieces: the estimate is within 2 us of the
+// measurement).
 enum { TILE_64 = 0, TILE_64x128 = 1, TILE_128 = 2 };
 struct TileModel {
   int bm, bn;
-  double L, f, tk, resident;
+  double L, f, tk, resident, stream;
 };
-static const TileModel TILE_MODELS[3] = {
-    {64, 64, 6.39, 0.79, 0.289, 1.0}, {64, 128, 6.54, 0.71, 0.552, 1.5}, {128, 128, 9.78, 0.48, 0.704, 1.0}};
+static const TileModel TILE_MODELS[3] = {{64, 64, 6.39, 0.79, 0.289, 1.0, 20e3},
+                                         {64, 128, 6.54, 0.71, 0.552, 1.5, 27e3},
+                                         {128, 128, 9.78, 0.48, 0.704, 1.0, 24e3}};
+constexpr double CHIP_STREAM = 5.3e6;     // bytes a microsecond
 
 static double tile_cost(int kind, int M, int N, int K, int num_cus, int pieces) {
   const TileModel& t = TILE_MODELS[kind];
   const double blocks = (double)((M + t.bm - 1) / t.bm) * ((N + t.bn - 1) / t.bn) * pieces;
   const double rounds = blocks / (num_cus * t.resident);
   const int nk = ((K + 63) / 64 + pieces - 1) / pieces;
-  return t.L + (rounds > 1.0 ? rounds : 1.0) * (t.f + nk * t.tk);
+  const double compute = (rounds > 1.0 ? rounds : 1.0) * (t.f + nk * t.tk);
+  const double rate = blocks * t.stream < CHIP_STREAM ? blocks * t.stream : CHIP_STREAM;
+  const double read = (double)N * K * 2.0 / rate;
+  return t.L + (compute > read ? compute : read);
 }
 
 // A tile can be forced for measurements (0 = choose; 64, 130 = 64 x 128, 129 = 128 x 128).
@@ -501,6 +510,11 @@ extern "C" void llmlab_linear_plan(int M, int N, int K, int num_cus, int max_pie
       }
     }
   }
+  // One tile of rows in pieces: the small tile, if its blocks still find a compute unit
+  // each (17 to 64 rows of matrices from 9 to 45 MB: 8.6 against 11.0, 12.4 against
+  // 15.8, 15.1 against 18.8 us; with more blocks than units it is the slower one)
+  if (M <= 64 && best_pieces > 1 && g_force_tile == 0 && (long)((N + 63) / 64) * best_pieces <= num_cus)
+    best_kind = TILE_64;
   out[0] = best_pieces;
   out[1] = best_kind;
 }

@@ -411,6 +411,24 @@ class HipOps:
     min_steps_per_split = 8       # K steps of 32 a piece should have at least (tests lower it)
     min_tiles_per_split = 8       # many rows: K tiles of 64 a piece should have at least
     force_tiled_pieces = 0        # many rows: this many pieces whatever the estimate says (tests)
+    TILED_PIECES_BYTES = 16e6     # from 17 rows on, a matrix of this size is cut by the tiled kernel:
+                                  # the few-row kernel reads it once per tile of 16 rows (64 rows of
+                                  # 3584 x 18944: 89 us against 34; of 1536 x 8960: 25 against 13)
+
+    PIECES_PER_BLOCK_BYTES = 1 << 20
+
+    def pieces_too_large_to_read_per_block(self, pending: Optional[PendingSums]) -> bool:
+        """A fused kernel that takes pieces on adds them as it reads the rows, in every one
+        of its blocks; beyond this size the norm kernel should fold them once instead
+        (32 rows of width 3584 in 7 pieces, 3.2 MB: 12 us a layer more in the fused kernels)."""
+        if pending is None:
+            return False
+        p = pending.parts
+        return pending.splits * p.shape[1] * p.shape[2] * 4 > self.PIECES_PER_BLOCK_BYTES
+
+    def _pieces_by_tiles(self, rows: int, n: int, k: int) -> bool:
+        """Whether a product left in pieces is cut by the tiled kernel (else by the few-row one)."""
+        return rows > self.FUSED_MAX_ROWS or (rows > self.FUSE_TILE_ROWS and 2.0 * n * k >= self.TILED_PIECES_BYTES)
 
     def split_count(self, rows: int, dtype, n: int, k: int) -> int:
         """Into how many pieces along the inner size a few-row product ``[rows, k] x
@@ -419,7 +437,7 @@ class HipOps:
         memory.  1: do not cut."""
         if dtype != torch.bfloat16 or rows <= 0:
             return 1
-        if rows > self.FUSED_MAX_ROWS:
+        if self._pieces_by_tiles(rows, n, k):
             # many rows, tiled kernel: its own estimate (rounds of blocks over the chip times
             # the K tiles of a block, plus a write and a read of the result for every piece)
             if k % 8:
@@ -453,7 +471,7 @@ class HipOps:
                              f"parts {tuple(parts.shape)} for {splits} pieces do not fit")
         if not 1 <= splits <= self.MAX_SPLITS:
             raise ValueError(f"linear_partials: {splits} pieces")
-        if m <= self.FUSED_MAX_ROWS:
+        if not self._pieces_by_tiles(m, n, k):
             self._skinny(x, False, None, None, 0.0, w, bias, EPI_PART, parts, m, n, k, parts.stride(1), n,
                          ksplit=splits, part_stride=parts.stride(0))
         else:

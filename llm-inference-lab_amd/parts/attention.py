@@ -105,7 +105,8 @@ class GQAAttention(Mixer):
         k_cache = entry.k_cache if entry.writes_cache else None
         v_cache = entry.v_cache if entry.writes_cache else None
         fuse = (isinstance(h, NormedInput) and ops.can_fuse(rows, self.dtype, self.hidden_size, self.q_size + 2 * self.kv_size)
-                and (self.position is None or table is not None))
+                and (self.position is None or table is not None)
+                and not ops.pieces_too_large_to_read_per_block(getattr(ctx, "pending", None)))
         rms = h.rms(accept_pending=True) if fuse else None
         pending = None
         if rms is not None:

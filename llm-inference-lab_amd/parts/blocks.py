@@ -101,7 +101,8 @@ class LinearHead(Part):
     takes_normed_input = True
 
     def forward(self, h, out):
-        fuse = isinstance(h, NormedInput) and self.ops.can_fuse(out.shape[0], self.dtype, self.hidden_size, out.shape[1])
+        fuse = (isinstance(h, NormedInput) and self.ops.can_fuse(out.shape[0], self.dtype, self.hidden_size, out.shape[1])
+                and not self.ops.pieces_too_large_to_read_per_block(getattr(h.ctx, "pending", None)))
         rms = h.rms(accept_pending=True) if fuse else None
         if rms is not None:
             # the last reader of the stream: pieces still owed to it are added on the fly

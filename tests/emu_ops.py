@@ -124,6 +124,9 @@ class EmuOps:
     FUSED_MAX_ROWS = 64
     fuse_max_rows = 16
 
+    def pieces_too_large_to_read_per_block(self, pending):
+        return False
+
     def can_fuse(self, rows, dtype, inner, outer=None):
         return self.fuse and dtype == torch.bfloat16 and 0 < rows <= self.fuse_max_rows
 

@@ -91,16 +91,22 @@ def test_sums_left_in_pieces_reach_every_reader(name, cut):
 
 
 @pytest.mark.parametrize("name", ["A", "B"])
-@pytest.mark.parametrize("cut", ["whole", "decode"])
-def test_sums_of_many_rows_left_in_pieces(name, cut):
+@pytest.mark.parametrize("cut,from_rows", [("whole", 65), ("decode", 65), ("whole", 17), ("portions", 17),
+                                           ("mixed", 17)])
+def test_sums_of_many_rows_left_in_pieces(name, cut, from_rows):
     """The same for steps of many rows (tiled product cut along its inner size): the next
     layer's norm folds the pieces into the stream as it reads it, the final norm of
-    gathered rows has them folded first."""
+    gathered rows has them folded first.  Large matrices take this path from 17 rows on
+    (the next reader is then a fused kernel of few rows or the norm): the tiny ones do
+    too with the size limit taken away."""
     seqs = sequences_of(name)
     want = {rid: H.plain_logits(name, 1, ids) for rid, ids in seqs.items()}
     engine = H.make_engine(name, 1, "bf16", page_size=16, num_pages=40, max_requests=4)
     engine.ops.force_tiled_pieces = 2
     cfg = H.config_of(name)
+    if from_rows == 17:
+        engine.ops.TILED_PIECES_BYTES = 0
+        assert engine.ops.split_count(17, torch.bfloat16, cfg.hidden_size, cfg.intermediate_size) == 2
     assert engine.ops.split_count(130, torch.bfloat16, cfg.hidden_size, cfg.intermediate_size) > 1
     got = H.run_trace(engine, seqs, CUTS[cut](seqs))
     bad = H.first_wrong(got, want, H.TOL["bf16"])
