@@ -635,7 +635,8 @@ __global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void attention_bf16_paired_ke
 //   out = sum_s w_s acc_s / sum_s w_s l_s,  w_s = 2^(m_s - max m).
 // Every wave takes a quarter of the splits (lane = element of the head), has all of
 // its partial sums on their way before the first is used (sixteen at a time: up to 64
-// splits cost one trip to memory), and the quarters meet in LDS in their order.
+// splits cost one trip to memory), and the quarters meet in LDS in their order.  Up to
+// sixteen splits are one wave's work, and the block is launched with one.
 // A kernel of its own: within one kernel, results of blocks on other dies would
 // need device-wide fences, which cost far more than a launch.
 constexpr int MERGE_WAVES = 4;
@@ -660,7 +661,8 @@ __global__ __launch_bounds__(64 * MERGE_WAVES) void attention_merge_kernel(
       ms[h] = ml_part[(at0 + h * 64 + lane) * 2];
       ls[h] = ml_part[(at0 + h * 64 + lane) * 2 + 1];
     }
-  const int quarter = (splits + MERGE_WAVES - 1) / MERGE_WAVES;
+  const int nw = (int)blockDim.x >> 6;      // four waves, or one for sixteen splits or fewer
+  const int quarter = (splits + nw - 1) / nw;
   const int u_lo = wave * quarter, u_hi = min(u_lo + quarter, splits);
   float num[PER];
 #pragma unroll
@@ -696,7 +698,7 @@ __global__ __launch_bounds__(64 * MERGE_WAVES) void attention_merge_kernel(
     const int dd = p * 64 + lane;
     float total = 0.f;
 #pragma unroll
-    for (int q = 0; q < MERGE_WAVES; ++q) total += s_num[q][dd];
+    for (int q = 0; q < nw; ++q) total += s_num[q][dd];
     if (dd < D) out[(size_t)row * out_stride + (size_t)head * D + dd] = (bf16_t)(total * inv);
   }
 }
@@ -797,7 +799,7 @@ static int launch_key_split_decode(AttnArgs a, int reqs, int live, int ctx_len, 
     hipLaunchKernelGGL((attention_bf16_kernel<1, true, 1>), grid, block, 0, stream, a);
   LLMLAB_LAUNCH_CHECK("attention(bfloat16, decode)");
   if (splits > 1) {
-    hipLaunchKernelGGL(attention_merge_kernel, dim3(total_rows, nq), dim3(64 * MERGE_WAVES), 0, stream, a.o_part,
+    hipLaunchKernelGGL(attention_merge_kernel, dim3(total_rows, nq), dim3(splits > 16 ? 64 * MERGE_WAVES : 64), 0, stream, a.o_part,
                        a.ml_part, (bf16_t*)out, out_stride, nq, splits, row_req, a.q_start, a.qlen_hi);
     LLMLAB_LAUNCH_CHECK("attention merge");
   }

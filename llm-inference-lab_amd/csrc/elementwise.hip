@@ -1,5 +1,7 @@
 // Embedding gather, RMSNorm, and rotary position encoding fused with the
 // write of keys and values into the paged cache.  gfx950 only.
+#include <type_traits>
+
 #include "common.h"
 
 extern "C" const char* llmlab_last_error() { return g_llmlab_error; }
@@ -84,19 +86,40 @@ __global__ void rmsnorm_kernel(float* __restrict__ x, const void* __restrict__ w
   const int stride = blockDim.x * W;
   float keep[KEEP][W], wk[KEEP][W];
   float ss = 0.f;
-  auto fetch = [&](int c, float* v) {       // the whole values of elements c .. c+W-1, written back if pieces came in
+  // Pieces come G at a time, loads unconditional (past the last piece: the last one again,
+  // not added), so that they travel together instead of one after the other; G = 2 for
+  // one or two pieces, which many rows bring, G = 4 for the many pieces of few rows.
+  auto fetch_by = [&](int c, float* v, auto group) {
+    constexpr int G = decltype(group)::value;
     if constexpr (VEC) {
       floatx4 t = *(const floatx4*)(src + c);
-      for (int s = 0; s < splits; ++s) t += *(const floatx4*)(prow + s * pend_stride + c);
+      for (int s0 = 0; s0 < splits; s0 += G) {
+        floatx4 p[G];
+#pragma unroll
+        for (int j = 0; j < G; ++j) p[j] = *(const floatx4*)(prow + (size_t)min(s0 + j, splits - 1) * pend_stride + c);
+#pragma unroll
+        for (int j = 0; j < G; ++j)
+          if (s0 + j < splits) t += p[j];
+      }
       if (splits > 0) *(floatx4*)(src + c) = t;
 #pragma unroll
       for (int e = 0; e < W; ++e) v[e] = t[e];
     } else {
       float t = src[c];
-      for (int s = 0; s < splits; ++s) t += prow[s * pend_stride + c];
+      for (int s0 = 0; s0 < splits; s0 += G) {
+        float p[G];
+#pragma unroll
+        for (int j = 0; j < G; ++j) p[j] = prow[(size_t)min(s0 + j, splits - 1) * pend_stride + c];
+#pragma unroll
+        for (int j = 0; j < G; ++j) t += s0 + j < splits ? p[j] : 0.f;
+      }
       if (splits > 0) src[c] = t;
       v[0] = t;
     }
+  };
+  auto fetch = [&](int c, float* v) {       // the whole values of elements c .. c+W-1, written back if pieces came in
+    if (splits > 2) fetch_by(c, v, std::integral_constant<int, 4>{});
+    else fetch_by(c, v, std::integral_constant<int, 2>{});
   };
 #pragma unroll
   for (int j = 0; j < KEEP; ++j) {
