@@ -426,7 +426,7 @@ class HipOps:
         p = pending.parts
         return pending.splits * p.shape[1] * p.shape[2] * 4 > self.PIECES_PER_BLOCK_BYTES
 
-    def _pieces_by_tiles(self, rows: int, n: int, k: int) -> bool:
+    def pieces_by_tiles(self, rows: int, n: int, k: int) -> bool:
         """Whether a product left in pieces is cut by the tiled kernel (else by the few-row one)."""
         return rows > self.FUSED_MAX_ROWS or (rows > self.FUSE_TILE_ROWS and 2.0 * n * k >= self.TILED_PIECES_BYTES)
 
@@ -437,7 +437,7 @@ class HipOps:
         memory.  1: do not cut."""
         if dtype != torch.bfloat16 or rows <= 0:
             return 1
-        if self._pieces_by_tiles(rows, n, k):
+        if self.pieces_by_tiles(rows, n, k):
             # many rows, tiled kernel: its own estimate (rounds of blocks over the chip times
             # the K tiles of a block, plus a write and a read of the result for every piece)
             if k % 8:
@@ -471,7 +471,7 @@ class HipOps:
                              f"parts {tuple(parts.shape)} for {splits} pieces do not fit")
         if not 1 <= splits <= self.MAX_SPLITS:
             raise ValueError(f"linear_partials: {splits} pieces")
-        if not self._pieces_by_tiles(m, n, k):
+        if not self.pieces_by_tiles(m, n, k):
             self._skinny(x, False, None, None, 0.0, w, bias, EPI_PART, parts, m, n, k, parts.stride(1), n,
                          ksplit=splits, part_stride=parts.stride(0))
         else:

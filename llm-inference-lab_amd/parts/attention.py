@@ -151,6 +151,15 @@ class GQAAttention(Mixer):
         if pending is not None:
             ops.linear_residual(out, self.w_o, residual, self.b_o, pending=pending)
             ctx.pending = None
+            return
+        splits = 1
+        if getattr(ctx, "pending", 0) is None and ops.pieces_by_tiles(rows, self.hidden_size, self.q_size):
+            splits = ops.split_count(rows, self.dtype, self.hidden_size, self.q_size)
+        if splits > 1:
+            # some rows of a large matrix: cut along the inner size, the pieces left for the
+            # norm that reads the stream next
+            parts = ctx.scratch("attention.pieces", (splits, rows, self.hidden_size), torch.float32)
+            ctx.pending = ops.linear_partials(out, self.w_o, parts, splits, self.b_o)
         else:
             ops.linear_residual(out, self.w_o, residual, self.b_o)
 

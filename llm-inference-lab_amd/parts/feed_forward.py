@@ -69,8 +69,10 @@ class SwiGLU(FeedForward):
     def forward(self, h, residual, ctx):
         rows = h.shape[0]
         act = ctx.scratch("swiglu.act", (rows, self.intermediate_size), self.dtype)
-        rms = h.rms() if isinstance(h, NormedInput) else None
-        if rms is not None and self.ops.can_fuse(rows, self.dtype, self.hidden_size, self.w_gate_up.shape[0]):
+        fuse = isinstance(h, NormedInput) and self.ops.can_fuse(rows, self.dtype, self.hidden_size,
+                                                                 self.w_gate_up.shape[0])
+        rms = h.rms() if fuse else None      # (folds pieces still owed to the stream; else the norm does)
+        if rms is not None:
             self.ops.fused_norm_swiglu(rms[0], rms[2], rms[3], self.w_gate_up, act)
         else:
             if isinstance(h, NormedInput):

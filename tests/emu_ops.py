@@ -127,6 +127,9 @@ class EmuOps:
     def pieces_too_large_to_read_per_block(self, pending):
         return False
 
+    def pieces_by_tiles(self, rows, n, k):
+        return False
+
     def can_fuse(self, rows, dtype, inner, outer=None):
         return self.fuse and dtype == torch.bfloat16 and 0 < rows <= self.fuse_max_rows
 
