@@ -463,6 +463,14 @@ static int choose_tile(int M, int N, int K, int num_cus) {
   if (g_force_tile == 64) return TILE_64;
   if (g_force_tile == 130) return TILE_64x128;
   if (g_force_tile == 129 || g_force_tile == 128) return TILE_128;
+  // One or two tiles of rows of a wide matrix (the head, gate and up at larger shapes):
+  // bound by the read of W, which the wider tiles stream better than the estimate
+  // knows, and the 128-row tile reads W once where two 64-row tiles read it twice
+  // (64 rows, 152064 x 3584: 220 us against 250 with the 64 x 64 tile; 128 rows,
+  // 55296 x 5120: 127 against 157).
+  const long wide = (N + 127) / 128;
+  if (M <= 64 && wide >= num_cus) return TILE_64x128;
+  if (M > 64 && M <= 128 && wide >= 3L * num_cus / 2) return TILE_128;
   int best = 0;
   double best_cost = 1e30;
   for (int kind = 0; kind < 3; ++kind) {
