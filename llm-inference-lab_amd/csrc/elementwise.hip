@@ -1,7 +1,5 @@
 // Embedding gather, RMSNorm, and rotary position encoding fused with the
 // write of keys and values into the paged cache.  gfx950 only.
-#include <type_traits>
-
 #include "common.h"
 
 extern "C" const char* llmlab_last_error() { return g_llmlab_error; }
@@ -73,7 +71,7 @@ extern "C" int llmlab_embed(const void* table, int dtype, int packed, const int*
 // registers, so a row of up to KEEP * W * blockDim.x elements costs one trip to
 // memory; what lies beyond is read again after the reduction.  VEC: groups of four
 // (hidden % 4 == 0 and 16-byte aligned rows).
-template <typename T, bool VEC>
+template <typename T, bool VEC, int G>
 __global__ void rmsnorm_kernel(float* __restrict__ x, const void* __restrict__ w, int w_bf16,
                                float eps, T* __restrict__ out, const int* __restrict__ rows,
                                int hidden, const float* __restrict__ pend, int splits, size_t pend_stride) {
@@ -87,10 +85,12 @@ __global__ void rmsnorm_kernel(float* __restrict__ x, const void* __restrict__ w
   float keep[KEEP][W], wk[KEEP][W];
   float ss = 0.f;
   // Pieces come G at a time, loads unconditional (past the last piece: the last one again,
-  // not added), so that they travel together instead of one after the other; G = 2 for
-  // one or two pieces, which many rows bring, G = 4 for the many pieces of few rows.
-  auto fetch_by = [&](int c, float* v, auto group) {
-    constexpr int G = decltype(group)::value;
+  // not added), so that they travel together instead of one after the other: G = 4 for
+  // the many pieces that few rows bring (a step bound by latency).  One or two pieces,
+  // which many rows bring, are taken one by one (G = 1, a kernel of its own): that step
+  // is bound by the memory rate, and the registers of a group would cost it waves (2,048
+  // rows of 896 with two pieces: 8.8 us one by one, 10.7 in pairs).
+  auto fetch = [&](int c, float* v) {       // the whole values of elements c .. c+W-1, written back if pieces came in
     if constexpr (VEC) {
       floatx4 t = *(const floatx4*)(src + c);
       for (int s0 = 0; s0 < splits; s0 += G) {
@@ -116,10 +116,6 @@ __global__ void rmsnorm_kernel(float* __restrict__ x, const void* __restrict__ w
       if (splits > 0) src[c] = t;
       v[0] = t;
     }
-  };
-  auto fetch = [&](int c, float* v) {       // the whole values of elements c .. c+W-1, written back if pieces came in
-    if (splits > 2) fetch_by(c, v, std::integral_constant<int, 4>{});
-    else fetch_by(c, v, std::integral_constant<int, 2>{});
   };
 #pragma unroll
   for (int j = 0; j < KEEP; ++j) {
@@ -169,9 +165,15 @@ extern "C" int llmlab_rmsnorm(float* x, const void* w, int w_dtype, float eps, v
   const bool vec = hidden % 4 == 0 && pend_stride % 4 == 0 &&
                    (((uintptr_t)x | (uintptr_t)pend | (uintptr_t)out) & 15) == 0;
   dim3 grid(n_out), block(hidden >= 8192 ? 512 : 256);
-#define LLMLAB_RMSNORM(T, VEC)                                                                      \
-  hipLaunchKernelGGL((rmsnorm_kernel<T, VEC>), grid, block, 0, stream, x, w, w_dtype == DT_BF16, eps, \
-                     (T*)out, rows, hidden, pend, splits, pend_stride)
+#define LLMLAB_RMSNORM(T, VEC)                                                                             \
+  do {                                                                                                     \
+    if (splits > 2)                                                                                        \
+      hipLaunchKernelGGL((rmsnorm_kernel<T, VEC, 4>), grid, block, 0, stream, x, w, w_dtype == DT_BF16, eps, \
+                         (T*)out, rows, hidden, pend, splits, pend_stride);                                \
+    else                                                                                                   \
+      hipLaunchKernelGGL((rmsnorm_kernel<T, VEC, 1>), grid, block, 0, stream, x, w, w_dtype == DT_BF16, eps, \
+                         (T*)out, rows, hidden, pend, splits, pend_stride);                                \
+  } while (0)
   if (out_dtype == DT_BF16) { if (vec) LLMLAB_RMSNORM(bf16_t, true); else LLMLAB_RMSNORM(bf16_t, false); }
   else                      { if (vec) LLMLAB_RMSNORM(float, true);  else LLMLAB_RMSNORM(float, false); }
 #undef LLMLAB_RMSNORM
