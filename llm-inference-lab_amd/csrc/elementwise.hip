@@ -164,7 +164,13 @@ extern "C" int llmlab_rmsnorm(float* x, const void* w, int w_dtype, float eps, v
   if (n_out == 0) return 0;
   const bool vec = hidden % 4 == 0 && pend_stride % 4 == 0 &&
                    (((uintptr_t)x | (uintptr_t)pend | (uintptr_t)out) & 15) == 0;
-  dim3 grid(n_out), block(hidden >= 8192 ? 512 : 256);
+  // few rows are bound by latency, not by the memory rate: then a row is spread over as
+  // many threads as it has groups of four numbers, so that every thread's loads (its
+  // numbers and the pieces owed to them) are one round
+  int threads = hidden >= 8192 ? 512 : 256;
+  if (n_out <= 128)
+    while (threads < 1024 && threads * 4 < hidden) threads *= 2;
+  dim3 grid(n_out), block(threads);
 #define LLMLAB_RMSNORM(T, VEC)                                                                             \
   do {                                                                                                     \
     if (splits > 2)                                                                                        \
