@@ -580,6 +580,21 @@ def test_attention_one_request_over_a_long_history(ops, emu, d, length, key):
     run_attention(ops, emu, torch.bfloat16, 4, 1, d, 64, None, [(length - 1, 1)], amplify=(0, key, 30.0))
 
 
+@pytest.mark.parametrize("splits", [1, 3, 16, 17, 50, 64, 65, 128])
+def test_attention_merge_of_any_number_of_splits(ops, emu, splits):
+    """The number of key splits is fixed from outside: one wave merges up to sixteen,
+    four waves more, a lane holds the weights of two; splits past the end of a short
+    history have no keys at all and must count for nothing."""
+    for d, length in ((64, 700), (128, 3000), (48, 90)):
+        lib = ops._attention_lib(d)
+        lib.llmlab_attention_force_splits(splits)
+        try:
+            run_attention(ops, emu, torch.bfloat16, 6, 2, d, 16, None, [(length - 1, 1), (40, 1), (length // 2, 2)],
+                          seed=96, amplify=(0, length // 3, 30.0))
+        finally:
+            lib.llmlab_attention_force_splits(0)
+
+
 @pytest.mark.parametrize("vocab", [1, 255, 256, 257, 4095, 4097, 151936])
 def test_argmax(ops, emu, vocab):
     """Vocabulary sizes and special rows of the reference's argmax tests
