@@ -4,7 +4,7 @@
 
 extern "C" const char* llmlab_last_error() { return g_llmlab_error; }
 
-extern "C" int llmlab_abi_version() { return 4; }
+extern "C" int llmlab_abi_version() { return 5; }
 
 // --------------------------------------------------------------- embedding
 // out[r, :] = float(table[ids[r], :]); an id outside [0, vocab) is clamped (the
@@ -283,6 +283,94 @@ extern "C" int llmlab_rope_kv_write(void* qkv, int dtype, int rows, int row_stri
                        nq, nkv, d, inv_freq, positions, row_req, table, table_stride, page_size,
                        (float*)kcache, (float*)vcache);
   LLMLAB_LAUNCH_CHECK("rope_kv_write");
+  return 0;
+}
+
+// The same from a q/k/v product that was left in pieces along its inner size
+// (float32 parts[s][row][ld], s < splits): one block per (row, head) sums the pieces in
+// their order, adds the bias, rotates q and k heads and writes q to q_out [rows, ldq] and
+// k and v into their cache pages (skipped without a cache).  One rounding, as in the
+// product kernels that have this epilogue.  For some rows of a large matrix: cut along
+// K the product spreads over the chip, which a head per block does not.
+__global__ __launch_bounds__(256) void qkv_from_pieces_kernel(
+    const float* __restrict__ parts, int splits, size_t part_stride, int ld, const void* __restrict__ bias,
+    int bias_bf16, int nq, int nkv, int d, const float* __restrict__ inv_freq,
+    const int* __restrict__ positions, const int* __restrict__ row_req, const int* __restrict__ table,
+    int table_stride, int page_size, bf16_t* __restrict__ kcache, bf16_t* __restrict__ vcache,
+    bf16_t* __restrict__ q_out, int ldq) {
+  const int r = blockIdx.x, head = blockIdx.y;
+  if (head >= nq && !kcache) return;
+  const int pos = positions[r];
+  size_t page = 0;
+  int off = 0;
+  if (head >= nq) {
+    page = (size_t)table[(size_t)row_req[r] * table_stride + pos / page_size];
+    off = pos % page_size;
+  }
+  const int half = d >> 1;
+  const float* src = parts + (size_t)r * ld + (size_t)head * d;
+  for (int i = threadIdx.x; i < half; i += blockDim.x) {
+    float lo = bias ? load_vec(bias, bias_bf16, head * d + i) : 0.f;
+    float hi = bias ? load_vec(bias, bias_bf16, head * d + i + half) : 0.f;
+    // four pieces at a time, loads unconditional (past the last piece: the last one again,
+    // not added), so that they travel together
+    for (int s0 = 0; s0 < splits; s0 += 4) {
+      float pl[4], ph[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float* ps = src + (size_t)min(s0 + j, splits - 1) * part_stride;
+        pl[j] = ps[i];
+        ph[j] = ps[i + half];
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        if (s0 + j < splits) {
+          lo += pl[j];
+          hi += ph[j];
+        }
+    }
+    if (inv_freq && head < nq + nkv) {
+      float sn, cs;
+      rope_sincos<bf16_t>((float)pos * inv_freq[i], &sn, &cs);
+      const float nlo = lo * cs - hi * sn, nhi = hi * cs + lo * sn;
+      lo = nlo;
+      hi = nhi;
+    }
+    if (head < nq) {
+      bf16_t* dst = q_out + (size_t)r * ldq + (size_t)head * d;
+      dst[i] = (bf16_t)lo;
+      dst[i + half] = (bf16_t)hi;
+    } else if (head < nq + nkv) {
+      bf16_t* kdst = kcache + (page * nkv + (head - nq)) * (size_t)page_size * d;
+      kdst[kcache_index(off, i, d)] = (bf16_t)lo;
+      kdst[kcache_index(off, i + half, d)] = (bf16_t)hi;
+    } else {
+      bf16_t* vdst = vcache + (page * nkv + (head - nq - nkv)) * (size_t)d * page_size;
+      vdst[vcache_index(off, i, d)] = (bf16_t)lo;
+      vdst[vcache_index(off, i + half, d)] = (bf16_t)hi;
+    }
+  }
+}
+
+extern "C" int llmlab_qkv_from_pieces(const float* parts, int splits, size_t part_stride, int ld,
+                                      const void* bias, int bias_dtype, int rows, int nq, int nkv, int d,
+                                      const float* inv_freq, const int* positions, const int* row_req,
+                                      const int* table, int table_stride, int page_size, void* kcache,
+                                      void* vcache, void* q_out, int ldq, hipStream_t stream) {
+  LLMLAB_REQUIRE(rows >= 0 && nq > 0 && nkv >= 0 && d > 0 && d % 2 == 0 && nq + 2 * nkv <= 65535,
+                 "qkv_from_pieces: bad sizes rows=%d nq=%d nkv=%d d=%d", rows, nq, nkv, d);
+  LLMLAB_REQUIRE(splits >= 1 && ld >= (nq + 2 * nkv) * d && part_stride >= (size_t)rows * ld && ldq >= nq * d,
+                 "qkv_from_pieces: %d pieces, row strides %d and %d", splits, ld, ldq);
+  LLMLAB_REQUIRE((kcache == nullptr) == (vcache == nullptr), "qkv_from_pieces: need both caches or none");
+  LLMLAB_REQUIRE(positions != nullptr && (kcache == nullptr || (table != nullptr && row_req != nullptr && page_size > 0)),
+                 "qkv_from_pieces: positions and, for a cache write, a block table are needed");
+  if (rows == 0) return 0;
+  const int half = d / 2;
+  dim3 grid(rows, nq + 2 * nkv), block(half >= 256 ? 256 : (half + 63) / 64 * 64);
+  hipLaunchKernelGGL(qkv_from_pieces_kernel, grid, block, 0, stream, parts, splits, part_stride, ld, bias,
+                     bias_dtype == DT_BF16, nq, nkv, d, inv_freq, positions, row_req, table, table_stride,
+                     page_size, (bf16_t*)kcache, (bf16_t*)vcache, (bf16_t*)q_out, ldq);
+  LLMLAB_LAUNCH_CHECK("qkv_from_pieces");
   return 0;
 }
 

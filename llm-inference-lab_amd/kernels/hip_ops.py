@@ -80,7 +80,7 @@ class HipOps:
             self.device = torch.device("cuda", torch.cuda.current_device())
         self._core = self._load(build.core_library())
         self._declare_core()
-        if self._core.llmlab_abi_version() != 4:
+        if self._core.llmlab_abi_version() != 5:
             raise RuntimeError("kernel library and Python bindings disagree on the interface")
         self._attn: Dict[int, ctypes.CDLL] = {}
         self._shared: Dict[int, tuple] = {}
@@ -126,6 +126,10 @@ class HipOps:
         c.llmlab_linear_tile.restype = _c_int
         c.llmlab_linear_partials.argtypes = [_c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_int, _c_int,
                                              _c_int, _c_int, _c_size, _c_int, _c_ptr]
+        c.llmlab_qkv_from_pieces.argtypes = [_c_ptr, _c_int, _c_size, _c_int, _c_ptr, _c_int, _c_int, _c_int,
+                                             _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int,
+                                             _c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr]
+        c.llmlab_qkv_from_pieces.restype = _c_int
         c.llmlab_linear_plan.argtypes = [_c_int, _c_int, _c_int, _c_int, _c_int, _c_int, _c_ptr]
         c.llmlab_linear_plan.restype = None
         c.llmlab_skinny_linear.argtypes = [
@@ -552,6 +556,7 @@ class HipOps:
                           nkv=num_kv_heads, d=head_dim), pending=pending)
 
     QKV_ROPE_MAX_ROWS = 64        # up to here the few-row kernel, beyond it the tiled one
+    QKV_PIECES_MIN_ROWS = 24      # from here to QKV_ROPE_MAX_ROWS a large matrix goes through pieces
 
     def can_fuse_qkv_rope(self, rows: int, dtype, head_dim: int, n: Optional[int] = None,
                           k: Optional[int] = None) -> bool:
@@ -577,6 +582,28 @@ class HipOps:
             raise ValueError(f"qkv_rope_cache: {rows} rows of {k}, heads of {head_dim} do not fit")
         self._qkv_checks("qkv_rope_cache", rows, w_qkv, b_qkv, num_heads, num_kv_heads, head_dim,
                          inv_freq, positions, row_req, block_table, page_size, k_cache, v_cache, q_out)
+        if self.QKV_PIECES_MIN_ROWS <= rows <= self.QKV_ROPE_MAX_ROWS and self.pieces_by_tiles(rows, n, k):
+            # some rows of a large matrix: a head per block leaves most of the chip idle, so
+            # the product is cut along K by the tiled kernel and a second kernel sums the
+            # pieces, rotates and writes the cache (64 rows of 7168 x 5120: 26 us against 52
+            # in one kernel, of 4608 x 3584: 19 against 24; the same at 24 rows, slower below)
+            pieces, tile = self._linear_plan(rows, n, k)
+            if self.force_tiled_pieces:
+                pieces = max(1, min(self.force_tiled_pieces, (k + 63) // 64, self.MAX_SPLITS))
+            if pieces > 1 and pieces * rows * n <= self.workspace.numel():
+                if b_qkv is not None:
+                    self._need(b_qkv, "bias")
+                parts = self.workspace[:pieces * rows * n].view(pieces, rows, n)
+                self._call(self._core.llmlab_linear_partials,
+                    self._ptr(h), self._ptr(w_qkv), self._ptr(parts), None, 0, rows, n, k, n, pieces,
+                    rows * n, tile, self._stream())
+                self._call(self._core.llmlab_qkv_from_pieces,
+                    self._ptr(parts), pieces, rows * n, n, self._ptr(b_qkv),
+                    _dt(b_qkv) if b_qkv is not None else 0, rows, num_heads, num_kv_heads, head_dim,
+                    self._ptr(inv_freq), self._ptr(positions), self._ptr(row_req), self._ptr(block_table),
+                    block_table.stride(0) if block_table is not None else 0, int(page_size),
+                    self._ptr(k_cache), self._ptr(v_cache), self._ptr(q_out), q_out.stride(0), self._stream())
+                return
         if rows <= self.QKV_ROPE_MAX_ROWS:
             self._skinny(h, False, None, None, 0.0, w_qkv, b_qkv, EPI_QKV, q_out, rows, n, k,
                          q_out.shape[1], n,

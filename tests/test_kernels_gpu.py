@@ -353,6 +353,22 @@ def test_qkv_rope_cache_of_normed_rows(ops, emu, nq, nkv, d, page, hidden, rows_
         ops._core.llmlab_gemm_force(0)
 
 
+@pytest.mark.parametrize("nq,nkv,d,page,hidden", [(4, 2, 16, 16, 64), (14, 2, 64, 64, 896), (6, 3, 48, 16, 72),
+                                                 (8, 8, 128, 64, 256), (2, 1, 256, 16, 64)])
+@pytest.mark.parametrize("rows_per", [[20, 1, 1, 3], [17, 30, 16], [5, 8, 11]])
+@pytest.mark.parametrize("pieces", [2, 5])
+def test_qkv_rope_cache_through_pieces(ops, emu, nq, nkv, d, page, hidden, rows_per, pieces):
+    """17 to 64 rows of a large matrix: the product is cut along its inner size and a second
+    kernel sums the pieces, adds the bias, rotates and writes the cache.  The small
+    matrices of the test take that way with the size limit taken away."""
+    ops.TILED_PIECES_BYTES, ops.force_tiled_pieces = 0, pieces
+    try:
+        assert ops.pieces_by_tiles(sum(rows_per), (nq + 2 * nkv) * d, hidden) and sum(rows_per) >= ops.QKV_PIECES_MIN_ROWS
+        check_qkv_rope_cache(ops, emu, nq, nkv, d, page, hidden, rows_per)
+    finally:
+        del ops.TILED_PIECES_BYTES, ops.force_tiled_pieces
+
+
 def check_qkv_rope_cache(ops, emu, nq, nkv, d, page, hidden, rows_per):
     bf = torch.bfloat16
     rows, reqs = sum(rows_per), len(rows_per)
