@@ -14,7 +14,8 @@
 //       large tile before).  Also measured and not adopted: 256x128 tiles with eight
 //       64x64 or four 128x64 wave tiles, K steps of 128, 128x256, 64x256, 128x64 and
 //       32x128 tiles with 1x4 waves (the second as good as 128x128, no better), eight
-//       waves 2x4 on 128x128 and 64x128, and 256x256 tiles with four 128x128 wave tiles (half the LDS traffic
+//       waves 2x4 on 128x128 and 64x128, a 64x256 tile with eight waves 1x8 for few rows of a wide
+//       matrix (as fast as 64x128, no faster), and 256x256 tiles with four 128x128 wave tiles (half the LDS traffic
 //       per product, one wave per SIMD: 833 against 793 TF/s on the largest product
 //       tried, slower on the rest).
 //     (products of few rows, as in decode steps, have kernels of their own in decode.hip)
