@@ -231,6 +231,31 @@ def test_decode_graph_replays_equal_eager(dtype):
     assert bad is None, f"first wrong logits at (request, position, error) = {bad}"
 
 
+@pytest.mark.parametrize("graph", [False, True])
+def test_many_decoding_requests_with_products_in_pieces(graph):
+    """26 requests decode together at layers of real size, with the size limit taken away so
+    that the rules for some rows of a large matrix hold: the down, the output and the
+    q/k/v product go through the tiled kernel in pieces, the norms fold the pieces (too
+    large for the fused kernels to read in every block), q/k/v is finished by the
+    kernel that sums, rotates and writes the cache.  Eager and from a replayed graph."""
+    cfg = H.config_of("R")
+    seqs = {f"r{i:02d}": H.random_ids(cfg, 19 + 12, 900 + i) for i in range(26)}
+    want = {rid: H.plain_logits("R", 1, ids) for rid, ids in seqs.items()}
+    engine = H.make_engine("R", 1, "bf16", page_size=64, num_pages=30, max_requests=32, max_batch_tokens=512,
+                           graph=graph)
+    ops = engine.ops
+    ops.TILED_PIECES_BYTES, ops.force_tiled_pieces, ops.PIECES_PER_BLOCK_BYTES = 0, 2, 1 << 16
+    assert ops.pieces_by_tiles(26, cfg.hidden_size, cfg.intermediate_size)
+    assert ops.split_count(26, torch.bfloat16, cfg.hidden_size, cfg.intermediate_size) == 2
+    steps = [([(rid, 19, True) for rid in seqs], [])]
+    steps += [([(rid, 1, True) for rid in seqs], []) for _ in range(12)]
+    got = H.run_trace(engine, seqs, steps)
+    if graph:
+        assert engine.step_fn.graph_replays >= 8
+    bad = H.first_wrong(got, want, TOL_REAL["bf16"][0])
+    assert bad is None, f"first wrong logits at (request, position, error) = {bad}"
+
+
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
 def test_temperature_sampling_on_the_gpu(dtype):
     cfg = H.config_of("B")
