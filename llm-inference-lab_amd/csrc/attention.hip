@@ -638,7 +638,9 @@ __global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void attention_bf16_paired_ke
 // splits cost one trip to memory), and the quarters meet in LDS in their order.  Up to
 // sixteen splits are one wave's work, and the block is launched with one.
 // A kernel of its own: within one kernel, results of blocks on other dies would
-// need device-wide fences, which cost far more than a launch.
+// need device-wide fences, which cost far more than a launch (measured: the last
+// block to arrive, found by an atomic counter behind a fence, merging in place of this
+// kernel made the decode step of 24 layers 1.88 ms instead of 0.97).
 constexpr int MERGE_WAVES = 4;
 __global__ __launch_bounds__(64 * MERGE_WAVES) void attention_merge_kernel(
     const float* __restrict__ o_part, const float* __restrict__ ml_part, bf16_t* __restrict__ out,
