@@ -47,7 +47,7 @@ class CapacityExhausted(RuntimeError):
     """The cache cannot hold the request even with nothing else running."""
 
 
-@dataclasses.dataclass
+@dataclasses.dataclass(eq=False)      # a request is itself, not its fields: compared and hashed by identity
 class Request:
     request_id: int
     prompt: List[int]
@@ -229,11 +229,13 @@ class Scheduler:
         started = None
         if plan:
             entries = []
+            # where the token of a request in flight lies among those chosen in the step before
+            place = {id(r): i for i, r in enumerate(self._pending[0])} if self._pending is not None else {}
             for p in plan:
                 r = p.request
                 start = r.computed
                 if r.in_flight:       # its input token is still on the GPU
-                    source = (self._pending[1].device_tokens, self._pending[0].index(r))
+                    source = (self._pending[1].device_tokens, place[id(r)])
                     entries.append(StepEntry(r.cache, [0], [0] if p.yields_token else [], source))
                 else:
                     entries.append(StepEntry(r.cache, r.tokens[start:start + p.count],

@@ -194,6 +194,25 @@ def test_overlap_gives_the_same_tokens_and_steps():
     assert results[False][1] == results[True][1]
 
 
+def test_equal_requests_are_told_apart():
+    """Two requests with the same prompt, sampling and progress are two requests: each finds
+    its own token in flight (requests compare by identity, and a step looks them up in
+    time that does not grow with the square of their number)."""
+    a = Request(0, [1, 2, 3], SamplingConfig(max_new_tokens=4, eos_token_id=[]))
+    b = Request(0, [1, 2, 3], SamplingConfig(max_new_tokens=4, eos_token_id=[]))
+    assert a != b and a == a and [a, b].index(b) == 1 and len({a, b}) == 2
+    cfg = H.config_of("A")
+    prompt = H.random_ids(cfg, 9, 5)
+    engine = engine_of("A", num_pages=24, max_requests=4)
+    sched = engine.scheduler(max_batch_tokens=64, overlap=True)
+    for _ in range(4):
+        sched.add_request(list(prompt), SamplingConfig(max_new_tokens=7, temperature=0.9, seed=11, eos_token_id=[]))
+    done = sched.run()
+    assert len({tuple(r.generated) for r in done.values()}) == 1 and len(done) == 4
+    assert all(len(r.generated) == 7 for r in done.values())
+    engine.cache.check()
+
+
 def test_overlap_drops_the_token_after_an_end_of_sequence():
     cfg = H.config_of("A")
     engine = engine_of(num_pages=16)
