@@ -163,9 +163,14 @@ class StepContext:
         for b, e in enumerate(entries):
             n = len(e.tokens)
             start = e.request.computed_len
-            h[o["token_ids"] + row:o["token_ids"] + row + n] = np.asarray(e.tokens, dtype=np.int32)
-            h[o["positions"] + row:o["positions"] + row + n] = np.arange(start, start + n, dtype=np.int32)
-            h[o["row_req"] + row:o["row_req"] + row + n] = b
+            if n == 1:          # (a decoding request: no arrays for one number)
+                h[o["token_ids"] + row] = e.tokens[0]
+                h[o["positions"] + row] = start
+                h[o["row_req"] + row] = b
+            else:
+                h[o["token_ids"] + row:o["token_ids"] + row + n] = np.asarray(e.tokens, dtype=np.int32)
+                h[o["positions"] + row:o["positions"] + row + n] = np.arange(start, start + n, dtype=np.int32)
+                h[o["row_req"] + row:o["row_req"] + row + n] = b
             h[o["q_start"] + b] = row
             h[o["start_pos"] + b] = start
             h[o["req_rows"] + b] = e.request.row
@@ -194,10 +199,10 @@ class StepContext:
         self.n_rows, self.n_reqs, self.n_want = n_rows, n_reqs, len(want)
         self.max_q_len, self.max_ctx_len = max_q, max_ctx
         used_pages = (max_ctx + cache.page_size - 1) // cache.page_size
+        cache_rows = self.host_req_rows
         for gi, at in enumerate(self._table_at):
             table = h[at:at + self.max_reqs * self.max_pages].reshape(self.max_reqs, self.max_pages)
-            for b, e in enumerate(entries):
-                table[b, :used_pages] = cache.tables[gi][e.request.row, :used_pages]
+            table[:n_reqs, :used_pages] = cache.tables[gi][cache_rows, :used_pages]
         for i, (dst, src) in enumerate(feeds):
             h[o["feed_dst"] + i] = dst
             h[o["feed_src"] + i] = src
@@ -301,7 +306,7 @@ class StepFunction:
             for r in reserved:
                 self.cache.cancel_reservation(r)
             raise
-        if self.use_graph and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries):
+        if self.use_graph and all(len(e.tokens) == 1 and len(e.want) == 1 and e.want[0] == 0 for e in entries):
             logits = self._decode_with_graph()
         else:
             logits = self.model.forward(self.ctx)
