@@ -10,6 +10,9 @@
 // a request's choices do not depend on the batch it ran in.  Each thread owns one
 // contiguous stretch of the row, so the cumulative sum has one fixed order.
 #include "common.h"
+#include "no_alloc.h"
+
+#include <mutex>
 
 constexpr int SAMPLE_THREADS = 1024;
 
@@ -184,6 +187,56 @@ extern "C" int llmlab_argmax(const float* logits, long row_stride, int rows, int
   LLMLAB_LAUNCH_CHECK("argmax (partial)");
   hipLaunchKernelGGL(argmax_final_kernel, dim3(rows), dim3(64), 0, stream, pvals, pidx, chunks, out);
   LLMLAB_LAUNCH_CHECK("argmax (final)");
+  return 0;
+}
+
+// The same selection for callers that cannot allocate: the partial maxima go to a
+// device array of this file.  The array's name is only a handle in host code; the
+// address on each GPU comes from hipGetSymbolAddress, asked for once per device with
+// that device current, and the kernels take that address as an argument.
+constexpr int STATIC_MAX_DEVICES = 64;
+static __device__ __align__(256) float scratch[2 * LLMLAB_ARGMAX_STATIC_PAIRS];
+static float* g_scratch_ptr[STATIC_MAX_DEVICES] = {};
+static std::mutex g_scratch_mutex;
+
+static int static_scratch(float** ptr) {
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  LLMLAB_REQUIRE(e == hipSuccess, "argmax_static: hipGetDevice failed: %s", hipGetErrorString(e));
+  LLMLAB_REQUIRE(device >= 0 && device < STATIC_MAX_DEVICES, "argmax_static: device %d is beyond %d",
+                 device, STATIC_MAX_DEVICES);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[device] == nullptr) {
+    float* p = nullptr;
+    e = hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch));
+    LLMLAB_REQUIRE(e == hipSuccess && p != nullptr, "argmax_static: hipGetSymbolAddress failed: %s",
+                   hipGetErrorString(e));
+    g_scratch_ptr[device] = p;
+  }
+  *ptr = g_scratch_ptr[device];
+  return 0;
+}
+
+extern "C" int llmlab_argmax_static(const float* logits, long row_stride, int rows, int vocab, int* out,
+                                    hipStream_t stream) {
+  LLMLAB_REQUIRE(rows >= 0 && vocab > 0 && row_stride >= vocab,
+                 "argmax_static: bad sizes rows=%d vocab=%d", rows, vocab);
+  if (rows == 0) return 0;
+  LLMLAB_REQUIRE(logits != nullptr && out != nullptr, "argmax_static: null logits or output");
+  const int chunks = (vocab + ARGMAX_CHUNK - 1) / ARGMAX_CHUNK;
+  LLMLAB_REQUIRE(rows <= 65535, "argmax_static: too many rows");
+  LLMLAB_REQUIRE((size_t)rows * chunks <= (size_t)LLMLAB_ARGMAX_STATIC_PAIRS,
+                 "argmax_static: %d rows of %d logits need %zu partial results, the static array "
+                 "holds %d", rows, vocab, (size_t)rows * chunks, LLMLAB_ARGMAX_STATIC_PAIRS);
+  float* base = nullptr;
+  if (static_scratch(&base) != 0) return 1;
+  float* pvals = base;
+  int* pidx = (int*)(base + (size_t)rows * chunks);
+  hipLaunchKernelGGL(argmax_partial_kernel, dim3(chunks, rows), dim3(256), 0, stream, logits, row_stride,
+                     vocab, pvals, pidx, chunks);
+  LLMLAB_LAUNCH_CHECK("argmax_static (partial)");
+  hipLaunchKernelGGL(argmax_final_kernel, dim3(rows), dim3(64), 0, stream, pvals, pidx, chunks, out);
+  LLMLAB_LAUNCH_CHECK("argmax_static (final)");
   return 0;
 }
 

@@ -27,6 +27,7 @@ LIB_DIR = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib")
 CORE_SOURCES = ("elementwise.hip", "gemm.hip", "decode.hip", "sampling.hip")
 ATTENTION_SOURCE = "attention.hip"
 HEADERS = ("common.h",)
+CORE_HEADERS = ("no_alloc.h",)      # included by the core sources only
 FLAGS = ("-O3", "-std=c++17", "-fPIC", "-shared", f"--offload-arch={ARCH}",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops")
 DEFAULT_HEAD_DIMS = (16, 32, 64, 128)
@@ -38,7 +39,8 @@ def _say(msg: str) -> None:
 
 def _hash(sources: Sequence[str], defines: Sequence[str]) -> str:
     h = hashlib.sha256()
-    for name in list(sources) + list(HEADERS):
+    extra = CORE_HEADERS if tuple(sources) == CORE_SOURCES else ()
+    for name in list(sources) + list(HEADERS) + list(extra):
         with open(os.path.join(CSRC, name), "rb") as f:
             h.update(name.encode() + b"\0" + f.read())
     h.update(" ".join(FLAGS).encode())
