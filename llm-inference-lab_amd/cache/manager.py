@@ -3,13 +3,14 @@ request, one page pool per group of layers with the same need, and slots for
 per-request state of fixed size.
 
 Storage of one group (``S`` cache-owning runs of layers, ``N`` pages of ``P``
-tokens, ``G`` kv heads of width ``d``), in the compute dtype::
+tokens): one tensor ``[S, N, *page_shape]`` for every named tensor of the group's
+``CacheSpec``.  For attention (``G`` kv heads of width ``d``), in the compute dtype::
 
-    keys    [S, N, G, P, d]     a page holds, per kv head, P keys of d numbers
-    values  [S, N, G, d, P]     and as many values
+    k   [S, N, G, P, d]     a page holds, per kv head, P keys of d numbers
+    v   [S, N, G, d, P]     and as many values
 
-A page number addresses the same page in every run of the group, so the group
-needs one block table.  Position ``p`` of a request lives in page
+A page number addresses the same page in every run of the group and in every one
+of its tensors, so the group needs one block table.  Position ``p`` of a request lives in page
 ``table[p // P]`` at offset ``p % P``.  Inside a (page, kv head) pair the
 ``P * d`` numbers lie in the order of the attention kernels' matrix-core
 fragments, not row by row (``cache/layout.py`` has the index maps); the manager
@@ -29,7 +30,7 @@ from typing import Dict, List, Optional, Sequence, Tuple
 import numpy as np
 import torch
 
-from ..parts.base import KVCacheSpec
+from ..parts.base import CacheSpec
 from .pages import OutOfPages, PagePool
 
 NO_PAGE = -1
@@ -39,7 +40,7 @@ NO_PAGE = -1
 class GroupLayout:
     """Layers (schedule entries) with one cache need."""
 
-    spec: KVCacheSpec
+    spec: CacheSpec
     entries: List[int]                     # schedule entries that own a cache in this group
     num_pages: int = 0
 
@@ -77,6 +78,7 @@ class RequestCache:
         self.pages: List[List[int]] = [[] for _ in range(num_groups)]   # logical page -> page or NO_PAGE
         self.first_live: List[int] = [0] * num_groups                   # first logical page still held
         self.released = False
+        self.invalid = False           # a step that wrote to it failed: it can only be released
 
 
 class CacheManager:
@@ -98,13 +100,16 @@ class CacheManager:
         # host mirror of the block tables; rows of dead requests are NO_PAGE
         self.tables = [np.full((self.max_requests, self.max_pages_per_request), NO_PAGE, dtype=np.int32)
                        for _ in self.groups]
-        self.keys: List[torch.Tensor] = []
-        self.values: List[torch.Tensor] = []
+        # per group: name -> [runs, pages, *page_shape].  Zeroed once: a masked position
+        # must never meet a NaN bit pattern.
+        self.storage: List[Dict[str, torch.Tensor]] = []
         for g in self.groups:
-            s, n, h, d = len(g.entries), g.num_pages, g.spec.num_kv_heads, g.spec.head_dim
-            # Zeroed once: a masked position must never meet a NaN bit pattern.
-            self.keys.append(torch.zeros((s, n, h, self.page_size, d), dtype=dtype, device=device))
-            self.values.append(torch.zeros((s, n, h, d, self.page_size), dtype=dtype, device=device))
+            if not isinstance(g.spec, CacheSpec):
+                raise TypeError(f"a cache group is described by a CacheSpec, got {type(g.spec).__name__}")
+            self.storage.append({
+                name: torch.zeros((len(g.entries), g.num_pages) + t.page_shape(self.page_size),
+                                  dtype=t.dtype or dtype, device=device)
+                for name, t in g.spec.tensors})
         self.entry_group: Dict[int, Tuple[int, int]] = {}
         for gi, g in enumerate(self.groups):
             for si, e in enumerate(g.entries):
@@ -139,10 +144,18 @@ class CacheManager:
         }
 
     def bytes_per_token(self) -> int:
-        """Cache bytes one token takes in the groups without a window."""
-        width = torch.empty((), dtype=self.dtype).element_size()
-        return sum(2 * len(g.entries) * g.spec.num_kv_heads * g.spec.head_dim * width
-                   for g in self.groups)
+        """Cache bytes one token takes in all groups (a windowed group holds them for the
+        latest ``window`` tokens only)."""
+        return sum(len(g.entries) * g.spec.bytes_per_token(self.dtype) for g in self.groups)
+
+    @property
+    def keys(self) -> List[torch.Tensor]:
+        """Per group the tensor named ``k`` (attention's keys; None for a group without)."""
+        return [st.get("k") for st in self.storage]
+
+    @property
+    def values(self) -> List[torch.Tensor]:
+        return [st.get("v") for st in self.storage]
 
     def page_need(self, total_tokens: int, max_step_tokens: int) -> List[int]:
         return [group_page_need(g.window, self.page_size, total_tokens, max_step_tokens)
@@ -173,6 +186,8 @@ class CacheManager:
         it had."""
         if req.released:
             raise ValueError(f"request {req.request_id!r} was released")
+        if req.invalid:
+            raise ValueError(f"request {req.request_id!r} was in a step that failed; release it")
         if new_tokens <= 0:
             raise ValueError("a step brings at least one token for each request in it")
         if req.reserved_len != req.computed_len:

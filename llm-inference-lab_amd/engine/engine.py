@@ -56,7 +56,7 @@ class Engine:
                  max_cache_tokens: Optional[int] = None, num_pages: Optional[int] = None,
                  max_requests: int = 64, max_batch_tokens: int = 512,
                  max_seq_len: Optional[int] = None, tensors=None, graph=False,
-                 progress: Optional[Callable[[str], None]] = None):
+                 progress: Optional[Callable[[str], None]] = None, strict_weights: bool = False):
         self.dtype = parse_dtype(dtype)
         if model_dir is not None:
             self.architecture, self.config = read_config(model_dir)
@@ -66,21 +66,30 @@ class Engine:
         else:
             raise ValueError("give a model_dir or a config")
         self.spec = self.architecture.build_spec(self.config)
+        # The model's end-of-sequence ids: those of generation_config.json if the folder
+        # has one that names any, else config.json's (engine.rs:403-407).  A request's own
+        # ids go before both.  The file's other fields are kept in ``generation_config``
+        # for callers that want them as defaults; requests carry their own options, as in
+        # the reference (model_runner.rs:612-614).
+        from ..sampling.params import read_generation_config
+        self.generation_config = read_generation_config(model_dir) if model_dir is not None else None
+        self.eos_token_ids = tuple(self.spec.eos_token_ids)
+        if self.generation_config is not None and self.generation_config.eos_token_id is not None:
+            self.eos_token_ids = self.generation_config.eos_ids()
+        self.model = CausalLM(self.spec)
         if ops is None:
-            # compile what this model needs before the GPU is first touched
+            # compile what this model's parts ask for before the GPU is first touched
             from ..kernels import build
             build.core_library()
-            for dim in sorted({b.mixer.params["head_dim"] for b in self.spec.blocks
-                               if "head_dim" in b.mixer.params}):
-                build.attention_library(int(dim))
+            for kind, parameter in self.model.kernel_libraries():
+                build.library(kind, parameter)
         self.ops = ops if ops is not None else default_ops(device)
         self.device = self.ops.device
-        self.model = CausalLM(self.spec)
         expected = self.model.tensor_specs()
         if model_dir is not None:
-            loaded = load_tensors(model_dir, expected, self.dtype, self.device, progress)
+            loaded = load_tensors(model_dir, expected, self.dtype, self.device, progress, strict_weights)
         elif tensors is not None:
-            loaded = place_tensors(tensors, expected, self.dtype, self.device)
+            loaded = place_tensors(tensors, expected, self.dtype, self.device, strict=strict_weights)
         else:
             loaded = place_tensors(random_tensors(expected, seed, torch.bfloat16), expected,
                                    self.dtype, self.device, "random weights")
@@ -107,9 +116,13 @@ class Engine:
                                   state_specs, self.dtype, self.device)
         self.model.attach_cache(self.cache)
         self.step_fn = StepFunction(self.model, self.cache, self.ops, self.max_batch_tokens,
-                                    graph=self._graph_choice(graph))
+                                    graph=graph)
         self._sampler = None
         self.last_scheduler = None
+        from .instruments import RequestInstruments
+        from .profiling import ranges_from_environment
+        self.request_instruments = RequestInstruments()
+        self.model.ranges = ranges_from_environment()
 
     CACHE_SHARE_OF_FREE_MEMORY = 0.9
 
@@ -118,29 +131,10 @@ class Engine:
         it for scratch buffers; at least one request of full length."""
         if self.device.type != "cuda":
             return 1 << 40
-        width = torch.empty((), dtype=self.dtype).element_size()
-        page_bytes = sum(2 * len(g.entries) * g.spec.num_kv_heads * g.spec.head_dim * width
-                         for g in groups) * self.page_size
+        page_bytes = sum(len(g.entries) * g.spec.bytes_per_token(self.dtype) for g in groups) * self.page_size
         free, _ = torch.cuda.mem_get_info(self.device)
         fit = int(free * self.CACHE_SHARE_OF_FREE_MEMORY) // max(page_bytes, 1)
         return max(fit, pages_for_tokens(self.max_seq_len, self.page_size))
-
-    # A decode step replayed from a HIP graph costs the host nothing, but the GPU about a
-    # microsecond more at every kernel boundary than kernels launched one by one by a host
-    # that runs ahead (measured: 4.05 against 3.90 ms a step at the 7B shape, 17.3 against
-    # 16.9 at the 32B shape; 0.97 against 1.7 at the 0.5B shape, where the host cannot keep
-    # up).  ``graph="auto"`` takes the graph unless the step's reading of the weights
-    # clearly outlasts the host's launching of its kernels.
-    HOST_SECONDS_PER_KERNEL = 12e-6
-    STREAMED_BYTES_PER_SECOND = 4.2e12
-
-    def _graph_choice(self, graph) -> bool:
-        if graph != "auto":
-            return bool(graph)
-        kernels = 6 * len(self.spec.schedule) + 6
-        host = kernels * self.HOST_SECONDS_PER_KERNEL
-        gpu = self.model.weight_bytes_per_step() / self.STREAMED_BYTES_PER_SECOND
-        return gpu < 1.25 * host
 
     # ------------------------------------------------------------- requests
     def open(self, request_id) -> RequestCache:
@@ -152,7 +146,17 @@ class Engine:
         self.cache.release(request)
 
     def step(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
+        """One step; an entry that cannot run raises before anything has run."""
         return self.step_fn(entries)
+
+    def run_step(self, entries: Sequence[StepEntry]):
+        """One step with a result for every entry (``StepResult``): entries that cannot run
+        carry their error, the others run as one batch."""
+        return self.step_fn.run(entries)
+
+    @property
+    def step_instruments(self):
+        return self.step_fn.instruments
 
     # ------------------------------------------------------------ generation
     def scheduler(self, max_batch_tokens: Optional[int] = None, on_token=None, trace=None,
@@ -196,8 +200,21 @@ class Engine:
         return self.model.weight_bytes_per_step()
 
     def metrics(self) -> Dict[str, object]:
-        return {"steps": self.step_fn.steps, "rows": self.step_fn.rows_total,
-                "cache": self.cache.metrics()}
+        """Counters and histograms as one dictionary of numbers: the step function's (steps
+        and input tokens by phase, host submit and step wall times, batch sizes, failed
+        steps, token readback), the decode graphs', the scratch buffers', the cache's, and
+        the requests' over every scheduler this engine has made."""
+        fn = self.step_fn
+        out = {"steps": fn.steps, "rows": fn.rows_total, "step": fn.instruments.snapshot(),
+               "graphs": {"enabled": fn.use_graph, "captures": fn.graph_captures,
+                          "replays": fn.graph_replays, "evictions": fn.graph_evictions,
+                          "kept": len(fn._graphs), "decode_calls": fn.decode_calls},
+               "scratch": {"bytes": fn.ctx.scratch_bytes, "allocations": fn.ctx.scratch_allocations},
+               "kernel_calls": getattr(self.ops, "calls_made", None),
+               "requests": self.request_instruments.snapshot(),
+               "cache": self.cache.metrics()}
+        out["step"]["failed_steps"] = fn.failed_steps
+        return out
 
 
 def write_random_model(model_dir: str, config, seed: int, dtype=torch.bfloat16) -> str:

@@ -30,9 +30,18 @@ class EntryView:
     group: Optional[int] = None     # cache group, None if the mixer keeps no cache
     slot: Optional[int] = None      # which of the group's layers
     writes_cache: bool = False
-    k_cache: Optional[torch.Tensor] = None     # [pages, kv_heads, page_size, head_dim]
-    v_cache: Optional[torch.Tensor] = None     # [pages, kv_heads, head_dim, page_size]
+    cache: Dict[str, torch.Tensor] = dataclasses.field(default_factory=dict)   # name -> [pages, *page_shape]
     state: Dict[str, torch.Tensor] = dataclasses.field(default_factory=dict)
+
+    @property
+    def k_cache(self) -> Optional[torch.Tensor]:
+        """Attention's keys, ``[pages, kv_heads, page_size, head_dim]``."""
+        return self.cache.get("k")
+
+    @property
+    def v_cache(self) -> Optional[torch.Tensor]:
+        """Attention's values, ``[pages, kv_heads, head_dim, page_size]``."""
+        return self.cache.get("v")
 
 
 class CausalLM:
@@ -49,6 +58,24 @@ class CausalLM:
         self.entries: List[EntryView] = [EntryView(i, e.block) for i, e in enumerate(spec.schedule)]
         self.ops = None
         self.dtype = None
+        self.ranges = None         # profiler ranges (engine/profiling.py), off by default
+
+    def parts(self):
+        return [self.embedding, *self.blocks, self.final_norm, self.head]
+
+    @property
+    def graph_safe(self) -> bool:
+        """Whether a decode step of this model may be replayed from a captured graph."""
+        return all(p.graph_safe for p in self.parts())
+
+    def kernel_libraries(self):
+        """What the parts want compiled before they are bound, each once."""
+        seen = []
+        for p in self.parts():
+            for lib in p.kernel_libraries():
+                if lib not in seen:
+                    seen.append(lib)
+        return seen
 
     # ---------------------------------------------------------------- weights
     def tensor_specs(self) -> Dict[str, TensorSpec]:
@@ -118,8 +145,7 @@ class CausalLM:
     def attach_cache(self, cache: CacheManager) -> None:
         for view in self.entries:
             if view.group is not None:
-                view.k_cache = cache.keys[view.group][view.slot]
-                view.v_cache = cache.values[view.group][view.slot]
+                view.cache = {name: t[view.slot] for name, t in cache.storage[view.group].items()}
             view.state = cache.state.get(view.index, {})
 
     # ---------------------------------------------------------------- forward
@@ -129,9 +155,14 @@ class CausalLM:
         rows, hidden = ctx.n_rows, self.spec.hidden_size
         x = ctx.scratch("model.residual", (rows, hidden), torch.float32)
         ctx.pending = None         # sums a product leaves in pieces for the next reader of x
-        self.embedding.forward(ctx.token_ids, x)
+        if self.ranges is not None:
+            return self._forward_with_ranges(x, ctx)
+        self.embedding.forward(ctx.token_ids, x, ctx)
         for view in self.entries:
             self.blocks[view.block].forward(x, ctx, view)
+        return self._head(x, ctx)
+
+    def _head(self, x, ctx) -> Optional[torch.Tensor]:
         if ctx.n_want == 0:
             ctx.pending = None
             return None
@@ -140,3 +171,14 @@ class CausalLM:
         logits = ctx.scratch("model.logits", (ctx.n_want, self.spec.vocab_size), torch.float32)
         self.head.forward(h if getattr(self.head, "takes_normed_input", False) else h.tensor(), logits)
         return logits
+
+    def _forward_with_ranges(self, x, ctx) -> Optional[torch.Tensor]:
+        """The same forward with a named range around every part's launches."""
+        r = self.ranges
+        with r.range("embedding"):
+            self.embedding.forward(ctx.token_ids, x, ctx)
+        for view in self.entries:
+            with r.range(f"block {view.index}"):
+                self.blocks[view.block].forward(x, ctx, view)
+        with r.range("final norm + head"):
+            return self._head(x, ctx)

@@ -40,7 +40,8 @@ import time
 from typing import Callable, Deque, Dict, List, Optional, Sequence, Tuple
 
 from ..sampling.params import SamplingConfig
-from .step import StepEntry
+from .instruments import RequestInstruments
+from .step import StepEntry, StepResult
 
 
 class CapacityExhausted(RuntimeError):
@@ -61,6 +62,7 @@ class Request:
     finish_reason: Optional[str] = None        # "eos", "length", "error"
     in_flight: bool = False                    # a token of this request is chosen but not read yet
     arrival: float = 0.0
+    admit_time: Optional[float] = None
     first_token_time: Optional[float] = None
     finish_time: Optional[float] = None
 
@@ -121,7 +123,7 @@ class Scheduler:
 
     ``engine`` needs: ``step(entries) -> logits``, ``cache`` (a ``CacheManager``),
     ``open(id)``, ``close(request_cache)``, ``spec`` (vocab_size, eos_token_ids),
-    ``max_seq_len``.  ``sampler.sample(logits, temperatures, seeds, counters)``
+    ``max_seq_len``, and optionally ``eos_token_ids`` (goes before the spec's).  ``sampler.sample(logits, temperatures, seeds, counters)``
     picks the tokens."""
 
     def __init__(self, engine, sampler, max_batch_tokens: Optional[int] = None,
@@ -139,8 +141,11 @@ class Scheduler:
         self.on_token = on_token
         self.trace = trace
         self.overlap = bool(overlap)
+        model_eos = getattr(engine, "eos_token_ids", None)
+        self._model_eos = tuple(model_eos if model_eos is not None else engine.spec.eos_token_ids)
         self._pending = None            # (requests, PendingTokens) of the step whose tokens are unread
         self.steps = 0
+        self.instruments = getattr(engine, "request_instruments", None) or RequestInstruments()
         self.step_log: List[List[Tuple[int, int]]] = []     # per step: (request id, tokens)
         self.keep_step_log = False
 
@@ -152,6 +157,7 @@ class Scheduler:
         request.tokens = list(request.prompt)
         request.remaining = request.sampling.new_tokens
         self.waiting.append(request)
+        self.instruments.received()
         return request.request_id
 
     # -------------------------------------------------------------- admission
@@ -209,6 +215,8 @@ class Scheduler:
             if fits:
                 r.cache = self.engine.open(("request", r.request_id))
                 r.promised_pages = need
+                r.admit_time = time.perf_counter()
+                self.instruments.admitted(r.admit_time - r.arrival)
                 self.active.append(r)
             elif self.active:
                 still_waiting.append(r)
@@ -219,10 +227,31 @@ class Scheduler:
         self.waiting = still_waiting
 
     # ------------------------------------------------------------------- step
+    def _run(self, entries: List[StepEntry]) -> StepResult:
+        """One step of the engine with a result for every entry.  Whatever the engine
+        raises for the step as a whole becomes every entry's error."""
+        run = getattr(self.engine, "run_step", None)
+        try:
+            if run is not None:
+                return run(entries)
+            logits = self.engine.step(entries)
+        except Exception as err:            # the batch failed as one (engine.rs:2041-2045)
+            return StepResult(None, [err] * len(entries), [None] * len(entries), shared_failure=err)
+        rows, at = [], 0
+        for e in entries:
+            rows.append(range(at, at + len(e.want)))
+            at += len(e.want)
+        return StepResult(logits, [None] * len(entries), rows)
+
     def step(self) -> List[Request]:
         """Admit, plan, run one step, choose tokens, finish.  Returns the requests that
         finished in this call.  With overlap the tokens read in this call are those of
-        the step before the one it starts."""
+        the step before the one it starts.
+
+        A request whose entry the engine refuses ends with that error and its peers run
+        on; if the step fails as a whole every request in it ends with the error; a
+        request whose logits row held no finite value ends alone (engine.rs:844-851).
+        Each gives its pages and its row back like any finished request."""
         before = set(self.finished)
         self._admit()
         plan = plan_step(self.active, self.max_batch_tokens)
@@ -241,21 +270,32 @@ class Scheduler:
                     entries.append(StepEntry(r.cache, r.tokens[start:start + p.count],
                                              [p.count - 1] if p.yields_token else []))
             t0 = time.perf_counter()
-            logits = self.engine.step(entries)
-            yielding = [p.request for p in plan if p.yields_token]
+            result = self._run(entries)
+            ran = []
+            for p, err in zip(plan, result.errors):
+                if err is None:
+                    ran.append(p)
+                else:
+                    self._fail(p.request, err)
+            yielding = [p.request for p in ran if p.yields_token]
+            phase = "decode" if all(p.request.decoding and p.count == 1 for p in plan) else "prefill"
             if yielding:
                 counters = [len(r.generated) + (1 if r.in_flight else 0) for r in yielding]
-                started = (yielding, self.sampler.sample_async(
-                    logits, [r.sampling.effective_temperature for r in yielding],
-                    [r.sampling.seed for r in yielding], counters))
+                try:
+                    handle = self.sampler.sample_async(
+                        result.logits, [r.sampling.effective_temperature for r in yielding],
+                        [r.sampling.seed for r in yielding], counters)
+                    started = (yielding, handle, t0, phase)
+                except Exception as err:
+                    for r in yielding:
+                        self._fail(r, err)
             self.steps += 1
             if self.keep_step_log:
                 self.step_log.append([(p.request.request_id, p.count) for p in plan])
             if self.trace is not None:
-                self.trace({"event": "step_submitted", "step": self.steps,
-                            "phase": "decode" if all(p.request.decoding and p.count == 1 for p in plan)
-                            else "prefill",
+                self.trace({"event": "step_submitted", "step": self.steps, "phase": phase,
                             "requests": len(plan), "tokens": sum(p.count for p in plan),
+                            "failed": len(plan) - len(ran),
                             "submit_seconds": time.perf_counter() - t0})
         # the tokens of the step before (with overlap), or of this one
         self._collect()
@@ -273,15 +313,36 @@ class Scheduler:
         """Read the tokens of the pending step and give them to their requests."""
         if self._pending is None:
             return
-        requests, handle = self._pending
+        requests, handle, submitted, phase = self._pending
         self._pending = None
-        tokens = handle.result()
+        wait_from = time.perf_counter()
+        try:
+            tokens = handle.tokens() if hasattr(handle, "tokens") else handle.result()
+        except Exception as err:
+            for r in requests:
+                r.in_flight = False
+                if not r.finished:
+                    self._fail(r, err)
+            return
         now = time.perf_counter()
+        step_metrics = getattr(self.engine, "step_instruments", None)
+        if step_metrics is not None:
+            step_metrics.readback_seconds.record(now - wait_from)
+            step_metrics.wall(phase, now - submitted)
         for r, token in zip(requests, tokens):
             r.in_flight = False
             if r.finished:
                 continue            # it ended a step earlier; this token was one too many
+            if token < 0:
+                self._fail(r, FloatingPointError(
+                    f"request {r.request_id}: non-finite logits, no token can be chosen"))
+                continue
             self._accept(r, token, now)
+
+    def _fail(self, r: Request, error: Exception) -> None:
+        """The request ends here with an error; ``step`` releases what it holds."""
+        if not r.finished:
+            r.finish_reason, r.error, r.remaining = "error", error, 0
 
     def _accept(self, r: Request, token: int, now: float) -> None:
         r.generated.append(token)
@@ -289,9 +350,10 @@ class Scheduler:
         r.remaining -= 1
         if r.first_token_time is None:
             r.first_token_time = now
+            self.instruments.first_token(now - r.arrival)
         if self.on_token is not None:
             self.on_token(r, token)
-        eos = r.sampling.eos_ids(self.engine.spec.eos_token_ids)
+        eos = r.sampling.eos_ids(self._model_eos)
         if token in eos:
             r.remaining = 0
             r.finish_reason = "eos"
@@ -305,11 +367,13 @@ class Scheduler:
             r.cache = None
         r.finish_time = time.perf_counter()
         self.finished[r.request_id] = r
+        self.instruments.finished(r.error is None, r.finish_time - r.arrival, len(r.generated))
 
     def _finish(self, r: Request, reason: str, error: Optional[Exception] = None) -> None:
         r.finish_reason, r.error, r.remaining = reason, error, 0
         r.finish_time = time.perf_counter()
         self.finished[r.request_id] = r
+        self.instruments.finished(error is None, r.finish_time - r.arrival, 0)
 
     @property
     def idle(self) -> bool:

@@ -17,12 +17,14 @@ from __future__ import annotations
 
 import collections
 import dataclasses
+import time
 from typing import Dict, List, Optional, Sequence, Tuple
 
 import numpy as np
 import torch
 
 from ..cache.manager import CacheManager, RequestCache
+from .instruments import StepInstruments
 from .model import CausalLM
 
 
@@ -46,6 +48,23 @@ class GroupView:
     window: Optional[int]
 
 
+class ScratchExhausted(RuntimeError):
+    """A step needs more scratch memory than the weights and the cache left free."""
+
+
+@dataclasses.dataclass
+class StepResult:
+    """What a step gives back.  ``errors[i]`` is None if entry i ran; ``rows[i]`` are then
+    the rows of ``logits`` that hold its wanted places (``logits`` has the wanted places of
+    the entries that ran, in their order).  ``shared_failure``: the batch as a whole
+    failed, every entry that was in it carries this error."""
+
+    logits: Optional[torch.Tensor]
+    errors: List[Optional[Exception]]
+    rows: List[Optional[range]]
+    shared_failure: Optional[Exception] = None
+
+
 class StepContext:
     """What the parts see of a step.  Device tensors (int32):
 
@@ -55,7 +74,8 @@ class StepContext:
     adjacent), ``start_pos [reqs]`` (tokens already cached before this step),
     ``req_rows [reqs]`` (the request's row in the state slots), ``want_rows
     [wanted]``.  Host-side: ``n_rows``, ``n_reqs``, ``n_want``, ``max_q_len``,
-    ``max_ctx_len``, ``host_q_start``, ``host_start_pos``, ``host_req_rows``."""
+    ``max_ctx_len``, ``host_q_start``, ``host_start_pos``, ``host_req_rows``, and ``memo``,
+    a dictionary for what a part works out once per step and its other layers use again."""
 
     def __init__(self, ops, device, max_rows: int, max_reqs: int, groups: List[Tuple[int, Optional[int]]],
                  max_pages_per_request: int):
@@ -88,9 +108,11 @@ class StepContext:
         self._uploaded = torch.cuda.Event() if pin else None
         self._scratch: Dict[Tuple[str, torch.dtype], torch.Tensor] = {}
         self.scratch_version = 0
+        self.scratch_bytes = 0
+        self.scratch_allocations = 0
         self.n_rows = self.n_reqs = self.n_want = 0
         self.max_q_len = self.max_ctx_len = 0
-        self._short = {}
+        self.memo: Dict[object, object] = {}     # notes of the parts about this step, emptied by fill()
         self.pending = None            # PendingSums owed to the residual stream, within a forward
         self.host_q_start: List[int] = []
         self.host_start_pos: List[int] = []
@@ -115,31 +137,39 @@ class StepContext:
 
     def scratch(self, name: str, shape: Tuple[int, ...], dtype: torch.dtype) -> torch.Tensor:
         """A reusable buffer: the same name and dtype give the same memory on
-        every step, grown when a larger shape is asked for."""
+        every step, grown when a larger shape is asked for.  Before it grows it asks
+        whether the GPU still has the memory (what is free, and what the allocator holds
+        unused): the page pool takes most of what the weights left, and a step that needs
+        more scratch than remains fails with ``ScratchExhausted`` instead of somewhere in
+        the allocator (rust/engine/src/runner/model/qwen2/workspace.rs:348-373)."""
         count = 1
         for s in shape:
             count *= int(s)
         key = (name, dtype)
         buf = self._scratch.get(key)
         if buf is None or buf.numel() < count:
+            width = torch.empty((), dtype=dtype).element_size()
+            need = max(count, 1) * width
+            have = self._memory_available()
+            if have is not None and need > have:
+                raise ScratchExhausted(f"scratch buffer '{name}' needs {need} bytes; {have} bytes are "
+                                       f"available after the weights and the cache")
+            self.scratch_bytes += need - (0 if buf is None else buf.numel() * width)
+            self.scratch_allocations += 1
+            buf = None                      # give the old one back before taking the new
+            self._scratch.pop(key, None)
             buf = torch.empty(max(count, 1), dtype=dtype, device=self.device)
             self._scratch[key] = buf
             self.scratch_version += 1
         return buf[:count].view(shape)
 
-    def short_requests(self, limit: int) -> Tuple[int, int]:
-        """How many of this step's requests bring at most ``limit`` tokens, and the
-        longest context among those (0 if none)."""
-        hit = self._short.get(limit)
-        if hit is None:
-            count = longest = 0
-            for b in range(self.n_reqs):
-                n = self.host_q_start[b + 1] - self.host_q_start[b]
-                if n <= limit:
-                    count += 1
-                    longest = max(longest, self.host_start_pos[b] + n)
-            hit = self._short[limit] = (count, longest)
-        return hit
+    def _memory_available(self) -> Optional[int]:
+        if torch.device(self.device).type != "cuda":
+            return None
+        free, _ = torch.cuda.mem_get_info(self.device)
+        stats = torch.cuda.memory_stats(self.device)
+        reusable = stats.get("reserved_bytes.all.current", 0) - stats.get("allocated_bytes.all.current", 0)
+        return int(free) + max(0, int(reusable))
 
     # ------------------------------------------------------------------ fill
     def fill(self, entries: Sequence[StepEntry], cache: CacheManager) -> None:
@@ -158,7 +188,7 @@ class StepContext:
         feeds: List[Tuple[int, int]] = []
         feed_tensor = None
         self.host_q_start, self.host_start_pos, self.host_req_rows = [], [], []
-        self._short = {}
+        self.memo = {}
         max_q = max_ctx = 0
         for b, e in enumerate(entries):
             n = len(e.tokens)
@@ -225,9 +255,18 @@ class StepFunction:
     """Owns the step's buffers; ``__call__`` runs one step."""
 
     MAX_GRAPHS = 16
+    # A decode step replayed from a HIP graph costs the host nothing, but the GPU about a
+    # microsecond more at every kernel boundary than kernels launched one by one by a host
+    # that runs ahead (measured: 4.05 against 3.90 ms a step at the 7B shape, 17.3 against
+    # 16.9 at the 32B shape; 0.97 against 1.7 at the 0.5B shape, where the host cannot keep
+    # up).  ``graph="auto"`` counts the calls into the kernel libraries that the model's
+    # first decode step makes and takes the graph unless the step's reading of the weights
+    # clearly outlasts the host's making of those calls.
+    HOST_SECONDS_PER_CALL = 12e-6
+    STREAMED_BYTES_PER_SECOND = 4.2e12
 
     def __init__(self, model: CausalLM, cache: CacheManager, ops, max_batch_tokens: int,
-                 graph: bool = False):
+                 graph=False):
         self.model = model
         self.cache = cache
         self.ops = ops
@@ -236,15 +275,34 @@ class StepFunction:
         # replayed from a captured HIP graph: buffers have fixed addresses and
         # everything that changes from step to step (tokens, positions, block
         # tables) lives in device memory that is rewritten before the replay.
-        self.use_graph = bool(graph)
+        # A model with a part that cannot be captured (``graph_safe`` False) runs
+        # eagerly whatever is asked for here.
+        self.use_graph = graph if graph == "auto" else bool(graph)
         self._graphs: "collections.OrderedDict" = collections.OrderedDict()
         self.graph_replays = 0
         self.graph_captures = 0
+        self.graph_evictions = 0
+        self.decode_calls: Optional[int] = None    # library calls of one decode step (measured)
         self.ctx = StepContext(
             ops, cache.device, self.max_batch_tokens, cache.max_requests,
             [(cache.page_size, g.window) for g in cache.groups], cache.max_pages_per_request)
         self.steps = 0
         self.rows_total = 0
+        self.failed_steps = 0
+        self.instruments = StepInstruments()
+
+    def _decode_choosing(self) -> torch.Tensor:
+        """``graph="auto"``: this decode step runs eagerly and its calls are counted."""
+        before = getattr(self.ops, "calls_made", None)
+        logits = self.model.forward(self.ctx)
+        if before is None:
+            self.use_graph = False
+            return logits
+        self.decode_calls = self.ops.calls_made - before
+        host = self.decode_calls * self.HOST_SECONDS_PER_CALL
+        gpu = self.model.weight_bytes_per_step() / self.STREAMED_BYTES_PER_SECOND
+        self.use_graph = gpu < 1.25 * host
+        return logits
 
     def _decode_with_graph(self) -> torch.Tensor:
         ctx = self.ctx
@@ -273,45 +331,122 @@ class StepFunction:
         self.graph_captures += 1
         while len(self._graphs) > self.MAX_GRAPHS:
             self._graphs.popitem(last=False)
+            self.graph_evictions += 1
         return logits
+
+    # ------------------------------------------------------------- validation
+    def _refusal(self, e: StepEntry, seen: set) -> Optional[Exception]:
+        """Why this entry cannot be part of a step, or None (the reference checks the
+        same per input: rust/engine/src/runner/model/qwen2/engine.rs:811-842)."""
+        vocab, max_pos = self.model.spec.vocab_size, self.model.spec.max_positions
+        rid = e.request.request_id
+        if id(e.request) in seen:
+            return ValueError(f"request {rid!r} appears twice in one step")
+        if e.request.released:
+            return ValueError(f"request {rid!r} was released")
+        if e.request.invalid:
+            return ValueError(f"request {rid!r} was in a step that failed: its cache is not "
+                              f"to be trusted any more, release it")
+        if e.request.reserved_len != e.request.computed_len:
+            return ValueError(f"request {rid!r} has a step pending")
+        n = len(e.tokens)
+        if n == 0:
+            return ValueError(f"request {rid!r} brings no token")
+        if e.source is None:
+            for t in e.tokens:
+                if not 0 <= int(t) < vocab:
+                    return ValueError(f"token id {t} is outside the vocabulary of {vocab}")
+        elif n != 1:
+            return ValueError("an entry fed from the device brings exactly one token")
+        end = e.request.computed_len + n
+        if end > max_pos:
+            return ValueError(f"request {rid!r}: position {end - 1} exceeds "
+                              f"max_position_embeddings {max_pos}")
+        if end > self.cache.max_seq_len:
+            return ValueError(f"request {rid!r}: {end} tokens exceed the cache's maximum "
+                              f"sequence length {self.cache.max_seq_len}")
+        for w in e.want:
+            if not 0 <= int(w) < n:
+                return ValueError(f"request {rid!r}: wanted place {w} is not among its {n} "
+                                  f"tokens of this step")
+        return None
+
+    def run(self, entries: Sequence[StepEntry]) -> "StepResult":
+        """One step with a result for every entry.  An entry that cannot run (a token id
+        outside the vocabulary, a position beyond the longest sequence, no page left for
+        it) gets its error and is left out; the others still run as one batch
+        (rust/engine/src/runner/model/qwen2/engine.rs:1943-2003).  If the batch itself
+        fails (a kernel refuses a size, a launch fails), every entry that was in it gets
+        that error (engine.rs:2041-2045), their reservations are dropped and their caches
+        are marked invalid (rust/engine/src/runner/kv_pool/api.rs:257-262): what the step
+        half wrote is not to be read, such a request can only be released."""
+        errors: List[Optional[Exception]] = [None] * len(entries)
+        seen: set = set()
+        for i, e in enumerate(entries):
+            errors[i] = self._refusal(e, seen)
+            if errors[i] is None:
+                seen.add(id(e.request))
+        # what is wrong with the step as a whole is the caller's mistake: nothing runs
+        n_rows = sum(len(e.tokens) for e, err in zip(entries, errors) if err is None)
+        if n_rows > self.max_batch_tokens:
+            raise ValueError(f"a step of {n_rows} tokens exceeds max_batch_tokens {self.max_batch_tokens}")
+        if sum(1 for err in errors if err is None) > self.cache.max_requests:
+            raise ValueError(f"a step of more than {self.cache.max_requests} requests (max_requests)")
+        for i, e in enumerate(entries):
+            if errors[i] is None:
+                try:
+                    self.cache.reserve(e.request, len(e.tokens))
+                except Exception as err:            # no page left: this entry sits out, with its reason
+                    errors[i] = err
+        valid = [e for e, err in zip(entries, errors) if err is None]
+        rows: List[Optional[range]] = []
+        at = 0
+        for e, err in zip(entries, errors):
+            rows.append(None if err is not None else range(at, at + len(e.want)))
+            at += 0 if err is not None else len(e.want)
+        if not valid:
+            return StepResult(None, errors, rows)
+        started = time.perf_counter()
+        try:
+            self.ctx.fill(valid, self.cache)
+            if (self.use_graph and self.model.graph_safe
+                    and all(len(e.tokens) == 1 and len(e.want) == 1 for e in valid)):
+                logits = self._decode_choosing() if self.use_graph == "auto" else self._decode_with_graph()
+            else:
+                logits = self.model.forward(self.ctx)
+        except Exception as err:
+            for e in valid:
+                self.cache.cancel_reservation(e.request)
+                e.request.invalid = True
+            for i, had in enumerate(errors):
+                if had is None:
+                    errors[i] = err
+            self.failed_steps += 1
+            return StepResult(None, errors, [None] * len(entries), shared_failure=err)
+        for e in valid:
+            self.cache.commit(e.request)
+        self.steps += 1
+        self.rows_total += self.ctx.n_rows
+        self.instruments.step(
+            prefill=any(e.request.computed_len == len(e.tokens) or len(e.tokens) > 1 for e in valid),
+            rows=self.ctx.n_rows, requests=len(valid), submit_seconds=time.perf_counter() - started)
+        return StepResult(logits, errors, rows)
 
     def __call__(self, entries: Sequence[StepEntry]) -> Optional[torch.Tensor]:
         """Reserve pages, run the rows, commit.  Returns float32 logits
         ``[wanted, vocab]`` in the order of the entries and of their ``want``
-        (None when nothing is wanted).  The tensor is reused by the next step."""
+        (None when nothing is wanted).  The tensor is reused by the next step.
+        Any entry that cannot run raises here, before anything has run."""
         if not entries:
             return None
-        vocab, max_pos = self.model.spec.vocab_size, self.model.spec.max_positions
-        seen = set()
+        seen: set = set()
         for e in entries:
-            if id(e.request) in seen:
-                raise ValueError(f"request {e.request.request_id!r} appears twice in one step")
+            refusal = self._refusal(e, seen)
+            if refusal is not None:
+                raise refusal
             seen.add(id(e.request))
-            if len(e.tokens) == 0:
-                raise ValueError(f"request {e.request.request_id!r} brings no token")
-            for t in (e.tokens if e.source is None else ()):
-                if not 0 <= int(t) < vocab:
-                    raise ValueError(f"token id {t} is outside the vocabulary of {vocab}")
-            if e.request.computed_len + len(e.tokens) > max_pos:
-                raise ValueError(
-                    f"request {e.request.request_id!r}: position "
-                    f"{e.request.computed_len + len(e.tokens) - 1} exceeds max_position_embeddings {max_pos}")
-        reserved: List[RequestCache] = []
-        try:
-            for e in entries:
-                self.cache.reserve(e.request, len(e.tokens))
-                reserved.append(e.request)
-            self.ctx.fill(entries, self.cache)
-        except Exception:
-            for r in reserved:
-                self.cache.cancel_reservation(r)
-            raise
-        if self.use_graph and all(len(e.tokens) == 1 and len(e.want) == 1 and e.want[0] == 0 for e in entries):
-            logits = self._decode_with_graph()
-        else:
-            logits = self.model.forward(self.ctx)
-        for e in entries:
-            self.cache.commit(e.request)
-        self.steps += 1
-        self.rows_total += self.ctx.n_rows
-        return logits
+        result = self.run(entries)
+        for err in result.errors:
+            if err is not None:
+                raise err
+        return result.logits

@@ -139,6 +139,16 @@ def attention_library(head_dim: int, force: bool = False) -> str:
     return _compile(f"attn_d{head_dim}", (ATTENTION_SOURCE,), (f"-DHEAD_DIM={head_dim}",), force)
 
 
+def library(kind: str, parameter=None, force: bool = False) -> str:
+    """The library a part names in ``kernel_libraries()``: ``("core", None)`` or
+    ``("attention", head_dim)``."""
+    if kind == "core":
+        return core_library(force)
+    if kind == "attention":
+        return attention_library(int(parameter), force)
+    raise ValueError(f"no kernel library of kind '{kind}'")
+
+
 def build_all(head_dims: Sequence[int] = DEFAULT_HEAD_DIMS, force: bool = True) -> Dict[str, str]:
     """Compile the core library and the attention libraries of the given head sizes."""
     out = {"core": core_library(force)}

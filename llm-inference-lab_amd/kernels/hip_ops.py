@@ -87,6 +87,7 @@ class HipOps:
         self.num_cus = int(torch.cuda.get_device_properties(self.device).multi_processor_count)
         self.workspace = torch.empty(self.WORKSPACE_FLOATS, dtype=torch.float32, device=self.device)
         self.loaded_libraries = [self._core._name]
+        self.calls_made = 0          # calls into the kernel libraries so far
 
     # ---------------------------------------------------------------- loading
     @staticmethod
@@ -232,6 +233,7 @@ class HipOps:
 
     def _call(self, fn, *args, lib=None) -> None:
         """One call into the kernel libraries; a failure raises with the library's message."""
+        self.calls_made += 1
         code = fn(*args)
         if code != 0:
             self._check(code, lib)
@@ -694,9 +696,22 @@ class HipOps:
             self._stream())
 
     # -------------------------------------------------------------- attention
+    def attention_short_limit(self, num_heads: int, num_kv_heads: int, dtype, max_q_len: int) -> int:
+        """A mixed step (portions of prompts beside decoding requests) is served by two
+        launches: its requests of a few tokens go to the one that splits their keys over
+        the chip, the portions to the tiled one.  Returns the most tokens a request may
+        bring to count as short in such a step, or 0 if the step is not divided."""
+        group = num_heads // num_kv_heads
+        if dtype == torch.bfloat16 and group <= 16 < max_q_len * group:
+            return 16 // group
+        return 0
+
     def paged_attention(self, qkv, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_table,
                         page_size, q_start, start_pos, n_reqs, max_q_len, max_ctx_len, window, scale,
-                        out, ctx=None) -> None:
+                        out, short=None) -> None:
+        """``short``: ``(row_req, limit, count, longest)`` for a step in which ``count`` of the
+        requests (not all) bring at most ``limit = attention_short_limit(...)`` tokens, the
+        longest context among those being ``longest``."""
         lib = self._attention_lib(head_dim)
         rows = qkv.shape[0]
         self._need(qkv, "queries", contiguous=False)
@@ -722,18 +737,15 @@ class HipOps:
         if page_size < 16 or page_size & (page_size - 1):
             raise UnsupportedSizeError(f"page size {page_size} is not a power of two >= 16")
         q_stride = qkv.stride(0) if rows > 1 else qkv.shape[1]
-        # a mixed step: its requests of a few tokens (decoding ones) go to the launch that
-        # splits their keys over the chip, the portions of prompts to the tiled one
         row_req, short_len, n_short, short_ctx = None, 0, 0, 0
-        group = num_heads // num_kv_heads
-        if (ctx is not None and qkv.dtype == torch.bfloat16 and group <= 16 < max_q_len * group
-                and hasattr(ctx, "short_requests")):
-            n_short, short_ctx = ctx.short_requests(16 // group)
-            if 0 < n_short < n_reqs:
-                row_req, short_len = ctx.row_req, 16 // group
-                self._need(row_req, "row -> request map", torch.int32)
-            else:
-                n_short = short_ctx = 0
+        if short is not None:
+            row_req, short_len, n_short, short_ctx = short
+            if (short_len != self.attention_short_limit(num_heads, num_kv_heads, qkv.dtype, max_q_len)
+                    or not 0 < n_short < n_reqs or short_ctx > max_ctx_len):
+                raise ValueError("attention: the description of the step's short requests does not fit")
+            self._need(row_req, "row -> request map", torch.int32)
+            if row_req.numel() < rows:
+                raise ValueError("attention: one request index per row")
         self._call(lib.llmlab_paged_attention,
             self._ptr(qkv), _dt(qkv), q_stride, num_heads, num_kv_heads, self._ptr(k_cache),
             self._ptr(v_cache), self._ptr(block_table), block_table.stride(0), page_size,

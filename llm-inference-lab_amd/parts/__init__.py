@@ -1,6 +1,6 @@
 from .registry import register_part, unregister_part, part_class, build_part, FAMILIES
 from .base import (Part, Norm, NormedInput, PendingSums, PositionEncoding, Mixer, FeedForward, Block,
-                   KVCacheSpec)
+                   KVCacheSpec, CacheSpec, PageTensor)
 from .norms import RMSNorm
 from .positions import RotaryEmbedding, NoPosition
 from .attention import GQAAttention

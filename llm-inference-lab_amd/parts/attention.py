@@ -147,7 +147,7 @@ class GQAAttention(Mixer):
             q, self.num_heads, self.num_kv_heads, self.head_dim,
             entry.k_cache, entry.v_cache, group.block_table, group.page_size,
             ctx.q_start, ctx.start_pos, ctx.n_reqs, ctx.max_q_len, ctx.max_ctx_len,
-            self.window, self.scale, out, ctx)
+            self.window, self.scale, out, self._short_requests(ctx))
         if pending is not None:
             ops.linear_residual(out, self.w_o, residual, self.b_o, pending=pending)
             ctx.pending = None
@@ -162,6 +162,27 @@ class GQAAttention(Mixer):
             ctx.pending = ops.linear_partials(out, self.w_o, parts, splits, self.b_o)
         else:
             ops.linear_residual(out, self.w_o, residual, self.b_o)
+
+    def _short_requests(self, ctx):
+        """Which of the step's requests bring only a few tokens (the kernels serve those by
+        another launch than the portions of prompts); worked out once per step, kept in
+        the step's notes for the other layers."""
+        limit = self.ops.attention_short_limit(self.num_heads, self.num_kv_heads, self.dtype, ctx.max_q_len)
+        if limit <= 0:
+            return None
+        key = ("attention.short", limit)
+        if key not in ctx.memo:
+            count = longest = 0
+            for b in range(ctx.n_reqs):
+                n = ctx.host_q_start[b + 1] - ctx.host_q_start[b]
+                if n <= limit:
+                    count += 1
+                    longest = max(longest, ctx.host_start_pos[b] + n)
+            ctx.memo[key] = (ctx.row_req, limit, count, longest) if 0 < count < ctx.n_reqs else None
+        return ctx.memo[key]
+
+    def kernel_libraries(self):
+        return [("attention", self.head_dim)]
 
     def weight_bytes(self):
         total = 0

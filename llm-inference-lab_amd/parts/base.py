@@ -20,15 +20,61 @@ from ..weights.loader import TensorSpec
 
 
 @dataclasses.dataclass(frozen=True)
-class KVCacheSpec:
-    """What a mixer keeps for each token: ``num_kv_heads * head_dim`` keys and as
-    many values.  ``window``: how many of the latest positions (the current one
-    included) it ever reads, or ``None`` for all.  Mixers with equal specs share
-    one group of pages and one block table."""
+class PageTensor:
+    """One named tensor of a mixer's per-token cache.  ``token_shape`` is what one token
+    keeps in it; a page of ``P`` tokens is a tensor of that shape with an axis of length
+    ``P`` put in at ``token_axis``.  Keys of ``G`` heads of width ``d`` with
+    ``token_axis=1``: pages ``[G, P, d]``; values with ``token_axis=2``: pages ``[G, d, P]``;
+    one latent vector of width ``r`` per token with ``token_axis=0``: pages ``[P, r]``.
+    ``dtype`` None means the engine's compute dtype."""
 
-    num_kv_heads: int
-    head_dim: int
+    token_shape: Tuple[int, ...]
+    token_axis: int = 0
+    dtype: Optional[torch.dtype] = None
+
+    def page_shape(self, page_size: int) -> Tuple[int, ...]:
+        shape = list(self.token_shape)
+        if not 0 <= self.token_axis <= len(shape):
+            raise ValueError(f"token_axis {self.token_axis} does not fit the shape {self.token_shape}")
+        shape.insert(self.token_axis, int(page_size))
+        return tuple(shape)
+
+    def token_elements(self) -> int:
+        n = 1
+        for s in self.token_shape:
+            n *= int(s)
+        return n
+
+
+@dataclasses.dataclass(frozen=True)
+class CacheSpec:
+    """What a mixer keeps for each token: named tensors in pages.  ``window``: how many
+    of the latest positions (the current one included) it ever reads, or ``None`` for
+    all.  Mixers with equal specs share one group of pages and one block table; the cache
+    manager allocates ``[runs, pages, *page_shape]`` per name and a run of the mixer finds
+    its slices in ``entry.cache[name]``."""
+
+    tensors: Tuple[Tuple[str, PageTensor], ...]
     window: Optional[int] = None
+
+    def __post_init__(self):
+        names = [n for n, _ in self.tensors]
+        if not names or len(set(names)) != len(names):
+            raise ValueError(f"a cache spec names at least one tensor, each once: {names}")
+        if self.window is not None and self.window <= 0:
+            raise ValueError(f"a window holds at least the current position, got {self.window}")
+
+    def bytes_per_token(self, dtype: torch.dtype) -> int:
+        return sum(t.token_elements() * torch.empty((), dtype=t.dtype or dtype).element_size()
+                   for _, t in self.tensors)
+
+
+def KVCacheSpec(num_kv_heads: int, head_dim: int, window: Optional[int] = None) -> CacheSpec:
+    """The cache of an attention mixer: ``k`` in pages ``[kv_heads, P, head_dim]`` and ``v``
+    in pages ``[kv_heads, head_dim, P]`` (values transposed, so that the probability-value
+    product reads runs of tokens)."""
+    return CacheSpec((("k", PageTensor((int(num_kv_heads), int(head_dim)), 1)),
+                      ("v", PageTensor((int(num_kv_heads), int(head_dim)), 2))), window)
 
 
 class Part:
@@ -52,6 +98,17 @@ class Part:
     def weight_bytes(self) -> int:
         """Bytes of weights one forward reads (for roofline accounting)."""
         return 0
+
+    # False: ``forward`` decides something on the host from this step's data (indexes a
+    # tensor with a host list, branches on a value) that a replayed graph would freeze.
+    # A model with such a part runs its decode steps eagerly even when graphs are asked for.
+    graph_safe = True
+
+    def kernel_libraries(self):
+        """Kernel libraries to have compiled before the model is bound, as ``(kind,
+        parameter)`` pairs that ``kernels.build.library`` knows (``("attention",
+        head_dim)``)."""
+        return []
 
 
 class Norm(Part):
@@ -150,8 +207,9 @@ class PositionEncoding(Part):
 class Mixer(Part):
     takes_normed_input = False     # True: ``forward`` gets a ``NormedInput`` and may fuse the norm
 
-    def cache_spec(self) -> Optional[KVCacheSpec]:
-        """Per-token cache need, or None."""
+    def cache_spec(self) -> Optional[CacheSpec]:
+        """Per-token cache need (``KVCacheSpec(...)`` for keys and values, or any
+        ``CacheSpec`` of named page tensors), or None."""
         return None
 
     def state_spec(self) -> Dict[str, Tuple[Tuple[int, ...], torch.dtype]]:
@@ -178,6 +236,13 @@ class Block(Part):
     def parts(self):
         """The parts this block is made of (for tensor lists and binding)."""
         raise NotImplementedError
+
+    @property
+    def graph_safe(self):
+        return all(p.graph_safe for p in self.parts())
+
+    def kernel_libraries(self):
+        return [lib for p in self.parts() for lib in p.kernel_libraries()]
 
     def mixer_part(self) -> Mixer:
         raise NotImplementedError

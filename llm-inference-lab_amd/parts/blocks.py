@@ -73,7 +73,9 @@ class TokenEmbedding(Part):
         # in the order the product kernels read, so that a tied output head shares it
         self.table = ops.prepare_weight(tensors[self.tensor_names["weight"]], shared=True)
 
-    def forward(self, ids, out):
+    def forward(self, ids, out, ctx=None):
+        """``ctx``: the step's batch description, for embeddings that need more than the
+        ids (positions, say); this one does not."""
         self.ops.embed(self.table, ids, out)
 
     def weight_bytes(self):

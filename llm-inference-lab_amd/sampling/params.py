@@ -57,12 +57,48 @@ class SamplingConfig:
         return tuple(int(e) for e in self.eos_token_id)
 
 
-def read_generation_config(model_dir: str) -> SamplingConfig:
-    """Optional ``generation_config.json`` of a model folder (loader.rs:199-205)."""
+def _check_generation_field(path: str, key: str, value):
+    """One field of ``generation_config.json``, type-checked; the error names the key."""
+    from ..config.errors import ConfigError
+
+    def bad(expected):
+        return ConfigError(f"{path}: '{key}' must be {expected}, got {value!r}")
+    if value is None:
+        return None
+    if key == "do_sample":
+        if not isinstance(value, bool):
+            raise bad("true or false")
+        return value
+    if key in ("temperature", "top_p"):
+        if isinstance(value, bool) or not isinstance(value, (int, float)) or not value >= 0:
+            raise bad("a number >= 0")
+        return float(value)
+    if key in ("top_k", "max_new_tokens"):
+        if isinstance(value, bool) or not isinstance(value, int) or value < 0:
+            raise bad("an integer >= 0")
+        return value
+    if key == "eos_token_id":
+        ids = value if isinstance(value, list) else [value]
+        if not all(isinstance(i, int) and not isinstance(i, bool) and i >= 0 for i in ids):
+            raise bad("a token id or a list of token ids")
+        return value if isinstance(value, int) else [int(i) for i in ids]
+    return value
+
+
+def read_generation_config(model_dir: str) -> Optional[SamplingConfig]:
+    """The optional ``generation_config.json`` of a model folder, or None if there is
+    none (rust/engine/src/runner/loader.rs:199-205).  The reference's fields are read
+    (loader.rs:30-44), every other key of the file is ignored."""
     path = os.path.join(model_dir, "generation_config.json")
     if not os.path.isfile(path):
-        return SamplingConfig()
+        return None
+    from ..config.errors import ConfigError
     with open(path, "r", encoding="utf-8") as f:
-        raw = json.load(f)
-    known = {f.name for f in dataclasses.fields(SamplingConfig)}
-    return SamplingConfig(**{k: v for k, v in raw.items() if k in known})
+        try:
+            raw = json.load(f)
+        except json.JSONDecodeError as e:
+            raise ConfigError(f"{path}: not valid JSON ({e})") from None
+    if not isinstance(raw, dict):
+        raise ConfigError(f"{path}: a JSON object is expected")
+    known = ("do_sample", "temperature", "top_k", "top_p", "max_new_tokens", "eos_token_id")
+    return SamplingConfig(**{k: _check_generation_field(path, k, raw[k]) for k in known if k in raw})

@@ -41,11 +41,15 @@ class PendingTokens:
         self._event = event
         self.rows = rows
 
-    def result(self) -> List[int]:
-        """Wait for the copy; raises if a row held no finite logit."""
+    def tokens(self) -> List[int]:
+        """Wait for the copy.  A row that held no finite logit gives -1."""
         if self._event is not None:
             self._event.synchronize()
-        tokens = self._host[:self.rows].tolist()
+        return self._host[:self.rows].tolist()
+
+    def result(self) -> List[int]:
+        """Wait for the copy; raises if a row held no finite logit."""
+        tokens = self.tokens()
         for t in tokens:
             if t < 0:
                 raise FloatingPointError("non-finite logits: no token can be chosen")
@@ -59,12 +63,18 @@ class Sampler:
         self.ops = ops
         self.device = ops.device
         self._cuda = torch.device(self.device).type == "cuda"
-        self._host = torch.zeros((2, max_requests), dtype=torch.float32, pin_memory=self._cuda)
-        self._dev = torch.zeros((2, max_requests), dtype=torch.float32, device=self.device)
+        # Every slot has its own staging of the inputs (temperatures, uniform numbers) as
+        # well as of the outputs: with one step of lookahead the host fills the next
+        # step's numbers while the copy of this step's may not have run yet.
+        self._host = [torch.zeros((2, max_requests), dtype=torch.float32, pin_memory=self._cuda)
+                      for _ in range(self.SLOTS)]
+        self._dev = [torch.zeros((2, max_requests), dtype=torch.float32, device=self.device)
+                     for _ in range(self.SLOTS)]
         self._out = [torch.zeros(max_requests, dtype=torch.int32, device=self.device)
                      for _ in range(self.SLOTS)]
         self._out_host = [torch.zeros(max_requests, dtype=torch.int32, pin_memory=self._cuda)
                           for _ in range(self.SLOTS)]
+        self._done = [None] * self.SLOTS      # recorded after a slot's last copy to the host
         self._slot = 0
 
     def sample_async(self, logits: torch.Tensor, temperatures: Sequence[float], seeds: Sequence[int],
@@ -73,21 +83,26 @@ class Sampler:
         to the host is started.  The buffers are reused after ``SLOTS`` further calls."""
         rows = logits.shape[0]
         self._slot = (self._slot + 1) % self.SLOTS
-        out, out_host = self._out[self._slot], self._out_host[self._slot]
+        slot = self._slot
+        out, out_host = self._out[slot], self._out_host[slot]
+        if self._done[slot] is not None:
+            # everything queued with this slot's buffers has run: they are free again
+            self._done[slot].synchronize()
         if all(t <= 0.0 for t in temperatures):
             self.ops.argmax(logits, out[:rows])
         else:
-            h = self._host.numpy()
+            host, dev = self._host[slot], self._dev[slot]
+            h = host.numpy()
             h[0, :rows] = np.asarray(temperatures, dtype=np.float32)
             h[1, :rows] = np.asarray([uniform(s, c) for s, c in zip(seeds, counters)], dtype=np.float32)
-            self._dev[0, :rows].copy_(self._host[0, :rows], non_blocking=True)
-            self._dev[1, :rows].copy_(self._host[1, :rows], non_blocking=True)
-            self.ops.sample(logits, self._dev[0, :rows], self._dev[1, :rows], out[:rows])
+            dev[:, :rows].copy_(host[:, :rows], non_blocking=True)
+            self.ops.sample(logits, dev[0, :rows], dev[1, :rows], out[:rows])
         event = None
         if self._cuda:
             out_host[:rows].copy_(out[:rows], non_blocking=True)
             event = torch.cuda.Event()
             event.record()
+            self._done[slot] = event
         else:
             out_host[:rows].copy_(out[:rows])
         return PendingTokens(out, out_host, event, rows)

@@ -222,9 +222,12 @@ class EmuOps:
             vflat[page][:, cache_layout.value_index(page_size, head_dim)[:, off]] = v[r].to(v_cache.dtype)
 
     # -------------------------------------------------------------- attention
+    def attention_short_limit(self, num_heads, num_kv_heads, dtype, max_q_len):
+        return 0
+
     def paged_attention(self, qkv, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_table,
                         page_size, q_start, start_pos, n_reqs, max_q_len, max_ctx_len, window, scale,
-                        out, ctx=None):
+                        out, short=None):
         self._count("paged_attention")
         group = num_heads // num_kv_heads
         qs = num_heads * head_dim

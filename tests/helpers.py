@@ -39,7 +39,23 @@ REAL_LAYER = dict(architectures=["Qwen2ForCausalLM"], model_type="qwen2", vocab_
                   intermediate_size=4864, num_hidden_layers=2, num_attention_heads=14,
                   num_key_value_heads=2, head_dim=64, rms_norm_eps=1e-6, rope_theta=1000000.0,
                   max_position_embeddings=4096, tie_word_embeddings=True, use_sliding_window=False)
-CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "R": REAL_LAYER}
+# The whole Qwen2.5-0.5B shape (24 layers, the real vocabulary), and one layer each with the
+# widths of Qwen2.5-7B and Qwen2.5-32B (a small odd vocabulary): the sizes at which the
+# kernels' rules for large matrices decide.
+FULL_05B = dict(architectures=["Qwen2ForCausalLM"], model_type="qwen2", vocab_size=151936, hidden_size=896,
+                intermediate_size=4864, num_hidden_layers=24, num_attention_heads=14,
+                num_key_value_heads=2, head_dim=64, rms_norm_eps=1e-6, rope_theta=1000000.0,
+                max_position_embeddings=32768, tie_word_embeddings=True, use_sliding_window=False)
+WIDE_7B = dict(architectures=["Qwen2ForCausalLM"], model_type="qwen2", vocab_size=5003, hidden_size=3584,
+               intermediate_size=18944, num_hidden_layers=1, num_attention_heads=28,
+               num_key_value_heads=4, head_dim=128, rms_norm_eps=1e-6, rope_theta=1000000.0,
+               max_position_embeddings=32768, tie_word_embeddings=False, use_sliding_window=False)
+WIDE_32B = dict(architectures=["Qwen2ForCausalLM"], model_type="qwen2", vocab_size=5003, hidden_size=5120,
+                intermediate_size=27648, num_hidden_layers=1, num_attention_heads=40,
+                num_key_value_heads=8, head_dim=128, rms_norm_eps=1e-6, rope_theta=1000000.0,
+                max_position_embeddings=32768, tie_word_embeddings=False, use_sliding_window=False)
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "R": REAL_LAYER, "F": FULL_05B, "W7": WIDE_7B,
+           "W32": WIDE_32B}
 
 # Decided before the first run and not widened since.  Logits of these models are
 # of order 1.  float32: sums in another order than the float64 reference.
@@ -80,11 +96,17 @@ def random_ids(cfg, n, seed):
 _PLAIN_CACHE = {}
 
 
+_PLAIN_WEIGHTS = {}      # the float64 weights of the model asked for last (one model: they are large)
+
+
 def plain_logits(name, seed, ids):
     key = (name, seed, tuple(ids))
     if key not in _PLAIN_CACHE:
         cfg = config_of(name)
-        _PLAIN_CACHE[key] = plain_qwen2.forward_logits(ids, make_tensors(cfg, seed), cfg.to_dict())
+        if (name, seed) not in _PLAIN_WEIGHTS:
+            _PLAIN_WEIGHTS.clear()
+            _PLAIN_WEIGHTS[(name, seed)] = {k: v.double() for k, v in make_tensors(cfg, seed).items()}
+        _PLAIN_CACHE[key] = plain_qwen2.forward_logits(ids, _PLAIN_WEIGHTS[(name, seed)], cfg.to_dict())
     return _PLAIN_CACHE[key]
 
 
@@ -217,3 +239,28 @@ def first_wrong(got, want, tol):
             if err > tol:
                 return rid, pos, err
     return None
+
+
+def check_drawn_tokens(name, seed, prompt, generated, temperature, stream_seed, slack=1e-5):
+    """Every generated token is the one the plain implementation predicts from the tokens
+    before it: the argmax at temperature 0, else the inverse-CDF draw from
+    ``softmax(plain logits / temperature)`` at ``uniform(stream_seed, n)`` for the n-th
+    token.  A draw closer than ``slack`` to a boundary of the cumulative sums may fall to
+    either side (float32 sums on the GPU, float64 here)."""
+    from llm_inference_lab_amd.sampling.sampler import uniform
+    ids = list(prompt)
+    for n, token in enumerate(generated):
+        logits = plain_logits(name, seed, ids)[-1]
+        if temperature <= 0.0:
+            best = plain_qwen2.argmax_smallest_index(logits)
+            assert token == best or float(logits[best] - logits[token]) < 1e-4, \
+                f"token {n}: {token} is not the argmax {best}"
+        else:
+            probs = plain_qwen2.temperature_probs(logits, temperature)
+            u = uniform(stream_seed, n)
+            cdf = torch.cumsum(probs, 0)
+            below = float(cdf[token - 1]) if token > 0 else 0.0
+            assert below - slack < u <= float(cdf[token]) + slack and float(probs[token]) > 0.0, \
+                (f"token {n}: {token} covers ({below}, {float(cdf[token])}], the draw is {u}; "
+                 f"plain predicts {plain_qwen2.inverse_cdf_token(probs, u)}")
+        ids.append(token)

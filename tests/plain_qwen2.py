@@ -190,3 +190,17 @@ def temperature_probs(logits: torch.Tensor, temperature: float) -> torch.Tensor:
     z = logits.to(torch.float64) / temperature
     e = torch.exp(z - z.max())
     return e / e.sum()
+
+
+def inverse_cdf_token(probs: torch.Tensor, u: float) -> int:
+    """The smallest token whose cumulative probability reaches ``u`` (a uniform number
+    in [0, 1)); tokens of probability 0 are never chosen."""
+    target = u * float(probs.sum())
+    run, last = 0.0, -1
+    for i, p in enumerate(probs.tolist()):
+        if p > 0.0:
+            last = i
+            run += p
+            if run >= target:
+                return i
+    return last

@@ -7,7 +7,7 @@ import torch
 
 from llm_inference_lab_amd.cache import (CacheManager, GroupLayout, OutOfPages, PagePool,
                                          group_page_need, pages_for_tokens)
-from llm_inference_lab_amd.parts import KVCacheSpec
+from llm_inference_lab_amd.parts import CacheSpec, KVCacheSpec, PageTensor
 
 
 def manager(pages=(8,), windows=(None,), page_size=16, max_requests=4, max_seq_len=256, state=None):
@@ -145,3 +145,28 @@ def test_random_orders_keep_every_invariant(seed):
         m.release(req)
     m.check()
     assert m.free_pages(0) == 24 and m.free_pages(1) == 10 and m.free_rows == 4
+
+
+def test_a_cache_is_described_by_named_page_tensors():
+    """Keys and values are two names among any: a group's storage is one tensor
+    ``[runs, pages, *page_shape]`` for every name of its spec, in the tensor's own dtype."""
+    kv = KVCacheSpec(2, 16, None)
+    assert [n for n, _ in kv.tensors] == ["k", "v"]
+    assert dict(kv.tensors)["k"].page_shape(32) == (2, 32, 16)
+    assert dict(kv.tensors)["v"].page_shape(32) == (2, 16, 32)
+    assert kv.bytes_per_token(torch.bfloat16) == 2 * 2 * 16 * 2 and kv == KVCacheSpec(2, 16)
+    latent = CacheSpec((("latent", PageTensor((24,), 0)), ("gate", PageTensor((3,), 1, torch.float32))), window=40)
+    assert latent.bytes_per_token(torch.bfloat16) == 24 * 2 + 3 * 4
+    groups = [GroupLayout(kv, [0, 2], 5), GroupLayout(latent, [1], 7)]
+    m = CacheManager(groups, 16, 2, 64, {}, torch.bfloat16, "cpu")
+    assert tuple(m.storage[0]["k"].shape) == (2, 5, 2, 16, 16) and m.storage[0]["v"].dtype == torch.bfloat16
+    assert tuple(m.storage[1]["latent"].shape) == (1, 7, 16, 24)
+    assert tuple(m.storage[1]["gate"].shape) == (1, 7, 3, 16) and m.storage[1]["gate"].dtype == torch.float32
+    assert m.bytes_per_token() == 2 * kv.bytes_per_token(torch.bfloat16) + latent.bytes_per_token(torch.bfloat16)
+    assert m.keys[0] is m.storage[0]["k"]
+    with pytest.raises(ValueError, match="each once"):
+        CacheSpec((("a", PageTensor((1,))), ("a", PageTensor((2,)))))
+    with pytest.raises(ValueError, match="token_axis"):
+        PageTensor((4,), 3).page_shape(16)
+    with pytest.raises(TypeError, match="CacheSpec"):
+        CacheManager([GroupLayout((2, 16, None), [0], 4)], 16, 2, 64, {}, torch.float32, "cpu")

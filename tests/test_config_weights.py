@@ -128,6 +128,24 @@ def test_one_error_lists_missing_unexpected_and_wrong_shapes(tmp_path):
         assert piece in text
 
 
+def test_tensors_the_model_does_not_use_are_left_unread(tmp_path):
+    """A file that holds all the model needs and more loads (the reference ignores extra
+    tensors, rust/engine/src/runner/loader.rs:218): the extra names are reported, and an
+    error only where the caller asks for strictness."""
+    cfg = H.config_of("A")
+    tensors = H.make_tensors(cfg, 0)
+    tensors["lm_head.weight"] = torch.zeros(256, 64, dtype=torch.bfloat16)     # tied: not used
+    tensors["model.rotary_emb.inv_freq"] = torch.zeros(8)
+    save_safetensors(str(tmp_path / "model.safetensors"), tensors.items())
+    said = []
+    loaded = load_tensors(str(tmp_path), H.expected_tensors(cfg), torch.float32, "cpu", progress=said.append)
+    assert sorted(loaded) == sorted(H.expected_tensors(cfg))
+    assert any("lm_head.weight" in line and "left unread" in line for line in said)
+    with pytest.raises(WeightError) as err:
+        load_tensors(str(tmp_path), H.expected_tensors(cfg), torch.float32, "cpu", strict=True)
+    assert err.value.unexpected == ["lm_head.weight", "model.rotary_emb.inv_freq"] and not err.value.missing
+
+
 def test_kept_dtypes():
     bf, f32 = torch.bfloat16, torch.float32
     assert kept_dtype(MATRIX, bf, bf) == bf and kept_dtype(MATRIX, f32, bf) == bf

@@ -205,7 +205,7 @@ def test_default_page_pool_fits_the_free_memory(monkeypatch):
     full = lab.Engine(config=cfg, tensors=tensors.items(), dtype="bf16", page_size=16, max_requests=4,
                       max_seq_len=512)
     assert full.cache.metrics()["groups"][0]["pages_total"] == 4 * 512 // 16
-    per_page = sum(2 * len(g.entries) * g.spec.num_kv_heads * g.spec.head_dim * 2 for g in full.model.cache_layout()[0]) * 16
+    per_page = sum(len(g.entries) * g.spec.bytes_per_token(torch.bfloat16) for g in full.model.cache_layout()[0]) * 16
     monkeypatch.setattr(torch.cuda, "mem_get_info", lambda device=None: (int(50 * per_page / 0.9) + 1, 1 << 40))
     small = lab.Engine(config=cfg, tensors=tensors.items(), dtype="bf16", page_size=16, max_requests=4,
                        max_seq_len=512)
@@ -273,6 +273,47 @@ def test_temperature_sampling_on_the_gpu(dtype):
         assert a == b
     else:
         assert [x[0] for x in a] == [x[0] for x in b]
+
+
+def test_drawn_tokens_are_those_the_plain_implementation_predicts():
+    """Config B in float32, three prompts, 24 tokens at temperature 0.8: token n of prompt
+    i is the inverse-CDF draw from softmax(plain logits / 0.8) at uniform(seed + i, n)."""
+    cfg = H.config_of("B")
+    prompts = [H.random_ids(cfg, n, 70 + n) for n in (5, 40, 61)]
+    engine = H.make_engine("B", 1, "f32", num_pages=30)
+    got = engine.generate(prompts, max_new_tokens=24, temperature=0.8, seed=11, eos_token_id=[])
+    for i, (prompt, tokens) in enumerate(zip(prompts, got)):
+        assert len(tokens) == 24
+        H.check_drawn_tokens("B", 1, prompt, tokens, 0.8, 11 + i)
+
+
+def test_sampling_with_the_gpu_lagging_behind_the_host():
+    """Greedy and sampled requests in one batch, of different lengths so that the batch
+    changes while it runs, and a GPU that is a millisecond behind the host at every step
+    (a sleeping kernel ahead of each): with one step of lookahead the host then fills the
+    next step's temperatures and uniform numbers while this step's have not been copied
+    yet.  Same tokens as without lookahead, and each the plain implementation's."""
+    from llm_inference_lab_amd.sampling import SamplingConfig
+    cfg = H.config_of("B")
+    prompts = [H.random_ids(cfg, n, 170 + n) for n in (3, 9, 30, 17)]
+    temps = [0.8, 0.0, 1.3, 0.0]
+    news = [20, 7, 12, 16]
+    sampling = [SamplingConfig(temperature=t, do_sample=t > 0, max_new_tokens=n, eos_token_id=[], seed=40 + i)
+                for i, (t, n) in enumerate(zip(temps, news))]
+    runs = {}
+    for overlap in (True, False):
+        engine = H.make_engine("B", 1, "f32", num_pages=30, max_batch_tokens=16)
+        step = engine.step_fn.__call__
+
+        def lagging(entries, step=step):
+            torch.cuda._sleep(2_000_000)
+            return step(entries)
+        engine.step = lagging
+        runs[overlap] = engine.generate(prompts, sampling=sampling, overlap=overlap)
+    assert runs[True] == runs[False]
+    for i, (prompt, tokens) in enumerate(zip(prompts, runs[True])):
+        assert len(tokens) == news[i]
+        H.check_drawn_tokens("B", 1, prompt, tokens, temps[i], 40 + i)
 
 
 def write_model_dir(path, name, seed=1):

@@ -535,18 +535,16 @@ def run_attention(ops, emu, dtype, nq, nkv, d, page, window, reqs_spec, seed=30,
 
     # the same step described as the engine describes it (which requests are short): a
     # mixed step is then served by two launches
-    class Described:
+    limit = ops.attention_short_limit(nq, nkv, dtype, max(n for _, n in reqs_spec))
+    short_reqs = [(s, n) for s, n in reqs_spec if n <= limit]
+    short = None
+    if 0 < len(short_reqs) < reqs:
         row_req = torch.cat([torch.full((n,), b) for b, (_, n) in enumerate(reqs_spec)]).int().to(DEV)
-
-        @staticmethod
-        def short_requests(limit):
-            short = [(s, n) for s, n in reqs_spec if n <= limit]
-            return len(short), max((s + n for s, n in short), default=0)
-
+        short = (row_req, limit, len(short_reqs), max(s + n for s, n in short_reqs))
     got2 = torch.zeros(rows, nq * d, dtype=dtype, device=DEV)
     ops.paged_attention(qkv.to(DEV), nq, nkv, d, kc.to(DEV), vc.to(DEV), table.to(DEV), page,
                         q_start_t.to(DEV), start_pos_t.to(DEV), reqs, max(n for _, n in reqs_spec),
-                        max_ctx, window, scale, got2, Described())
+                        max_ctx, window, scale, got2, short)
     err = (got2.float().cpu() - want.float()).abs().max().item()
     assert err <= tol * max(1.0, want.float().abs().max().item()), f"attention error {err} (described step)"
 

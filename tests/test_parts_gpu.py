@@ -11,8 +11,8 @@ import helpers as H
 import plain_qwen2 as P
 from llm_inference_lab_amd.config import (BlockSpec, ModelSpec, PartSpec, ScheduleEntry,
                                           register_architecture, unregister_architecture)
-from llm_inference_lab_amd.parts import (Mixer, RMSNorm, RotaryEmbedding, SwiGLU, TokenEmbedding,
-                                         LinearHead, register_part, build_part)
+from llm_inference_lab_amd.parts import (CacheSpec, Mixer, PageTensor, Part, RMSNorm, RotaryEmbedding, SwiGLU,
+                                         TokenEmbedding, LinearHead, register_part, build_part)
 from llm_inference_lab_amd.parts.registry import unregister_part
 from llm_inference_lab_amd.weights import TensorSpec, MATRIX
 
@@ -178,6 +178,8 @@ class RunningMean(Mixer):
     projection of the mean of all inputs of its request so far.  The state (sum
     and count) lives in the cache manager's per-request slots."""
 
+    graph_safe = False        # it finds its state rows through host lists: not for a replayed graph
+
     def __init__(self, hidden_size, tensors):
         super().__init__(tensors)
         self.hidden_size = hidden_size
@@ -288,6 +290,20 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(dtype):
             got = H.run_trace(engine, seqs, steps)
             bad = H.first_wrong(got, want, H.TOL[dtype])
             assert bad is None, f"first wrong logits at (request, position, error) = {bad}"
+        # Graphs asked for: the mixer says that it cannot be captured (it indexes its state
+        # with host lists, which a replay would freeze), so the model's decode steps run
+        # eagerly and are right; the same model without that mixer's word would be captured.
+        assert not engine.model.graph_safe
+        graphed = H.lab.Engine(config=cfg, tensors=tensors.items(), dtype=dtype, page_size=16, num_pages=16,
+                               max_requests=3, max_batch_tokens=128, max_seq_len=256, graph=True)
+        three = {rid: seqs[rid] for rid in ("r0", "r1", "r3")}
+        steps = [([(rid, 12, True) for rid in three], [])]
+        steps += [([(rid, 1, True) for rid in three], []) for _ in range(30)]
+        got = H.run_trace(graphed, three, steps)
+        assert graphed.step_fn.use_graph is True
+        assert graphed.step_fn.graph_captures == 0 and graphed.step_fn.graph_replays == 0
+        for rid in three:
+            assert (got[rid][:42].double() - want[rid][:42]).abs().max() <= H.TOL[dtype]
     finally:
         unregister_part("mixer", "toy_running_mean")
         unregister_architecture("ToyForCausalLM")
@@ -448,3 +464,169 @@ def test_toy_routed_feed_forward_and_other_position_encoding(dtype):
         unregister_part("feed_forward", "toy_top_one_experts")
         unregister_part("position", "toy_half_rotary")
         unregister_architecture("Toy2ForCausalLM")
+
+
+# ------------------- toy embedding that reads positions, toy mixer with a cache of its own shape
+class PositionalEmbedding(Part):
+    """``x = table[id] + places[position]``: a learned table of absolute positions beside
+    the token table.  It needs the step's positions, which the embedding part is handed
+    with the step's description."""
+
+    def __init__(self, vocab_size, hidden_size, max_positions, tensors):
+        super().__init__(tensors)
+        self.vocab_size, self.hidden_size, self.max_positions = vocab_size, hidden_size, max_positions
+
+    def tensor_specs(self):
+        t = self.tensor_names
+        return {t["weight"]: TensorSpec((self.vocab_size, self.hidden_size), MATRIX),
+                t["places"]: TensorSpec((self.max_positions, self.hidden_size), MATRIX)}
+
+    def bind(self, tensors, ops, dtype):
+        super().bind(tensors, ops, dtype)
+        self.table = ops.prepare_weight(tensors[self.tensor_names["weight"]], shared=True)
+        self.places = tensors[self.tensor_names["places"]].float()
+
+    def forward(self, ids, out, ctx=None):
+        self.ops.embed(self.table, ids, out)
+        out += self.places[ctx.positions.long()]
+
+
+class LatentMixer(Mixer):
+    """A mixer that keeps ONE vector of width r per token (not keys and values): c = h Wc^T
+    goes to the cache, and the output at a token is ``(softmax(q . c_j / sqrt(r)) c) Wo^T``
+    over the tokens j up to it, with q = h Wq^T.  Its cache is a page tensor ``[P, r]`` under
+    the name "latent"; it finds pages through the group's block table like attention does."""
+
+    graph_safe = False
+
+    def __init__(self, hidden_size, latent_size, tensors):
+        super().__init__(tensors)
+        self.hidden_size, self.latent_size = hidden_size, latent_size
+
+    def tensor_specs(self):
+        t, h, r = self.tensor_names, self.hidden_size, self.latent_size
+        return {t["down"]: TensorSpec((r, h), MATRIX), t["query"]: TensorSpec((r, h), MATRIX),
+                t["up"]: TensorSpec((h, r), MATRIX)}
+
+    def bind(self, tensors, ops, dtype):
+        super().bind(tensors, ops, dtype)
+        t = self.tensor_names
+        self.w_down, self.w_query, self.w_up = (ops.prepare_weight(tensors[t[n]].contiguous())
+                                                for n in ("down", "query", "up"))
+
+    def cache_spec(self):
+        return CacheSpec((("latent", PageTensor((self.latent_size,), 0)),), window=None)
+
+    def forward(self, h, residual, ctx, entry):
+        rows, r = h.shape[0], self.latent_size
+        group = ctx.group(entry.group)
+        page = group.page_size
+        c = ctx.scratch("latent.c", (rows, r), self.dtype)
+        q = ctx.scratch("latent.q", (rows, r), self.dtype)
+        self.ops.linear(h, self.w_down, c)
+        self.ops.linear(h, self.w_query, q)
+        store = entry.cache["latent"]                                  # [pages, P, r]
+        pos = ctx.positions.long()
+        pages = group.block_table[ctx.row_req.long(), pos // page].long()
+        store[pages, pos % page] = c
+        mixed = torch.empty((rows, r), dtype=torch.float32, device=h.device)
+        for b in range(ctx.n_reqs):
+            r0, r1 = ctx.host_q_start[b], ctx.host_q_start[b + 1]
+            end = ctx.host_start_pos[b] + (r1 - r0)
+            used = group.block_table[b, :(end + page - 1) // page].long()
+            seen = store[used].reshape(-1, r)[:end].float()            # the request's latents, in order
+            scores = q[r0:r1].float() @ seen.t() / math.sqrt(r)
+            late = torch.arange(end, device=h.device)[None, :] > pos[r0:r1, None]
+            mixed[r0:r1] = torch.softmax(scores.masked_fill(late, float("-inf")), dim=-1) @ seen
+        self.ops.linear_residual(mixed.to(self.dtype), self.w_up, residual)
+
+
+@dataclasses.dataclass(frozen=True)
+class Toy3Config:
+    vocab_size: int
+    hidden_size: int
+    latent_size: int
+    max_positions: int
+    eps: float
+    architecture: str = "Toy3ForCausalLM"
+
+    @classmethod
+    def from_dict(cls, raw, where="config.json"):
+        return cls(*(raw[k] for k in ("vocab_size", "hidden_size", "latent_size", "max_positions", "eps")))
+
+    def to_dict(self):
+        return {"architectures": [self.architecture], **dataclasses.asdict(self)}
+
+
+def toy3_spec(cfg):
+    h = cfg.hidden_size
+    norm = lambda n: PartSpec("rmsnorm", dict(size=h, eps=cfg.eps), dict(weight=n))
+    def block(p):
+        return BlockSpec(
+            "prenorm",
+            mixer=PartSpec("toy_latent_mixer", dict(hidden_size=h, latent_size=cfg.latent_size),
+                           dict(down=p + "down", query=p + "query", up=p + "up")),
+            feed_forward=PartSpec("swiglu", dict(hidden_size=h, intermediate_size=2 * h),
+                                  dict(gate_weight=p + "gate", up_weight=p + "ffn_up", down_weight=p + "ffn_down")),
+            norm1=norm(p + "n1"), norm2=norm(p + "n2"), params=dict(hidden_size=h))
+    sizes = dict(vocab_size=cfg.vocab_size, hidden_size=h)
+    return ModelSpec("Toy3ForCausalLM", cfg.vocab_size, h, cfg.max_positions,
+                     PartSpec("toy_positional_embedding", dict(max_positions=cfg.max_positions, **sizes),
+                              dict(weight="embed", places="places")),
+                     (block("a."), block("b.")), (ScheduleEntry(0), ScheduleEntry(1)),
+                     norm("final"), PartSpec("linear_head", sizes, dict(weight="head")))
+
+
+def toy3_plain(ids, w, cfg):
+    t, r = len(ids), cfg.latent_size
+    x = w["embed"][torch.tensor(ids)] + w["places"][:t]
+    late = torch.arange(t)[None, :] > torch.arange(t)[:, None]
+    for p in ("a.", "b."):
+        n = P.rms_norm(x, w[p + "n1"], cfg.eps)
+        c, q = P.linear(n, w[p + "down"]), P.linear(n, w[p + "query"])
+        probs = torch.softmax((q @ c.t() / math.sqrt(r)).masked_fill(late, float("-inf")), dim=-1)
+        x = x + P.linear(probs @ c, w[p + "up"])
+        x = x + P.swiglu_mlp(P.rms_norm(x, w[p + "n2"], cfg.eps), w[p + "gate"], w[p + "ffn_up"], w[p + "ffn_down"])
+    return P.linear(P.rms_norm(x, w["final"], cfg.eps), w["head"])
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_toy_embedding_with_positions_and_mixer_with_a_cache_of_its_own_shape(dtype):
+    """An embedding that adds a learned vector per absolute position, and a mixer whose
+    per-token cache is one latent vector (a page tensor [P, r] by the name it chose, in a
+    group and with a block table of its own): registered, built and stepped in every cut,
+    with pages used again, without a change to the framework's files."""
+    register_part("embedding", "toy_positional_embedding", PositionalEmbedding, replace=True)
+    register_part("mixer", "toy_latent_mixer", LatentMixer, replace=True)
+    register_architecture("Toy3ForCausalLM", Toy3Config, toy3_spec, replace=True)
+    try:
+        cfg = Toy3Config(vocab_size=83, hidden_size=64, latent_size=24, max_positions=256, eps=1e-5)
+        from llm_inference_lab_amd.engine.model import CausalLM
+        from llm_inference_lab_amd.weights import random_tensors
+        tensors = dict(random_tensors(CausalLM(toy3_spec(cfg)).tensor_specs(), 7, torch.bfloat16,
+                                      is_norm=lambda n: n.endswith(("n1", "n2", "final"))))
+        for n in tensors:
+            if n in ("embed", "places") or n.endswith(("down", "query")) and "ffn" not in n:
+                tensors[n] = (tensors[n].float() * 8).to(torch.bfloat16)
+        engine = H.lab.Engine(config=cfg, tensors=tensors.items(), dtype=dtype, page_size=16, num_pages=14,
+                              max_requests=3, max_batch_tokens=128, max_seq_len=256)
+        groups, _ = engine.model.cache_layout()
+        assert len(groups) == 1 and groups[0].entries == [0, 1]
+        assert tuple(engine.cache.storage[0]["latent"].shape) == (2, 14, 16, 24)
+        assert engine.model.entries[1].cache["latent"].shape[0] == 14 and engine.model.entries[1].k_cache is None
+        g = torch.Generator().manual_seed(4)
+        seqs = {f"r{i}": torch.randint(0, 83, (n,), generator=g).tolist() for i, n in enumerate([45, 80, 23, 60])}
+        w64 = {k: v.double() for k, v in tensors.items()}
+        want = {rid: toy3_plain(ids, w64, cfg) for rid, ids in seqs.items()}
+        for steps in (H.steps_whole(seqs), H.steps_prefill_then_decode(seqs), H.steps_portions(seqs),
+                      H.steps_mixed(seqs, seed=2, max_live=3)):
+            got = H.run_trace(engine, seqs, steps)
+            bad = H.first_wrong(got, want, H.TOL[dtype])
+            assert bad is None, f"first wrong logits at (request, position, error) = {bad}"
+        engine.cache.check()
+        m = engine.cache.metrics()
+        assert m["rows_used"] == 0 and m["groups"][0]["pages_used"] == 0 and m["groups"][0]["pages_high_water"] >= 10
+    finally:
+        unregister_part("embedding", "toy_positional_embedding")
+        unregister_part("mixer", "toy_latent_mixer")
+        unregister_architecture("Toy3ForCausalLM")
