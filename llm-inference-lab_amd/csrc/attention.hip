@@ -706,9 +706,18 @@ __global__ __launch_bounds__(64 * MERGE_WAVES) void attention_merge_kernel(
 }
 
 // ------------------------------------------------------------ f32, scalar
-__global__ __launch_bounds__(64) void attention_f32_kernel(AttnArgs a) {
+// A block of NW waves per (token, head).  The waves take the chunks of 64 visible keys in
+// turn and merge at the end in LDS.  In a chunk every lane takes one key for the score
+// (q . k in 32 bits, the numbers of the head in order); the wave takes the chunk's maximum
+// and sum; for the values the lanes turn to the numbers of the head: lane c adds p_j v_j[c]
+// for the chunk's keys j, whose p_j, page and place go round by lane reads.
+template <int NW>
+__global__ __launch_bounds__(64 * NW) void attention_f32_kernel(AttnArgs a) {
+  constexpr int DPL = (D + 63) / 64;       // numbers of the head per lane
   __shared__ float qs[D];
-  const int lane = threadIdx.x;
+  __shared__ float s_m[NW], s_l[NW];
+  __shared__ float s_o[NW][D];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int t = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
   const int r0 = a.q_start[b], qlen = a.q_start[b + 1] - r0;
   if (t >= qlen) return;
@@ -719,39 +728,64 @@ __global__ __launch_bounds__(64) void attention_f32_kernel(AttnArgs a) {
   const float* q = (const float*)a.q + (size_t)(r0 + t) * a.q_stride + (size_t)h * D;
   const float* kc = (const float*)a.kc;
   const float* vc = (const float*)a.vc;
-  for (int dd = lane; dd < D; dd += 64) qs[dd] = q[dd];
+  for (int dd = threadIdx.x; dd < D; dd += 64 * NW) qs[dd] = q[dd];
   __syncthreads();
 
-  float o[D];
+  float o[DPL];
 #pragma unroll
-  for (int dd = 0; dd < D; ++dd) o[dd] = 0.f;
+  for (int i = 0; i < DPL; ++i) o[i] = 0.f;
   float m = NEG_INF, l = 0.f;
-  for (int j = lo + lane; j <= p; j += 64) {
-    const int page = a.table[(size_t)b * a.table_stride + (j >> a.page_shift)];
-    const int off = j & (P - 1);
+  for (int j0 = lo + 64 * wave; j0 <= p; j0 += 64 * NW) {
+    const int j = j0 + lane;
+    const bool valid = j <= p;
+    const int jc = valid ? j : p;           // clamped: read, weight 0
+    const int page = a.table[(size_t)b * a.table_stride + (jc >> a.page_shift)];
+    const int off = jc & (P - 1);
     const float* kp = kc + ((size_t)page * a.nkv + kvh) * P * D;
-    const float* vp = vc + ((size_t)page * a.nkv + kvh) * P * D;
     float dot = 0.f;
-#pragma unroll
+#pragma unroll 16
     for (int dd = 0; dd < D; ++dd) dot = fmaf(qs[dd], kp[kcache_index(off, dd, D)], dot);
-    const float s = dot * a.scale;
-    const float m_new = fmaxf(m, s);
-    const float alpha = expf(m - m_new);  // m = -inf on the first key: exp(-inf) = 0
-    const float pr = expf(s - m_new);
-    l = l * alpha + pr;
+    const float s = valid ? dot * a.scale : NEG_INF;
+    const float m_new = fmaxf(m, wave_max(s));        // the chunk's first key is always visible
+    const float alpha = expf(m - m_new);              // m = -inf before the first chunk: exp(-inf) = 0
+    const float pr = valid ? expf(s - m_new) : 0.f;
+    l = l * alpha + wave_sum(pr);
 #pragma unroll
-    for (int dd = 0; dd < D; ++dd) o[dd] = fmaf(pr, vp[vcache_index(off, dd, D)], o[dd] * alpha);
+    for (int i = 0; i < DPL; ++i) o[i] *= alpha;
     m = m_new;
+    const int count = min(64, p - j0 + 1);
+    for (int jj = 0; jj < count; ++jj) {
+      const float pj = __shfl(pr, jj, WAVE);
+      const int pg = __shfl(page, jj, WAVE), of = __shfl(off, jj, WAVE);
+      const float* vp = vc + ((size_t)pg * a.nkv + kvh) * P * D;
+#pragma unroll
+      for (int i = 0; i < DPL; ++i) {
+        const int dd = lane + 64 * i;
+        if (dd < D) o[i] = fmaf(pj, vp[vcache_index(of, dd, D)], o[i]);
+      }
+    }
   }
-  const float mmax = wave_max(m);
-  const float w = m == NEG_INF ? 0.f : expf(m - mmax);
-  const float ltot = wave_sum(l * w);
+  if (lane == 0) {
+    s_m[wave] = m;
+    s_l[wave] = l;
+  }
+#pragma unroll
+  for (int i = 0; i < DPL; ++i)
+    if (lane + 64 * i < D) s_o[wave][lane + 64 * i] = o[i];
+  __syncthreads();
+  float mmax = NEG_INF;
+#pragma unroll
+  for (int w = 0; w < NW; ++w) mmax = fmaxf(mmax, s_m[w]);
+  float ltot = 0.f;
+#pragma unroll
+  for (int w = 0; w < NW; ++w) ltot += s_m[w] == NEG_INF ? 0.f : s_l[w] * expf(s_m[w] - mmax);
   const float inv = ltot > 0.f ? 1.f / ltot : 0.f;
   float* dst = (float*)a.out + (size_t)(r0 + t) * a.out_stride + (size_t)h * D;
+  for (int dd = threadIdx.x; dd < D; dd += 64 * NW) {
+    float tot = 0.f;
 #pragma unroll
-  for (int dd = 0; dd < D; ++dd) {
-    const float tot = wave_sum(o[dd] * w);
-    if ((dd & 63) == lane) dst[dd] = tot * inv;
+    for (int w = 0; w < NW; ++w) tot += s_m[w] == NEG_INF ? 0.f : s_o[w][dd] * expf(s_m[w] - mmax);
+    dst[dd] = tot * inv;
   }
 }
 
@@ -760,9 +794,10 @@ extern "C" const char* llmlab_last_error() { return g_llmlab_error; }
 
 extern "C" int llmlab_attention_head_dim() { return D; }
 
-// Tests and tuning runs may fix the number of key splits (0: chosen here).
+// Debug interface (kernels/debug.py): the number of key splits can be fixed, for tests and
+// measurements (0: chosen here).
 static int g_force_splits = 0;
-extern "C" void llmlab_attention_force_splits(int splits) { g_force_splits = splits; }
+extern "C" void llmlab_debug_attention_splits(int splits) { g_force_splits = splits; }
 
 // The decode-like launch: a block of DECODE_WAVES waves per (request, kv head, split); a
 // wave gets about two steps of 32 keys, a block's waves merge in LDS, and only what is
@@ -846,8 +881,17 @@ extern "C" int llmlab_paged_attention(const void* q, int dtype, int q_stride, in
   a.qlen_lo = 0; a.qlen_hi = 0x7fffffff;
   while ((1 << a.page_shift) < page_size) ++a.page_shift;
   if (dtype == DT_F32) {
-    dim3 grid(max_q_len, nq, reqs), block(64);
-    hipLaunchKernelGGL(attention_f32_kernel, grid, block, 0, stream, a);
+    // waves per (token, head): as many as the longest history has chunks of 64 keys for, up
+    // to 16; four at most where the rows alone fill the chip
+    dim3 grid(max_q_len, nq, reqs);
+    const int chunks = (max_ctx_len + 63) / 64;
+    const bool many_rows = (long)total_rows * nq >= 8L * num_cus;
+    if (chunks <= 2)
+      hipLaunchKernelGGL(attention_f32_kernel<1>, grid, dim3(64), 0, stream, a);
+    else if (chunks <= 16 || many_rows)
+      hipLaunchKernelGGL(attention_f32_kernel<4>, grid, dim3(256), 0, stream, a);
+    else
+      hipLaunchKernelGGL(attention_f32_kernel<16>, grid, dim3(1024), 0, stream, a);
     LLMLAB_LAUNCH_CHECK("attention(float32)");
     return 0;
   }

@@ -97,12 +97,7 @@ __device__ __forceinline__ float sk_silu(float z) { return z / (1.f + __expf(-z)
 // ring of registers that is refilled slot by slot, so a wave always has R loads
 // in flight and never waits for all of them at once.  Measured at depths 4, 8 and
 // 12: no difference once the stream is continuous, so the shallow ring it is.
-#ifndef SK_RING_STAGE
-#define SK_RING_STAGE 4
-#endif
-#ifndef SK_RING_DIRECT
-#define SK_RING_DIRECT 4
-#endif
+constexpr int SK_RING_STAGE = 4, SK_RING_DIRECT = 4;
 __host__ __device__ constexpr int sk_ring(int mb, bool stage) {
   return stage ? SK_RING_STAGE : (mb >= 4 ? SK_RING_DIRECT / 2 : SK_RING_DIRECT);
 }
@@ -531,16 +526,17 @@ static int skinny_launch_stage(const SkinnyArgs& a, bool stage, int mb, int bloc
   }
 }
 
-// A choice of block shape can be forced for measurements (0 = choose).
+// Debug interface (kernels/debug.py): a block shape can be forced, for tests and
+// measurements (0 = choose).
 static int g_force_nsb = 0, g_force_kw = 0, g_force_stage = -1, g_force_mb = 0, g_force_epi = -1;
-extern "C" void llmlab_skinny_force(int nsb, int kw, int stage, int mb) {
+extern "C" void llmlab_debug_skinny_shape(int nsb, int kw, int stage, int mb) {
   g_force_nsb = nsb;
   g_force_kw = kw;
   g_force_stage = stage;
   g_force_mb = mb;
 }
 // ... for one epilogue only (-1: for all)
-extern "C" void llmlab_skinny_force_epilogue(int epilogue) { g_force_epi = epilogue; }
+extern "C" void llmlab_debug_skinny_epilogue(int epilogue) { g_force_epi = epilogue; }
 
 struct SkinnyShape {
   int nsb, kw;

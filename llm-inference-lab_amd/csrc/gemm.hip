@@ -19,8 +19,9 @@
 //       per product, one wave per SIMD: 833 against 793 TF/s on the largest product
 //       tried, slower on the rest).
 //     (products of few rows, as in decode steps, have kernels of their own in decode.hip)
-//   float32: a plain FMA kernel (64x64 tile, 4x4 outputs per thread): true 32-bit
-//     products and sums, no matrix-core shortcut.
+//   float32: a plain FMA kernel (tiles of 64x64 to 128x128, 4x4 to 8x8 outputs per thread) and, for up to 64
+//     rows, one in which a wave owns four rows of W and its lanes split the inner size:
+//     true 32-bit products and sums, no matrix-core shortcut.
 //
 // Fragment layout of the 16x16x32 MFMA (wave of 64 lanes, lane l):
 //   A operand: row l%16, k = 8*(l/16) .. +7      B operand: column l%16, same k
@@ -103,7 +104,6 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __
   // every die a band of neighbouring column tiles, rows running fastest, so that
   // what its blocks read at one time is a few column tiles of W and the rows of x.
   int bx = blockIdx.x, by = blockIdx.y;
-#ifndef GEMM_NO_REMAP
   {
     const int gx = gridDim.x, gy = gridDim.y, total = gx * gy;
     const int lin = by * gx + bx;
@@ -112,7 +112,6 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __
     bx = mapped / gy;
     by = mapped - bx * gy;
   }
-#endif
   const int m0 = by * BM, n0 = bx * BN;
   const int c = lane & 15, g = lane >> 4;
 
@@ -360,53 +359,84 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __
 }
 
 // ================================================================ float32
-// 64x64 outputs per block of 256 threads; thread (ty, tx) owns rows ty + 16*i and
-// columns tx + 16*j (i, j in 0..3), so for SWIGLU columns j = 0, 2 are gate and
-// j = 1, 3 the up values of the same outputs.
-template <int EPI>
+// BM x BN outputs per block of 256 threads (16 x 16); thread (ty, tx) owns the TM = BM/16
+// rows ty*TM + i and the TN = BN/16 columns tx + 16*j, so for SWIGLU columns j = 0, 2, ..
+// are gate and j = 1, 3, .. the up values of the same outputs.  K steps of 8 through LDS
+// (both operands transposed, so that a thread reads its TM rows as vectors); the next
+// step's numbers are on their way from memory while this one is multiplied.  Plain FMAs.
+template <int EPI, int BM, int BN>
 __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__ A,
                                                         const float* __restrict__ W, EpiArgs e, int M,
-                                                        int N, int K) {
-  constexpr int BK = 16;
-  __shared__ float As[BK][64 + 1];
-  __shared__ float Bs[BK][64 + 1];
+                                                        int N, int K, int vec) {
+  constexpr int BK = 8, TM = BM / 16, TN = BN / 16;
+  constexpr int LA = BM * BK / 256, LB = BN * BK / 256;      // numbers per thread and step: 2 or 4
+  __shared__ __attribute__((aligned(16))) float As[BK][BM + 4];
+  __shared__ __attribute__((aligned(16))) float Bs[BK][BN + 4];
   const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
-  const int m0 = blockIdx.y * 64, n0 = blockIdx.x * 64;
-  float acc[4][4];
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  float acc[TM][TN];
 #pragma unroll
-  for (int i = 0; i < 4; ++i)
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
-  const int lrow = tid >> 2, lk = (tid & 3) * 4;  // this thread loads 4 k values of one row
-  for (int k0 = 0; k0 < K; k0 += BK) {
+    for (int j = 0; j < TN; ++j) acc[i][j] = 0.f;
+  // a thread fetches LA (LB) consecutive k of one row of x (of W)
+  const int arow = tid / (BK / LA), ak = (tid % (BK / LA)) * LA;
+  const int brow = tid / (BK / LB), bk = (tid % (BK / LB)) * LB;
+  const float* ap = A + (size_t)min(m0 + arow, M - 1) * K;
+  const float* bp = W + (size_t)min(n0 + brow, N - 1) * K;
+  float ra[LA], rb[LB];
+  auto fetch = [&](int k0) {
+    if (vec && k0 + BK <= K) {
+      if constexpr (LA == 4) {
+        const floatx4 v = *(const floatx4*)(ap + k0 + ak);
+        ra[0] = v[0]; ra[1] = v[1]; ra[2] = v[2]; ra[3] = v[3];
+      } else {
+        ra[0] = ap[k0 + ak]; ra[1] = ap[k0 + ak + 1];
+      }
+      if constexpr (LB == 4) {
+        const floatx4 v = *(const floatx4*)(bp + k0 + bk);
+        rb[0] = v[0]; rb[1] = v[1]; rb[2] = v[2]; rb[3] = v[3];
+      } else {
+        rb[0] = bp[k0 + bk]; rb[1] = bp[k0 + bk + 1];
+      }
+    } else {
 #pragma unroll
-    for (int x = 0; x < 4; ++x) {
-      const int k = k0 + lk + x;
-      const int m = m0 + lrow, n = n0 + lrow;
-      As[lk + x][lrow] = (m < M && k < K) ? A[(size_t)m * K + k] : 0.f;
-      Bs[lk + x][lrow] = (n < N && k < K) ? W[(size_t)n * K + k] : 0.f;
+      for (int x = 0; x < LA; ++x) ra[x] = k0 + ak + x < K ? ap[k0 + ak + x] : 0.f;
+#pragma unroll
+      for (int x = 0; x < LB; ++x) rb[x] = k0 + bk + x < K ? bp[k0 + bk + x] : 0.f;
     }
+  };
+  fetch(0);
+  for (int k0 = 0; k0 < K; k0 += BK) {
     __syncthreads();
+#pragma unroll
+    for (int x = 0; x < LA; ++x) As[ak + x][arow] = ra[x];
+#pragma unroll
+    for (int x = 0; x < LB; ++x) Bs[bk + x][brow] = rb[x];
+    __syncthreads();
+    if (k0 + BK < K) fetch(k0 + BK);
 #pragma unroll
     for (int kk = 0; kk < BK; ++kk) {
-      float a[4], b[4];
+      float a[TM], b[TN];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) a[i] = As[kk][ty + 16 * i];
+      for (int i = 0; i < TM; i += 4) {
+        const floatx4 v = *(const floatx4*)&As[kk][ty * TM + i];
+        a[i] = v[0]; a[i + 1] = v[1]; a[i + 2] = v[2]; a[i + 3] = v[3];
+      }
 #pragma unroll
-      for (int j = 0; j < 4; ++j) b[j] = Bs[kk][tx + 16 * j];
+      for (int j = 0; j < TN; ++j) b[j] = Bs[kk][tx + 16 * j];
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int i = 0; i < TM; ++i)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+        for (int j = 0; j < TN; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
     }
-    __syncthreads();
   }
 #pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int m = m0 + ty + 16 * i;
+  for (int i = 0; i < TM; ++i) {
+    const int m = m0 + ty * TM + i;
     if (m >= M) continue;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < TN; ++j) {
       if constexpr (EPI == EPI_SWIGLU) {
         if (j & 1) continue;
         const int nb = n0 + 16 * j;
@@ -422,6 +452,125 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__
     }
   }
 }
+
+// The largest tile that still gives every compute unit a block.
+template <int EPI>
+static void launch_f32_tiled(const float* A, const float* W, const EpiArgs& e, int M, int N, int K,
+                             int num_cus, hipStream_t stream) {
+  const int vec = (K % 4 == 0) && ((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0);
+  auto blocks = [&](int bm, int bn) { return (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
+  if (blocks(128, 128) >= num_cus)
+    hipLaunchKernelGGL((gemm_f32_kernel<EPI, 128, 128>), dim3((N + 127) / 128, (M + 127) / 128), dim3(256), 0,
+                       stream, A, W, e, M, N, K, vec);
+  else if (blocks(128, 64) >= num_cus)
+    hipLaunchKernelGGL((gemm_f32_kernel<EPI, 128, 64>), dim3((N + 63) / 64, (M + 127) / 128), dim3(256), 0,
+                       stream, A, W, e, M, N, K, vec);
+  else
+    hipLaunchKernelGGL((gemm_f32_kernel<EPI, 64, 64>), dim3((N + 63) / 64, (M + 63) / 64), dim3(256), 0,
+                       stream, A, W, e, M, N, K, vec);
+}
+
+// Few rows in float32 (decode steps, short portions): one wave owns NB = 4 rows of W and
+// its lanes split the inner size, four numbers a lane and step, so that a wave instruction
+// reads 1 KB of a row of W in a row (any inner size: one number at a time where rows are
+// not 16-byte aligned).  MB rows of x go with them (they stay in the caches); the MB x NB
+// sums meet by lane shuffles.  For SWIGLU the four rows are two gate rows and the up rows
+// of the same two outputs.  Still plain FMAs in 32 bits.
+template <int EPI, int MB>
+__global__ __launch_bounds__(64) void gemm_f32_rows_kernel(const float* __restrict__ A,
+                                                            const float* __restrict__ W, EpiArgs e, int M,
+                                                            int N, int K, int vec) {
+  constexpr int NB = 4;
+  const int lane = threadIdx.x;
+  const int m0 = blockIdx.y * MB;
+  int rows_w[NB];
+  if constexpr (EPI == EPI_SWIGLU) {
+    const int n = (blockIdx.x >> 3) * 32 + (blockIdx.x & 7) * 2;     // two gate rows; their up rows 16 on
+    rows_w[0] = n; rows_w[1] = n + 1; rows_w[2] = n + 16; rows_w[3] = n + 17;
+  } else {
+#pragma unroll
+    for (int j = 0; j < NB; ++j) rows_w[j] = blockIdx.x * NB + j;
+  }
+  const float* wp[NB];
+  const float* xp[MB];
+#pragma unroll
+  for (int j = 0; j < NB; ++j) wp[j] = W + (size_t)min(rows_w[j], N - 1) * K;   // clamped: read, never stored
+#pragma unroll
+  for (int i = 0; i < MB; ++i) xp[i] = A + (size_t)min(m0 + i, M - 1) * K;
+  float acc[MB][NB];
+#pragma unroll
+  for (int i = 0; i < MB; ++i)
+#pragma unroll
+    for (int j = 0; j < NB; ++j) acc[i][j] = 0.f;
+  if (vec) {
+    for (int k = lane * 4; k < K; k += 256) {
+      floatx4 w4[NB], x4[MB];
+#pragma unroll
+      for (int j = 0; j < NB; ++j) w4[j] = *(const floatx4*)(wp[j] + k);
+#pragma unroll
+      for (int i = 0; i < MB; ++i) x4[i] = *(const floatx4*)(xp[i] + k);
+#pragma unroll
+      for (int i = 0; i < MB; ++i)
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+#pragma unroll
+          for (int c = 0; c < 4; ++c) acc[i][j] = fmaf(x4[i][c], w4[j][c], acc[i][j]);
+    }
+  } else {
+    for (int k = lane; k < K; k += 64) {
+      float w1[NB], x1[MB];
+#pragma unroll
+      for (int j = 0; j < NB; ++j) w1[j] = wp[j][k];
+#pragma unroll
+      for (int i = 0; i < MB; ++i) x1[i] = xp[i][k];
+#pragma unroll
+      for (int i = 0; i < MB; ++i)
+#pragma unroll
+        for (int j = 0; j < NB; ++j) acc[i][j] = fmaf(x1[i], w1[j], acc[i][j]);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < MB; ++i)
+#pragma unroll
+    for (int j = 0; j < NB; ++j) acc[i][j] = wave_sum(acc[i][j]);
+  if (lane != 0) return;
+#pragma unroll
+  for (int i = 0; i < MB; ++i) {
+    const int m = m0 + i;
+    if (m >= M) continue;
+    if constexpr (EPI == EPI_SWIGLU) {
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        const int o = (rows_w[j] >> 5) * 16 + (rows_w[j] & 15);
+        if (o < e.n_out) {
+          const float z = acc[i][j];
+          ((float*)e.out)[(size_t)m * e.ldo + o] = z / (1.f + expf(-z)) * acc[i][j + 2];
+        }
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < NB; ++j)
+        if (rows_w[j] < N) epi_store<float, EPI>(e, m, rows_w[j], acc[i][j]);
+    }
+  }
+}
+
+template <int EPI>
+static void launch_f32_rows(const float* A, const float* W, const EpiArgs& e, int M, int N, int K,
+                            hipStream_t stream) {
+  const int vec = (K % 4 == 0) && ((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0);
+  const unsigned groups = EPI == EPI_SWIGLU ? (unsigned)(N / 32) * 8 : (unsigned)((N + 3) / 4);
+  if (M == 1)
+    hipLaunchKernelGGL((gemm_f32_rows_kernel<EPI, 1>), dim3(groups, 1), dim3(64), 0, stream, A, W, e, M, N, K, vec);
+  else if (M == 2)
+    hipLaunchKernelGGL((gemm_f32_rows_kernel<EPI, 2>), dim3(groups, 1), dim3(64), 0, stream, A, W, e, M, N, K, vec);
+  else if (M <= 4)
+    hipLaunchKernelGGL((gemm_f32_rows_kernel<EPI, 4>), dim3(groups, 1), dim3(64), 0, stream, A, W, e, M, N, K, vec);
+  else
+    hipLaunchKernelGGL((gemm_f32_rows_kernel<EPI, 8>), dim3(groups, (M + 7) / 8), dim3(64), 0, stream, A, W, e, M, N,
+                       K, vec);
+}
+constexpr int F32_ROWS_MAX = 64;     // up to here the few-row kernel (the tiled one would run on N / 64 blocks)
 
 // ================================================================ dispatch
 // Three tile shapes, all with four waves, x through LDS and W straight from the packed
@@ -456,9 +605,10 @@ static double tile_cost(int kind, int M, int N, int K, int num_cus, int pieces) 
   return t.L + (compute > read ? compute : read);
 }
 
-// A tile can be forced for measurements (0 = choose; 64, 130 = 64 x 128, 129 = 128 x 128).
+// Debug interface (kernels/debug.py): a tile can be forced, for tests and measurements
+// (0 = choose; 64, 130 = 64 x 128, 129 = 128 x 128).
 static int g_force_tile = 0;
-extern "C" void llmlab_gemm_force(int tile) { g_force_tile = tile; }
+extern "C" void llmlab_debug_gemm_tile(int tile) { g_force_tile = tile; }
 
 static int choose_tile(int M, int N, int K, int num_cus) {
   if (g_force_tile == 64) return TILE_64;
@@ -616,14 +766,23 @@ extern "C" int llmlab_linear(const void* x, const void* w, int dtype, int epilog
       default: launch_tile<EPI_SWIGLU>(kind, A, W, e, M, N, K, 1, stream); break;
     }
   } else {
-    dim3 grid((N + 63) / 64, (M + 63) / 64), block(256);
     const float* A = (const float*)x;
     const float* W = (const float*)w;
+    if (M <= F32_ROWS_MAX) {
+      switch (epilogue) {
+        case EPI_STORE: launch_f32_rows<EPI_STORE>(A, W, e, M, N, K, stream); break;
+        case EPI_RESID: launch_f32_rows<EPI_RESID>(A, W, e, M, N, K, stream); break;
+        case EPI_F32: launch_f32_rows<EPI_F32>(A, W, e, M, N, K, stream); break;
+        default: launch_f32_rows<EPI_SWIGLU>(A, W, e, M, N, K, stream); break;
+      }
+      LLMLAB_LAUNCH_CHECK("linear(float32, few rows)");
+      return 0;
+    }
     switch (epilogue) {
-      case EPI_STORE: hipLaunchKernelGGL(gemm_f32_kernel<EPI_STORE>, grid, block, 0, stream, A, W, e, M, N, K); break;
-      case EPI_RESID: hipLaunchKernelGGL(gemm_f32_kernel<EPI_RESID>, grid, block, 0, stream, A, W, e, M, N, K); break;
-      case EPI_F32: hipLaunchKernelGGL(gemm_f32_kernel<EPI_F32>, grid, block, 0, stream, A, W, e, M, N, K); break;
-      default: hipLaunchKernelGGL(gemm_f32_kernel<EPI_SWIGLU>, grid, block, 0, stream, A, W, e, M, N, K); break;
+      case EPI_STORE: launch_f32_tiled<EPI_STORE>(A, W, e, M, N, K, num_cus, stream); break;
+      case EPI_RESID: launch_f32_tiled<EPI_RESID>(A, W, e, M, N, K, num_cus, stream); break;
+      case EPI_F32: launch_f32_tiled<EPI_F32>(A, W, e, M, N, K, num_cus, stream); break;
+      default: launch_f32_tiled<EPI_SWIGLU>(A, W, e, M, N, K, num_cus, stream); break;
     }
   }
   LLMLAB_LAUNCH_CHECK("linear");

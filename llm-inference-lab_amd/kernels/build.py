@@ -85,8 +85,7 @@ def _lib_name(kind: str, sources, defines) -> str:
 
 
 def _compile(kind: str, sources: Sequence[str], defines: Sequence[str], force: bool) -> str:
-    # extra -D flags for experiments (they are part of the library's name)
-    defines = tuple(defines) + tuple(os.environ.get("LLMLAB_EXTRA_DEFINES", "").split())
+    defines = tuple(defines)
     name = _lib_name(kind, sources, defines)
     if not force:
         for d in _search_dirs():

@@ -1,0 +1,94 @@
+"""The debug interface of the kernel set: the one place through which a choice that the
+kernels make for themselves can be fixed from outside.
+
+The product never calls it.  Tests do, to reach every kernel variant at small sizes (the
+chooser would pick one tile per size, tiny matrices would never be cut along their inner
+size), and measurements do, to compare variants.
+
+Two kinds of choices:
+
+* ``DispatchRules`` (``HipOps.rules``): the measured thresholds by which ``HipOps`` picks a
+  path from the shape of a product.  One object, every field with its product value and
+  what it was measured on.
+* forced kernel shapes (``HipOps.debug.force(...)``, a context manager that restores on
+  exit): the tile of the tiled products, the block shape of the few-row products, the
+  number of key splits of decode attention, the number of pieces of a product cut by the
+  tiled kernel.  These are process-wide switches inside the kernel libraries
+  (``llmlab_debug_*`` entry points), so two ``HipOps`` in one process share them.
+"""
+from __future__ import annotations
+
+import contextlib
+import dataclasses
+from typing import Optional, Tuple
+
+
+@dataclasses.dataclass
+class DispatchRules:
+    # Fused norm + product kernels beyond one tile of 16 rows: only while the matrix, read
+    # once per tile of rows, stays below this many bytes in all (else norm + tiled product
+    # wins: 64 rows of a 55 MB matrix take 38 us fused, 26 us in two kernels).
+    fuse_read_bytes: float = 128e6
+    # From 17 rows on, a matrix of this many bytes that adds into the stream is cut along its
+    # inner size by the tiled kernel: the few-row kernel reads it once per tile of 16 rows
+    # (64 rows of 3584 x 18944: 89 us against 34; of 1536 x 8960: 25 against 13).
+    tiled_pieces_bytes: float = 16e6
+    # Pieces beyond this many bytes are folded once by the norm kernel instead of being
+    # added on the fly by every block of a fused kernel (32 rows of width 3584 in 7 pieces,
+    # 3.2 MB: 12 us a layer more in the fused kernels).
+    pieces_per_block_bytes: int = 1 << 20
+    # A piece of a few-row product has at least this many K steps of 32 ...
+    min_steps_per_split: int = 8
+    # ... and of a many-row product this many K tiles of 64.
+    min_tiles_per_split: int = 8
+    # q/k/v of this many rows up to 64 goes through pieces when the matrix is a large one
+    # (64 rows of 7168 x 5120: 26 us against 52 with a head per block; slower below 24 rows).
+    qkv_pieces_min_rows: int = 24
+    # Debug only: a product that the tiled kernel cuts gets this many pieces whatever the
+    # estimate says (0: the estimate decides).
+    forced_tiled_pieces: int = 0
+
+
+class KernelDebug:
+    def __init__(self, ops):
+        self._ops = ops
+
+    @contextlib.contextmanager
+    def force(self, *, gemm_tile: Optional[int] = None,
+              skinny_shape: Optional[Tuple[int, int, int, int]] = None,
+              skinny_epilogue: Optional[int] = None,
+              attention_splits: Optional[Tuple[int, int]] = None, **rules):
+        """``gemm_tile``: 64 (64 x 64), 130 (64 x 128) or 129 (128 x 128).  ``skinny_shape``:
+        (strips per block, K slices, staged rows 0/1 or -1, rows per tile) of the few-row
+        product kernel, 0 = chosen by the kernel.  ``skinny_epilogue``: the force holds for
+        this epilogue only.  ``attention_splits``: (head size, key splits of the decode
+        launch).  Other keywords: fields of ``DispatchRules`` for the time of the block."""
+        ops = self._ops
+        core = ops._core
+        saved = dataclasses.replace(ops.rules)
+        for key, value in rules.items():
+            if not hasattr(ops.rules, key):
+                raise TypeError(f"no dispatch rule named '{key}'")
+            setattr(ops.rules, key, value)
+        lib = None
+        try:
+            if gemm_tile is not None:
+                core.llmlab_debug_gemm_tile(int(gemm_tile))
+            if skinny_shape is not None:
+                core.llmlab_debug_skinny_shape(*[int(v) for v in skinny_shape])
+            if skinny_epilogue is not None:
+                core.llmlab_debug_skinny_epilogue(int(skinny_epilogue))
+            if attention_splits is not None:
+                lib = ops._attention_lib(int(attention_splits[0]))
+                lib.llmlab_debug_attention_splits(int(attention_splits[1]))
+            yield ops
+        finally:
+            ops.rules = saved
+            if gemm_tile is not None:
+                core.llmlab_debug_gemm_tile(0)
+            if skinny_shape is not None:
+                core.llmlab_debug_skinny_shape(0, 0, -1, 0)
+            if skinny_epilogue is not None:
+                core.llmlab_debug_skinny_epilogue(-1)
+            if lib is not None:
+                lib.llmlab_debug_attention_splits(0)

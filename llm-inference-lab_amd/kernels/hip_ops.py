@@ -17,6 +17,7 @@ import torch
 from ..config.errors import UnsupportedSizeError
 from ..parts.base import PendingSums
 from . import build
+from .debug import DispatchRules, KernelDebug
 
 DT_F32, DT_BF16 = 0, 1
 EPI_STORE, EPI_RESID, EPI_F32, EPI_SWIGLU, EPI_QKV, EPI_PART = 0, 1, 2, 3, 4, 5
@@ -88,6 +89,8 @@ class HipOps:
         self.workspace = torch.empty(self.WORKSPACE_FLOATS, dtype=torch.float32, device=self.device)
         self.loaded_libraries = [self._core._name]
         self.calls_made = 0          # calls into the kernel libraries so far
+        self.rules = DispatchRules()         # the measured thresholds of the dispatch, in one place
+        self.debug = KernelDebug(self)       # forcing kernel choices from outside (tests, measurements)
 
     # ---------------------------------------------------------------- loading
     @staticmethod
@@ -371,9 +374,6 @@ class HipOps:
     skinny_max_rows = 64          # plain products up to here may take the few-row kernel
     fuse_max_rows = 64            # steps up to here may take the fused kernels
     FUSE_TILE_ROWS = 16           # the few-row kernels cut the rows into tiles of so many
-    FUSE_READ_BYTES = 128e6       # beyond 16 rows: only while the matrix, read once per tile of 16
-                                  # rows, stays below this in all (else norm + tiled product wins:
-                                  # 64 rows of a 55 MB matrix 38 us fused, 26 us in two kernels)
     STAGE_BYTES = 118 * 1024      # most LDS the staged rows of a fused kernel may take
 
     def can_fuse(self, rows: int, dtype, inner: int, outer: Optional[int] = None) -> bool:
@@ -383,7 +383,7 @@ class HipOps:
         if dtype != torch.bfloat16 or not 0 < rows <= self.fuse_max_rows:
             return False
         tiles = (rows + self.FUSE_TILE_ROWS - 1) // self.FUSE_TILE_ROWS
-        if tiles > 1 and (outer is None or 2.0 * outer * inner * tiles >= self.FUSE_READ_BYTES):
+        if tiles > 1 and (outer is None or 2.0 * outer * inner * tiles >= self.rules.fuse_read_bytes):
             return False
         return min(rows, self.FUSE_TILE_ROWS) * ((inner + 31) // 32 * 32 + 8) * 2 <= self.STAGE_BYTES
 
@@ -415,15 +415,7 @@ class HipOps:
 
     # --------------------------------------------- sums left in pieces (deferred)
     MAX_SPLITS = 8
-    split_max_rows = 32           # most rows of a product that is left in pieces
-    min_steps_per_split = 8       # K steps of 32 a piece should have at least (tests lower it)
-    min_tiles_per_split = 8       # many rows: K tiles of 64 a piece should have at least
-    force_tiled_pieces = 0        # many rows: this many pieces whatever the estimate says (tests)
-    TILED_PIECES_BYTES = 16e6     # from 17 rows on, a matrix of this size is cut by the tiled kernel:
-                                  # the few-row kernel reads it once per tile of 16 rows (64 rows of
-                                  # 3584 x 18944: 89 us against 34; of 1536 x 8960: 25 against 13)
-
-    PIECES_PER_BLOCK_BYTES = 1 << 20
+    split_max_rows = 32           # most rows of a few-row product that is left in pieces
 
     def pieces_too_large_to_read_per_block(self, pending: Optional[PendingSums]) -> bool:
         """A fused kernel that takes pieces on adds them as it reads the rows, in every one
@@ -432,11 +424,11 @@ class HipOps:
         if pending is None:
             return False
         p = pending.parts
-        return pending.splits * p.shape[1] * p.shape[2] * 4 > self.PIECES_PER_BLOCK_BYTES
+        return pending.splits * p.shape[1] * p.shape[2] * 4 > self.rules.pieces_per_block_bytes
 
     def pieces_by_tiles(self, rows: int, n: int, k: int) -> bool:
         """Whether a product left in pieces is cut by the tiled kernel (else by the few-row one)."""
-        return rows > self.FUSED_MAX_ROWS or (rows > self.FUSE_TILE_ROWS and 2.0 * n * k >= self.TILED_PIECES_BYTES)
+        return rows > self.FUSED_MAX_ROWS or (rows > self.FUSE_TILE_ROWS and 2.0 * n * k >= self.rules.tiled_pieces_bytes)
 
     def split_count(self, rows: int, dtype, n: int, k: int) -> int:
         """Into how many pieces along the inner size a few-row product ``[rows, k] x
@@ -450,19 +442,19 @@ class HipOps:
             # the K tiles of a block, plus a write and a read of the result for every piece)
             if k % 8:
                 return 1
-            if self.force_tiled_pieces:         # (tests: tiny products would never be cut)
-                return max(1, min(self.force_tiled_pieces, (k + 63) // 64, self.MAX_SPLITS))
+            if self.rules.forced_tiled_pieces:
+                return max(1, min(self.rules.forced_tiled_pieces, (k + 63) // 64, self.MAX_SPLITS))
             return self._linear_plan(rows, n, k)[0]
         if rows > self.split_max_rows:
             return 1
         strips, steps = (n + 15) // 16, (k + 31) // 32
         want = self.num_cus // max(strips, 1)
-        return max(1, min(want, steps // self.min_steps_per_split, self.MAX_SPLITS))
+        return max(1, min(want, steps // self.rules.min_steps_per_split, self.MAX_SPLITS))
 
     def _linear_plan(self, rows: int, n: int, k: int):
         """(pieces, tile) for a many-row product that adds into float32 rows."""
         out = (_c_int * 2)()
-        self._core.llmlab_linear_plan(rows, n, k, self.num_cus, self.MAX_SPLITS, self.min_tiles_per_split, out)
+        self._core.llmlab_linear_plan(rows, n, k, self.num_cus, self.MAX_SPLITS, self.rules.min_tiles_per_split, out)
         return out[0], out[1]
 
     def linear_partials(self, x, w, parts: torch.Tensor, splits: int, bias=None) -> PendingSums:
@@ -560,7 +552,6 @@ class HipOps:
                           nkv=num_kv_heads, d=head_dim), pending=pending)
 
     QKV_ROPE_MAX_ROWS = 64        # up to here the few-row kernel, beyond it the tiled one
-    QKV_PIECES_MIN_ROWS = 24      # from here to QKV_ROPE_MAX_ROWS a large matrix goes through pieces
 
     def can_fuse_qkv_rope(self, rows: int, dtype, head_dim: int, n: Optional[int] = None,
                           k: Optional[int] = None) -> bool:
@@ -586,14 +577,14 @@ class HipOps:
             raise ValueError(f"qkv_rope_cache: {rows} rows of {k}, heads of {head_dim} do not fit")
         self._qkv_checks("qkv_rope_cache", rows, w_qkv, b_qkv, num_heads, num_kv_heads, head_dim,
                          inv_freq, positions, row_req, block_table, page_size, k_cache, v_cache, q_out)
-        if self.QKV_PIECES_MIN_ROWS <= rows <= self.QKV_ROPE_MAX_ROWS and self.pieces_by_tiles(rows, n, k):
+        if self.rules.qkv_pieces_min_rows <= rows <= self.QKV_ROPE_MAX_ROWS and self.pieces_by_tiles(rows, n, k):
             # some rows of a large matrix: a head per block leaves most of the chip idle, so
             # the product is cut along K by the tiled kernel and a second kernel sums the
             # pieces, rotates and writes the cache (64 rows of 7168 x 5120: 26 us against 52
             # in one kernel, of 4608 x 3584: 19 against 24; the same at 24 rows, slower below)
             pieces, tile = self._linear_plan(rows, n, k)
-            if self.force_tiled_pieces:
-                pieces = max(1, min(self.force_tiled_pieces, (k + 63) // 64, self.MAX_SPLITS))
+            if self.rules.forced_tiled_pieces:
+                pieces = max(1, min(self.rules.forced_tiled_pieces, (k + 63) // 64, self.MAX_SPLITS))
             if pieces > 1 and pieces * rows * n <= self.workspace.numel():
                 if b_qkv is not None:
                     self._need(b_qkv, "bias")

@@ -22,6 +22,8 @@ class EmuOps:
         self.device = torch.device(device)
         self.calls = {}
         self.fuse = fuse
+        import types
+        self.rules = types.SimpleNamespace(min_steps_per_split=8)
 
     def _count(self, name):
         self.calls[name] = self.calls.get(name, 0) + 1
@@ -74,7 +76,6 @@ class EmuOps:
     # ---------------------------------------------------- sums left in pieces
     MAX_SPLITS = 8
     num_cus = 256
-    min_steps_per_split = 8
 
     @staticmethod
     def _owed(pending):
@@ -84,7 +85,7 @@ class EmuOps:
         if not self.fuse or dtype != torch.bfloat16 or not 0 < rows <= 64:
             return 1
         strips, steps = (n + 15) // 16, (k + 31) // 32
-        return max(1, min(self.num_cus // max(strips, 1), steps // self.min_steps_per_split, self.MAX_SPLITS))
+        return max(1, min(self.num_cus // max(strips, 1), steps // self.rules.min_steps_per_split, self.MAX_SPLITS))
 
     def linear_partials(self, x, w, parts, splits, bias=None):
         """Piece s covers the K steps from s * ceil(steps / splits) on; a step is 32 wide

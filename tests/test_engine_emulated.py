@@ -67,7 +67,7 @@ def test_sums_left_in_pieces_reach_every_reader(name, cut):
     seqs = sequences_of(name)
     want = {rid: H.plain_logits(name, 1, ids) for rid, ids in seqs.items()}
     engine = engine_of(name, "bf16", page_size=16, num_pages=14, max_requests=4)
-    engine.ops.min_steps_per_split = 1
+    engine.ops.rules.min_steps_per_split = 1
     steps = {"decode": H.steps_prefill_then_decode, "mixed": H.steps_mixed}[cut](seqs)
     got = H.run_trace(engine, seqs, steps)
     bad = H.first_wrong(got, want, H.TOL["bf16"])

@@ -82,7 +82,7 @@ def test_sums_left_in_pieces_reach_every_reader(name, cut):
     seqs = sequences_of(name)
     want = {rid: H.plain_logits(name, 1, ids) for rid, ids in seqs.items()}
     engine = H.make_engine(name, 1, "bf16", page_size=16, num_pages=40, max_requests=4)
-    engine.ops.min_steps_per_split = 1
+    engine.ops.rules.min_steps_per_split = 1
     cfg = H.config_of(name)
     assert engine.ops.split_count(4, torch.bfloat16, cfg.hidden_size, cfg.intermediate_size) > 1
     got = H.run_trace(engine, seqs, CUTS[cut](seqs))
@@ -102,10 +102,10 @@ def test_sums_of_many_rows_left_in_pieces(name, cut, from_rows):
     seqs = sequences_of(name)
     want = {rid: H.plain_logits(name, 1, ids) for rid, ids in seqs.items()}
     engine = H.make_engine(name, 1, "bf16", page_size=16, num_pages=40, max_requests=4)
-    engine.ops.force_tiled_pieces = 2
+    engine.ops.rules.forced_tiled_pieces = 2
     cfg = H.config_of(name)
     if from_rows == 17:
-        engine.ops.TILED_PIECES_BYTES = 0
+        engine.ops.rules.tiled_pieces_bytes = 0
         assert engine.ops.split_count(17, torch.bfloat16, cfg.hidden_size, cfg.intermediate_size) == 2
     assert engine.ops.split_count(130, torch.bfloat16, cfg.hidden_size, cfg.intermediate_size) > 1
     got = H.run_trace(engine, seqs, CUTS[cut](seqs))
@@ -244,7 +244,7 @@ def test_many_decoding_requests_with_products_in_pieces(graph):
     engine = H.make_engine("R", 1, "bf16", page_size=64, num_pages=30, max_requests=32, max_batch_tokens=512,
                            graph=graph)
     ops = engine.ops
-    ops.TILED_PIECES_BYTES, ops.force_tiled_pieces, ops.PIECES_PER_BLOCK_BYTES = 0, 2, 1 << 16
+    ops.rules.tiled_pieces_bytes, ops.rules.forced_tiled_pieces, ops.rules.pieces_per_block_bytes = 0, 2, 1 << 16
     assert ops.pieces_by_tiles(26, cfg.hidden_size, cfg.intermediate_size)
     assert ops.split_count(26, torch.bfloat16, cfg.hidden_size, cfg.intermediate_size) == 2
     steps = [([(rid, 19, True) for rid in seqs], [])]

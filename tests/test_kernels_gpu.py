@@ -132,8 +132,7 @@ def test_every_tile_shape_of_the_tiled_products(ops, emu, tile, m, n, k):
     in all three dimensions (the chooser would pick only one of them per size)."""
     from llm_inference_lab_amd.parts.feed_forward import interleave_gate_up
     bf = torch.bfloat16
-    ops._core.llmlab_gemm_force(tile)
-    try:
+    with ops.debug.force(gemm_tile=tile):
         x, w, bias = rnd((m, k), bf, 5), rnd((n, k), bf, 6, 0.1), rnd((n,), torch.float32, 7)
         pw = ops.prepare_weight(w.to(DEV))
         want = torch.empty(m, n, dtype=bf)
@@ -163,8 +162,6 @@ def test_every_tile_shape_of_the_tiled_products(ops, emu, tile, m, n, k):
         ops.linear_partials(x.to(DEV), pw, parts, 3)
         whole = x.float() @ w.float().t()
         close(parts.sum(0), whole, torch.float32, "pieces", whole.abs().max().item())
-    finally:
-        ops._core.llmlab_gemm_force(0)
 
 
 def test_linear_reference_vectors(ops):
@@ -253,15 +250,13 @@ def test_few_row_products_in_every_block_shape(ops, emu, nsb, kw, stage, mb):
         xd, wd, gd = x.to(DEV), ops.prepare_weight(w.to(DEV)), ops.prepare_weight(gate_up.to(DEV))
         def forced(fn):
             """Runs fn under the forced shape; False if the kernel refused the shape."""
-            ops._core.llmlab_skinny_force(nsb, kw, stage, mb)
             try:
-                fn()
+                with ops.debug.force(skinny_shape=(nsb, kw, stage, mb)):
+                    fn()
                 return True
             except KernelError as err:
                 assert "does not fit" in str(err) or "no block shape" in str(err), err
                 return False
-            finally:
-                ops._core.llmlab_skinny_force(0, 0, -1, 0)
 
         got = torch.full((m, n), float("nan"), dtype=dtype, device=DEV)
         if forced(lambda: ops.linear(xd, wd, got, bias.to(DEV))):
@@ -345,12 +340,9 @@ def test_fused_norm_qkv_rope_write(ops, emu, nq, nkv, d, page, hidden, rotate, r
                                                  (8, 8, 128, 64, 256), (2, 1, 256, 16, 64)])
 @pytest.mark.parametrize("rows_per", [[5, 1, 9], [20, 1, 1, 3], [17, 30, 16], [70, 1, 130], [300, 2, 2, 90]])
 def test_qkv_rope_cache_of_normed_rows(ops, emu, nq, nkv, d, page, hidden, rows_per):
-    if d == 128 and sum(rows_per) > 64:
-        ops._core.llmlab_gemm_force(128)      # the large tile, which this few rows would not get
-    try:
+    # (heads of 128: the large tile, which this few rows would not get)
+    with ops.debug.force(gemm_tile=128 if d == 128 and sum(rows_per) > 64 else 0):
         check_qkv_rope_cache(ops, emu, nq, nkv, d, page, hidden, rows_per)
-    finally:
-        ops._core.llmlab_gemm_force(0)
 
 
 @pytest.mark.parametrize("nq,nkv,d,page,hidden", [(4, 2, 16, 16, 64), (14, 2, 64, 64, 896), (6, 3, 48, 16, 72),
@@ -361,12 +353,11 @@ def test_qkv_rope_cache_through_pieces(ops, emu, nq, nkv, d, page, hidden, rows_
     """17 to 64 rows of a large matrix: the product is cut along its inner size and a second
     kernel sums the pieces, adds the bias, rotates and writes the cache.  The small
     matrices of the test take that way with the size limit taken away."""
-    ops.TILED_PIECES_BYTES, ops.force_tiled_pieces = 0, pieces
-    try:
-        assert ops.pieces_by_tiles(sum(rows_per), (nq + 2 * nkv) * d, hidden) and sum(rows_per) >= ops.QKV_PIECES_MIN_ROWS
+    with ops.debug.force(tiled_pieces_bytes=0, forced_tiled_pieces=pieces):
+        assert ops.pieces_by_tiles(sum(rows_per), (nq + 2 * nkv) * d, hidden)
+        assert sum(rows_per) >= ops.rules.qkv_pieces_min_rows
         check_qkv_rope_cache(ops, emu, nq, nkv, d, page, hidden, rows_per)
-    finally:
-        del ops.TILED_PIECES_BYTES, ops.force_tiled_pieces
+    assert ops.rules.forced_tiled_pieces == 0 and ops.rules.tiled_pieces_bytes == 16e6
 
 
 def check_qkv_rope_cache(ops, emu, nq, nkv, d, page, hidden, rows_per):
@@ -600,13 +591,9 @@ def test_attention_merge_of_any_number_of_splits(ops, emu, splits):
     four waves more, a lane holds the weights of two; splits past the end of a short
     history have no keys at all and must count for nothing."""
     for d, length in ((64, 700), (128, 3000), (48, 90)):
-        lib = ops._attention_lib(d)
-        lib.llmlab_attention_force_splits(splits)
-        try:
+        with ops.debug.force(attention_splits=(d, splits)):
             run_attention(ops, emu, torch.bfloat16, 6, 2, d, 16, None, [(length - 1, 1), (40, 1), (length // 2, 2)],
                           seed=96, amplify=(0, length // 3, 30.0))
-        finally:
-            lib.llmlab_attention_force_splits(0)
 
 
 @pytest.mark.parametrize("vocab", [1, 255, 256, 257, 4095, 4097, 151936])

@@ -73,7 +73,7 @@ def assert_large_matrix_rules_fire(ops, cfg):
     # ... the fused norm + product kernels stop at one tile of rows ...
     assert ops.can_fuse(8, bf, h, qkv) and not ops.can_fuse(26, bf, h, 2 * inter) and not ops.can_fuse(64, bf, h, qkv)
     # ... q/k/v of 24 to 64 rows goes through pieces, of more rows through the tiled epilogue
-    assert ops.QKV_PIECES_MIN_ROWS <= 26 <= ops.QKV_ROPE_MAX_ROWS and ops.pieces_by_tiles(26, qkv, h)
+    assert ops.rules.qkv_pieces_min_rows <= 26 <= ops.QKV_ROPE_MAX_ROWS and ops.pieces_by_tiles(26, qkv, h)
     assert ops._linear_plan(26, qkv, h)[0] > 1 and ops._linear_plan(64, qkv, h)[0] > 1
     # (a head of 128 needs the 128-wide tile for that; steps whose product gets the 64-wide
     # one take the product, then the kernel that rotates and writes the cache)
