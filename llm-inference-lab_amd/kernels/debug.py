@@ -41,6 +41,10 @@ class DispatchRules:
     min_steps_per_split: int = 8
     # ... and of a many-row product this many K tiles of 64.
     min_tiles_per_split: int = 8
+    # A few-row product of more strips than compute units is cut along its inner size when
+    # the last round of its blocks would leave the chip this much slower than even rounds
+    # (1.25 rounds of blocks take the time of 2: a waste of 1.6).
+    uneven_rounds_waste: float = 1.3
     # q/k/v of this many rows up to 64 goes through pieces when the matrix is a large one
     # (64 rows of 7168 x 5120: 26 us against 52 with a head per block; slower below 24 rows).
     qkv_pieces_min_rows: int = 24
