@@ -798,6 +798,11 @@ extern "C" int llmlab_attention_head_dim() { return D; }
 // measurements (0: chosen here).
 static int g_force_splits = 0;
 extern "C" void llmlab_debug_attention_splits(int splits) { g_force_splits = splits; }
+// ... and the launch that steps of many rows take: 1 = the waves of a block split the keys of
+// a tile of 32 rows, 2 = tiles of 32 rows per wave, 3 = late and early tiles in pairs,
+// 4 = tiles of 16 rows per wave (0: chosen here).
+static int g_force_path = 0;
+extern "C" void llmlab_debug_attention_path(int path) { g_force_path = path; }
 
 // The decode-like launch: a block of DECODE_WAVES waves per (request, kv head, split); a
 // wave gets about two steps of 32 keys, a block's waves merge in LDS, and only what is
@@ -919,7 +924,7 @@ extern "C" int llmlab_paged_attention(const void* q, int dtype, int q_stride, in
   // that the work still spreads over the chip.  Else every wave owns its rows and
   // the block's waves share the keys through LDS.
   const long blocks16 = ((max_rows + 63) / 64) * nkv * live;
-  if (blocks16 < num_cus) {
+  if (g_force_path == 1 || (g_force_path == 0 && blocks16 < num_cus)) {
     const int steps32 = (max_ctx_len + 31) / 32 + 1;
     const int steps_per_wave = (steps32 + DECODE_WAVES - 1) / DECODE_WAVES;
     dim3 grid((unsigned)((max_rows + 31) / 32), nkv, reqs), block(64 * DECODE_WAVES);
@@ -933,10 +938,11 @@ extern "C" int llmlab_paged_attention(const void* q, int dtype, int q_stride, in
   // rows per wave: 32 when that still gives every compute unit two blocks (or for
   // nothing smaller), else 16; always 16 for the largest heads (registers)
   const long blocks32 = ((max_rows + 127) / 128) * nkv * live;
-  if (D <= 128 && blocks32 >= 2L * num_cus) {
+  if (g_force_path == 2 || (g_force_path == 0 && D <= 128 && blocks32 >= 2L * num_cus)) {
     dim3 grid((unsigned)((max_rows + 127) / 128), nkv, reqs), block(256);
     hipLaunchKernelGGL((attention_bf16_kernel<2, false>), grid, block, 0, stream, a);
-  } else if (window <= 0 && blocks16 >= (3L * num_cus) / 2 && 16L * (max_ctx_len - max_q_len) <= max_q_len) {
+  } else if (g_force_path == 3 || (g_force_path == 0 && window <= 0 && blocks16 >= (3L * num_cus) / 2 &&
+                                   16L * (max_ctx_len - max_q_len) <= max_q_len)) {
     // not enough tiles to keep every unit busy with what the longest ones leave over:
     // pair late and early tiles (no window: then the loads add up evenly).  Only at the
     // start of a prompt: behind a history all tiles carry about the same load, and the

@@ -61,12 +61,16 @@ class KernelDebug:
     def force(self, *, gemm_tile: Optional[int] = None,
               skinny_shape: Optional[Tuple[int, int, int, int]] = None,
               skinny_epilogue: Optional[int] = None,
-              attention_splits: Optional[Tuple[int, int]] = None, **rules):
+              attention_splits: Optional[Tuple[int, int]] = None,
+              attention_path: Optional[Tuple[int, int]] = None, **rules):
         """``gemm_tile``: 64 (64 x 64), 130 (64 x 128) or 129 (128 x 128).  ``skinny_shape``:
         (strips per block, K slices, staged rows 0/1 or -1, rows per tile) of the few-row
         product kernel, 0 = chosen by the kernel.  ``skinny_epilogue``: the force holds for
         this epilogue only.  ``attention_splits``: (head size, key splits of the decode
-        launch).  Other keywords: fields of ``DispatchRules`` for the time of the block."""
+        launch).  ``attention_path``: (head size, launch of a step of many rows: 1 = the waves of a
+        block split the keys of a tile of 32 rows, 2 = tiles of 32 rows per wave, 3 = late and
+        early tiles in pairs, 4 = tiles of 16 rows per wave).  Other keywords: fields of
+        ``DispatchRules`` for the time of the block."""
         ops = self._ops
         core = ops._core
         saved = dataclasses.replace(ops.rules)
@@ -74,8 +78,11 @@ class KernelDebug:
             if not hasattr(ops.rules, key):
                 raise TypeError(f"no dispatch rule named '{key}'")
             setattr(ops.rules, key, value)
-        lib = None
+        lib = plib = None
         try:
+            if attention_path is not None:
+                plib = ops._attention_lib(int(attention_path[0]))
+                plib.llmlab_debug_attention_path(int(attention_path[1]))
             if gemm_tile is not None:
                 core.llmlab_debug_gemm_tile(int(gemm_tile))
             if skinny_shape is not None:
@@ -96,3 +103,5 @@ class KernelDebug:
                 core.llmlab_debug_skinny_epilogue(-1)
             if lib is not None:
                 lib.llmlab_debug_attention_splits(0)
+            if plib is not None:
+                plib.llmlab_debug_attention_path(0)
