@@ -218,7 +218,7 @@ class Runs:
         limit = 1e-3 if self.dtype == "f32" else 0.5
         prompts = [self.random_ids(n) for n in (5, 130, 700)]
         first = engine.generate(prompts, max_new_tokens=12, eos_token_id=[])
-        second = engine.generate(prompts, max_new_tokens=12, eos_token_id=[], max_batch_tokens=256)
+        second = engine.generate(prompts, max_new_tokens=12, eos_token_id=[])      # pages and rows used again
         after = engine.cache.metrics()
         for m in (initial, after):
             for g in m["groups"]:

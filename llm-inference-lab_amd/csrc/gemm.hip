@@ -115,6 +115,26 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __
   const int m0 = by * BM, n0 = bx * BN;
   const int c = lane & 15, g = lane >> 4;
 
+  // QKV: what the epilogue needs from global memory per row of the tile (position, and the
+  // page of that position for the tiles that hold k or v heads) and per column (bias,
+  // rotary frequencies) is fetched now, so that those round trips (the page follows the
+  // position follows the request) pass behind the product instead of after it.
+  constexpr bool QKV = EPI == EPI_QKV;
+  __shared__ int s_pos[QKV ? BM : 1], s_page[QKV ? BM : 1];
+  __shared__ float s_freq[QKV ? 128 : 1], s_bias[QKV ? BN : 1];
+  if constexpr (QKV) {
+    if (tid < BM) {
+      const int m = min(m0 + tid, M - 1);
+      const int pos = e.positions[m];
+      s_pos[tid] = pos;
+      s_page[tid] = (e.kcache && n0 + BN > e.nq * e.d)
+                        ? e.table[(size_t)e.row_req[m] * e.table_stride + pos / e.page_size] : 0;
+    }
+    for (int i = tid; i < (e.d >> 1); i += NT) s_freq[i] = e.inv_freq ? e.inv_freq[i] : 0.f;
+    for (int i = tid; i < BN; i += NT)
+      s_bias[i] = (e.bias && n0 + i < N) ? load_vec(e.bias, e.bias_bf16, n0 + i) : 0.f;
+  }
+
   floatx4 acc[TM][TN];
 #pragma unroll
   for (int i = 0; i < TM; ++i)
@@ -239,19 +259,18 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __
       if (m >= M || head >= e.nq + 2 * e.nkv) continue;
       const float* src = Cs + row * C_STRIDE + hh * d + i;
       floatx4 lo = *(const floatx4*)src, hi = *(const floatx4*)(src + dh);
-      if (e.bias)
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          lo[q] += load_vec(e.bias, e.bias_bf16, head * d + i + q);
-          hi[q] += load_vec(e.bias, e.bias_bf16, head * d + dh + i + q);
-        }
+      for (int q = 0; q < 4; ++q) {
+        lo[q] += s_bias[hh * d + i + q];
+        hi[q] += s_bias[hh * d + dh + i + q];
+      }
       const bool is_q = head < e.nq, is_k = !is_q && head < e.nq + e.nkv;
-      const int pos = e.positions[m];
+      const int pos = s_pos[row];
       if ((is_q || is_k) && e.inv_freq) {
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
           // the hardware sine and cosine of r = frac(angle / 2 pi)
-          float r = (float)pos * e.inv_freq[i + q] * 0.15915494309189535f;
+          float r = (float)pos * s_freq[i + q] * 0.15915494309189535f;
           r -= floorf(r);
           const float sn = __builtin_amdgcn_sinf(r), cs = __builtin_amdgcn_cosf(r);
           const float nlo = lo[q] * cs - hi[q] * sn, nhi = hi[q] * cs + lo[q] * sn;
@@ -277,7 +296,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __
           }
         }
       } else if (e.kcache) {
-        const size_t page = (size_t)e.table[(size_t)e.row_req[m] * e.table_stride + pos / e.page_size];
+        const size_t page = (size_t)s_page[row];
         const int off = pos % e.page_size;
         if (is_k) {
           // four neighbours of one octet of d lie next to each other in the key order
