@@ -590,7 +590,11 @@ static SkinnyShape skinny_choose_tile(int epilogue, bool norm, int mb, int M, in
         // stand for)
         const bool large = (double)N * K * 2.0 >= 64e6;
         double rate = (large ? 3.2e3 : 3.5e3) * resident * nsb * kw;
-        const double cap = large ? 50.0e3 : 25.0e3;
+        // (more than one tile of rows of a wide output: all but the first tile of a set of
+        // columns find W in the L2 of their die, and sixteen waves a block draw what eight
+        // cannot: gate/up of the 0.5B shape at 48 rows, 10.5 us with 8 strips x 2 slices, 14.3
+        // with 4 x 2; a narrow output gains nothing from more slices)
+        const double cap = (large || (tiles > 1 && strips >= num_cus)) ? 50.0e3 : 25.0e3;
         if (rate > cap) rate = cap;
         const double t_stream = per_cu * (16.0 * nsb * K * 2.0) / rate;
         const double x_bytes = (double)(stage ? 1 : 2 * nsb) * M * K * (norm ? 4.0 : 2.0);

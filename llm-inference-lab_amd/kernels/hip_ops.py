@@ -459,7 +459,7 @@ class HipOps:
             if waste(1) < self.rules.uneven_rounds_waste:
                 return 1
             for p in range(2, max(most, 1) + 1):
-                if waste(p) <= 1.05:
+                if waste(p) <= 1.07:       # (3 pieces, 3.75 rounds, do as well as 4 and cost the next reader less)
                     return p
             return 1
         want = self.num_cus // max(strips, 1)

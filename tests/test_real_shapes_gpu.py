@@ -69,8 +69,8 @@ def assert_large_matrix_rules_fire(ops, cfg):
     assert ops.pieces_by_tiles(26, h, inter) and ops.pieces_by_tiles(64, h, q) and not ops.pieces_by_tiles(8, h, inter)
     assert ops.split_count(26, bf, h, inter) > 1 and ops.split_count(64, bf, h, q) > 1
     # ... while a step of one tile of rows has strips enough for the chip: 224 strips on 256
-    # units are not cut, 320 strips (1.25 rounds of blocks) are cut in four (5 even rounds) ...
-    assert ops.split_count(8, bf, h, inter) == {3584: 1, 5120: 4}[h]
+    # units are not cut, 320 strips (1.25 rounds of blocks) are cut in three (3.75 rounds) ...
+    assert ops.split_count(8, bf, h, inter) == {3584: 1, 5120: 3}[h]
     # ... the fused norm + product kernels stop at one tile of rows ...
     assert ops.can_fuse(8, bf, h, qkv) and not ops.can_fuse(26, bf, h, 2 * inter) and not ops.can_fuse(64, bf, h, qkv)
     # ... q/k/v of 24 to 64 rows goes through pieces, of more rows through the tiled epilogue
