@@ -823,6 +823,14 @@ static int launch_key_split_decode(AttnArgs a, int reqs, int live, int ctx_len, 
   const int most = (steps32 + DECODE_WAVES - 1) / DECODE_WAVES;      // one step per wave at least
   if (splits > most) splits = most;
   if (splits > MAX_KEY_SPLITS) splits = MAX_KEY_SPLITS;       // what the merge kernel takes: two per lane
+  // A split costs the merge kernel (4 to 5 us with its launch), which a short history does
+  // not earn back: one block reads 256 KB of keys and values in about that time, and with
+  // few splits to be had (many blocks already) twice as much (64 requests of 2 kv heads of
+  // 64 over 1,024 keys: 10.3 us unsplit, 13.2 in two splits; 32 requests of 4 kv heads of
+  // 128 over 1,024 keys: 20.3 and 22.8; 8 requests of those over 1,024 keys: 14.8 unsplit,
+  // 13.5 in eight splits).
+  const size_t block_bytes = (size_t)visible * D * 2 * sizeof(bf16_t);
+  if (block_bytes < (384u << 10) || (splits <= 4 && block_bytes < (768u << 10))) splits = 1;
   if (g_force_splits > 0) splits = min(g_force_splits, MAX_KEY_SPLITS);
   if (splits < 1) splits = 1;
   const size_t per_split = (size_t)total_rows * nq * (D + 2);
