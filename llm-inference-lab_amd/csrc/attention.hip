@@ -102,7 +102,12 @@ constexpr int DECODE_WAVES = D <= 64 ? 8 : (D <= 128 ? 4 : 2);
 // RING (decode only): key steps a wave keeps in flight; 1 when a wave has one or two
 // steps at all (nothing to run ahead of), 2 for longer shares (deeper rings measured
 // no faster).
-template <int QB, bool DECODE, int RING>
+// PH (prefill only): the block has PH groups of four waves; group ph takes the ph-th 64 keys
+// of every 64*PH the block stages, and the groups' sums meet in LDS at the end.  Two
+// groups double the waves of a launch whose tiles of rows would leave a SIMD with one
+// wave or none: a wave's step is a chain (LDS, scores, maximum, exponentials, products)
+// that only another wave can fill.
+template <int QB, bool DECODE, int RING, int PH = 1>
 __device__ __forceinline__ void attention_tile(const AttnArgs& a, const int xblk) {
   constexpr int DC = (D + 31) / 32;  // 32-wide chunks of d for Q.K
   constexpr int DB = D / 16;         // 16-wide blocks of d for P.V
@@ -115,8 +120,10 @@ __device__ __forceinline__ void attention_tile(const AttnArgs& a, const int xblk
   const int G = a.nq / a.nkv;
   const int r0 = a.q_start[b], qlen = a.q_start[b + 1] - r0, sp = a.start_pos[b];
   const int rows_total = qlen * G;
-  const int row0 = DECODE ? xblk * (16 * QB) : (xblk * nw + wave) * (16 * QB);
-  if ((DECODE ? row0 : xblk * nw * (16 * QB)) >= rows_total) return;   // the whole block is past the rows
+  const int nwr = DECODE ? 1 : nw / PH;          // prefill: waves side by side along the rows
+  const int ph = DECODE ? 0 : wave / nwr;        // ... and this wave's group
+  const int row0 = DECODE ? xblk * (16 * QB) : (xblk * nwr + wave % nwr) * (16 * QB);
+  if ((DECODE ? row0 : xblk * nwr * (16 * QB)) >= rows_total) return;   // the whole block is past the rows
   if (qlen < a.qlen_lo || qlen > a.qlen_hi) return;                     // another launch's request
   const bool wave_live = row0 < rows_total;      // a wave without rows still helps to stage keys
   const bf16_t* q = (const bf16_t*)a.q;
@@ -261,6 +268,11 @@ __device__ __forceinline__ void attention_tile(const AttnArgs& a, const int xblk
     }
   };
 
+  // prefill: the keys and values of a staged tile (64 keys for each group of waves)
+  static_assert(PH == 1 || PH == 2, "one or two groups of waves");
+  constexpr int KT = 64 * PH;
+  constexpr int STAGES = PH;                   // of keys and values in LDS
+  __shared__ __attribute__((aligned(16))) bf16_t kv_lds[DECODE ? 8 : STAGES * 2 * KT * D];
   if constexpr (PIPE) {
     // The loads of the next steps are in flight while this one is computed.  Every
     // load in the loop is unconditional (a load under a branch makes the compiler
@@ -320,27 +332,33 @@ __device__ __forceinline__ void attention_tile(const AttnArgs& a, const int xblk
   } else {
     // ---- prefill: tiles of 64 keys go through LDS once per block and serve all its
     // waves; the next tile is fetched into registers while this one is multiplied
-    constexpr int NCH = D / 16;                     // 16-byte pieces per thread and tile (256 threads)
-    // the tile's four 16-key blocks as they lie in the cache (fragment order): the
+    constexpr int NCH = D / 16;                     // 16-byte pieces per thread and tile (64 threads per 16 keys)
+    constexpr int NT = 256 * PH;                    // threads of the block
+    constexpr int KT_SHIFT = PH == 1 ? 6 : 7;
+    // the tile's 16-key blocks as they lie in the cache (fragment order): the
     // copy is straight, and every fragment read below is lane-contiguous
-    __shared__ __attribute__((aligned(16))) bf16_t Ks[64 * D];
-    __shared__ __attribute__((aligned(16))) bf16_t Vs[64 * D];
+    // With two groups of waves two stages, the tile after this one being put in while this
+    // one is multiplied: one barrier per tile, and the copy of one wave passes behind the
+    // arithmetic of the others (a block of eight waves is alone on its compute unit; two
+    // blocks of four fill each other's waits, and measured no faster with two stages).
+    auto ks_of = [&](int stage) { return kv_lds + stage * (2 * KT * D); };
+    auto vs_of = [&](int stage) { return kv_lds + stage * (2 * KT * D) + KT * D; };
     // The values lie in LDS so that one 16-byte read gives a lane its MFMA operand of a
     // step of 32 keys: [pair of 16-key blocks][16-wide block of d][lane][even block's 4 |
     // odd block's 4].  A 16-byte piece as it comes from the cache (two lanes' values of
     // one 16-key block) goes there in two halves.
     auto vs_at = [&](int sub, int db, int ln) { return (((sub >> 1) * DB + db) * 64 + ln) * 8 + (sub & 1) * 4; };
-    auto vs_store = [&](int sub, int rem, const bf16x8& v) {     // piece `rem` of 16-key block `sub`
+    auto vs_store = [&](bf16_t* Vs, int sub, int rem, const bf16x8& v) {     // piece `rem` of 16-key block `sub`
       bf16_t* dst = Vs + vs_at(sub, rem >> 5, (rem & 31) * 2);
       *(bf16x4*)dst = __builtin_shufflevector(v, v, 0, 1, 2, 3);
       *(bf16x4*)(dst + 8) = __builtin_shufflevector(v, v, 4, 5, 6, 7);
     };
-    __shared__ int s_ok[4];
+    __shared__ int s_ok_all[STAGES][4 * PH];
     constexpr int PAGE_CAP = 2048;
-    __shared__ int s_pages[PAGE_CAP];               // the block's slice of its request's block table
+    __shared__ int s_pages[PAGE_CAP + 1];           // the block's slice of its request's block table (a slice that starts inside a page touches one more)
     const int tid = threadIdx.x;
-    const int blk_row0 = xblk * nw * (16 * QB);
-    const int blk_last = min(blk_row0 + nw * 16 * QB, rows_total) - 1;
+    const int blk_row0 = xblk * nwr * (16 * QB);
+    const int blk_last = min(blk_row0 + nwr * 16 * QB, rows_total) - 1;
     const int bkey_hi = sp + blk_last / G;
     const int bkey_lo = a.window > 0 ? max(0, sp + blk_row0 / G - a.window + 1) : 0;
     // PD tiles are on their way from memory at any time (a ring of register buffers):
@@ -350,16 +368,16 @@ __device__ __forceinline__ void attention_tile(const AttnArgs& a, const int xblk
     constexpr int PD = NCH <= 4 ? 3 : 2;
     bf16x8 regs[PD][NCH];
     bool rok[PD][NCH];
-    const int tile_lo = bkey_lo >> 6, tile_hi = bkey_hi >> 6;
+    const int tile_lo = bkey_lo >> KT_SHIFT, tile_hi = bkey_hi >> KT_SHIFT;
     // The page numbers come from LDS, PAGE_CAP pages at a time (one slice is enough
     // for any common context), so that a tile costs one memory round trip, not two.
-    const int tiles_per_slice = (PAGE_CAP << pshift) >> 6;
+    const int tiles_per_slice = (PAGE_CAP << pshift) >> KT_SHIFT;
     for (int ct = tile_lo; ct <= tile_hi; ct += tiles_per_slice) {
       const int ce = min(ct + tiles_per_slice - 1, tile_hi);
-      const int page_first = page_index(ct * 64);
-      const int page_count = page_index(ce * 64 + 63) - page_first + 1;
+      const int page_first = page_index(ct * KT);
+      const int page_count = page_index(ce * KT + KT - 1) - page_first + 1;
       __syncthreads();
-      for (int i = tid; i < page_count; i += 256) {
+      for (int i = tid; i < page_count; i += NT) {
         const int pi = page_first + i;
         s_pages[i] = pi < a.table_stride ? a.table[(size_t)b * a.table_stride + pi] : -1;
       }
@@ -372,7 +390,7 @@ __device__ __forceinline__ void attention_tile(const AttnArgs& a, const int xblk
         if constexpr (FAST_PIECES) {
           // wave w copies the w-th 16-key block of the tile, keys and values: one page
           // lookup and one address for all pieces of a thread
-          const int pos16 = tl * 64 + wave * 16;
+          const int pos16 = tl * KT + wave * 16;
           const int page = s_pages[page_index(pos16) - page_first];
           const bool ok = tile <= ce && pos16 <= bkey_hi && pos16 + 15 >= bkey_lo && page >= 0;
           const size_t at = ((size_t)max(page, 0) * a.nkv + kvh) * P * D +
@@ -387,11 +405,11 @@ __device__ __forceinline__ void attention_tile(const AttnArgs& a, const int xblk
         }
 #pragma unroll
         for (int n = 0; n < NCH; ++n) {
-          const int i = tid + n * 256;
-          const bool is_v = i >= 8 * D;
-          const int j = is_v ? i - 8 * D : i;
+          const int i = tid + n * NT;
+          const bool is_v = i >= 8 * D * PH;
+          const int j = is_v ? i - 8 * D * PH : i;
           const int sub = j / (2 * D), rem = j - sub * (2 * D);
-          const int pos16 = tl * 64 + sub * 16;
+          const int pos16 = tl * KT + sub * 16;
           const int page = s_pages[page_index(pos16) - page_first];
           rok[slot][n] = tile <= ce && pos16 <= bkey_hi && pos16 + 15 >= bkey_lo && page >= 0;
           const size_t blk16 = ((size_t)max(page, 0) * a.nkv + kvh) * P * D +
@@ -399,48 +417,68 @@ __device__ __forceinline__ void attention_tile(const AttnArgs& a, const int xblk
           regs[slot][n] = *(const bf16x8*)((is_v ? vc : kc) + blk16 + rem * 8);
         }
       };
-      auto store_tile = [&](int slot) {
+      auto store_tile = [&](int slot, int stage) {
+        bf16_t* Ks = ks_of(stage);
+        bf16_t* Vs = vs_of(stage);
+        int* s_ok = s_ok_all[stage];
         if constexpr (FAST_PIECES) {
 #pragma unroll
           for (int n = 0; n < NCH / 2; ++n) {
             // (what came for a 16-key block that is not there goes in as it is: s_ok keeps
             // the keys out of the scores, and the values are zeroed where they are read)
             *(bf16x8*)(Ks + wave * (16 * D) + (lane + n * 64) * 8) = regs[slot][n];
-            vs_store(wave, lane + n * 64, regs[slot][n + NCH / 2]);
+            vs_store(Vs, wave, lane + n * 64, regs[slot][n + NCH / 2]);
           }
           if (lane == 0) s_ok[wave] = rok[slot][0];
           return;
         }
 #pragma unroll
         for (int n = 0; n < NCH; ++n) {
-          const int i = tid + n * 256;
-          const bool is_v = i >= 8 * D;
-          const int j = is_v ? i - 8 * D : i;
+          const int i = tid + n * NT;
+          const bool is_v = i >= 8 * D * PH;
+          const int j = is_v ? i - 8 * D * PH : i;
           const int sub = j / (2 * D), rem = j - sub * (2 * D);
           const bf16x8 v = rok[slot][n] ? regs[slot][n] : zero8;
-          if (is_v) vs_store(sub, rem, v);
+          if (is_v) vs_store(Vs, sub, rem, v);
           else *(bf16x8*)(Ks + sub * (16 * D) + rem * 8) = v;
           if (!is_v && rem == 0) s_ok[sub] = rok[slot][n];
         }
       };
 #pragma unroll
       for (int p = 0; p < PD; ++p) fetch_tile(p, ct + p);
+      // two stages: tile t lies in stage t & 1; it is put there during tile t - 1 (the first one: now)
+      if constexpr (STAGES == 2) {
+        store_tile(0, ct & 1);
+        fetch_tile(0, ct + PD);
+        __syncthreads();
+      }
       for (int tile0 = ct; tile0 <= ce; tile0 += PD) {
 #pragma unroll
         for (int p = 0; p < PD; ++p) {
           const int tile = tile0 + p;
           const bool live = tile <= ce;
-          if (live) {
-            store_tile(p);
-            __syncthreads();
+          const int stage = STAGES == 2 ? (tile & 1) : 0;
+          if constexpr (STAGES == 2) {
+            const int pn = (p + 1) % PD;              // ring slot of the next tile (a constant once unrolled)
+            if (tile + 1 <= ce) store_tile(pn, stage ^ 1);
+            fetch_tile(pn, tile + 1 + PD);
+          } else {
+            if (live) {
+              store_tile(p, 0);
+              __syncthreads();
+            }
+            fetch_tile(p, tile + PD);
           }
-          fetch_tile(p, tile + PD);
           __builtin_amdgcn_sched_barrier(0);
-          const int kb0 = tile * 64;
-          // a tile below the diagonal of all rows of the wave and inside their windows,
-          // with all its pages there: the whole tile in one piece, without comparisons
+          const bf16_t* Ks = ks_of(stage);
+          const bf16_t* Vs = vs_of(stage);
+          const int* s_ok = s_ok_all[stage];
+          const int kb0 = tile * KT + ph * 64;      // this group's 64 keys of the tile
+          const int sub0 = ph * 4;                  // ... and their first 16-key block in LDS
+          // 64 keys below the diagonal of all rows of the wave and inside their windows,
+          // with all their pages there: in one piece, without comparisons
           const bool interior = live && wave_live && kb0 + 63 <= p_first && kb0 >= full_lo &&
-                                (s_ok[0] & s_ok[1] & s_ok[2] & s_ok[3]) != 0;
+                                (s_ok[sub0] & s_ok[sub0 + 1] & s_ok[sub0 + 2] & s_ok[sub0 + 3]) != 0;
           if (interior) {
             // with one row block the whole tile of 64 keys at once, with two in halves of
             // 32 (registers): scores of the piece, one maximum, exponentials, products
@@ -451,7 +489,7 @@ __device__ __forceinline__ void attention_tile(const AttnArgs& a, const int xblk
               bf16x8 vf[SUBS / 2][DB];
 #pragma unroll
               for (int u = 0; u < SUBS; ++u) {
-                const int sub = piece * SUBS + u;
+                const int sub = sub0 + piece * SUBS + u;
 #pragma unroll
                 for (int dc = 0; dc < DC; ++dc)
                   kf[u][dc] = *(const bf16x8*)(Ks + sub * (16 * D) + min(dc * 4 + g, D / 8 - 1) * 128 + c * 8);
@@ -461,7 +499,7 @@ __device__ __forceinline__ void attention_tile(const AttnArgs& a, const int xblk
               for (int st = 0; st < SUBS / 2; ++st)
 #pragma unroll
                 for (int db = 0; db < DB; ++db)
-                  vf[st][db] = *(const bf16x8*)(Vs + vs_at(piece * SUBS + st * 2, db, lane));
+                  vf[st][db] = *(const bf16x8*)(Vs + vs_at(sub0 + piece * SUBS + st * 2, db, lane));
               floatx4 s4[SUBS][QB];
 #pragma unroll
               for (int u = 0; u < SUBS; ++u)
@@ -520,12 +558,12 @@ __device__ __forceinline__ void attention_tile(const AttnArgs& a, const int xblk
           } else if (live) {
 #pragma unroll
             for (int st = 0; st < 2; ++st) {
-              const int kb = tile * 64 + st * 32;
+              const int kb = kb0 + st * 32;
               if (kb <= key_hi && kb + 31 >= key_lo) {        // this wave sees some of these keys
                 KeyStep<DC, DB> f;
 #pragma unroll
                 for (int h2 = 0; h2 < 2; ++h2) {
-                  const int sub = st * 2 + h2;
+                  const int sub = sub0 + st * 2 + h2;
                   f.ok[h2] = s_ok[sub] != 0;
 #pragma unroll
                   for (int dc = 0; dc < DC; ++dc)
@@ -544,6 +582,37 @@ __device__ __forceinline__ void attention_tile(const AttnArgs& a, const int xblk
     }
   }
 
+  if constexpr (!DECODE && PH > 1) {
+    // The second group hands its sums to the first, lane to lane (both hold the same rows in
+    // the same places); the staged keys are done with after the last tile's barrier.
+    //   o = 2^(m0 - m) o0 + 2^(m1 - m) o1,  l likewise,  m = max(m0, m1)
+    float* xo = (float*)kv_lds;                        // [row tile][qb][db][lane][4]
+    __shared__ float x_m[4][QB][64], x_l[4][QB][64];
+    const int rt = wave % nwr;
+    if (ph == 1) {
+#pragma unroll
+      for (int qb = 0; qb < QB; ++qb) {
+        x_m[rt][qb][lane] = m[qb];
+        x_l[rt][qb][lane] = lsum[qb];
+#pragma unroll
+        for (int db = 0; db < DB; ++db) *(floatx4*)(xo + (((rt * QB + qb) * DB + db) * 64 + lane) * 4) = o[qb][db];
+      }
+    }
+    __syncthreads();
+    if (ph != 0) return;
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+      const float m1 = x_m[rt][qb][lane], m_new = fmaxf(m[qb], m1);
+      const float a0 = m[qb] == NEG_INF ? 0.f : fast_exp2(m[qb] - m_new);
+      const float a1 = m1 == NEG_INF ? 0.f : fast_exp2(m1 - m_new);
+      lsum[qb] = lsum[qb] * a0 + x_l[rt][qb][lane] * a1;
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        const floatx4 o1 = *(const floatx4*)(xo + (((rt * QB + qb) * DB + db) * 64 + lane) * 4);
+        o[qb][db] = o[qb][db] * a0 + o1 * a1;
+      }
+    }
+  }
   if constexpr (!DECODE) {
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
@@ -612,21 +681,21 @@ __device__ __forceinline__ void attention_tile(const AttnArgs& a, const int xblk
 
 // One tile of rows per block; the blocks with the longest histories (the last rows)
 // are dispatched first.
-template <int QB, bool DECODE, int RING = 1>
-__global__ __launch_bounds__(DECODE ? 64 * DECODE_WAVES : 256, (!DECODE && D <= 64) ? 2 : 1) void attention_bf16_kernel(AttnArgs a) {
-  attention_tile<QB, DECODE, RING>(a, (int)(gridDim.x - 1 - blockIdx.x));
+template <int QB, bool DECODE, int RING = 1, int PH = 1>
+__global__ __launch_bounds__(DECODE ? 64 * DECODE_WAVES : 256 * PH, (!DECODE && D <= 64 && PH == 1) ? 2 : 1) void attention_bf16_kernel(AttnArgs a) {
+  attention_tile<QB, DECODE, RING, PH>(a, (int)(gridDim.x - 1 - blockIdx.x));
 }
 
 // Two tiles of rows per block, one after the other: tile t from the end and tile t
 // from the start.  Under a causal mask their histories add up to the same length for
 // every t, so all blocks of a prompt carry the same load; with one tile per block the
 // last tiles' blocks run on while the units of the first ones idle.
-template <int QB>
-__global__ __launch_bounds__(256, D <= 64 ? 2 : 1) void attention_bf16_paired_kernel(AttnArgs a) {
+template <int QB, int PH = 1>
+__global__ __launch_bounds__(256 * PH, (D <= 64 && PH == 1) ? 2 : 1) void attention_bf16_paired_kernel(AttnArgs a) {
   const int late = a.tiles - 1 - (int)blockIdx.x, early = (int)blockIdx.x;
   for (int pass = 0; pass < 2; ++pass) {
     if (pass == 1 && early >= late) break;
-    attention_tile<QB, false, 1>(a, pass == 0 ? late : early);
+    attention_tile<QB, false, 1, PH>(a, pass == 0 ? late : early);
     __syncthreads();
   }
 }
@@ -800,7 +869,8 @@ static int g_force_splits = 0;
 extern "C" void llmlab_debug_attention_splits(int splits) { g_force_splits = splits; }
 // ... and the launch that steps of many rows take: 1 = the waves of a block split the keys of
 // a tile of 32 rows, 2 = tiles of 32 rows per wave, 3 = late and early tiles in pairs,
-// 4 = tiles of 16 rows per wave (0: chosen here).
+// 4 = tiles of 16 rows per wave, 5 and 6 = 3 and 4 with two groups of waves that take the
+// staged keys in turn (0: chosen here).
 static int g_force_path = 0;
 extern "C" void llmlab_debug_attention_path(int path) { g_force_path = path; }
 
@@ -927,12 +997,46 @@ extern "C" int llmlab_paged_attention(const void* q, int dtype, int q_stride, in
     a.qlen_lo = short_len + 1;
     live = reqs - n_short;
   }
-  // Few tiles of rows (a short portion, with or without a long history behind it):
-  // the waves of a block split the keys of one tile of 32 rows and merge in LDS, so
-  // that the work still spreads over the chip.  Else every wave owns its rows and
-  // the block's waves share the keys through LDS.
+  // The launch, from measurements of 64 to 4,096 tokens behind 0 and 4,096 keys, one to
+  // eight requests, heads of 64 (14 over 2) and 128 (28 over 4, 40 over 8):
+  //   1  few tiles of rows behind a long history: the waves of a block split the keys of
+  //      one tile of 32 rows and merge in LDS, so that the work still spreads over the
+  //      chip (64 to 512 tokens behind 4,096 keys, heads of 64: 27 to 31 us against 41 to
+  //      46 for the next best; at the start of a prompt it is the slowest, 17 against 8)
+  //   6  every wave owns 16 rows, the block's two groups of four waves take the staged
+  //      keys in turn: for heads above 64, where a block of four waves is alone on its
+  //      compute unit (2,048 tokens behind 4,096 keys, 28 heads of 128: 313 us against
+  //      374 to 470 for the others), and for heads of 64 when the tiles of rows would
+  //      leave a SIMD with one wave or none, or the longest tile of a long prompt's
+  //      triangle decides (2,048 tokens from 0: 32 us against 38; four prompts of 512: 19
+  //      against 15, so not for those)
+  //   4  the same with one group of four waves (two blocks share a compute unit at heads
+  //      of 64)
+  //   2  32 rows per wave, when that still gives every compute unit two blocks
+  //   3  late and early tiles in pairs (see below)
+  constexpr bool TWO_GROUPS = D <= 128;      // (the staged keys and values of two groups at larger heads: more LDS than there is)
   const long blocks16 = ((max_rows + 63) / 64) * nkv * live;
-  if (g_force_path == 1 || (g_force_path == 0 && blocks16 < num_cus)) {
+  const long blocks32 = ((max_rows + 127) / 128) * nkv * live;
+  const bool long_history = (long)max_ctx_len >= 8L * max_q_len;
+  const bool triangle = window <= 0 && 16L * (max_ctx_len - max_q_len) <= max_q_len;
+  int path = g_force_path;
+  if (!TWO_GROUPS && (path == 5 || path == 6)) path = 0;
+  if (path == 0) {
+    if (blocks16 <= num_cus / 2 && long_history) path = 1;
+    else if (TWO_GROUPS && D > 64 && !(blocks16 >= 4L * num_cus && max_ctx_len <= 1024)) path = 6;
+    else if (TWO_GROUPS && D <= 64 && blocks16 > num_cus / 2 &&
+             (blocks16 <= num_cus || (blocks16 <= 3L * num_cus && triangle && max_q_len >= 1536))) path = 6;
+    else if (blocks16 < num_cus) path = 4;
+    else if (D <= 128 && blocks32 >= 2L * num_cus) path = 2;
+    // not enough tiles to keep every unit busy with what the longest ones leave over:
+    // pair late and early tiles (no window: then the loads add up evenly).  Only at the
+    // start of a prompt: behind a history all tiles carry about the same load, and the
+    // pairs only halve the blocks (2,048 tokens behind 8,192, head size 64: 246 us in
+    // pairs, 172 without)
+    else if (triangle && blocks16 >= (3L * num_cus) / 2) path = 3;
+    else path = 4;
+  }
+  if (path == 1) {
     const int steps32 = (max_ctx_len + 31) / 32 + 1;
     const int steps_per_wave = (steps32 + DECODE_WAVES - 1) / DECODE_WAVES;
     dim3 grid((unsigned)((max_rows + 31) / 32), nkv, reqs), block(64 * DECODE_WAVES);
@@ -943,19 +1047,21 @@ extern "C" int llmlab_paged_attention(const void* q, int dtype, int q_stride, in
     LLMLAB_LAUNCH_CHECK("attention(bfloat16, key split)");
     return 0;
   }
-  // rows per wave: 32 when that still gives every compute unit two blocks (or for
-  // nothing smaller), else 16; always 16 for the largest heads (registers)
-  const long blocks32 = ((max_rows + 127) / 128) * nkv * live;
-  if (g_force_path == 2 || (g_force_path == 0 && D <= 128 && blocks32 >= 2L * num_cus)) {
+  if (path == 2) {
     dim3 grid((unsigned)((max_rows + 127) / 128), nkv, reqs), block(256);
     hipLaunchKernelGGL((attention_bf16_kernel<2, false>), grid, block, 0, stream, a);
-  } else if (g_force_path == 3 || (g_force_path == 0 && window <= 0 && blocks16 >= (3L * num_cus) / 2 &&
-                                   16L * (max_ctx_len - max_q_len) <= max_q_len)) {
-    // not enough tiles to keep every unit busy with what the longest ones leave over:
-    // pair late and early tiles (no window: then the loads add up evenly).  Only at the
-    // start of a prompt: behind a history all tiles carry about the same load, and the
-    // pairs only halve the blocks (2,048 tokens behind 8,192, head size 64: 246 us in
-    // pairs, 172 without)
+  } else if (path == 5) {
+    if constexpr (TWO_GROUPS) {
+      a.tiles = (int)((max_rows + 63) / 64);
+      dim3 grid((unsigned)((a.tiles + 1) / 2), nkv, reqs), block(512);
+      hipLaunchKernelGGL((attention_bf16_paired_kernel<1, 2>), grid, block, 0, stream, a);
+    }
+  } else if (path == 6) {
+    if constexpr (TWO_GROUPS) {
+      dim3 grid((unsigned)((max_rows + 63) / 64), nkv, reqs), block(512);
+      hipLaunchKernelGGL((attention_bf16_kernel<1, false, 1, 2>), grid, block, 0, stream, a);
+    }
+  } else if (path == 3) {
     a.tiles = (int)((max_rows + 63) / 64);
     dim3 grid((unsigned)((a.tiles + 1) / 2), nkv, reqs), block(256);
     hipLaunchKernelGGL((attention_bf16_paired_kernel<1>), grid, block, 0, stream, a);

@@ -5,10 +5,12 @@
 //   bfloat16:  v_mfma_f32_16x16x32_bf16 everywhere.
 //     * tiled kernel: 256 threads = 4 waves, block tile 64x64 (waves 2x2), 64x128 or
 //       128x128 (waves 1x4, side by side along the columns), K step 64; x staged through
-//       two stages of LDS (rows padded to 72 elements so that the 16-byte fragment reads
-//       of 8 lanes cover all banks), the fragments of W read straight from the packed
-//       matrix into registers; three or four tiles are on their way from memory in a
-//       ring of register buffers while one is multiplied.  With the waves 1x4 every
+//       three stages of LDS (rows padded to 80 elements: a wave's 16-byte fragment reads
+//       then take 8.4 clocks, as lane-contiguous ones do; 9.5 with 72, 16 unpadded), its
+//       fragments read into registers half a tile ahead of their products, the fragments
+//       of W read straight from the packed matrix into registers; three or four tiles
+//       are on their way from memory in a ring of register buffers while one is
+//       multiplied.  With the waves 1x4 every
 //       fragment of W is read by one wave only and all four share the rows of x in LDS:
 //       5 to 35 % faster than 2x2 waves with W staged through LDS too (which was the
 //       large tile before).  Also measured and not adopted: 256x128 tiles with eight
@@ -17,7 +19,11 @@
 //       waves 2x4 on 128x128 and 64x128, a 64x256 tile with eight waves 1x8 for few rows of a wide
 //       matrix (as fast as 64x128, no faster), and 256x256 tiles with four 128x128 wave tiles (half the LDS traffic
 //       per product, one wave per SIMD: 833 against 793 TF/s on the largest product
-//       tried, slower on the rest).
+//       tried, slower on the rest).  Counters of the 128x128 tile on a product of
+//       2048 x 37888 x 3584 (900 TF/s; two blocks share a compute unit, the clock is at
+//       2.0 GHz under this load): matrix pipes busy 40 % of the time, LDS 52 % (and
+//       counted in bank conflicts for another 21 %), the texture address units 56 %: no
+//       unit is the limit alone, the waves wait for one another's turns at three of them.
 //     (products of few rows, as in decode steps, have kernels of their own in decode.hip)
 //   float32: a plain FMA kernel (tiles of 64x64 to 128x128, 4x4 to 8x8 outputs per thread) and, for up to 64
 //     rows, one in which a wave owns four rows of W and its lanes split the inner size:
@@ -81,19 +87,19 @@ template <int BM, int BN, int BK, int WM, int WN, int EPI>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __restrict__ A,
                                                         const bf16_t* __restrict__ W, EpiArgs e, int M,
                                                         int N, int K) {
-  constexpr int LDS_STRIDE = BK + 8;         // padded rows: 16-byte reads of 8 lanes cover all banks
+  constexpr int LDS_STRIDE = BK + 16;        // padded rows: the fragment reads of a wave spread evenly over the banks
   constexpr int NT = 64 * WM * WN;           // threads: WM x WN waves
   constexpr int WTM = BM / WM, WTN = BN / WN;  // wave tile
   constexpr int TM = WTM / 16, TN = WTN / 16;
   constexpr int KCH = BK / 8;                // 16-byte chunks in a row of a tile
   constexpr int A_CHUNKS = BM * KCH / NT;    // chunks of x per thread
   static_assert(A_CHUNKS >= 1 && BM * KCH % NT == 0, "tile too small");
-  // two stages of LDS for x: the next tile is put in while this one is multiplied, one
-  // barrier per tile
+  // three stages of LDS for x: the tile after the next is put in while this one is
+  // multiplied and the next one's fragments are read, one barrier per tile
   constexpr int A_STAGE = BM * LDS_STRIDE;
   // (one array: after the last tile it holds the block's results for the epilogue)
   constexpr int C_STRIDE = BN + 4;           // floats per row of the result tile in LDS
-  constexpr size_t STAGE_BYTES = (size_t)(2 * A_STAGE) * sizeof(bf16_t);
+  constexpr size_t STAGE_BYTES = (size_t)(3 * A_STAGE) * sizeof(bf16_t);
   constexpr size_t C_BYTES = (size_t)BM * C_STRIDE * sizeof(float);
   __shared__ __attribute__((aligned(16))) char smem[STAGE_BYTES > C_BYTES ? STAGE_BYTES : C_BYTES];
   bf16_t* As2 = (bf16_t*)smem;
@@ -200,38 +206,53 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __
     fetch(p, kbase + p * BK);
     fetch_b(p, kbase + p * BK);
   }
-  // tile kt lies in stage kt & 1; it was put there during tile kt - 1 (tile 0: now)
+  // Tile t lies in stage t % 3.  It is put there during tile t - 2, and its fragments are
+  // read into registers half a tile ahead of their products (those of its first 32
+  // columns of K during the second half of tile t - 1), so that the reads of LDS pass
+  // behind the matrix instructions of the half before: with one wave on a SIMD nothing
+  // else would hide them.  One barrier per tile: what is overwritten during tile t (stage
+  // (t + 2) % 3) was last read during tile t - 1.
+  auto frags = [&](bf16x8 (&a)[TM], int stage, int ks) {
+    const bf16_t* As = As2 + stage * A_STAGE;
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+      a[i] = *(const bf16x8*)(As + (wm * WTM + i * 16 + c) * LDS_STRIDE + ks * 32 + g * 8);
+  };
+  static_assert(BK == 64, "two half tiles");
+  bf16x8 a0[TM], a1[TM];
   stash(0, 0);
   fetch(0, kbase + PD * BK);
+  if (nk > 1) stash(1 % PD, 1);
+  fetch(1 % PD, kbase + (PD + 1) * BK);
   __syncthreads();
+  frags(a0, 0, 0);
+  int stage = 0;                                 // t % 3
   for (int kt = 0; kt < nk; kt += PD) {
 #pragma unroll
     for (int p = 0; p < PD; ++p) {
       const int t = kt + p;
       const bool live = t < nk;
-      const int stage = t & 1;
-      const int pn = (p + 1) % PD;              // ring slot of tile t + 1 (a constant once unrolled)
-      if (t + 1 < nk) stash(pn, stage ^ 1);
-      fetch(pn, kbase + (t + 1 + PD) * BK);
+      const int p2 = (p + 2) % PD;              // ring slot of tile t + 2 (a constant once unrolled)
+      const int stage1 = stage == 2 ? 0 : stage + 1, stage2 = stage1 == 2 ? 0 : stage1 + 1;
       if (live) {
-        const bf16_t* As = As2 + stage * A_STAGE;
+        frags(a1, stage, 1);
 #pragma unroll
-        for (int ks = 0; ks < BK / 32; ++ks) {
-          bf16x8 a[TM], b[TN];
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-          for (int i = 0; i < TM; ++i)
-            a[i] = *(const bf16x8*)(As + (wm * WTM + i * 16 + c) * LDS_STRIDE + ks * 32 + g * 8);
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0[i], rbd[p][0][j], acc[i][j], 0, 0, 0);
+        frags(a0, stage1, 0);
+        if (t + 2 < nk) stash(p2, stage2);
+        fetch(p2, kbase + (t + 2 + PD) * BK);
 #pragma unroll
-          for (int j = 0; j < TN; ++j) b[j] = rbd[p][ks][j];
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-          for (int i = 0; i < TM; ++i)
-#pragma unroll
-            for (int j = 0; j < TN; ++j)
-              acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
-        }
+          for (int j = 0; j < TN; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1[i], rbd[p][1][j], acc[i][j], 0, 0, 0);
         __syncthreads();
       }
       fetch_b(p, kbase + (t + PD) * BK);
+      stage = stage1;
     }
   }
 

@@ -69,7 +69,9 @@ class KernelDebug:
         this epilogue only.  ``attention_splits``: (head size, key splits of the decode
         launch).  ``attention_path``: (head size, launch of a step of many rows: 1 = the waves of a
         block split the keys of a tile of 32 rows, 2 = tiles of 32 rows per wave, 3 = late and
-        early tiles in pairs, 4 = tiles of 16 rows per wave).  Other keywords: fields of
+        early tiles in pairs, 4 = tiles of 16 rows per wave, 5 and 6 = 3 and 4 with two groups of
+        waves that take the staged keys in turn; heads above 128 have no 5 and 6 and choose
+        for themselves).  Other keywords: fields of
         ``DispatchRules`` for the time of the block."""
         ops = self._ops
         core = ops._core

@@ -431,6 +431,22 @@ def test_attention_tilings_of_many_rows(ops, emu, window, cus, nq, nkv, d, page)
         ops.num_cus = real
 
 
+@pytest.mark.parametrize("window", [None, 40])
+@pytest.mark.parametrize("path", [1, 2, 3, 4, 5, 6])
+@pytest.mark.parametrize("nq,nkv,d,page", [(14, 2, 64, 64), (6, 3, 48, 16), (8, 1, 128, 32), (3, 1, 96, 16)])
+def test_attention_every_launch_of_many_rows(ops, emu, window, path, nq, nkv, d, page):
+    """Each launch for steps of many rows, fixed from outside whatever the rule would take:
+    keys split over the waves of a block, tiles of 32 and of 16 rows per wave, late and
+    early tiles in pairs, and the last two with two groups of waves that take the staged
+    keys in turn and merge at the end (a tile of rows whose second group sees no key at all,
+    a history that ends inside the first group's keys)."""
+    with ops.debug.force(attention_path=(d, path)):
+        run_attention(ops, emu, torch.bfloat16, nq, nkv, d, page, window, [(0, 300), (0, 70), (0, 129)], seed=96,
+                      amplify=(0, 70, 30.0))
+        run_attention(ops, emu, torch.bfloat16, nq, nkv, d, page, window, [(500, 300), (64, 200), (900, 1)], seed=97,
+                      amplify=(0, 130 if window is None else 770, 30.0))
+
+
 @pytest.mark.parametrize("start", [0, 3000])
 def test_attention_of_a_long_portion(ops, emu, start):
     """2,048 tokens of a prompt at the 0.5B head counts, at its start and behind a
