@@ -243,7 +243,6 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __
             acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a0[i], rbd[p][0][j], acc[i][j], 0, 0, 0);
         frags(a0, stage1, 0);
         if (t + 2 < nk) stash(p2, stage2);
-        fetch(p2, kbase + (t + 2 + PD) * BK);
 #pragma unroll
         for (int i = 0; i < TM; ++i)
 #pragma unroll
@@ -251,6 +250,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __
             acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a1[i], rbd[p][1][j], acc[i][j], 0, 0, 0);
         __syncthreads();
       }
+      // (outside the branch, like every load of the loop: see above)
+      fetch(p2, kbase + (t + 2 + PD) * BK);
       fetch_b(p, kbase + (t + PD) * BK);
       stage = stage1;
     }
@@ -617,8 +618,8 @@ constexpr int F32_ROWS_MAX = 64;     // up to here the few-row kernel (the tiled
 // matrix: 64 x 64 (waves 2 x 2) for small products, 64 x 128 and 128 x 128 with the waves
 // side by side along the columns (1 x 4), so that every fragment of W is read by one wave
 // only and the rows of x in LDS are shared by all four.  The shape is picked by an
-// estimate of the time, fitted to sweeps of the three products of a layer at two model
-// shapes and 576 to 4096 rows (its picks cost 1.4 % over the best shape there):
+// estimate of the time, fitted to sweeps of the four products of a layer at three model
+// shapes and 576 to 8192 rows (its picks cost 0.7 % over the best shape there):
 //   time = L + rounds * (f + K tiles * tk),  rounds = max(1, blocks / (units * resident)).
 // With few rows the product is bound by the read of W instead: a block draws `stream`
 // bytes a microsecond, the chip 5.3e6 at most (one tile of rows, 17 to 64 of them, of
@@ -630,8 +631,8 @@ struct TileModel {
   double L, f, tk, resident, stream;
 };
 static const TileModel TILE_MODELS[3] = {{64, 64, 6.39, 0.79, 0.289, 1.0, 20e3},
-                                         {64, 128, 6.54, 0.71, 0.552, 1.5, 27e3},
-                                         {128, 128, 9.78, 0.48, 0.704, 1.0, 24e3}};
+                                         {64, 128, 6.54, 0.71, 0.5, 1.5, 27e3},
+                                         {128, 128, 8.0, 0.48, 0.66, 1.0, 24e3}};
 constexpr double CHIP_STREAM = 5.3e6;     // bytes a microsecond
 
 static double tile_cost(int kind, int M, int N, int K, int num_cus, int pieces) {
