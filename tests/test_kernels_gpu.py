@@ -433,7 +433,8 @@ def test_attention_tilings_of_many_rows(ops, emu, window, cus, nq, nkv, d, page)
 
 @pytest.mark.parametrize("window", [None, 40])
 @pytest.mark.parametrize("path", [1, 2, 3, 4, 5, 6])
-@pytest.mark.parametrize("nq,nkv,d,page", [(14, 2, 64, 64), (6, 3, 48, 16), (8, 1, 128, 32), (3, 1, 96, 16)])
+@pytest.mark.parametrize("nq,nkv,d,page", [(14, 2, 64, 64), (6, 3, 48, 16), (8, 1, 128, 32), (3, 1, 96, 16),
+                                           (4, 2, 16, 16), (5, 5, 112, 32), (2, 1, 256, 16)])
 def test_attention_every_launch_of_many_rows(ops, emu, window, path, nq, nkv, d, page):
     """Each launch for steps of many rows, fixed from outside whatever the rule would take:
     keys split over the waves of a block, tiles of 32 and of 16 rows per wave, late and
