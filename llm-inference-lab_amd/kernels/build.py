@@ -2,7 +2,8 @@
 
 Two kinds of library: ``core`` (embedding, norm, rotary + cache write, matrix
 products, sampling) and ``attn_d<D>`` (attention for head size D; one per head
-size that a model needs).  A library's file name carries a hash of its sources
+size that a model needs); beside them the plain C++ references of the same operations,
+built with the host compiler for the tests.  A library's file name carries a hash of its sources
 and flags, so a library built from other sources is never loaded.  Libraries are
 kept in ``kernels/lib`` inside the package, or, if that folder cannot be written,
 in a per-user folder under the system's temporary directory (or
@@ -138,6 +139,42 @@ def attention_library(head_dim: int, force: bool = False) -> str:
     return _compile(f"attn_d{head_dim}", (ATTENTION_SOURCE,), (f"-DHEAD_DIM={head_dim}",), force)
 
 
+REFERENCE_SOURCE = "reference.cpp"
+
+
+def reference_library(force: bool = False) -> str:
+    """The plain C++ references of the kernels' operations (``csrc/reference.cpp``), built with
+    the host compiler.  Tests load it; the product never does."""
+    with open(os.path.join(CSRC, REFERENCE_SOURCE), "rb") as f:
+        digest = hashlib.sha256(f.read()).hexdigest()[:12]
+    name = f"libllmlab_reference.{digest}.so"
+    if not force:
+        for d in _search_dirs():
+            if os.path.isfile(os.path.join(d, name)):
+                return os.path.join(d, name)
+    compiler = next((c for c in (os.environ.get("CXX"), shutil.which("g++"), shutil.which("c++"),
+                                 shutil.which("clang++")) if c), None)
+    if compiler is None:
+        raise RuntimeError("no host C++ compiler found for the plain references")
+    out_dir = _writable_dir()
+    path = os.path.join(out_dir, name)
+    tmp = f"{path}.{os.getpid()}.tmp"
+    proc = subprocess.run([compiler, "-O2", "-std=c++17", "-fPIC", "-shared",
+                           os.path.join(CSRC, REFERENCE_SOURCE), "-o", tmp],
+                          stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise RuntimeError("the host compiler failed for the plain references:\n" + proc.stdout[-4000:])
+    os.replace(tmp, path)
+    for old in glob.glob(os.path.join(out_dir, "libllmlab_reference.*.so")):
+        if old != path:
+            try:
+                os.remove(old)
+            except OSError:
+                pass
+    _say(f"built {name}")
+    return path
+
+
 def library(kind: str, parameter=None, force: bool = False) -> str:
     """The library a part names in ``kernel_libraries()``: ``("core", None)`` or
     ``("attention", head_dim)``."""
@@ -153,4 +190,5 @@ def build_all(head_dims: Sequence[int] = DEFAULT_HEAD_DIMS, force: bool = True) 
     out = {"core": core_library(force)}
     for d in head_dims:
         out[f"attn_d{d}"] = attention_library(d, force)
+    out["reference"] = reference_library(force)
     return out
