@@ -385,6 +385,8 @@ def main():
     ap.add_argument("--requests", type=int, default=64)
     ap.add_argument("--chunk", type=int, default=512)
     ap.add_argument("--outputs", type=int, default=64)
+    ap.add_argument("--prefill-tokens", type=int, default=2048,
+                    help="with --only-prefill: the length of the prompt (at most 8192, one step)")
     ap.add_argument("--only-prefill", action="store_true",
                     help="run nothing but the 2,048-token prefill (for profiling); prints its numbers")
     ap.add_argument("--side", choices=["7b", "32b", "f32"], help=argparse.SUPPRESS)
@@ -419,7 +421,9 @@ def main():
     runs = Runs(engine, cfg, context, args.dtype)
 
     if args.only_prefill:
-        print(json.dumps({"prefill": runs.prefill()}))
+        if not 0 < args.prefill_tokens <= min(FILL_TOKENS, context):
+            sys.exit(f"--prefill-tokens must be between 1 and {min(FILL_TOKENS, context)}")
+        print(json.dumps({"prefill": runs.prefill(args.prefill_tokens)}))
         return
 
     validation = dict(side_validation)
