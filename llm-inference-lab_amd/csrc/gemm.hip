@@ -4,7 +4,8 @@
 //
 //   bfloat16:  v_mfma_f32_16x16x32_bf16 everywhere.
 //     * tiled kernel: 256 threads = 4 waves, block tile 64x64 (waves 2x2), 64x128 or
-//       128x128 (waves 1x4, side by side along the columns), K step 64; x staged through
+//       128x128 (waves 1x4, side by side along the columns), or 512 threads = 8 waves on
+//       128x256 (1x8), K step 64; x staged through
 //       three stages of LDS (rows padded to 80 elements: a wave's 16-byte fragment reads
 //       then take 8.4 clocks, as lane-contiguous ones do; 9.5 with 72, 16 unpadded), its
 //       fragments read into registers half a tile ahead of their products, the fragments
@@ -614,31 +615,40 @@ static void launch_f32_rows(const float* A, const float* W, const EpiArgs& e, in
 constexpr int F32_ROWS_MAX = 64;     // up to here the few-row kernel (the tiled one would run on N / 64 blocks)
 
 // ================================================================ dispatch
-// Three tile shapes, all with four waves, x through LDS and W straight from the packed
-// matrix: 64 x 64 (waves 2 x 2) for small products, 64 x 128 and 128 x 128 with the waves
-// side by side along the columns (1 x 4), so that every fragment of W is read by one wave
-// only and the rows of x in LDS are shared by all four.  The shape is picked by an
-// estimate of the time, fitted to sweeps of the four products of a layer at three model
-// shapes and 576 to 8192 rows (its picks cost 0.7 % over the best shape there):
+// Four tile shapes, x through LDS and W straight from the packed matrix: 64 x 64 (four
+// waves 2 x 2) for small products; 64 x 128 and 128 x 128 with four waves and 128 x 256
+// with eight, side by side along the columns (1 x 4, 1 x 8), so that every fragment of W
+// is read by one wave only and the rows of x in LDS are shared by all of them.  The shape
+// is picked by an estimate of the time, fitted to sweeps of the four products of a layer
+// at three model shapes and 576 to 8192 rows (its picks cost 0.8 % over the best shape
+// there):
 //   time = L + rounds * (f + K tiles * tk),  rounds = max(1, blocks / (units * resident)).
+// One block of the 128 x 256 tile fills a compute unit (its epilogue stages 133 KB), so
+// its rounds are whole: ceil(blocks / units).  Where its blocks fill their rounds it is
+// the fastest by 5 to 20 % (2048 rows, 3584 x 18944: 301 us against 337 with 128 x 128;
+// 8192 rows, 37888 x 3584: 2320 against 2577), where the last round is nearly empty the
+// slowest (2048 rows, 5120 x 27648: 852 against 731).
 // With few rows the product is bound by the read of W instead: a block draws `stream`
 // bytes a microsecond, the chip 5.3e6 at most (one tile of rows, 17 to 64 of them, of
 // matrices from 9 to 283 MB, in 4 or 8 pieces: the estimate is within 2 us of the
 // measurement).
-enum { TILE_64 = 0, TILE_64x128 = 1, TILE_128 = 2 };
+enum { TILE_64 = 0, TILE_64x128 = 1, TILE_128 = 2, TILE_128x256 = 3, TILE_KINDS = 4 };
 struct TileModel {
   int bm, bn;
   double L, f, tk, resident, stream;
+  int whole_rounds;
 };
-static const TileModel TILE_MODELS[3] = {{64, 64, 6.39, 0.79, 0.289, 1.0, 20e3},
-                                         {64, 128, 6.54, 0.71, 0.5, 1.5, 27e3},
-                                         {128, 128, 8.0, 0.48, 0.66, 1.0, 24e3}};
+static const TileModel TILE_MODELS[TILE_KINDS] = {{64, 64, 6.39, 0.79, 0.289, 1.0, 20e3, 0},
+                                                  {64, 128, 6.54, 0.71, 0.5, 1.5, 27e3, 0},
+                                                  {128, 128, 8.0, 0.48, 0.66, 1.0, 24e3, 0},
+                                                  {128, 256, 0.0, 6.16, 0.945, 1.0, 24e3, 1}};
 constexpr double CHIP_STREAM = 5.3e6;     // bytes a microsecond
 
 static double tile_cost(int kind, int M, int N, int K, int num_cus, int pieces) {
   const TileModel& t = TILE_MODELS[kind];
   const double blocks = (double)((M + t.bm - 1) / t.bm) * ((N + t.bn - 1) / t.bn) * pieces;
-  const double rounds = blocks / (num_cus * t.resident);
+  double rounds = blocks / (num_cus * t.resident);
+  if (t.whole_rounds) rounds = ceil(rounds - 1e-9);
   const int nk = ((K + 63) / 64 + pieces - 1) / pieces;
   const double compute = (rounds > 1.0 ? rounds : 1.0) * (t.f + nk * t.tk);
   const double rate = blocks * t.stream < CHIP_STREAM ? blocks * t.stream : CHIP_STREAM;
@@ -647,14 +657,19 @@ static double tile_cost(int kind, int M, int N, int K, int num_cus, int pieces) 
 }
 
 // Debug interface (kernels/debug.py): a tile can be forced, for tests and measurements
-// (0 = choose; 64, 130 = 64 x 128, 129 = 128 x 128).
-static int g_force_tile = 0;
-extern "C" void llmlab_debug_gemm_tile(int tile) { g_force_tile = tile; }
+// (0 = choose; 64, 130 = 64 x 128, 129 = 128 x 128, 131 = 128 x 256; -131 = choose among
+// the other three).
+static int g_force_tile = 0, g_without_wide = 0;
+extern "C" void llmlab_debug_gemm_tile(int tile) {
+  g_force_tile = tile > 0 ? tile : 0;
+  g_without_wide = tile == -131;
+}
 
 static int choose_tile(int M, int N, int K, int num_cus) {
   if (g_force_tile == 64) return TILE_64;
   if (g_force_tile == 130) return TILE_64x128;
   if (g_force_tile == 129 || g_force_tile == 128) return TILE_128;
+  if (g_force_tile == 131) return TILE_128x256;
   // One or two tiles of rows of a wide matrix (the head, gate and up at larger shapes):
   // bound by the read of W, which the wider tiles stream better than the estimate
   // knows, and the 128-row tile reads W once where two 64-row tiles read it twice
@@ -663,19 +678,23 @@ static int choose_tile(int M, int N, int K, int num_cus) {
   const long wide = (N + 127) / 128;
   if (M <= 64 && wide >= num_cus) return TILE_64x128;
   if (M > 64 && M <= 128 && wide >= 3L * num_cus / 2) return TILE_128;
-  // Enough 128 x 128 tiles for four rounds of blocks: the large tile, whatever the
+  // The 128 x 256 tile from 2048 rows on: with 576 and 1024 rows it wins or loses a few
+  // percent by the product alone, and a prefill step of 1024 tokens as a whole is 1 to
+  // 2 % slower with it than without (steps of 2048: from 0.6 % slower to 3 % faster by
+  // the shape of the model, of 4096 and 8192: 3 to 7 % faster at the larger shapes), and
+  // an inner size of 1024 on: with 896 its one block per unit shows its start and its
+  // epilogue, and steps of 4096 are 1.7 % slower with it.
+  const int kinds = M >= 2048 && K >= 1024 && !g_without_wide ? TILE_KINDS : TILE_128x256;
+  double cost[TILE_KINDS];
+  int best = 0;
+  for (int kind = 0; kind < kinds; ++kind) {
+    cost[kind] = tile_cost(kind, M, N, K, num_cus, 1);
+    if (cost[kind] < cost[best]) best = kind;
+  }
+  // Enough 128 x 128 tiles for four rounds of blocks: a large tile, whatever the
   // estimate makes of the rows it pads (576 rows, 37888 x 3584: 206 us against 221 with
   // 64 x 128; 1024 rows: 324 against 370).
-  if (((long)(M + 127) / 128) * wide >= 4L * num_cus) return TILE_128;
-  int best = 0;
-  double best_cost = 1e30;
-  for (int kind = 0; kind < 3; ++kind) {
-    const double c = tile_cost(kind, M, N, K, num_cus, 1);
-    if (c < best_cost) {
-      best_cost = c;
-      best = kind;
-    }
-  }
+  if (((long)(M + 127) / 128) * wide >= 4L * num_cus && best != TILE_128x256) return TILE_128;
   return best;
 }
 
@@ -688,8 +707,10 @@ static void launch_tile(int kind, const bf16_t* A, const bf16_t* W, const EpiArg
     hipLaunchKernelGGL((gemm_bf16_tiled<64, 64, 64, 2, 2, EPI>), grid, dim3(256), 0, stream, A, W, e, M, N, K);
   else if (kind == TILE_64x128)
     hipLaunchKernelGGL((gemm_bf16_tiled<64, 128, 64, 1, 4, EPI>), grid, dim3(256), 0, stream, A, W, e, M, N, K);
-  else
+  else if (kind == TILE_128)
     hipLaunchKernelGGL((gemm_bf16_tiled<128, 128, 64, 1, 4, EPI>), grid, dim3(256), 0, stream, A, W, e, M, N, K);
+  else
+    hipLaunchKernelGGL((gemm_bf16_tiled<128, 256, 64, 1, 8, EPI>), grid, dim3(512), 0, stream, A, W, e, M, N, K);
 }
 
 // Whether (and into how many pieces along K) a product that adds into float32 rows should
@@ -751,7 +772,7 @@ extern "C" int llmlab_linear_qkv(const void* x, const void* w, const void* bias,
   return 0;
 }
 
-// The width of the tile (64 or 128 columns) that a product of these sizes gets: for
+// The width of the tile (64, 128 or 256 columns) that a product of these sizes gets: for
 // callers that must know whether a head fits it.
 extern "C" int llmlab_linear_tile(int M, int N, int K, int num_cus) {
   if (num_cus <= 0) num_cus = 256;
@@ -766,7 +787,7 @@ extern "C" int llmlab_linear_partials(const void* x, const void* w, float* parts
   LLMLAB_REQUIRE(M >= 0 && N > 0 && K > 0 && K % 8 == 0, "linear_partials: bad sizes M=%d N=%d K=%d", M, N, K);
   LLMLAB_REQUIRE(ksplit >= 1 && ksplit <= 16 && ldo >= N && part_stride >= (size_t)M * ldo,
                  "linear_partials: %d pieces, row stride %d", ksplit, ldo);
-  LLMLAB_REQUIRE(tile >= TILE_64 && tile <= TILE_128, "linear_partials: unknown tile %d", tile);
+  LLMLAB_REQUIRE(tile >= TILE_64 && tile < TILE_KINDS, "linear_partials: unknown tile %d", tile);
   LLMLAB_REQUIRE(((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0),
                  "linear_partials: operands must be 16-byte aligned");
   if (M == 0) return 0;
