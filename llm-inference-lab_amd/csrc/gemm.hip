@@ -693,8 +693,17 @@ static int choose_tile(int M, int N, int K, int num_cus) {
   }
   // Enough 128 x 128 tiles for four rounds of blocks: a large tile, whatever the
   // estimate makes of the rows it pads (576 rows, 37888 x 3584: 206 us against 221 with
-  // 64 x 128; 1024 rows: 324 against 370).
-  if (((long)(M + 127) / 128) * wide >= 4L * num_cus && best != TILE_128x256) return TILE_128;
+  // 64 x 128; 1024 rows: 324 against 370).  Which of the two, the estimates cannot tell
+  // here (they err by 10 % in opposite directions): the 128 x 256 tile unless its last
+  // round is less than half full and one of few (2048 rows, 37888 x 3584, 9.25 rounds:
+  // 640 us against 588 inside a prefill step; 18.5 rounds: 1246 against 1273; 37: 2302
+  // against 2517; 3.5 rounds, 7168 x 5120: 359 against 379).
+  if (((long)(M + 127) / 128) * wide >= 4L * num_cus) {
+    if (kinds <= TILE_128x256) return TILE_128;
+    const double rounds = (double)((M + 127) / 128) * ((N + 255) / 256) / num_cus;
+    const double last = rounds - floor(rounds);
+    return (last < 1e-9 || last >= 0.5 || rounds >= 16.0) ? TILE_128x256 : TILE_128;
+  }
   return best;
 }
 
