@@ -25,6 +25,10 @@
 //       2.0 GHz under this load): matrix pipes busy 40 % of the time, LDS 52 % (and
 //       counted in bank conflicts for another 21 %), the texture address units 56 %: no
 //       unit is the limit alone, the waves wait for one another's turns at three of them.
+//     * the largest products (from 1024 rows on, where its blocks fill the chip): a 256x256
+//       tile whose eight waves form two groups that alternate between reading LDS and
+//       issuing MFMAs, both operands loaded from global memory straight into LDS
+//       (gemm_bf16_pingpong): 1.1 to 1.17 PF/s where the tiles above reach 0.9 to 0.97.
 //     (products of few rows, as in decode steps, have kernels of their own in decode.hip)
 //   float32: a plain FMA kernel (tiles of 64x64 to 128x128, 4x4 to 8x8 outputs per thread) and, for up to 64
 //     rows, one in which a wave owns four rows of W and its lanes split the inner size:
@@ -81,6 +85,144 @@ __device__ __forceinline__ void epi_store(const EpiArgs& e, int m, int n, float 
     ((float*)e.out)[at] += acc;
   else
     ((float*)e.out)[at] = acc;
+}
+
+// The epilogue of a tile of BM x BN sums that lies in LDS (rows of BN + 4 floats), by the NT
+// threads of the block: global memory is written (and the residual read) in pieces of 16 bytes,
+// consecutive lanes next to each other.  s_pos, s_page, s_freq and s_bias are what the QKV
+// epilogue fetched per row and per column of the tile before the product.
+template <int BM, int BN, int NT, int EPI>
+__device__ __forceinline__ void tile_epilogue(const float* Cs, const EpiArgs& e, int m0, int n0, int M, int N,
+                                              int tid, const int* s_pos, const int* s_page, const float* s_freq,
+                                              const float* s_bias) {
+  constexpr int C_STRIDE = BN + 4;
+  if constexpr (EPI == EPI_QKV) {
+    // a unit of work: four pairs (i .. i+3, and those + d/2) of one head of one row
+    const int d = e.d, dh = d >> 1, heads = BN / d, cpl = dh >> 2;
+    const int units = BM * heads * cpl;
+    const bool vec = (e.ldo & 3) == 0 && ((uintptr_t)e.out & 7) == 0;
+    for (int u = tid; u < units; u += NT) {
+      const int jc = u % cpl, t = u / cpl, hh = t % heads, row = t / heads;
+      const int m = m0 + row, head = n0 / d + hh, i = jc * 4;
+      if (m >= M || head >= e.nq + 2 * e.nkv) continue;
+      const float* src = Cs + row * C_STRIDE + hh * d + i;
+      floatx4 lo = *(const floatx4*)src, hi = *(const floatx4*)(src + dh);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        lo[q] += s_bias[hh * d + i + q];
+        hi[q] += s_bias[hh * d + dh + i + q];
+      }
+      const bool is_q = head < e.nq, is_k = !is_q && head < e.nq + e.nkv;
+      const int pos = s_pos[row];
+      if ((is_q || is_k) && e.inv_freq) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          // the hardware sine and cosine of r = frac(angle / 2 pi)
+          float r = (float)pos * s_freq[i + q] * 0.15915494309189535f;
+          r -= floorf(r);
+          const float sn = __builtin_amdgcn_sinf(r), cs = __builtin_amdgcn_cosf(r);
+          const float nlo = lo[q] * cs - hi[q] * sn, nhi = hi[q] * cs + lo[q] * sn;
+          lo[q] = nlo;
+          hi[q] = nhi;
+        }
+      }
+      bf16x4 blo, bhi;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        blo[q] = (bf16_t)lo[q];
+        bhi[q] = (bf16_t)hi[q];
+      }
+      if (is_q) {
+        bf16_t* dst = (bf16_t*)e.out + (size_t)m * e.ldo + (size_t)head * d + i;
+        if (vec) {
+          *(bf16x4*)dst = blo;
+          *(bf16x4*)(dst + dh) = bhi;
+        } else {
+          for (int q = 0; q < 4; ++q) {
+            dst[q] = blo[q];
+            dst[dh + q] = bhi[q];
+          }
+        }
+      } else if (e.kcache) {
+        const size_t page = (size_t)s_page[row];
+        const int off = pos % e.page_size;
+        if (is_k) {
+          // four neighbours of one octet of d lie next to each other in the key order
+          bf16_t* dst = e.kcache + (page * e.nkv + (head - e.nq)) * (size_t)e.page_size * d;
+          *(bf16x4*)(dst + kcache_index(off, i, d)) = blo;
+          *(bf16x4*)(dst + kcache_index(off, i + dh, d)) = bhi;
+        } else {
+          bf16_t* dst = e.vcache + (page * e.nkv + (head - e.nq - e.nkv)) * (size_t)e.page_size * d;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            dst[vcache_index(off, i + q, d)] = blo[q];
+            dst[vcache_index(off, i + dh + q, d)] = bhi[q];
+          }
+        }
+      }
+    }
+  } else if constexpr (EPI == EPI_SWIGLU) {
+    // columns of the tile alternate in runs of 16: gate, up of the same 16 outputs
+    constexpr int OUTS = BN / 2, CH = OUTS / 8;      // outputs per row of the tile, chunks of 8 of them
+    bf16_t* out = (bf16_t*)e.out;
+    const int o0 = n0 >> 1;
+    const bool vec = (e.ldo & 7) == 0 && ((uintptr_t)out & 15) == 0;
+    for (int ch = tid; ch < BM * CH; ch += NT) {
+      const int row = ch / CH, oc = (ch % CH) * 8;      // 8 outputs within one run of 16
+      const int m = m0 + row;
+      if (m >= M) continue;
+      const float* gp = Cs + row * C_STRIDE + (oc >> 4) * 32 + (oc & 15);
+      const floatx4 g0 = *(const floatx4*)gp, g1 = *(const floatx4*)(gp + 4);
+      const floatx4 u0 = *(const floatx4*)(gp + 16), u1 = *(const floatx4*)(gp + 20);
+      bf16x8 v;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        v[q] = (bf16_t)(silu_f(g0[q]) * u0[q]);
+        v[4 + q] = (bf16_t)(silu_f(g1[q]) * u1[q]);
+      }
+      bf16_t* dst = out + (size_t)m * e.ldo + o0 + oc;
+      if (vec && o0 + oc + 8 <= e.n_out) *(bf16x8*)dst = v;
+      else
+        for (int q = 0; q < 8; ++q)
+          if (o0 + oc + q < e.n_out) dst[q] = v[q];
+    }
+  } else {
+    constexpr int CH = BN / 4;                         // chunks of 4 columns per row of the tile
+    constexpr bool OUT32 = EPI != EPI_STORE;
+    const bool vec = (e.ldo & 3) == 0 && ((uintptr_t)e.out & 15) == 0 && (OUT32 || (e.ldo & 7) == 0);
+    for (int ch = tid; ch < BM * CH; ch += NT) {
+      const int row = ch / CH, col = (ch % CH) * 4;
+      const int m = m0 + row, n = n0 + col;
+      if (m >= M || n >= N) continue;
+      floatx4 v = *(const floatx4*)(Cs + row * C_STRIDE + col);
+      if (e.bias)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) v[q] += load_vec(e.bias, e.bias_bf16, min(n + q, N - 1));
+      const size_t at = (size_t)m * e.ldo + n;
+      const bool whole = vec && n + 4 <= N;
+      if constexpr (EPI == EPI_STORE) {
+        bf16_t* dst = (bf16_t*)e.out + at;
+        if (whole) {
+          bf16x4 o;
+#pragma unroll
+          for (int q = 0; q < 4; ++q) o[q] = (bf16_t)v[q];
+          *(bf16x4*)dst = o;
+        } else {
+          for (int q = 0; q < 4; ++q)
+            if (n + q < N) dst[q] = (bf16_t)v[q];
+        }
+      } else {
+        float* dst = (float*)e.out + at;
+        if (whole) {
+          if constexpr (EPI == EPI_RESID) v += *(const floatx4*)dst;
+          *(floatx4*)dst = v;
+        } else {
+          for (int q = 0; q < 4; ++q)
+            if (n + q < N) dst[q] = (EPI == EPI_RESID ? dst[q] : 0.f) + v[q];
+        }
+      }
+    }
+  }
 }
 
 // ============================================================ bf16, tiled
@@ -271,132 +413,170 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __
       for (int x = 0; x < 4; ++x)
         Cs[(wm * WTM + i * 16 + g * 4 + x) * C_STRIDE + wn * WTN + j * 16 + c] = acc[i][j][x];
   __syncthreads();
-  if constexpr (EPI == EPI_QKV) {
-    // a unit of work: four pairs (i .. i+3, and those + d/2) of one head of one row
-    const int d = e.d, dh = d >> 1, heads = BN / d, cpl = dh >> 2;
-    const int units = BM * heads * cpl;
-    const bool vec = (e.ldo & 3) == 0 && ((uintptr_t)e.out & 7) == 0;
-    for (int u = tid; u < units; u += NT) {
-      const int jc = u % cpl, t = u / cpl, hh = t % heads, row = t / heads;
-      const int m = m0 + row, head = n0 / d + hh, i = jc * 4;
-      if (m >= M || head >= e.nq + 2 * e.nkv) continue;
-      const float* src = Cs + row * C_STRIDE + hh * d + i;
-      floatx4 lo = *(const floatx4*)src, hi = *(const floatx4*)(src + dh);
+  tile_epilogue<BM, BN, NT, EPI>(Cs, e, m0, n0, M, N, tid, s_pos, s_page, s_freq, s_bias);
+}
+
+// ============================================================ bf16, 256 x 256 by two groups of waves
+// The largest products.  Eight waves, each with a 128 x 64 part of a 256 x 256 tile; both
+// operands come by direct loads from global memory into LDS (no registers in between), in
+// steps of 32 of the inner size, four stages of 32 KB.  The lanes of a load address the
+// 16-byte pieces of one MFMA fragment (16 rows of x, or one 1 KB tile of the packed W), which
+// the hardware lays down lane after lane: LDS holds fragments, and a fragment read is 1 KB
+// of consecutive bytes.  The waves form two groups with a wave on every SIMD each, half a
+// step apart: between two barriers one group reads its twelve fragments and issues its
+// loads while the other issues its 32 MFMAs, then they change roles, so that the reads of
+// LDS and the matrix instructions of a compute unit overlap by construction and not by
+// the luck of the scheduler (all eight waves in step: 975 TF/s on 8192 x 37888 x 3584,
+// the groups apart: 1065; the 128 x 256 tile of the kernel above: 966).  Under this load
+// the chip holds 1.45 to 1.85 GHz, and a step takes 1340 clocks where the MFMAs alone
+// need 1024.  A block fills a compute unit; the epilogue takes the two halves of the rows
+// through LDS one after the other.
+//
+// The direct loads are written in assembly: the compiler then knows nothing of them, the
+// waits (vmcnt) are placed by hand, and the loop holds no other load that it would count.
+template <int EPI>
+__global__ __launch_bounds__(512) void gemm_bf16_pingpong(const bf16_t* __restrict__ A,
+                                                          const bf16_t* __restrict__ W, EpiArgs e, int M,
+                                                          int N, int K) {
+  constexpr int BM = 256, BN = 256, NT = 512, HALF = 128;
+  constexpr int STAGE = (BM / 16 + BN / 16) * 1024;     // bytes: 16 fragments of x, then 16 of W
+  constexpr int C_STRIDE = BN + 4;
+  constexpr size_t C_BYTES = (size_t)HALF * C_STRIDE * sizeof(float);
+  static_assert(EPI != EPI_PART, "no pieces along K with this tile");
+  __shared__ __attribute__((aligned(1024))) char smem[C_BYTES > 4 * STAGE ? C_BYTES : 4 * STAGE];
+
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int grp = wave >> 2;                             // waves 0-3 and 4-7: one of each on every SIMD
+  const int wm = wave & 1, wn = ((wave >> 1) & 1) | (grp << 1);   // rows wm * 128, columns wn * 64
+  int bx = blockIdx.x, by = blockIdx.y;
+  {                                                      // a band of column tiles per die, as above
+    const int gx = gridDim.x, gy = gridDim.y, total = gx * gy;
+    const int lin = by * gx + bx;
+    const int whole = total & ~7;
+    const int mapped = lin < whole ? (lin & 7) * (whole >> 3) + (lin >> 3) : lin;
+    bx = mapped / gy;
+    by = mapped - bx * gy;
+  }
+  const int m0 = by * BM, n0 = bx * BN;
+  const int c = lane & 15, g = lane >> 4;
+
+  constexpr bool QKV = EPI == EPI_QKV;
+  __shared__ int s_pos[QKV ? BM : 1], s_page[QKV ? BM : 1];
+  __shared__ float s_freq[QKV ? 128 : 1], s_bias[QKV ? BN : 1];
+  if constexpr (QKV) {
+    if (tid < BM) {
+      const int m = min(m0 + tid, M - 1);
+      const int pos = e.positions[m];
+      s_pos[tid] = pos;
+      s_page[tid] = (e.kcache && n0 + BN > e.nq * e.d)
+                        ? e.table[(size_t)e.row_req[m] * e.table_stride + pos / e.page_size] : 0;
+    }
+    for (int i = tid; i < (e.d >> 1); i += NT) s_freq[i] = e.inv_freq ? e.inv_freq[i] : 0.f;
+    for (int i = tid; i < BN; i += NT)
+      s_bias[i] = (e.bias && n0 + i < N) ? load_vec(e.bias, e.bias_bf16, n0 + i) : 0.f;
+  }
+
+  // Per step a wave fetches four fragments: the even waves of x, the odd ones of W (so
+  // that both groups fetch both).  Rows past M, strips past N and pieces past K read a
+  // valid piece instead: they land in rows and columns that nobody stores, or meet the
+  // zeros of the padded W.
+  const int T = (K + 31) >> 5, nstrips = (N + 15) >> 4;
+  const bool fetches_x = (wave & 1) == 0;
+  const int quarter = wave >> 1;
+  const bf16_t* src[4];
+  unsigned dst[4];
+  const unsigned lds0 = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        lo[q] += s_bias[hh * d + i + q];
-        hi[q] += s_bias[hh * d + dh + i + q];
-      }
-      const bool is_q = head < e.nq, is_k = !is_q && head < e.nq + e.nkv;
-      const int pos = s_pos[row];
-      if ((is_q || is_k) && e.inv_freq) {
+  for (int i = 0; i < 4; ++i) {
+    const int f = quarter * 4 + i;
+    if (fetches_x) {
+      src[i] = A + (size_t)min(m0 + f * 16 + c, M - 1) * K;
+      dst[i] = lds0 + f * 1024;
+    } else {
+      src[i] = W + (size_t)min((n0 >> 4) + f, nstrips - 1) * T * 512 + lane * 8;
+      dst[i] = lds0 + (16 + f) * 1024;
+    }
+  }
+  auto fetch = [&](int stage, int t) {
+    const size_t off = fetches_x ? (size_t)min(t * 32 + g * 8, K - 8) : (size_t)t * 512;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-          // the hardware sine and cosine of r = frac(angle / 2 pi)
-          float r = (float)pos * s_freq[i + q] * 0.15915494309189535f;
-          r -= floorf(r);
-          const float sn = __builtin_amdgcn_sinf(r), cs = __builtin_amdgcn_cosf(r);
-          const float nlo = lo[q] * cs - hi[q] * sn, nhi = hi[q] * cs + lo[q] * sn;
-          lo[q] = nlo;
-          hi[q] = nhi;
-        }
-      }
-      bf16x4 blo, bhi;
+    for (int i = 0; i < 4; ++i)
+      asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                   :
+                   : "v"(src[i] + off), "s"(dst[i] + stage * STAGE)
+                   : "memory", "m0");
+  };
+
+  floatx4 acc[8][4];
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        blo[q] = (bf16_t)lo[q];
-        bhi[q] = (bf16_t)hi[q];
-      }
-      if (is_q) {
-        bf16_t* dst = (bf16_t*)e.out + (size_t)m * e.ldo + (size_t)head * d + i;
-        if (vec) {
-          *(bf16x4*)dst = blo;
-          *(bf16x4*)(dst + dh) = bhi;
-        } else {
-          for (int q = 0; q < 4; ++q) {
-            dst[q] = blo[q];
-            dst[dh + q] = bhi[q];
-          }
-        }
-      } else if (e.kcache) {
-        const size_t page = (size_t)s_page[row];
-        const int off = pos % e.page_size;
-        if (is_k) {
-          // four neighbours of one octet of d lie next to each other in the key order
-          bf16_t* dst = e.kcache + (page * e.nkv + (head - e.nq)) * (size_t)e.page_size * d;
-          *(bf16x4*)(dst + kcache_index(off, i, d)) = blo;
-          *(bf16x4*)(dst + kcache_index(off, i + dh, d)) = bhi;
-        } else {
-          bf16_t* dst = e.vcache + (page * e.nkv + (head - e.nq - e.nkv)) * (size_t)e.page_size * d;
+  for (int i = 0; i < 8; ++i)
 #pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            dst[vcache_index(off, i + q, d)] = blo[q];
-            dst[vcache_index(off, i + dh + q, d)] = bhi[q];
-          }
-        }
+    for (int j = 0; j < 4; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
+  bf16x8 a[8], b[4];
+
+  // every wave passes the same barriers; nothing may move across one
+  auto barrier = [&]() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("" ::: "memory");
+  };
+  constexpr int WAIT_ALL_BUT_TWO_STEPS = 0x0070 | 8;    // lgkmcnt(0), vmcnt(8): two steps of four loads
+  const int nk = T;
+  // Step t lies in stage t % 4.  A wave's memory phase of step t reads its fragments,
+  // issues its loads of step t + 3 (into the stage that both groups read last in step
+  // t - 1, at least one barrier ago) and waits for its own loads of step t + 1; the
+  // barrier after the other group's same phase then says that step t + 1 is whole.
+  fetch(0, 0);
+  fetch(1, min(1, nk - 1));
+  fetch(2, min(2, nk - 1));
+  __builtin_amdgcn_s_waitcnt(WAIT_ALL_BUT_TWO_STEPS);
+  barrier();
+  if (grp == 1) barrier();                               // the second group runs half a step behind
+  for (int t0 = 0; t0 < nk; t0 += 4) {
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int t = t0 + u;
+      if (t < nk) {                                      // (the same for every wave of the block)
+        const char* stage = smem + u * STAGE;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) b[j] = *(const bf16x8*)(stage + (16 + wn * 4 + j) * 1024 + lane * 16);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) a[i] = *(const bf16x8*)(stage + (wm * 8 + i) * 1024 + lane * 16);
+        fetch((u + 3) & 3, min(t + 3, nk - 1));
+        __builtin_amdgcn_s_waitcnt(WAIT_ALL_BUT_TWO_STEPS);
+        barrier();
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
+        barrier();
       }
     }
-  } else if constexpr (EPI == EPI_SWIGLU) {
-    // columns of the tile alternate in runs of 16: gate, up of the same 16 outputs
-    constexpr int OUTS = BN / 2, CH = OUTS / 8;      // outputs per row of the tile, chunks of 8 of them
-    bf16_t* out = (bf16_t*)e.out;
-    const int o0 = n0 >> 1;
-    const bool vec = (e.ldo & 7) == 0 && ((uintptr_t)out & 15) == 0;
-    for (int ch = tid; ch < BM * CH; ch += NT) {
-      const int row = ch / CH, oc = (ch % CH) * 8;      // 8 outputs within one run of 16
-      const int m = m0 + row;
-      if (m >= M) continue;
-      const float* gp = Cs + row * C_STRIDE + (oc >> 4) * 32 + (oc & 15);
-      const floatx4 g0 = *(const floatx4*)gp, g1 = *(const floatx4*)(gp + 4);
-      const floatx4 u0 = *(const floatx4*)(gp + 16), u1 = *(const floatx4*)(gp + 20);
-      bf16x8 v;
+  }
+  if (grp == 0) barrier();
+  __builtin_amdgcn_s_waitcnt(0x0070);                    // the last loads (past K, never read) are in
+  barrier();
+
+  // ---- epilogue: the rows 0-127 of the tile through LDS, then the rows 128-255
+  float* Cs = (float*)smem;
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        v[q] = (bf16_t)(silu_f(g0[q]) * u0[q]);
-        v[4 + q] = (bf16_t)(silu_f(g1[q]) * u1[q]);
-      }
-      bf16_t* dst = out + (size_t)m * e.ldo + o0 + oc;
-      if (vec && o0 + oc + 8 <= e.n_out) *(bf16x8*)dst = v;
-      else
-        for (int q = 0; q < 8; ++q)
-          if (o0 + oc + q < e.n_out) dst[q] = v[q];
+  for (int half = 0; half < 2; ++half) {
+    if (wm == half) {
+#pragma unroll
+      for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+          for (int x = 0; x < 4; ++x)
+            Cs[(i * 16 + g * 4 + x) * C_STRIDE + wn * 64 + j * 16 + c] = acc[i][j][x];
     }
-  } else {
-    constexpr int CH = BN / 4;                         // chunks of 4 columns per row of the tile
-    constexpr bool OUT32 = EPI != EPI_STORE;
-    const bool vec = (e.ldo & 3) == 0 && ((uintptr_t)e.out & 15) == 0 && (OUT32 || (e.ldo & 7) == 0);
-    for (int ch = tid; ch < BM * CH; ch += NT) {
-      const int row = ch / CH, col = (ch % CH) * 4;
-      const int m = m0 + row, n = n0 + col;
-      if (m >= M || n >= N) continue;
-      floatx4 v = *(const floatx4*)(Cs + row * C_STRIDE + col);
-      if (e.bias)
-#pragma unroll
-        for (int q = 0; q < 4; ++q) v[q] += load_vec(e.bias, e.bias_bf16, min(n + q, N - 1));
-      const size_t at = (size_t)m * e.ldo + n;
-      const bool whole = vec && n + 4 <= N;
-      if constexpr (EPI == EPI_STORE) {
-        bf16_t* dst = (bf16_t*)e.out + at;
-        if (whole) {
-          bf16x4 o;
-#pragma unroll
-          for (int q = 0; q < 4; ++q) o[q] = (bf16_t)v[q];
-          *(bf16x4*)dst = o;
-        } else {
-          for (int q = 0; q < 4; ++q)
-            if (n + q < N) dst[q] = (bf16_t)v[q];
-        }
-      } else {
-        float* dst = (float*)e.out + at;
-        if (whole) {
-          if constexpr (EPI == EPI_RESID) v += *(const floatx4*)dst;
-          *(floatx4*)dst = v;
-        } else {
-          for (int q = 0; q < 4; ++q)
-            if (n + q < N) dst[q] = (EPI == EPI_RESID ? dst[q] : 0.f) + v[q];
-        }
-      }
-    }
+    __syncthreads();
+    tile_epilogue<HALF, BN, NT, EPI>(Cs, e, m0 + half * HALF, n0, M, N, tid, s_pos + (QKV ? half * HALF : 0),
+                                     s_page + (QKV ? half * HALF : 0), s_freq, s_bias);
+    __syncthreads();
   }
 }
 
@@ -615,10 +795,11 @@ static void launch_f32_rows(const float* A, const float* W, const EpiArgs& e, in
 constexpr int F32_ROWS_MAX = 64;     // up to here the few-row kernel (the tiled one would run on N / 64 blocks)
 
 // ================================================================ dispatch
-// Four tile shapes, x through LDS and W straight from the packed matrix: 64 x 64 (four
+// Four tile shapes with x through LDS and W straight from the packed matrix: 64 x 64 (four
 // waves 2 x 2) for small products; 64 x 128 and 128 x 128 with four waves and 128 x 256
 // with eight, side by side along the columns (1 x 4, 1 x 8), so that every fragment of W
-// is read by one wave only and the rows of x in LDS are shared by all of them.  The shape
+// is read by one wave only and the rows of x in LDS are shared by all of them; and the
+// 256 x 256 tile of gemm_bf16_pingpong for the largest products.  The shape
 // is picked by an estimate of the time, fitted to sweeps of the four products of a layer
 // at three model shapes and 576 to 8192 rows (its picks cost 0.8 % over the best shape
 // there):
@@ -632,7 +813,7 @@ constexpr int F32_ROWS_MAX = 64;     // up to here the few-row kernel (the tiled
 // bytes a microsecond, the chip 5.3e6 at most (one tile of rows, 17 to 64 of them, of
 // matrices from 9 to 283 MB, in 4 or 8 pieces: the estimate is within 2 us of the
 // measurement).
-enum { TILE_64 = 0, TILE_64x128 = 1, TILE_128 = 2, TILE_128x256 = 3, TILE_KINDS = 4 };
+enum { TILE_64 = 0, TILE_64x128 = 1, TILE_128 = 2, TILE_128x256 = 3, TILE_256 = 4, TILE_KINDS = 5 };
 struct TileModel {
   int bm, bn;
   double L, f, tk, resident, stream;
@@ -641,10 +822,24 @@ struct TileModel {
 static const TileModel TILE_MODELS[TILE_KINDS] = {{64, 64, 6.39, 0.79, 0.289, 1.0, 20e3, 0},
                                                   {64, 128, 6.54, 0.71, 0.5, 1.5, 27e3, 0},
                                                   {128, 128, 8.0, 0.48, 0.66, 1.0, 24e3, 0},
-                                                  {128, 256, 0.0, 6.16, 0.945, 1.0, 24e3, 1}};
+                                                  {128, 256, 0.0, 6.16, 0.945, 1.0, 24e3, 1},
+                                                  {256, 256, 0.0, 9.2, 1.8, 1.0, 24e3, 1}};
 constexpr double CHIP_STREAM = 5.3e6;     // bytes a microsecond
 
+// The 256 x 256 tile: whole rounds of one block a unit, a step of 32 of the inner size
+// 0.82 us in a full round and from 0.51 us in a round of few blocks (the chip clocks
+// higher), 9.3 us before and after the loop (fitted to the same sweeps: 6 % rms).
+static double pingpong_cost(int M, int N, int K, int num_cus) {
+  const double rounds = (double)((M + 255) / 256) * ((N + 255) / 256) / num_cus;
+  const double whole = floor(rounds + 1e-9), last = rounds - whole;
+  const int steps = (K + 31) / 32;
+  double t = 0.7 + whole * (9.3 + steps * 0.824);
+  if (last > 1e-9) t += 9.3 + steps * (0.506 + (0.824 - 0.506) * last);
+  return t;
+}
+
 static double tile_cost(int kind, int M, int N, int K, int num_cus, int pieces) {
+  if (kind == TILE_256) return pingpong_cost(M, N, K, num_cus);
   const TileModel& t = TILE_MODELS[kind];
   const double blocks = (double)((M + t.bm - 1) / t.bm) * ((N + t.bn - 1) / t.bn) * pieces;
   double rounds = blocks / (num_cus * t.resident);
@@ -657,8 +852,8 @@ static double tile_cost(int kind, int M, int N, int K, int num_cus, int pieces) 
 }
 
 // Debug interface (kernels/debug.py): a tile can be forced, for tests and measurements
-// (0 = choose; 64, 130 = 64 x 128, 129 = 128 x 128, 131 = 128 x 256; -131 = choose among
-// the other three).
+// (0 = choose; 64, 130 = 64 x 128, 129 = 128 x 128, 131 = 128 x 256, 132 = 256 x 256; -131 =
+// choose among the first three).
 static int g_force_tile = 0, g_without_wide = 0;
 extern "C" void llmlab_debug_gemm_tile(int tile) {
   g_force_tile = tile > 0 ? tile : 0;
@@ -670,6 +865,7 @@ static int choose_tile(int M, int N, int K, int num_cus) {
   if (g_force_tile == 130) return TILE_64x128;
   if (g_force_tile == 129 || g_force_tile == 128) return TILE_128;
   if (g_force_tile == 131) return TILE_128x256;
+  if (g_force_tile == 132) return TILE_256;
   // One or two tiles of rows of a wide matrix (the head, gate and up at larger shapes):
   // bound by the read of W, which the wider tiles stream better than the estimate
   // knows, and the 128-row tile reads W once where two 64-row tiles read it twice
@@ -684,7 +880,7 @@ static int choose_tile(int M, int N, int K, int num_cus) {
   // the shape of the model, of 4096 and 8192: 3 to 7 % faster at the larger shapes), and
   // an inner size of 1024 on: with 896 its one block per unit shows its start and its
   // epilogue, and steps of 4096 are 1.7 % slower with it.
-  const int kinds = M >= 2048 && K >= 1024 && !g_without_wide ? TILE_KINDS : TILE_128x256;
+  const int kinds = M >= 2048 && K >= 1024 && !g_without_wide ? TILE_256 : TILE_128x256;
   double cost[TILE_KINDS];
   int best = 0;
   for (int kind = 0; kind < kinds; ++kind) {
@@ -699,11 +895,23 @@ static int choose_tile(int M, int N, int K, int num_cus) {
   // 640 us against 588 inside a prefill step; 18.5 rounds: 1246 against 1273; 37: 2302
   // against 2517; 3.5 rounds, 7168 x 5120: 359 against 379).
   if (((long)(M + 127) / 128) * wide >= 4L * num_cus) {
-    if (kinds <= TILE_128x256) return TILE_128;
-    const double rounds = (double)((M + 127) / 128) * ((N + 255) / 256) / num_cus;
-    const double last = rounds - floor(rounds);
-    return (last < 1e-9 || last >= 0.5 || rounds >= 16.0) ? TILE_128x256 : TILE_128;
+    best = TILE_128;
+    if (kinds > TILE_128x256) {
+      const double rounds = (double)((M + 127) / 128) * ((N + 255) / 256) / num_cus;
+      const double last = rounds - floor(rounds);
+      if (last < 1e-9 || last >= 0.5 || rounds >= 16.0) best = TILE_128x256;
+    }
   }
+  // The 256 x 256 tile of the two groups of waves where its estimate is the lower one
+  // (over the sweeps it is then 10 to 24 % faster than the best of the others: 2048 rows,
+  // 37888 x 3584: 501 us against 623; 55296 x 5120: 999 against 1245; 576 rows, 37888 x
+  // 3584: 178 against 195; with a quarter of a round of blocks it is twice as slow).
+  // From 1024 rows on, and with an inner size below 1024 from 2048 rows on: by the products
+  // alone it would win from 576 rows, but a step of 576 rows as a whole is 1.5 % slower
+  // with it at the 7B shape, one of 1024 rows 3 % slower at the 0.5B shape.
+  if (M >= 1024 && (K >= 1024 || M >= 2048) && !g_without_wide &&
+      pingpong_cost(M, N, K, num_cus) < tile_cost(best, M, N, K, num_cus, 1))
+    best = TILE_256;
   return best;
 }
 
@@ -718,8 +926,10 @@ static void launch_tile(int kind, const bf16_t* A, const bf16_t* W, const EpiArg
     hipLaunchKernelGGL((gemm_bf16_tiled<64, 128, 64, 1, 4, EPI>), grid, dim3(256), 0, stream, A, W, e, M, N, K);
   else if (kind == TILE_128)
     hipLaunchKernelGGL((gemm_bf16_tiled<128, 128, 64, 1, 4, EPI>), grid, dim3(256), 0, stream, A, W, e, M, N, K);
-  else
+  else if (kind == TILE_128x256)
     hipLaunchKernelGGL((gemm_bf16_tiled<128, 256, 64, 1, 8, EPI>), grid, dim3(512), 0, stream, A, W, e, M, N, K);
+  else if constexpr (EPI != EPI_PART)
+    hipLaunchKernelGGL((gemm_bf16_pingpong<EPI>), grid, dim3(512), 0, stream, A, W, e, M, N, K);
 }
 
 // Whether (and into how many pieces along K) a product that adds into float32 rows should
@@ -749,6 +959,7 @@ extern "C" void llmlab_linear_plan(int M, int N, int K, int num_cus, int max_pie
   // 15.8, 15.1 against 18.8 us; with more blocks than units it is the slower one)
   if (M <= 64 && best_pieces > 1 && g_force_tile == 0 && (long)((N + 63) / 64) * best_pieces <= num_cus)
     best_kind = TILE_64;
+  if (best_kind == TILE_256) best_kind = TILE_128x256;   // (the 256 x 256 tile makes no pieces)
   out[0] = best_pieces;
   out[1] = best_kind;
 }
@@ -796,7 +1007,7 @@ extern "C" int llmlab_linear_partials(const void* x, const void* w, float* parts
   LLMLAB_REQUIRE(M >= 0 && N > 0 && K > 0 && K % 8 == 0, "linear_partials: bad sizes M=%d N=%d K=%d", M, N, K);
   LLMLAB_REQUIRE(ksplit >= 1 && ksplit <= 16 && ldo >= N && part_stride >= (size_t)M * ldo,
                  "linear_partials: %d pieces, row stride %d", ksplit, ldo);
-  LLMLAB_REQUIRE(tile >= TILE_64 && tile < TILE_KINDS, "linear_partials: unknown tile %d", tile);
+  LLMLAB_REQUIRE(tile >= TILE_64 && tile <= TILE_128x256, "linear_partials: unknown tile %d", tile);
   LLMLAB_REQUIRE(((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0),
                  "linear_partials: operands must be 16-byte aligned");
   if (M == 0) return 0;
