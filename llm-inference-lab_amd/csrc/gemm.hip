@@ -906,10 +906,13 @@ static int choose_tile(int M, int N, int K, int num_cus) {
   // (over the sweeps it is then 10 to 24 % faster than the best of the others: 2048 rows,
   // 37888 x 3584: 501 us against 623; 55296 x 5120: 999 against 1245; 576 rows, 37888 x
   // 3584: 178 against 195; with a quarter of a round of blocks it is twice as slow).
-  // From 1024 rows on, and with an inner size below 1024 from 2048 rows on: by the products
-  // alone it would win from 576 rows, but a step of 576 rows as a whole is 1.5 % slower
-  // with it at the 7B shape, one of 1024 rows 3 % slower at the 0.5B shape.
-  if (M >= 1024 && (K >= 1024 || M >= 2048) && !g_without_wide &&
+  // From 1024 rows and an inner size of 1024 on: by the products alone it would win from
+  // 576 rows and with an inner size of 896 too, but a step of 576 rows as a whole is 1.5 %
+  // slower with it at the 7B shape, steps of 1024 and 4096 rows 1 to 3 % at the 0.5B shape.
+  // (The same two groups of waves on a 128 x 256 tile, 64 x 64 a wave, are as fast as the
+  // 128 x 256 tile above and no faster: a wave then reads as many bytes from LDS per MFMA
+  // as there, and LDS is the limit of both.)
+  if (M >= 1024 && K >= 1024 && !g_without_wide &&
       pingpong_cost(M, N, K, num_cus) < tile_cost(best, M, N, K, num_cus, 1))
     best = TILE_256;
   return best;
