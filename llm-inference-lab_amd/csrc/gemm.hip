@@ -434,12 +434,18 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_bf16_tiled(const bf16_t* __
 //
 // The direct loads are written in assembly: the compiler then knows nothing of them, the
 // waits (vmcnt) are placed by hand, and the loop holds no other load that it would count.
-template <int EPI>
+//
+// BM = 192 is the same with 96 x 64 a wave, for steps whose rows fill tiles of 192 better
+// than tiles of 256 (576 rows: three tiles instead of three of which one is a quarter full).
+template <int BM, int EPI>
 __global__ __launch_bounds__(512) void gemm_bf16_pingpong(const bf16_t* __restrict__ A,
                                                           const bf16_t* __restrict__ W, EpiArgs e, int M,
                                                           int N, int K) {
-  constexpr int BM = 256, BN = 256, NT = 512, HALF = 128;
-  constexpr int STAGE = (BM / 16 + BN / 16) * 1024;     // bytes: 16 fragments of x, then 16 of W
+  static_assert(BM == 256 || BM == 192, "a wave has 128 or 96 rows");
+  constexpr int BN = 256, NT = 512, HALF = 128;
+  constexpr int TM = BM / 32;                           // blocks of 16 rows of a wave
+  constexpr int XF = BM / 16;                           // fragments of x in a step
+  constexpr int STAGE = (XF + BN / 16) * 1024;          // bytes: the fragments of x, then 16 of W
   constexpr int C_STRIDE = BN + 4;
   constexpr size_t C_BYTES = (size_t)HALF * C_STRIDE * sizeof(float);
   static_assert(EPI != EPI_PART, "no pieces along K with this tile");
@@ -447,7 +453,7 @@ __global__ __launch_bounds__(512) void gemm_bf16_pingpong(const bf16_t* __restri
 
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int grp = wave >> 2;                             // waves 0-3 and 4-7: one of each on every SIMD
-  const int wm = wave & 1, wn = ((wave >> 1) & 1) | (grp << 1);   // rows wm * 128, columns wn * 64
+  const int wm = wave & 1, wn = ((wave >> 1) & 1) | (grp << 1);   // rows wm * BM / 2, columns wn * 64
   int bx = blockIdx.x, by = blockIdx.y;
   {                                                      // a band of column tiles per die, as above
     const int gx = gridDim.x, gy = gridDim.y, total = gx * gy;
@@ -476,43 +482,58 @@ __global__ __launch_bounds__(512) void gemm_bf16_pingpong(const bf16_t* __restri
       s_bias[i] = (e.bias && n0 + i < N) ? load_vec(e.bias, e.bias_bf16, n0 + i) : 0.f;
   }
 
-  // Per step a wave fetches four fragments: the even waves of x, the odd ones of W (so
-  // that both groups fetch both).  Rows past M, strips past N and pieces past K read a
+  // Per step a wave fetches four fragments (three of x with BM = 192): the even waves of x,
+  // the odd ones of W (so that both groups fetch both).  Rows past M, strips past N and pieces past K read a
   // valid piece instead: they land in rows and columns that nobody stores, or meet the
   // zeros of the padded W.
   const int T = (K + 31) >> 5, nstrips = (N + 15) >> 4;
   const bool fetches_x = (wave & 1) == 0;
   const int quarter = wave >> 1;
+  constexpr int NFX = XF / 4;                           // fragments of x that one of its four waves fetches
   const bf16_t* src[4];
   unsigned dst[4];
   const unsigned lds0 = (unsigned)(uintptr_t)(__attribute__((address_space(3))) char*)smem;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const int f = quarter * 4 + i;
     if (fetches_x) {
+      const int f = min(quarter * NFX + i, XF - 1);
       src[i] = A + (size_t)min(m0 + f * 16 + c, M - 1) * K;
       dst[i] = lds0 + f * 1024;
     } else {
+      const int f = quarter * 4 + i;
       src[i] = W + (size_t)min((n0 >> 4) + f, nstrips - 1) * T * 512 + lane * 8;
-      dst[i] = lds0 + (16 + f) * 1024;
+      dst[i] = lds0 + (XF + f) * 1024;
     }
   }
+  auto load_to_lds = [&](const bf16_t* from, unsigned to) {
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                 :
+                 : "v"(from), "s"(to)
+                 : "memory", "m0");
+  };
   auto fetch = [&](int stage, int t) {
-    const size_t off = fetches_x ? (size_t)min(t * 32 + g * 8, K - 8) : (size_t)t * 512;
+    if (fetches_x) {
+      const size_t off = (size_t)min(t * 32 + g * 8, K - 8);
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
-                   :
-                   : "v"(src[i] + off), "s"(dst[i] + stage * STAGE)
-                   : "memory", "m0");
+      for (int i = 0; i < NFX; ++i) load_to_lds(src[i] + off, dst[i] + stage * STAGE);
+    } else {
+      const size_t off = (size_t)t * 512;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) load_to_lds(src[i] + off, dst[i] + stage * STAGE);
+    }
+  };
+  // lgkmcnt(0) and vmcnt(the loads of two steps): what a wave waits for before a barrier
+  auto wait_all_but_two_steps = [&]() {
+    if (NFX == 4 || !fetches_x) __builtin_amdgcn_s_waitcnt(0x0070 | 8);
+    else __builtin_amdgcn_s_waitcnt(0x0070 | (2 * NFX));
   };
 
-  floatx4 acc[8][4];
+  floatx4 acc[TM][4];
 #pragma unroll
-  for (int i = 0; i < 8; ++i)
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[i][j] = floatx4{0.f, 0.f, 0.f, 0.f};
-  bf16x8 a[8], b[4];
+  bf16x8 a[TM], b[4];
 
   // every wave passes the same barriers; nothing may move across one
   auto barrier = [&]() {
@@ -522,7 +543,6 @@ __global__ __launch_bounds__(512) void gemm_bf16_pingpong(const bf16_t* __restri
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("" ::: "memory");
   };
-  constexpr int WAIT_ALL_BUT_TWO_STEPS = 0x0070 | 8;    // lgkmcnt(0), vmcnt(8): two steps of four loads
   const int nk = T;
   // Step t lies in stage t % 4.  A wave's memory phase of step t reads its fragments,
   // issues its loads of step t + 3 (into the stage that both groups read last in step
@@ -531,7 +551,7 @@ __global__ __launch_bounds__(512) void gemm_bf16_pingpong(const bf16_t* __restri
   fetch(0, 0);
   fetch(1, min(1, nk - 1));
   fetch(2, min(2, nk - 1));
-  __builtin_amdgcn_s_waitcnt(WAIT_ALL_BUT_TWO_STEPS);
+  wait_all_but_two_steps();
   barrier();
   if (grp == 1) barrier();                               // the second group runs half a step behind
   for (int t0 = 0; t0 < nk; t0 += 4) {
@@ -541,14 +561,14 @@ __global__ __launch_bounds__(512) void gemm_bf16_pingpong(const bf16_t* __restri
       if (t < nk) {                                      // (the same for every wave of the block)
         const char* stage = smem + u * STAGE;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) b[j] = *(const bf16x8*)(stage + (16 + wn * 4 + j) * 1024 + lane * 16);
+        for (int j = 0; j < 4; ++j) b[j] = *(const bf16x8*)(stage + (XF + wn * 4 + j) * 1024 + lane * 16);
 #pragma unroll
-        for (int i = 0; i < 8; ++i) a[i] = *(const bf16x8*)(stage + (wm * 8 + i) * 1024 + lane * 16);
+        for (int i = 0; i < TM; ++i) a[i] = *(const bf16x8*)(stage + (wm * TM + i) * 1024 + lane * 16);
         fetch((u + 3) & 3, min(t + 3, nk - 1));
-        __builtin_amdgcn_s_waitcnt(WAIT_ALL_BUT_TWO_STEPS);
+        wait_all_but_two_steps();
         barrier();
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
           for (int j = 0; j < 4; ++j)
             acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[i], b[j], acc[i][j], 0, 0, 0);
@@ -560,24 +580,28 @@ __global__ __launch_bounds__(512) void gemm_bf16_pingpong(const bf16_t* __restri
   __builtin_amdgcn_s_waitcnt(0x0070);                    // the last loads (past K, never read) are in
   barrier();
 
-  // ---- epilogue: the rows 0-127 of the tile through LDS, then the rows 128-255
+  // ---- epilogue: the rows 0-127 of the tile through LDS, then the rest
   float* Cs = (float*)smem;
+  auto to_lds = [&](int part) {
 #pragma unroll
-  for (int half = 0; half < 2; ++half) {
-    if (wm == half) {
-#pragma unroll
-      for (int i = 0; i < 8; ++i)
+    for (int i = 0; i < TM; ++i) {
+      const int row = wm * (BM / 2) + i * 16;             // of the tile
+      if (row / HALF == part) {
 #pragma unroll
         for (int j = 0; j < 4; ++j)
 #pragma unroll
           for (int x = 0; x < 4; ++x)
-            Cs[(i * 16 + g * 4 + x) * C_STRIDE + wn * 64 + j * 16 + c] = acc[i][j][x];
+            Cs[(row % HALF + g * 4 + x) * C_STRIDE + wn * 64 + j * 16 + c] = acc[i][j][x];
+      }
     }
     __syncthreads();
-    tile_epilogue<HALF, BN, NT, EPI>(Cs, e, m0 + half * HALF, n0, M, N, tid, s_pos + (QKV ? half * HALF : 0),
-                                     s_page + (QKV ? half * HALF : 0), s_freq, s_bias);
-    __syncthreads();
-  }
+  };
+  to_lds(0);
+  tile_epilogue<HALF, BN, NT, EPI>(Cs, e, m0, n0, M, N, tid, s_pos, s_page, s_freq, s_bias);
+  __syncthreads();
+  to_lds(1);
+  tile_epilogue<BM - HALF, BN, NT, EPI>(Cs, e, m0 + HALF, n0, M, N, tid, s_pos + (QKV ? HALF : 0),
+                                        s_page + (QKV ? HALF : 0), s_freq, s_bias);
 }
 
 // ================================================================ float32
@@ -813,7 +837,7 @@ constexpr int F32_ROWS_MAX = 64;     // up to here the few-row kernel (the tiled
 // bytes a microsecond, the chip 5.3e6 at most (one tile of rows, 17 to 64 of them, of
 // matrices from 9 to 283 MB, in 4 or 8 pieces: the estimate is within 2 us of the
 // measurement).
-enum { TILE_64 = 0, TILE_64x128 = 1, TILE_128 = 2, TILE_128x256 = 3, TILE_256 = 4, TILE_KINDS = 5 };
+enum { TILE_64 = 0, TILE_64x128 = 1, TILE_128 = 2, TILE_128x256 = 3, TILE_256 = 4, TILE_192 = 5, TILE_KINDS = 6 };
 struct TileModel {
   int bm, bn;
   double L, f, tk, resident, stream;
@@ -823,23 +847,26 @@ static const TileModel TILE_MODELS[TILE_KINDS] = {{64, 64, 6.39, 0.79, 0.289, 1.
                                                   {64, 128, 6.54, 0.71, 0.5, 1.5, 27e3, 0},
                                                   {128, 128, 8.0, 0.48, 0.66, 1.0, 24e3, 0},
                                                   {128, 256, 0.0, 6.16, 0.945, 1.0, 24e3, 1},
-                                                  {256, 256, 0.0, 9.2, 1.8, 1.0, 24e3, 1}};
+                                                  {256, 256, 0.0, 9.2, 1.8, 1.0, 24e3, 1},
+                                                  {192, 256, 0.0, 9.2, 1.4, 1.0, 24e3, 1}};
 constexpr double CHIP_STREAM = 5.3e6;     // bytes a microsecond
 
-// The 256 x 256 tile: whole rounds of one block a unit, a step of 32 of the inner size
-// 0.82 us in a full round and from 0.51 us in a round of few blocks (the chip clocks
-// higher), 9.3 us before and after the loop (fitted to the same sweeps: 6 % rms).
-static double pingpong_cost(int M, int N, int K, int num_cus) {
-  const double rounds = (double)((M + 255) / 256) * ((N + 255) / 256) / num_cus;
+// The tiles of the two groups of waves: whole rounds of one block a unit; with 256 rows a
+// step of 32 of the inner size takes 0.82 us in a full round and from 0.51 us in a round of
+// few blocks (the chip clocks higher), and 9.3 us pass before and after the loop; with 192
+// rows 0.70 and 0.44 us (fitted to the same sweeps: 5 and 7 % rms).
+static double pingpong_cost(int bm, int M, int N, int K, int num_cus) {
+  const double rounds = (double)((M + bm - 1) / bm) * ((N + 255) / 256) / num_cus;
   const double whole = floor(rounds + 1e-9), last = rounds - whole;
   const int steps = (K + 31) / 32;
-  double t = 0.7 + whole * (9.3 + steps * 0.824);
-  if (last > 1e-9) t += 9.3 + steps * (0.506 + (0.824 - 0.506) * last);
+  const double before_after = bm == 256 ? 9.3 : 0.8, full = bm == 256 ? 0.824 : 0.70, few = bm == 256 ? 0.506 : 0.441;
+  double t = (bm == 256 ? 0.7 : 0.0) + whole * (before_after + steps * full);
+  if (last > 1e-9) t += before_after + steps * (few + (full - few) * last);
   return t;
 }
 
 static double tile_cost(int kind, int M, int N, int K, int num_cus, int pieces) {
-  if (kind == TILE_256) return pingpong_cost(M, N, K, num_cus);
+  if (kind == TILE_256 || kind == TILE_192) return pingpong_cost(TILE_MODELS[kind].bm, M, N, K, num_cus);
   const TileModel& t = TILE_MODELS[kind];
   const double blocks = (double)((M + t.bm - 1) / t.bm) * ((N + t.bn - 1) / t.bn) * pieces;
   double rounds = blocks / (num_cus * t.resident);
@@ -852,7 +879,7 @@ static double tile_cost(int kind, int M, int N, int K, int num_cus, int pieces) 
 }
 
 // Debug interface (kernels/debug.py): a tile can be forced, for tests and measurements
-// (0 = choose; 64, 130 = 64 x 128, 129 = 128 x 128, 131 = 128 x 256, 132 = 256 x 256; -131 =
+// (0 = choose; 64, 130 = 64 x 128, 129 = 128 x 128, 131 = 128 x 256, 132 = 256 x 256, 133 = 192 x 256; -131 =
 // choose among the first three).
 static int g_force_tile = 0, g_without_wide = 0;
 extern "C" void llmlab_debug_gemm_tile(int tile) {
@@ -866,6 +893,7 @@ static int choose_tile(int M, int N, int K, int num_cus) {
   if (g_force_tile == 129 || g_force_tile == 128) return TILE_128;
   if (g_force_tile == 131) return TILE_128x256;
   if (g_force_tile == 132) return TILE_256;
+  if (g_force_tile == 133) return TILE_192;
   // One or two tiles of rows of a wide matrix (the head, gate and up at larger shapes):
   // bound by the read of W, which the wider tiles stream better than the estimate
   // knows, and the 128-row tile reads W once where two 64-row tiles read it twice
@@ -902,19 +930,27 @@ static int choose_tile(int M, int N, int K, int num_cus) {
       if (last < 1e-9 || last >= 0.5 || rounds >= 16.0) best = TILE_128x256;
     }
   }
-  // The 256 x 256 tile of the two groups of waves where its estimate is the lower one
-  // (over the sweeps it is then 10 to 24 % faster than the best of the others: 2048 rows,
-  // 37888 x 3584: 501 us against 623; 55296 x 5120: 999 against 1245; 576 rows, 37888 x
-  // 3584: 178 against 195; with a quarter of a round of blocks it is twice as slow).
-  // From 1024 rows and an inner size of 1024 on: by the products alone it would win from
+  // The tiles of the two groups of waves where the estimate of one is the lowest (over the
+  // sweeps the 256 x 256 tile is then 10 to 24 % faster than the best of the others: 2048
+  // rows, 37888 x 3584: 501 us against 623; 55296 x 5120: 999 against 1245; with a quarter
+  // of a round of blocks it is twice as slow; the 192 x 256 tile where its blocks fill
+  // their rounds better: 2048 rows, 5120 x 27648: 534 us against 655 with 256 rows).
+  // From 1024 rows and an inner size of 1024 on: by the products alone they would win from
   // 576 rows and with an inner size of 896 too, but a step of 576 rows as a whole is 1.5 %
-  // slower with it at the 7B shape, steps of 1024 and 4096 rows 1 to 3 % at the 0.5B shape.
-  // (The same two groups of waves on a 128 x 256 tile, 64 x 64 a wave, are as fast as the
-  // 128 x 256 tile above and no faster: a wave then reads as many bytes from LDS per MFMA
-  // as there, and LDS is the limit of both.)
-  if (M >= 1024 && K >= 1024 && !g_without_wide &&
-      pingpong_cost(M, N, K, num_cus) < tile_cost(best, M, N, K, num_cus, 1))
-    best = TILE_256;
+  // slower with the larger one at the 7B shape, steps of 1024 and 4096 rows 1 to 3 % at the
+  // 0.5B shape.  (The same two groups of waves on a 128 x 256 tile, 64 x 64 a wave, are as
+  // fast as the 128 x 256 tile above and no faster: a wave then reads as many bytes from
+  // LDS per MFMA as there, and LDS is the limit of both.)
+  if (M >= 1024 && K >= 1024 && !g_without_wide) {
+    double least = tile_cost(best, M, N, K, num_cus, 1);
+    for (int kind = TILE_256; kind <= TILE_192; ++kind) {
+      const double c = tile_cost(kind, M, N, K, num_cus, 1);
+      if (c < least) {
+        least = c;
+        best = kind;
+      }
+    }
+  }
   return best;
 }
 
@@ -931,8 +967,12 @@ static void launch_tile(int kind, const bf16_t* A, const bf16_t* W, const EpiArg
     hipLaunchKernelGGL((gemm_bf16_tiled<128, 128, 64, 1, 4, EPI>), grid, dim3(256), 0, stream, A, W, e, M, N, K);
   else if (kind == TILE_128x256)
     hipLaunchKernelGGL((gemm_bf16_tiled<128, 256, 64, 1, 8, EPI>), grid, dim3(512), 0, stream, A, W, e, M, N, K);
-  else if constexpr (EPI != EPI_PART)
-    hipLaunchKernelGGL((gemm_bf16_pingpong<EPI>), grid, dim3(512), 0, stream, A, W, e, M, N, K);
+  else if constexpr (EPI != EPI_PART) {
+    if (kind == TILE_256)
+      hipLaunchKernelGGL((gemm_bf16_pingpong<256, EPI>), grid, dim3(512), 0, stream, A, W, e, M, N, K);
+    else
+      hipLaunchKernelGGL((gemm_bf16_pingpong<192, EPI>), grid, dim3(512), 0, stream, A, W, e, M, N, K);
+  }
 }
 
 // Whether (and into how many pieces along K) a product that adds into float32 rows should
@@ -962,7 +1002,7 @@ extern "C" void llmlab_linear_plan(int M, int N, int K, int num_cus, int max_pie
   // 15.8, 15.1 against 18.8 us; with more blocks than units it is the slower one)
   if (M <= 64 && best_pieces > 1 && g_force_tile == 0 && (long)((N + 63) / 64) * best_pieces <= num_cus)
     best_kind = TILE_64;
-  if (best_kind == TILE_256) best_kind = TILE_128x256;   // (the 256 x 256 tile makes no pieces)
+  if (best_kind >= TILE_256) best_kind = TILE_128x256;   // (the tiles of the two groups of waves make no pieces)
   out[0] = best_pieces;
   out[1] = best_kind;
 }

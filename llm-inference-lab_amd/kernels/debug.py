@@ -63,7 +63,7 @@ class KernelDebug:
               skinny_epilogue: Optional[int] = None,
               attention_splits: Optional[Tuple[int, int]] = None,
               attention_path: Optional[Tuple[int, int]] = None, **rules):
-        """``gemm_tile``: 64 (64 x 64), 130 (64 x 128), 129 (128 x 128), 131 (128 x 256) or 132 (256 x 256); -131: the
+        """``gemm_tile``: 64 (64 x 64), 130 (64 x 128), 129 (128 x 128), 131 (128 x 256), 132 (256 x 256) or 133 (192 x 256); -131: the
         choice among the first three.  ``skinny_shape``:
         (strips per block, K slices, staged rows 0/1 or -1, rows per tile) of the few-row
         product kernel, 0 = chosen by the kernel.  ``skinny_epilogue``: the force holds for

@@ -125,10 +125,10 @@ def test_linear_residual_and_logits(ops, emu, dtype, m, n, k):
     close(got, want, torch.float32, f"linear_logits {m}x{n}x{k}", want.abs().max().item())
 
 
-@pytest.mark.parametrize("tile", [64, 130, 129, 131, 132])
+@pytest.mark.parametrize("tile", [64, 130, 129, 131, 132, 133])
 @pytest.mark.parametrize("m,n,k", [(65, 130, 72), (200, 1152, 896), (300, 257, 136), (513, 384, 264), (129, 64, 1160)])
 def test_every_tile_shape_of_the_tiled_products(ops, emu, tile, m, n, k):
-    """Every epilogue with each of the five tile shapes forced, on sizes with ragged edges
+    """Every epilogue with each of the six tile shapes forced, on sizes with ragged edges
     in all three dimensions (the chooser would pick only one of them per size)."""
     from llm_inference_lab_amd.parts.feed_forward import interleave_gate_up
     bf = torch.bfloat16
@@ -348,7 +348,7 @@ def test_qkv_rope_cache_of_normed_rows(ops, emu, nq, nkv, d, page, hidden, rows_
 @pytest.mark.parametrize("nq,nkv,d,page,hidden", [(4, 2, 16, 16, 64), (14, 2, 64, 64, 896), (7, 1, 32, 16, 72),
                                                  (8, 8, 128, 64, 256), (2, 1, 256, 16, 64)])
 @pytest.mark.parametrize("rows_per", [[70, 1, 130], [300, 2, 2, 90]])
-@pytest.mark.parametrize("tile", [131, 132])
+@pytest.mark.parametrize("tile", [131, 132, 133])
 def test_qkv_rope_cache_with_the_widest_tiles(ops, emu, nq, nkv, d, page, hidden, rows_per, tile):
     """The tiles of 256 columns and eight waves, which only large products get by
     themselves: heads of every size that divides them, a head of 256 among them."""

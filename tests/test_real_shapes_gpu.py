@@ -105,12 +105,12 @@ def test_one_layer_at_the_widths_of_larger_models(name, dtype, cut):
 @pytest.mark.parametrize("cut", ["whole", "mixed"])
 def test_one_layer_with_the_tiles_of_large_steps(name, cut):
     """The tiles that only steps of a thousand rows and more get by themselves (128 x 256,
-    and 256 x 256 with its two groups of waves), forced on every product of more than 64
+    and 256 x 256 and 192 x 256 with their two groups of waves), forced on every product of more than 64
     rows of these shorter steps: q/k/v with rotation and cache write, both products into the
     stream, gate/up with SwiGLU and the logits."""
     seqs = sequences_of(name)
     want = {rid: H.plain_logits(name, 1, ids) for rid, ids in seqs.items()}
-    for tile in (131, 132):
+    for tile in (131, 132, 133):
         engine = H.make_engine(name, 1, "bf16", page_size=64, num_pages=19, max_requests=4, max_batch_tokens=512)
         with engine.ops.debug.force(gemm_tile=tile):
             got = H.run_trace(engine, seqs, CUTS[cut](seqs))
