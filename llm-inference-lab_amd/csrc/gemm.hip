@@ -879,12 +879,14 @@ static double tile_cost(int kind, int M, int N, int K, int num_cus, int pieces) 
 }
 
 // Debug interface (kernels/debug.py): a tile can be forced, for tests and measurements
-// (0 = choose; 64, 130 = 64 x 128, 129 = 128 x 128, 131 = 128 x 256, 132 = 256 x 256, 133 = 192 x 256; -131 =
-// choose among the first three).
-static int g_force_tile = 0, g_without_wide = 0;
+// (0 = choose; 64, 130 = 64 x 128, 129 = 128 x 128, 131 = 128 x 256, 132 = 256 x 256, 133 =
+// 192 x 256; -131 = choose among the first three; -256 and below: the tiles of two groups
+// of waves from so many rows on).
+static int g_force_tile = 0, g_without_wide = 0, g_pp_min_rows = 512;
 extern "C" void llmlab_debug_gemm_tile(int tile) {
   g_force_tile = tile > 0 ? tile : 0;
   g_without_wide = tile == -131;
+  g_pp_min_rows = tile <= -256 ? -tile : 512;
 }
 
 static int choose_tile(int M, int N, int K, int num_cus) {
@@ -935,13 +937,14 @@ static int choose_tile(int M, int N, int K, int num_cus) {
   // rows, 37888 x 3584: 501 us against 623; 55296 x 5120: 999 against 1245; with a quarter
   // of a round of blocks it is twice as slow; the 192 x 256 tile where its blocks fill
   // their rounds better: 2048 rows, 5120 x 27648: 534 us against 655 with 256 rows).
-  // From 1024 rows and an inner size of 1024 on: by the products alone they would win from
-  // 576 rows and with an inner size of 896 too, but a step of 576 rows as a whole is 1.5 %
-  // slower with the larger one at the 7B shape, steps of 1024 and 4096 rows 1 to 3 % at the
-  // 0.5B shape.  (The same two groups of waves on a 128 x 256 tile, 64 x 64 a wave, are as
+  // From 512 rows and an inner size of 1024 on (prefill steps of 512 to 960 tokens as a
+  // whole: 2.4 to 6.8 % faster at the 7B shape, 3 to 4.6 % at the 32B shape; from 256 rows
+  // a step of 384 tokens would be 13 % slower at the 7B shape: the estimates are not fitted
+  // there; with an inner size of 896 steps of 1024 and 4096 rows are 1 to 3 % slower at the
+  // 0.5B shape though the products alone are faster).  (The same two groups of waves on a 128 x 256 tile, 64 x 64 a wave, are as
   // fast as the 128 x 256 tile above and no faster: a wave then reads as many bytes from
   // LDS per MFMA as there, and LDS is the limit of both.)
-  if (M >= 1024 && K >= 1024 && !g_without_wide) {
+  if (M >= g_pp_min_rows && K >= 1024 && !g_without_wide) {
     double least = tile_cost(best, M, N, K, num_cus, 1);
     for (int kind = TILE_256; kind <= TILE_192; ++kind) {
       const double c = tile_cost(kind, M, N, K, num_cus, 1);

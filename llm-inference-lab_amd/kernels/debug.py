@@ -63,8 +63,9 @@ class KernelDebug:
               skinny_epilogue: Optional[int] = None,
               attention_splits: Optional[Tuple[int, int]] = None,
               attention_path: Optional[Tuple[int, int]] = None, **rules):
-        """``gemm_tile``: 64 (64 x 64), 130 (64 x 128), 129 (128 x 128), 131 (128 x 256), 132 (256 x 256) or 133 (192 x 256); -131: the
-        choice among the first three.  ``skinny_shape``:
+        """``gemm_tile``: 64 (64 x 64), 130 (64 x 128), 129 (128 x 128), 131 (128 x 256), 132 (256 x
+        256) or 133 (192 x 256); -131: the choice among the first three; -256 and below: the
+        tiles of two groups of waves (132, 133) from so many rows on.  ``skinny_shape``:
         (strips per block, K slices, staged rows 0/1 or -1, rows per tile) of the few-row
         product kernel, 0 = chosen by the kernel.  ``skinny_epilogue``: the force holds for
         this epilogue only.  ``attention_splits``: (head size, key splits of the decode
