@@ -448,7 +448,6 @@ __global__ __launch_bounds__(512) void gemm_bf16_pingpong(const bf16_t* __restri
   constexpr int STAGE = (XF + BN / 16) * 1024;          // bytes: the fragments of x, then 16 of W
   constexpr int C_STRIDE = BN + 4;
   constexpr size_t C_BYTES = (size_t)HALF * C_STRIDE * sizeof(float);
-  static_assert(EPI != EPI_PART, "no pieces along K with this tile");
   __shared__ __attribute__((aligned(1024))) char smem[C_BYTES > 4 * STAGE ? C_BYTES : 4 * STAGE];
 
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -511,7 +510,17 @@ __global__ __launch_bounds__(512) void gemm_bf16_pingpong(const bf16_t* __restri
                  : "v"(from), "s"(to)
                  : "memory", "m0");
   };
-  auto fetch = [&](int stage, int t) {
+  // this block's steps: all of them, or (PART) its group's share of the inner size from
+  // step `first` on, whose sums go to the group's own piece of the output
+  int first = 0, nk = T;
+  if constexpr (EPI == EPI_PART) {
+    first = (int)blockIdx.z * e.kt_per_split * 2;
+    nk = max(0, min(T - first, e.kt_per_split * 2));
+    e.out = (float*)e.out + (size_t)blockIdx.z * e.part_stride;
+    if (blockIdx.z > 0) e.bias = nullptr;
+  }
+  auto fetch = [&](int stage, int step) {
+    const int t = min(first + step, T - 1);
     if (fetches_x) {
       const size_t off = (size_t)min(t * 32 + g * 8, K - 8);
 #pragma unroll
@@ -543,14 +552,13 @@ __global__ __launch_bounds__(512) void gemm_bf16_pingpong(const bf16_t* __restri
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("" ::: "memory");
   };
-  const int nk = T;
   // Step t lies in stage t % 4.  A wave's memory phase of step t reads its fragments,
   // issues its loads of step t + 3 (into the stage that both groups read last in step
   // t - 1, at least one barrier ago) and waits for its own loads of step t + 1; the
   // barrier after the other group's same phase then says that step t + 1 is whole.
   fetch(0, 0);
-  fetch(1, min(1, nk - 1));
-  fetch(2, min(2, nk - 1));
+  fetch(1, 1);
+  fetch(2, 2);
   wait_all_but_two_steps();
   barrier();
   if (grp == 1) barrier();                               // the second group runs half a step behind
@@ -564,7 +572,7 @@ __global__ __launch_bounds__(512) void gemm_bf16_pingpong(const bf16_t* __restri
         for (int j = 0; j < 4; ++j) b[j] = *(const bf16x8*)(stage + (XF + wn * 4 + j) * 1024 + lane * 16);
 #pragma unroll
         for (int i = 0; i < TM; ++i) a[i] = *(const bf16x8*)(stage + (wm * TM + i) * 1024 + lane * 16);
-        fetch((u + 3) & 3, min(t + 3, nk - 1));
+        fetch((u + 3) & 3, t + 3);
         wait_all_but_two_steps();
         barrier();
 #pragma unroll
@@ -855,10 +863,10 @@ constexpr double CHIP_STREAM = 5.3e6;     // bytes a microsecond
 // step of 32 of the inner size takes 0.82 us in a full round and from 0.51 us in a round of
 // few blocks (the chip clocks higher), and 9.3 us pass before and after the loop; with 192
 // rows 0.70 and 0.44 us (fitted to the same sweeps: 5 and 7 % rms).
-static double pingpong_cost(int bm, int M, int N, int K, int num_cus) {
-  const double rounds = (double)((M + bm - 1) / bm) * ((N + 255) / 256) / num_cus;
+static double pingpong_cost(int bm, int M, int N, int K, int num_cus, int pieces) {
+  const double rounds = (double)((M + bm - 1) / bm) * ((N + 255) / 256) * pieces / num_cus;
   const double whole = floor(rounds + 1e-9), last = rounds - whole;
-  const int steps = (K + 31) / 32;
+  const int steps = pieces > 1 ? 2 * (((K + 63) / 64 + pieces - 1) / pieces) : (K + 31) / 32;
   const double before_after = bm == 256 ? 9.3 : 0.8, full = bm == 256 ? 0.824 : 0.70, few = bm == 256 ? 0.506 : 0.441;
   double t = (bm == 256 ? 0.7 : 0.0) + whole * (before_after + steps * full);
   if (last > 1e-9) t += before_after + steps * (few + (full - few) * last);
@@ -866,7 +874,7 @@ static double pingpong_cost(int bm, int M, int N, int K, int num_cus) {
 }
 
 static double tile_cost(int kind, int M, int N, int K, int num_cus, int pieces) {
-  if (kind == TILE_256 || kind == TILE_192) return pingpong_cost(TILE_MODELS[kind].bm, M, N, K, num_cus);
+  if (kind == TILE_256 || kind == TILE_192) return pingpong_cost(TILE_MODELS[kind].bm, M, N, K, num_cus, pieces);
   const TileModel& t = TILE_MODELS[kind];
   const double blocks = (double)((M + t.bm - 1) / t.bm) * ((N + t.bn - 1) / t.bn) * pieces;
   double rounds = blocks / (num_cus * t.resident);
@@ -970,7 +978,7 @@ static void launch_tile(int kind, const bf16_t* A, const bf16_t* W, const EpiArg
     hipLaunchKernelGGL((gemm_bf16_tiled<128, 128, 64, 1, 4, EPI>), grid, dim3(256), 0, stream, A, W, e, M, N, K);
   else if (kind == TILE_128x256)
     hipLaunchKernelGGL((gemm_bf16_tiled<128, 256, 64, 1, 8, EPI>), grid, dim3(512), 0, stream, A, W, e, M, N, K);
-  else if constexpr (EPI != EPI_PART) {
+  else {
     if (kind == TILE_256)
       hipLaunchKernelGGL((gemm_bf16_pingpong<256, EPI>), grid, dim3(512), 0, stream, A, W, e, M, N, K);
     else
@@ -988,7 +996,9 @@ extern "C" void llmlab_linear_plan(int M, int N, int K, int num_cus, int max_pie
   const double piece = (double)M * N * 2.2e-6 + 0.3;
   int best_kind = choose_tile(M, N, K, num_cus), best_pieces = 1;
   double best_cost = tile_cost(best_kind, M, N, K, num_cus, 1);
-  for (int kind = TILE_64x128; kind <= TILE_128; ++kind) {
+  for (int kind = TILE_64x128; kind < TILE_KINDS; ++kind) {
+    if (kind == TILE_128x256) continue;
+    if (kind >= TILE_256 && !(M >= g_pp_min_rows && K >= 1024 && !g_without_wide)) continue;
     if (g_force_tile != 0 && kind != choose_tile(M, N, K, num_cus)) continue;
     for (int s = 2; s <= max_pieces; ++s) {
       if ((nk + s - 1) / s < min_tiles_per_piece) break;
@@ -1005,7 +1015,6 @@ extern "C" void llmlab_linear_plan(int M, int N, int K, int num_cus, int max_pie
   // 15.8, 15.1 against 18.8 us; with more blocks than units it is the slower one)
   if (M <= 64 && best_pieces > 1 && g_force_tile == 0 && (long)((N + 63) / 64) * best_pieces <= num_cus)
     best_kind = TILE_64;
-  if (best_kind >= TILE_256) best_kind = TILE_128x256;   // (the tiles of the two groups of waves make no pieces)
   out[0] = best_pieces;
   out[1] = best_kind;
 }
@@ -1053,7 +1062,7 @@ extern "C" int llmlab_linear_partials(const void* x, const void* w, float* parts
   LLMLAB_REQUIRE(M >= 0 && N > 0 && K > 0 && K % 8 == 0, "linear_partials: bad sizes M=%d N=%d K=%d", M, N, K);
   LLMLAB_REQUIRE(ksplit >= 1 && ksplit <= 16 && ldo >= N && part_stride >= (size_t)M * ldo,
                  "linear_partials: %d pieces, row stride %d", ksplit, ldo);
-  LLMLAB_REQUIRE(tile >= TILE_64 && tile <= TILE_128x256, "linear_partials: unknown tile %d", tile);
+  LLMLAB_REQUIRE(tile >= TILE_64 && tile < TILE_KINDS, "linear_partials: unknown tile %d", tile);
   LLMLAB_REQUIRE(((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0),
                  "linear_partials: operands must be 16-byte aligned");
   if (M == 0) return 0;
