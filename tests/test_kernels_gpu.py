@@ -126,7 +126,8 @@ def test_linear_residual_and_logits(ops, emu, dtype, m, n, k):
 
 
 @pytest.mark.parametrize("tile", [64, 130, 129, 131, 132, 133])
-@pytest.mark.parametrize("m,n,k", [(65, 130, 72), (200, 1152, 896), (300, 257, 136), (513, 384, 264), (129, 64, 1160)])
+@pytest.mark.parametrize("m,n,k", [(65, 130, 72), (200, 1152, 896), (300, 257, 136), (513, 384, 264), (129, 64, 1160),
+                                   (70, 300, 24), (130, 90, 40), (257, 520, 8)])
 def test_every_tile_shape_of_the_tiled_products(ops, emu, tile, m, n, k):
     """Every epilogue with each of the six tile shapes forced, on sizes with ragged edges
     in all three dimensions (the chooser would pick only one of them per size)."""
