@@ -860,15 +860,16 @@ static const TileModel TILE_MODELS[TILE_KINDS] = {{64, 64, 6.39, 0.79, 0.289, 1.
 constexpr double CHIP_STREAM = 5.3e6;     // bytes a microsecond
 
 // The tiles of the two groups of waves: whole rounds of one block a unit; with 256 rows a
-// step of 32 of the inner size takes 0.82 us in a full round and from 0.51 us in a round of
-// few blocks (the chip clocks higher), and 9.3 us pass before and after the loop; with 192
-// rows 0.70 and 0.44 us (fitted to the same sweeps: 5 and 7 % rms).
+// step of 32 of the inner size takes 0.82 us in a full round and from 0.56 us in a round of
+// few blocks (the chip clocks higher), and 9.6 us pass before and after the loop; with 192
+// rows 0.64, 0.47 and 7.6 us (fitted to the same sweeps, inner sizes from 896 to 27648: 8
+// and 9 % rms).
 static double pingpong_cost(int bm, int M, int N, int K, int num_cus, int pieces) {
   const double rounds = (double)((M + bm - 1) / bm) * ((N + 255) / 256) * pieces / num_cus;
   const double whole = floor(rounds + 1e-9), last = rounds - whole;
   const int steps = pieces > 1 ? 2 * (((K + 63) / 64 + pieces - 1) / pieces) : (K + 31) / 32;
-  const double before_after = bm == 256 ? 9.3 : 0.8, full = bm == 256 ? 0.824 : 0.70, few = bm == 256 ? 0.506 : 0.441;
-  double t = (bm == 256 ? 0.7 : 0.0) + whole * (before_after + steps * full);
+  const double before_after = bm == 256 ? 9.6 : 7.6, full = bm == 256 ? 0.816 : 0.637, few = bm == 256 ? 0.555 : 0.472;
+  double t = whole * (before_after + steps * full);
   if (last > 1e-9) t += before_after + steps * (few + (full - few) * last);
   return t;
 }
@@ -891,6 +892,7 @@ static double tile_cost(int kind, int M, int N, int K, int num_cus, int pieces) 
 // 192 x 256; -131 = choose among the first three; -256 and below: the tiles of two groups
 // of waves from so many rows on).
 static int g_force_tile = 0, g_without_wide = 0, g_pp_min_rows = 512;
+constexpr int PP_MIN_INNER = 896;      // the shortest inner size the estimates of those tiles were fitted to
 extern "C" void llmlab_debug_gemm_tile(int tile) {
   g_force_tile = tile > 0 ? tile : 0;
   g_without_wide = tile == -131;
@@ -945,14 +947,14 @@ static int choose_tile(int M, int N, int K, int num_cus) {
   // rows, 37888 x 3584: 501 us against 623; 55296 x 5120: 999 against 1245; with a quarter
   // of a round of blocks it is twice as slow; the 192 x 256 tile where its blocks fill
   // their rounds better: 2048 rows, 5120 x 27648: 534 us against 655 with 256 rows).
-  // From 512 rows and an inner size of 1024 on (prefill steps of 512 to 960 tokens as a
-  // whole: 2.4 to 6.8 % faster at the 7B shape, 3 to 4.6 % at the 32B shape; from 256 rows
-  // a step of 384 tokens would be 13 % slower at the 7B shape: the estimates are not fitted
-  // there; with an inner size of 896 steps of 1024 and 4096 rows are 1 to 3 % slower at the
-  // 0.5B shape though the products alone are faster).  (The same two groups of waves on a 128 x 256 tile, 64 x 64 a wave, are as
-  // fast as the 128 x 256 tile above and no faster: a wave then reads as many bytes from
-  // LDS per MFMA as there, and LDS is the limit of both.)
-  if (M >= g_pp_min_rows && K >= 1024 && !g_without_wide) {
+  // From 512 rows on (prefill steps of 512 to 960 tokens as a whole: 2.4 to 6.8 % faster at
+  // the 7B shape, 3 to 4.6 % at the 32B shape; from 256 rows a step of 384 tokens would be
+  // 13 % slower at the 7B shape: the estimates are not fitted there) and an inner size of
+  // 896, the shortest measured (steps of 1024 / 4096 / 8192 tokens of the 0.5B shape: 5.8 /
+  // 3.5 / 5.8 % faster, 576 and 2048 unchanged).  (The same two groups of waves on a 128 x
+  // 256 tile, 64 x 64 a wave, are as fast as the 128 x 256 tile above and no faster: a wave
+  // then reads as many bytes from LDS per MFMA as there, and LDS is the limit of both.)
+  if (M >= g_pp_min_rows && K >= PP_MIN_INNER && !g_without_wide) {
     double least = tile_cost(best, M, N, K, num_cus, 1);
     for (int kind = TILE_256; kind <= TILE_192; ++kind) {
       const double c = tile_cost(kind, M, N, K, num_cus, 1);
@@ -998,7 +1000,7 @@ extern "C" void llmlab_linear_plan(int M, int N, int K, int num_cus, int max_pie
   double best_cost = tile_cost(best_kind, M, N, K, num_cus, 1);
   for (int kind = TILE_64x128; kind < TILE_KINDS; ++kind) {
     if (kind == TILE_128x256) continue;
-    if (kind >= TILE_256 && !(M >= g_pp_min_rows && K >= 1024 && !g_without_wide)) continue;
+    if (kind >= TILE_256 && !(M >= g_pp_min_rows && K >= PP_MIN_INNER && !g_without_wide)) continue;
     if (g_force_tile != 0 && kind != choose_tile(M, N, K, num_cus)) continue;
     for (int s = 2; s <= max_pieces; ++s) {
       if ((nk + s - 1) / s < min_tiles_per_piece) break;
