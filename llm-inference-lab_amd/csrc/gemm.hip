@@ -97,26 +97,33 @@ __device__ __forceinline__ void tile_epilogue(const float* Cs, const EpiArgs& e,
                                               const float* s_bias) {
   constexpr int C_STRIDE = BN + 4;
   if constexpr (EPI == EPI_QKV) {
-    // a unit of work: four pairs (i .. i+3, and those + d/2) of one head of one row
-    const int d = e.d, dh = d >> 1, heads = BN / d, cpl = dh >> 2;
+    // q and k heads.  A unit of work: eight pairs (i .. i+7, and those + d/2) of one head of
+    // one row, rotated and stored 16 bytes at a time (eight neighbours of one octet of d lie
+    // next to each other in the key order too).
+    const int d = e.d, dh = d >> 1, heads = BN / d, cpl = dh >> 3, head0 = n0 / d;
     const int units = BM * heads * cpl;
-    const bool vec = (e.ldo & 3) == 0 && ((uintptr_t)e.out & 7) == 0;
+    const bool vec = (e.ldo & 7) == 0 && ((uintptr_t)e.out & 15) == 0;
     for (int u = tid; u < units; u += NT) {
       const int jc = u % cpl, t = u / cpl, hh = t % heads, row = t / heads;
-      const int m = m0 + row, head = n0 / d + hh, i = jc * 4;
-      if (m >= M || head >= e.nq + 2 * e.nkv) continue;
+      const int m = m0 + row, head = head0 + hh, i = jc * 8;
+      if (m >= M || head >= e.nq + e.nkv) continue;          // (values: below)
+      const bool is_q = head < e.nq;
+      if (!is_q && !e.kcache) continue;
       const float* src = Cs + row * C_STRIDE + hh * d + i;
-      floatx4 lo = *(const floatx4*)src, hi = *(const floatx4*)(src + dh);
+      float lo[8], hi[8];
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        lo[q] += s_bias[hh * d + i + q];
-        hi[q] += s_bias[hh * d + dh + i + q];
+      for (int q = 0; q < 8; q += 4) {
+        const floatx4 l4 = *(const floatx4*)(src + q), h4 = *(const floatx4*)(src + dh + q);
+#pragma unroll
+        for (int x = 0; x < 4; ++x) {
+          lo[q + x] = l4[x] + s_bias[hh * d + i + q + x];
+          hi[q + x] = h4[x] + s_bias[hh * d + dh + i + q + x];
+        }
       }
-      const bool is_q = head < e.nq, is_k = !is_q && head < e.nq + e.nkv;
       const int pos = s_pos[row];
-      if ((is_q || is_k) && e.inv_freq) {
+      if (e.inv_freq) {
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
+        for (int q = 0; q < 8; ++q) {
           // the hardware sine and cosine of r = frac(angle / 2 pi)
           float r = (float)pos * s_freq[i + q] * 0.15915494309189535f;
           r -= floorf(r);
@@ -126,37 +133,75 @@ __device__ __forceinline__ void tile_epilogue(const float* Cs, const EpiArgs& e,
           hi[q] = nhi;
         }
       }
-      bf16x4 blo, bhi;
+      bf16x8 blo, bhi;
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
+      for (int q = 0; q < 8; ++q) {
         blo[q] = (bf16_t)lo[q];
         bhi[q] = (bf16_t)hi[q];
       }
       if (is_q) {
         bf16_t* dst = (bf16_t*)e.out + (size_t)m * e.ldo + (size_t)head * d + i;
         if (vec) {
-          *(bf16x4*)dst = blo;
-          *(bf16x4*)(dst + dh) = bhi;
+          *(bf16x8*)dst = blo;
+          *(bf16x8*)(dst + dh) = bhi;
         } else {
-          for (int q = 0; q < 4; ++q) {
+          for (int q = 0; q < 8; ++q) {
             dst[q] = blo[q];
             dst[dh + q] = bhi[q];
           }
         }
-      } else if (e.kcache) {
-        const size_t page = (size_t)s_page[row];
+      } else {
+        bf16_t* dst = e.kcache + ((size_t)s_page[row] * e.nkv + (head - e.nq)) * (size_t)e.page_size * d;
         const int off = pos % e.page_size;
-        if (is_k) {
-          // four neighbours of one octet of d lie next to each other in the key order
-          bf16_t* dst = e.kcache + (page * e.nkv + (head - e.nq)) * (size_t)e.page_size * d;
-          *(bf16x4*)(dst + kcache_index(off, i, d)) = blo;
-          *(bf16x4*)(dst + kcache_index(off, i + dh, d)) = bhi;
-        } else {
-          bf16_t* dst = e.vcache + (page * e.nkv + (head - e.nq - e.nkv)) * (size_t)e.page_size * d;
+        *(bf16x8*)(dst + kcache_index(off, i, d)) = blo;
+        *(bf16x8*)(dst + kcache_index(off, i + dh, d)) = bhi;
+      }
+    }
+    // v heads.  In the value order four consecutive keys of one number of d lie next to each
+    // other, and the numbers of a 16-wide block of d after one another: a unit is four rows
+    // by four numbers, 32 consecutive bytes of the page when the rows are four consecutive
+    // positions of one request that start at a multiple of four (rows of a prompt mostly are;
+    // single numbers of 2 bytes, which memory would have to merge into what it holds, else).
+    const int hv0 = max(0, e.nq + e.nkv - head0), hv1 = min(heads, e.nq + 2 * e.nkv - head0);
+    if (e.vcache && hv1 > hv0) {
+      const int nv = hv1 - hv0, chunks = d >> 2;
+      for (int u = tid; u < (BM / 4) * nv * chunks; u += NT) {
+        const int jc = u % chunks, t = u / chunks, hh = hv0 + t % nv, r0 = (t / nv) * 4;
+        if (m0 + r0 >= M) continue;
+        const int dd0 = jc * 4, head = head0 + hh;
+        float val[4][4];
 #pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            dst[vcache_index(off, i + q, d)] = blo[q];
-            dst[vcache_index(off, i + dh + q, d)] = bhi[q];
+        for (int k = 0; k < 4; ++k) {
+          const floatx4 v4 = *(const floatx4*)(Cs + (r0 + k) * C_STRIDE + hh * d + dd0);
+#pragma unroll
+          for (int x = 0; x < 4; ++x) val[k][x] = v4[x] + s_bias[hh * d + dd0 + x];
+        }
+        const int pos0 = s_pos[r0];
+        bool together = m0 + r0 + 3 < M && (pos0 & 3) == 0;
+#pragma unroll
+        for (int k = 1; k < 4; ++k) together = together && s_pos[r0 + k] == pos0 + k && s_page[r0 + k] == s_page[r0];
+        const size_t per_page = (size_t)e.page_size * d;
+        if (together) {
+          bf16x8 w0, w1;
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            w0[k] = (bf16_t)val[k][0];
+            w0[4 + k] = (bf16_t)val[k][1];
+            w1[k] = (bf16_t)val[k][2];
+            w1[4 + k] = (bf16_t)val[k][3];
+          }
+          bf16_t* dst = e.vcache + ((size_t)s_page[r0] * e.nkv + (head - e.nq - e.nkv)) * per_page +
+                        vcache_index(pos0 % e.page_size, dd0, d);
+          *(bf16x8*)dst = w0;
+          *(bf16x8*)(dst + 8) = w1;
+        } else {
+#pragma unroll
+          for (int k = 0; k < 4; ++k) {
+            if (m0 + r0 + k >= M) continue;
+            bf16_t* dst = e.vcache + ((size_t)s_page[r0 + k] * e.nkv + (head - e.nq - e.nkv)) * per_page;
+            const int off = s_pos[r0 + k] % e.page_size;
+#pragma unroll
+            for (int x = 0; x < 4; ++x) dst[vcache_index(off, dd0 + x, d)] = (bf16_t)val[k][x];
           }
         }
       }
@@ -1035,7 +1080,7 @@ extern "C" int llmlab_linear_qkv(const void* x, const void* w, const void* bias,
   LLMLAB_REQUIRE(positions != nullptr && (kcache == nullptr || (table && row_req && page_size > 0)),
                  "linear_qkv: positions and block table are needed");
   LLMLAB_REQUIRE(((uintptr_t)x % 16 == 0) && ((uintptr_t)w % 16 == 0) &&
-                 ((uintptr_t)kcache % 8 == 0) && ((uintptr_t)vcache % 8 == 0),
+                 ((uintptr_t)kcache % 16 == 0) && ((uintptr_t)vcache % 16 == 0),
                  "linear_qkv: operands must be 16-byte aligned");
   if (M == 0) return 0;
   if (num_cus <= 0) num_cus = 256;

@@ -373,10 +373,10 @@ def test_qkv_rope_cache_through_pieces(ops, emu, nq, nkv, d, page, hidden, rows_
     assert ops.rules.forced_tiled_pieces == 0 and ops.rules.tiled_pieces_bytes == 16e6
 
 
-def check_qkv_rope_cache(ops, emu, nq, nkv, d, page, hidden, rows_per):
+def check_qkv_rope_cache(ops, emu, nq, nkv, d, page, hidden, rows_per, starts=(3, 40, 0, 7)):
     bf = torch.bfloat16
     rows, reqs = sum(rows_per), len(rows_per)
-    num_pages = 16 + sum((40 + c + page - 1) // page for c in rows_per)
+    num_pages = 16 + sum((max(starts) + c + page - 1) // page for c in rows_per)
     if not ops.can_fuse_qkv_rope(rows, bf, d, (nq + 2 * nkv) * d, hidden):
         with pytest.raises(ValueError):
             ops.qkv_rope_cache(torch.zeros(rows, hidden, dtype=bf, device=DEV),
@@ -384,7 +384,7 @@ def check_qkv_rope_cache(ops, emu, nq, nkv, d, page, hidden, rows_per):
                                None, nq, nkv, d, None, torch.zeros(rows, dtype=torch.int32, device=DEV), None,
                                None, page, None, None, torch.empty(rows, nq * d, dtype=bf, device=DEV))
         return
-    starts = [3, 40, 0, 7][:reqs]
+    starts = list(starts)[:reqs]
     h = rnd((rows, hidden), bf, 70)
     n = (nq + 2 * nkv) * d
     w, b = rnd((n, hidden), bf, 72, 0.2), rnd((n,), bf, 73)
@@ -412,6 +412,22 @@ def check_qkv_rope_cache(ops, emu, nq, nkv, d, page, hidden, rows_per):
     close(got_v, want_v, bf, "value cache", scale)
     untouched = (want_k == kc)
     assert torch.equal(got_k.cpu()[untouched], kc[untouched])
+    untouched = (want_v == vc)
+    assert torch.equal(got_v.cpu()[untouched], vc[untouched])
+
+
+@pytest.mark.parametrize("nq,nkv,d,page,hidden", [(4, 2, 16, 16, 64), (14, 2, 64, 64, 896), (8, 8, 128, 64, 256),
+                                                 (2, 1, 256, 16, 64)])
+@pytest.mark.parametrize("rows_per,starts", [([72, 4, 124], (0, 64, 8)), ([70, 6, 125], (2, 61, 9)),
+                                             ([8, 4, 4, 180], (12, 0, 28, 100))])
+@pytest.mark.parametrize("tile", [0, 129, 132, 133])
+def test_values_of_four_positions_written_together(ops, emu, nq, nkv, d, page, hidden, rows_per, starts, tile):
+    """The values of four consecutive positions of a request that start at a multiple of four go
+    to their page as one piece of 32 bytes per four numbers of a head, others number by number:
+    requests whose rows and positions line up so (a prompt from its start, a portion that starts
+    at a multiple of four), requests that do not, and short requests between them."""
+    with ops.debug.force(gemm_tile=tile):
+        check_qkv_rope_cache(ops, emu, nq, nkv, d, page, hidden, rows_per, starts)
 
 
 @pytest.mark.parametrize("window", [None, 40])
