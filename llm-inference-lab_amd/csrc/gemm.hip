@@ -160,49 +160,54 @@ __device__ __forceinline__ void tile_epilogue(const float* Cs, const EpiArgs& e,
     // v heads.  In the value order four consecutive keys of one number of d lie next to each
     // other, and the numbers of a 16-wide block of d after one another: four rows that are
     // four consecutive positions of one request, the first a multiple of four, put four
-    // numbers of a head into 32 consecutive bytes of the page.  The row of the first of such
-    // four (wherever in the tile it lies: a portion of a prompt may follow the rows of
-    // decoding requests) stores for all of them; rows that belong to no whole group of the
-    // tile store number by number (2 bytes each, which memory has to merge into what it
-    // holds: a tile of value heads stored so finished long after the others).
+    // numbers of a head into 32 consecutive bytes of the page.  The rows of the tile are
+    // taken in fours from the first row on whose position is a multiple of four if the tile
+    // continues as its first row begins (a prompt from its start does; so does a portion
+    // that follows the rows of decoding requests, from its second tile on); a unit of work
+    // is such a group of rows by four numbers.  Groups that are not four positions in a row
+    // of one request (and the rows before the first group and after the last) store number
+    // by number: 2 bytes each, which memory has to merge into what it holds; a tile of
+    // value heads stored so finished long after the others.
     const int hv0 = max(0, e.nq + e.nkv - head0), hv1 = min(heads, e.nq + 2 * e.nkv - head0);
     if (e.vcache && hv1 > hv0) {
       const int nv = hv1 - hv0, chunks = d >> 2;
-      auto leads_four = [&](int l) {      // rows l .. l+3 of the tile are such a group
-        if (l < 0 || l + 3 >= BM || m0 + l + 3 >= M || (s_pos[l] & 3) != 0) return false;
-        bool ok = true;
-#pragma unroll
-        for (int k = 1; k < 4; ++k) ok = ok && s_pos[l + k] == s_pos[l] + k && s_page[l + k] == s_page[l];
-        return ok;
-      };
+      const int shift = (4 - (s_pos[0] & 3)) & 3;
       const size_t per_page = (size_t)e.page_size * d;
-      for (int u = tid; u < BM * nv * chunks; u += NT) {
-        const int jc = u % chunks, t = u / chunks, hh = hv0 + t % nv, row = t / nv;
-        if (m0 + row >= M) continue;
-        const int dd0 = jc * 4, head = head0 + hh, pos = s_pos[row], first = row - (pos & 3);
-        const bool grouped = leads_four(first);
-        if (grouped && first != row) continue;               // the first row of the group stores
-        const float* src = Cs + row * C_STRIDE + hh * d + dd0;
+      for (int u = tid; u < (BM / 4 + 1) * nv * chunks; u += NT) {
+        const int jc = u % chunks, t = u / chunks, hh = hv0 + t % nv, r0 = shift - 4 + 4 * (t / nv);
+        const int dd0 = jc * 4, head = head0 + hh;
         const float* bias = s_bias + hh * d + dd0;
-        bf16_t* dst = e.vcache + ((size_t)s_page[row] * e.nkv + (head - e.nq - e.nkv)) * per_page;
-        if (grouped) {
+        bool together = r0 >= 0 && r0 + 3 < BM && m0 + r0 + 3 < M;
+        if (together) {
+          const int pos0 = s_pos[r0];
+          together = (pos0 & 3) == 0;
+#pragma unroll
+          for (int k = 1; k < 4; ++k) together = together && s_pos[r0 + k] == pos0 + k && s_page[r0 + k] == s_page[r0];
+        }
+        if (together) {
           bf16x8 w0, w1;
 #pragma unroll
           for (int k = 0; k < 4; ++k) {
-            const floatx4 v4 = *(const floatx4*)(src + k * C_STRIDE);
+            const floatx4 v4 = *(const floatx4*)(Cs + (r0 + k) * C_STRIDE + hh * d + dd0);
             w0[k] = (bf16_t)(v4[0] + bias[0]);
             w0[4 + k] = (bf16_t)(v4[1] + bias[1]);
             w1[k] = (bf16_t)(v4[2] + bias[2]);
             w1[4 + k] = (bf16_t)(v4[3] + bias[3]);
           }
-          dst += vcache_index(pos % e.page_size, dd0, d);
+          bf16_t* dst = e.vcache + ((size_t)s_page[r0] * e.nkv + (head - e.nq - e.nkv)) * per_page +
+                        vcache_index(s_pos[r0] % e.page_size, dd0, d);
           *(bf16x8*)dst = w0;
           *(bf16x8*)(dst + 8) = w1;
         } else {
-          const floatx4 v4 = *(const floatx4*)src;
-          const int off = pos % e.page_size;
+          for (int k = 0; k < 4; ++k) {
+            const int row = r0 + k;
+            if (row < 0 || row >= BM || m0 + row >= M) continue;
+            const floatx4 v4 = *(const floatx4*)(Cs + row * C_STRIDE + hh * d + dd0);
+            bf16_t* dst = e.vcache + ((size_t)s_page[row] * e.nkv + (head - e.nq - e.nkv)) * per_page;
+            const int off = s_pos[row] % e.page_size;
 #pragma unroll
-          for (int x = 0; x < 4; ++x) dst[vcache_index(off, dd0 + x, d)] = (bf16_t)(v4[x] + bias[x]);
+            for (int x = 0; x < 4; ++x) dst[vcache_index(off, dd0 + x, d)] = (bf16_t)(v4[x] + bias[x]);
+          }
         }
       }
     }
