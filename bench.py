@@ -56,8 +56,21 @@ SHAPES = {   # layer sizes of the published Qwen2.5 checkpoints; weights are ran
     "32b": dict(COMMON, vocab_size=152064, hidden_size=5120, intermediate_size=27648,
                 num_hidden_layers=64, num_attention_heads=40, num_key_value_heads=8, head_dim=128,
                 tie_word_embeddings=False),
+    # further sizes of the same family, for measurements beside the three above
+    "1.5b": dict(COMMON, vocab_size=151936, hidden_size=1536, intermediate_size=8960,
+                 num_hidden_layers=28, num_attention_heads=12, num_key_value_heads=2, head_dim=128,
+                 tie_word_embeddings=True),
+    "3b": dict(COMMON, vocab_size=151936, hidden_size=2048, intermediate_size=11008,
+               num_hidden_layers=36, num_attention_heads=16, num_key_value_heads=2, head_dim=128,
+               tie_word_embeddings=True),
+    "14b": dict(COMMON, vocab_size=152064, hidden_size=5120, intermediate_size=13824,
+                num_hidden_layers=48, num_attention_heads=40, num_key_value_heads=8, head_dim=128,
+                tie_word_embeddings=False),
+    "72b": dict(COMMON, vocab_size=152064, hidden_size=8192, intermediate_size=29568,
+                num_hidden_layers=80, num_attention_heads=64, num_key_value_heads=8, head_dim=128,
+                tie_word_embeddings=False),
 }
-DEFAULT_CONTEXT = {"0.5b": 4096, "7b": 4096, "32b": 8192}
+DEFAULT_CONTEXT = {"0.5b": 4096, "7b": 4096, "32b": 8192, "1.5b": 4096, "3b": 4096, "14b": 4096, "72b": 4096}
 
 
 def prefill_flops(cfg, tokens):
