@@ -115,6 +115,7 @@ class RequestInstruments:
     def __init__(self):
         self.requests = 0
         self.failures = 0
+        self.cancelled = 0
         self.in_flight = 0
         self.generated_tokens = 0
         self.duration_seconds = {"success": Histogram(), "error": Histogram()}
@@ -132,17 +133,21 @@ class RequestInstruments:
     def first_token(self, seconds: float) -> None:
         self.first_token_seconds.record(seconds)
 
-    def finished(self, ok: bool, seconds: float, generated: int) -> None:
+    def finished(self, ok: bool, seconds: float, generated: int, cancelled: bool = False) -> None:
         self.in_flight -= 1
-        self.duration_seconds["success" if ok else "error"].record(seconds)
         self.generated_tokens += int(generated)
+        if cancelled:
+            self.cancelled += 1         # neither a success nor a failure: no duration is recorded
+            return
+        self.duration_seconds["success" if ok else "error"].record(seconds)
         if not ok:
             self.failures += 1
         elif generated > 0 and seconds > 0:
             self.output_tokens_per_second.record(generated / seconds)
 
     def snapshot(self):
-        return {"requests": self.requests, "failures": self.failures, "in_flight": self.in_flight,
+        return {"requests": self.requests, "failures": self.failures, "cancelled": self.cancelled,
+                "in_flight": self.in_flight,
                 "generated_tokens": self.generated_tokens,
                 "duration_seconds": {k: h.snapshot() for k, h in self.duration_seconds.items()},
                 "queue_wait_seconds": self.queue_wait_seconds.snapshot(),

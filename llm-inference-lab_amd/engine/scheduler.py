@@ -59,7 +59,7 @@ class Request:
     remaining: int = 0
     promised_pages: List[int] = dataclasses.field(default_factory=list)
     error: Optional[Exception] = None
-    finish_reason: Optional[str] = None        # "eos", "length", "error"
+    finish_reason: Optional[str] = None        # "eos", "length", "error", "cancelled"
     in_flight: bool = False                    # a token of this request is chosen but not read yet
     arrival: float = 0.0
     admit_time: Optional[float] = None
@@ -367,13 +367,47 @@ class Scheduler:
             r.cache = None
         r.finish_time = time.perf_counter()
         self.finished[r.request_id] = r
-        self.instruments.finished(r.error is None, r.finish_time - r.arrival, len(r.generated))
+        self.instruments.finished(r.error is None, r.finish_time - r.arrival, len(r.generated),
+                                  cancelled=r.finish_reason == "cancelled")
 
     def _finish(self, r: Request, reason: str, error: Optional[Exception] = None) -> None:
         r.finish_reason, r.error, r.remaining = reason, error, 0
         r.finish_time = time.perf_counter()
         self.finished[r.request_id] = r
         self.instruments.finished(error is None, r.finish_time - r.arrival, 0)
+
+    def cancel(self, request_id: int) -> bool:
+        """End a waiting or running request now, between two steps: it leaves its queue,
+        gives its pages and its row back at once (what the GPU still writes there is
+        ordered before the next step's work on the same stream) and is reported as
+        finished with ``finish_reason="cancelled"`` and the tokens it had been given.  A
+        token of it that is still on its way is dropped when it arrives.  Returns False
+        if no such request is waiting or running.  The reference cancels the runner as a
+        whole, which drops every active and waiting turn
+        (rust/engine/src/runner/model_runner.rs:899-910, test 1796-1827); ``cancel_all``
+        is that."""
+        for r in self.waiting:
+            if r.request_id == request_id:
+                self.waiting.remove(r)
+                r.finish_reason, r.remaining = "cancelled", 0
+                r.finish_time = time.perf_counter()
+                self.finished[r.request_id] = r
+                self.instruments.finished(True, r.finish_time - r.arrival, 0, cancelled=True)
+                return True
+        for r in self.active:
+            if r.request_id == request_id:
+                if not r.finished:
+                    r.finish_reason, r.remaining = "cancelled", 0
+                self._release(r)
+                return True
+        return False
+
+    def cancel_all(self) -> List[int]:
+        """Cancel everything that waits or runs; returns the ids."""
+        ids = [r.request_id for r in list(self.waiting) + list(self.active)]
+        for i in ids:
+            self.cancel(i)
+        return ids
 
     @property
     def idle(self) -> bool:

@@ -378,7 +378,7 @@ class StepFunction:
                                   f"tokens of this step")
         return None
 
-    def run(self, entries: Sequence[StepEntry]) -> "StepResult":
+    def run(self, entries: Sequence[StepEntry], strict: bool = False) -> "StepResult":
         """One step with a result for every entry.  An entry that cannot run (a token id
         outside the vocabulary, a position beyond the longest sequence, no page left for
         it) gets its error and is left out; the others still run as one batch
@@ -386,13 +386,19 @@ class StepFunction:
         fails (a kernel refuses a size, a launch fails), every entry that was in it gets
         that error (engine.rs:2041-2045), their reservations are dropped and their caches
         are marked invalid (rust/engine/src/runner/kv_pool/api.rs:257-262): what the step
-        half wrote is not to be read, such a request can only be released."""
+        half wrote is not to be read, such a request can only be released.
+
+        ``strict``: all or nothing.  The first entry that cannot run (also one that finds
+        no page) raises its error before anything has run, and every reservation this
+        call made is given back: lengths and pages of all entries are as before."""
         errors: List[Optional[Exception]] = [None] * len(entries)
         seen: set = set()
         for i, e in enumerate(entries):
             errors[i] = self._refusal(e, seen)
             if errors[i] is None:
                 seen.add(id(e.request))
+            elif strict:
+                raise errors[i]
         # what is wrong with the step as a whole is the caller's mistake: nothing runs
         n_rows = sum(len(e.tokens) for e, err in zip(entries, errors) if err is None)
         if n_rows > self.max_batch_tokens:
@@ -404,6 +410,10 @@ class StepFunction:
                 try:
                     self.cache.reserve(e.request, len(e.tokens))
                 except Exception as err:            # no page left: this entry sits out, with its reason
+                    if strict:
+                        for earlier in entries[:i]:
+                            self.cache.cancel_reservation(earlier.request)
+                        raise
                     errors[i] = err
         valid = [e for e, err in zip(entries, errors) if err is None]
         rows: List[Optional[range]] = []
@@ -443,16 +453,13 @@ class StepFunction:
         """Reserve pages, run the rows, commit.  Returns float32 logits
         ``[wanted, vocab]`` in the order of the entries and of their ``want``
         (None when nothing is wanted).  The tensor is reused by the next step.
-        Any entry that cannot run raises here, before anything has run."""
+        All or nothing: an entry that cannot run (an invalid token, a position too far, no
+        page left for it) raises here before anything has run, with the lengths and the
+        pages of every entry as they were, so the caller may try again with other entries.
+        A batch that fails while it runs raises too; its requests are then invalid."""
         if not entries:
             return None
-        seen: set = set()
-        for e in entries:
-            refusal = self._refusal(e, seen)
-            if refusal is not None:
-                raise refusal
-            seen.add(id(e.request))
-        result = self.run(entries)
+        result = self.run(entries, strict=True)
         for err in result.errors:
             if err is not None:
                 raise err

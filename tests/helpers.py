@@ -38,7 +38,7 @@ TINY_C = dict(architectures=["Qwen2ForCausalLM"], model_type="qwen2", vocab_size
 REAL_LAYER = dict(architectures=["Qwen2ForCausalLM"], model_type="qwen2", vocab_size=4099, hidden_size=896,
                   intermediate_size=4864, num_hidden_layers=2, num_attention_heads=14,
                   num_key_value_heads=2, head_dim=64, rms_norm_eps=1e-6, rope_theta=1000000.0,
-                  max_position_embeddings=4096, tie_word_embeddings=True, use_sliding_window=False)
+                  max_position_embeddings=8192, tie_word_embeddings=True, use_sliding_window=False)
 # The whole Qwen2.5-0.5B shape (24 layers, the real vocabulary), and one layer each with the
 # widths of Qwen2.5-7B and Qwen2.5-32B (a small odd vocabulary): the sizes at which the
 # kernels' rules for large matrices decide.
@@ -61,6 +61,13 @@ CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C, "R": REAL_LAYER, "F": FULL_05B
 # of order 1.  float32: sums in another order than the float64 reference.
 # bfloat16: activations rounded to 8 bits of mantissa between kernels.
 TOL = {"f32": 1e-4, "bf16": 2e-2}
+# Layers 896 wide (configuration R): float32 within 1e-3 of the float64 plain implementation
+# (sums of 896 to 4864 terms).  For bfloat16 the floor is what rounding the activations to 8
+# bits of mantissa at the engine's rounding points costs at this width: the emulation of the
+# kernels on the CPU (tests/emu_ops.py, float32 arithmetic, the same roundings) is off the
+# plain implementation by 0.09 to 0.10 at most and 0.016 to 0.017 in the root mean square
+# over the logits of such sequences; the GPU may be off by half as much again.
+TOL_REAL = {"f32": (1e-3, 1e-3), "bf16": (0.15, 0.025)}     # (max, root mean square)
 
 
 def config_of(name):

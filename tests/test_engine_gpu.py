@@ -22,13 +22,7 @@ CUTS = {"whole": H.steps_whole, "decode": H.steps_prefill_then_decode, "portions
         "mixed": H.steps_mixed}
 
 
-# Layers 896 wide: float32 within 1e-3 of the float64 plain implementation (sums of 896
-# to 4864 terms).  For bfloat16 the floor is what rounding the activations to 8 bits of
-# mantissa at the engine's rounding points costs at this width: the emulation of the
-# kernels on the CPU (tests/emu_ops.py, float32 arithmetic, the same roundings) is off
-# the plain implementation by 0.09 to 0.10 at most and 0.016 to 0.017 in the root mean
-# square over the logits of these sequences; the GPU may be off by half as much again.
-TOL_REAL = {"f32": (1e-3, 1e-3), "bf16": (0.15, 0.025)}     # (max, root mean square)
+TOL_REAL = H.TOL_REAL
 
 
 def sequences_of(name, seed=0):

@@ -157,6 +157,39 @@ def test_the_strict_step_raises_before_anything_runs():
     assert roomy.cache.free_pages(0) == 40 and c.reserved_len == 0
 
 
+def test_the_strict_step_leaves_everything_as_it_was_when_a_page_is_missing():
+    """``engine.step`` with an entry that finds no page raises before anything runs: the
+    lengths, reservations and pages of every entry, also of those that came before it in
+    the list and had got their pages, are as before, so the same peers can be fed the
+    same tokens again at the same positions."""
+    cfg = H.config_of("A")
+    engine = engine_of(EmuOps(), num_pages=4, max_seq_len=64)
+    initial = initial_metrics(engine)
+    a, b, c = engine.open("a"), engine.open("b"), engine.open("c")
+    first = H.random_ids(cfg, 10, 1)
+    engine.step([lab.StepEntry(a, first, [])])                       # a holds 1 page of 4
+    held = [list(r.pages[0]) for r in (a, b, c)]
+    steps_before = engine.step_fn.steps
+    more_a, ids_b, ids_c = H.random_ids(cfg, 20, 2), H.random_ids(cfg, 17, 3), H.random_ids(cfg, 20, 4)
+    with pytest.raises(OutOfPages):
+        engine.step([lab.StepEntry(a, more_a, [19]),                # 1 more page
+                     lab.StepEntry(b, ids_b, [16]),                 # 2 pages: the pool is empty now
+                     lab.StepEntry(c, ids_c, [19])])                # none left
+    assert engine.step_fn.steps == steps_before
+    assert (a.computed_len, a.reserved_len) == (10, 10) and not a.invalid
+    for r in (b, c):
+        assert (r.computed_len, r.reserved_len) == (0, 0) and not r.invalid
+    assert [list(r.pages[0]) for r in (a, b, c)] == held and engine.cache.free_pages(0) == 3
+    engine.cache.check()
+    # the caller tries again without the one that did not fit: same logits as plain
+    logits = engine.step([lab.StepEntry(a, more_a, [19]), lab.StepEntry(b, ids_b, [16])])
+    assert (logits[0].double() - H.plain_logits("A", 1, first + more_a)[29]).abs().max() <= H.TOL["f32"]
+    assert (logits[1].double() - H.plain_logits("A", 1, ids_b)[16]).abs().max() <= H.TOL["f32"]
+    for r in (a, b, c):
+        engine.close(r)
+    pool_is_as_new(engine, initial)
+
+
 @pytest.mark.parametrize("overlap", [False, True])
 def test_scheduler_ends_the_requests_of_a_failed_step_and_goes_on(overlap):
     cfg = H.config_of("A")

@@ -176,6 +176,52 @@ def test_finished_request_frees_before_the_next_step():
     engine.cache.check()
 
 
+@pytest.mark.parametrize("overlap", [False, True])
+def test_cancelling_releases_running_and_waiting_requests(overlap):
+    """A running request that is cancelled between two steps gives its pages and its row
+    back at once, a waiting one leaves the queue, a token of the cancelled one that was
+    still on its way is dropped, its peers' tokens are what they are without it, the one
+    that waited for its pages is admitted at the next step, and at the end the pool is as
+    new (the reference drops every active and waiting turn when its runner is cancelled:
+    rust/engine/src/runner/model_runner.rs:899-910, 1796-1827)."""
+    cfg = H.config_of("A")
+    engine = engine_of("A", num_pages=6, max_requests=2)
+    initial = engine.cache.metrics()
+    prompts = [H.random_ids(cfg, n, 40 + n) for n in (20, 9, 30, 5)]
+    alone = [engine.generate([p], max_new_tokens=8, eos_token_id=[], overlap=overlap)[0] for p in prompts]
+    sched = engine.scheduler(overlap=overlap)
+    ids = [sched.add_request(p, SamplingConfig(max_new_tokens=8, eos_token_id=[])) for p in prompts]
+    for _ in range(3):
+        sched.step()
+    assert [r.request_id for r in sched.active] == ids[:2] and [r.request_id for r in sched.waiting] == ids[2:]
+    given = list(sched.active[0].generated)
+    assert sched.cancel(ids[0]) and sched.cancel(ids[3]) and not sched.cancel(ids[0]) and not sched.cancel(99)
+    assert engine.cache.live_requests == 1
+    engine.cache.check()
+    done = sched.run()
+    assert done[ids[0]].finish_reason == "cancelled" and done[ids[0]].error is None
+    assert done[ids[0]].generated == given == alone[0][:len(given)] and 0 < len(given) < 8
+    assert done[ids[3]].finish_reason == "cancelled" and done[ids[3]].generated == []
+    assert done[ids[1]].generated == alone[1] and done[ids[2]].generated == alone[2]
+    engine.cache.check()
+    now = engine.cache.metrics()
+    for m in (initial, now):
+        for g in m["groups"]:
+            g.pop("pages_high_water")
+    assert now == initial
+    m = engine.request_instruments.snapshot()
+    assert m["cancelled"] == 2 and m["failures"] == 0 and m["in_flight"] == 0
+    # everything at once
+    sched = engine.scheduler(overlap=overlap)
+    ids = [sched.add_request(p, SamplingConfig(max_new_tokens=8, eos_token_id=[])) for p in prompts]
+    sched.step()
+    sched.step()
+    assert sorted(sched.cancel_all()) == ids and sched.active == [] and not sched.waiting
+    sched.run()
+    assert sched.idle and all(sched.finished[i].finish_reason == "cancelled" for i in ids)
+    assert engine.cache.live_requests == 0 and engine.cache.free_pages(0) == 6
+
+
 def test_overlap_gives_the_same_tokens_and_steps():
     cfg = H.config_of("B")
     prompts = [H.random_ids(cfg, n, 90 + n) for n in (5, 40, 61, 3)]
