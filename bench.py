@@ -480,10 +480,10 @@ def main():
         p50, p95 = runs.step_latencies(args.batch)
         result["step_ms"] = {"p50": p50, "p95": p95}
         if not args.no_graph:             # the same steps the other way: kernel by kernel, or from a graph
-            chosen = bool(engine.step_fn.use_graph)
-            engine.step_fn.use_graph = not chosen
+            chosen, auto = bool(engine.step_fn.use_graph), engine.step_fn.auto_graph
+            engine.step_fn.use_graph, engine.step_fn.auto_graph = not chosen, False
             s, _ = runs.decode(args.batch, half_steps, half_warmup)
-            engine.step_fn.use_graph = chosen
+            engine.step_fn.use_graph, engine.step_fn.auto_graph = chosen, auto
             result["eager" if chosen else "graph"] = {
                 "value": round(args.batch * half_steps / s, 1),
                 "ms_per_step": round(s / half_steps * 1e3, 4)}

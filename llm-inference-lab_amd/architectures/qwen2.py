@@ -35,9 +35,9 @@ def build_qwen2_spec(cfg: Qwen2Config) -> ModelSpec:
                          down_weight=p + "mlp.down_proj.weight"))
         norm = lambda name: PartSpec("rmsnorm", params=dict(size=cfg.hidden_size, eps=cfg.rms_norm_eps),
                                      tensors=dict(weight=p + name + ".weight"))
-        blocks.append(BlockSpec("prenorm", mixer=mixer, feed_forward=ffn,
-                                norm1=norm("input_layernorm"),
-                                norm2=norm("post_attention_layernorm"),
+        blocks.append(BlockSpec("prenorm",
+                                parts=dict(norm1=norm("input_layernorm"), mixer=mixer,
+                                           norm2=norm("post_attention_layernorm"), feed_forward=ffn),
                                 params=dict(hidden_size=cfg.hidden_size)))
     embed_name = "model.embed_tokens.weight"
     head_name = embed_name if cfg.tie_word_embeddings else "lm_head.weight"
@@ -57,4 +57,10 @@ def build_qwen2_spec(cfg: Qwen2Config) -> ModelSpec:
     return spec
 
 
-register_architecture(Qwen2Config.ARCHITECTURE, Qwen2Config, build_qwen2_spec, replace=True)
+# The two-message prompt that the reference's command line writes out for this model
+# (rust/engine/examples/qwen2.rs:122-124).
+QWEN2_CHAT_TEMPLATE = ("<|im_start|>system\nYou are Qwen, created by Alibaba Cloud. You are a helpful "
+                       "assistant.<|im_end|>\n<|im_start|>user\n{prompt}<|im_end|>\n<|im_start|>assistant\n")
+
+register_architecture(Qwen2Config.ARCHITECTURE, Qwen2Config, build_qwen2_spec, replace=True,
+                      chat_template=QWEN2_CHAT_TEMPLATE)

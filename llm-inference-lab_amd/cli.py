@@ -51,10 +51,6 @@ def build_parser() -> argparse.ArgumentParser:
     return ap
 
 
-CHAT_TEMPLATE = ("<|im_start|>system\nYou are Qwen, created by Alibaba Cloud. You are a helpful "
-                 "assistant.<|im_end|>\n<|im_start|>user\n{prompt}<|im_end|>\n<|im_start|>assistant\n")
-
-
 def _load_tokenizer(model_dir: str):
     path = os.path.join(model_dir, "tokenizer.json")
     if not os.path.isfile(path):
@@ -68,8 +64,8 @@ def main(argv: Optional[List[str]] = None) -> int:
     if args.max_new_tokens <= 0:
         print("--max-new-tokens must be positive", file=sys.stderr)
         return 2
-    from . import Engine, Qwen2Config, write_random_model
-    from .config.registry import architecture_of
+    from . import Engine, write_random_model
+    from .config.registry import architecture_of, read_config
     from .engine.step import StepEntry
 
     tmp = None
@@ -77,7 +73,6 @@ def main(argv: Optional[List[str]] = None) -> int:
     if args.random_weights:
         with open(args.random_weights, "r", encoding="utf-8") as f:
             raw = json.load(f)
-        raw.setdefault("architectures", ["Qwen2ForCausalLM"])
         arch = architecture_of(raw, args.random_weights)
         tmp = tempfile.TemporaryDirectory(prefix="llmlab_random_")
         model_dir = write_random_model(tmp.name, arch.config_class.from_dict(raw, args.random_weights),
@@ -94,7 +89,11 @@ def main(argv: Optional[List[str]] = None) -> int:
         if tokenizer is None:
             print(f"{model_dir} has no tokenizer.json: give --prompt-ids", file=sys.stderr)
             return 2
-        prompts = [tokenizer.encode(CHAT_TEMPLATE.format(prompt=args.prompt), add_special_tokens=False).ids]
+        # the architecture's registry entry says how a user's text is wrapped before it is
+        # tokenised (rust/engine/examples/qwen2.rs:122-124 writes out the one of its model)
+        template = read_config(model_dir)[0].chat_template
+        text = template.replace("{prompt}", args.prompt) if template else args.prompt
+        prompts = [tokenizer.encode(text, add_special_tokens=False).ids]
 
     reference = None
     if args.reference_dir:

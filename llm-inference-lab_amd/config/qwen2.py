@@ -69,6 +69,7 @@ class Qwen2Config:
     model_type: str = "qwen2"
 
     ARCHITECTURE = "Qwen2ForCausalLM"
+    MODEL_TYPE = "qwen2"
 
     # ------------------------------------------------------------------ read
     @classmethod

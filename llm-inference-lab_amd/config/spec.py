@@ -25,14 +25,16 @@ class PartSpec:
 
 @dataclasses.dataclass(frozen=True)
 class BlockSpec:
-    """One layer: how ``norm1 -> mixer -> norm2 -> feed_forward`` are arranged
-    is the block kind's business (``prenorm``: norm, sublayer, residual add)."""
+    """One layer: a block kind (a name in the parts registry) and the parts it is made of,
+    by the names that this kind gives them.  Which parts a block has and how they are
+    arranged is the kind's business: ``prenorm`` takes ``norm1, mixer, norm2,
+    feed_forward`` (norm, sublayer, residual add, twice); a kind with one norm and two
+    parallel sublayers, with norms on both sides of a sublayer, or without a feed-forward
+    names its own.  The block class receives the named ``PartSpec``s and ``params`` as
+    keyword arguments."""
 
     kind: str
-    mixer: PartSpec
-    feed_forward: PartSpec
-    norm1: PartSpec
-    norm2: PartSpec
+    parts: Dict[str, PartSpec] = dataclasses.field(default_factory=dict)
     params: Dict[str, Any] = dataclasses.field(default_factory=dict)
 
 

@@ -91,8 +91,8 @@ class Engine:
         elif tensors is not None:
             loaded = place_tensors(tensors, expected, self.dtype, self.device, strict=strict_weights)
         else:
-            loaded = place_tensors(random_tensors(expected, seed, torch.bfloat16), expected,
-                                   self.dtype, self.device, "random weights")
+            loaded = place_tensors(draw_random_tensors(self.architecture, self.config, expected, seed),
+                                   expected, self.dtype, self.device, "random weights")
         self.model.bind(loaded, self.ops, self.dtype)
         del loaded
         # ------------------------------------------------------------- cache
@@ -217,9 +217,19 @@ class Engine:
         return out
 
 
+def draw_random_tensors(architecture, config, expected, seed: int, dtype=torch.bfloat16):
+    """The (name, tensor) pairs of the random-weights mode: drawn by the architecture's own
+    ``random_init(config, expected, seed, dtype)`` if its registry entry has one, else
+    every tensor as the part that owns it says (``TensorSpec.init``)."""
+    if architecture.random_init is not None:
+        return architecture.random_init(config, expected, seed, dtype)
+    return random_tensors(expected, seed, dtype)
+
+
 def write_random_model(model_dir: str, config, seed: int, dtype=torch.bfloat16) -> str:
     """Random-weights mode: write ``config.json`` and ``model.safetensors``."""
     arch_name = getattr(config, "architecture", None) or getattr(config, "ARCHITECTURE")
     arch = get_architecture(arch_name)
     expected = CausalLM(arch.build_spec(config)).tensor_specs()
-    return write_model_dir(model_dir, config, expected, seed, dtype)
+    return write_model_dir(model_dir, config, expected, seed, dtype,
+                           tensors=draw_random_tensors(arch, config, expected, seed, dtype))

@@ -49,10 +49,7 @@ class CausalLM:
         spec.validate()
         self.spec = spec
         self.embedding = build_part("embedding", spec.embedding)
-        self.blocks = [
-            part_class("block", b.kind)(norm1=b.norm1, mixer=b.mixer, norm2=b.norm2,
-                                        feed_forward=b.feed_forward, **dict(b.params))
-            for b in spec.blocks]
+        self.blocks = [part_class("block", b.kind)(**dict(b.parts), **dict(b.params)) for b in spec.blocks]
         self.final_norm = build_part("norm", spec.final_norm)
         self.head = build_part("head", spec.head)
         self.entries: List[EntryView] = [EntryView(i, e.block) for i, e in enumerate(spec.schedule)]

@@ -255,15 +255,6 @@ class StepFunction:
     """Owns the step's buffers; ``__call__`` runs one step."""
 
     MAX_GRAPHS = 16
-    # A decode step replayed from a HIP graph costs the host nothing, but the GPU about a
-    # microsecond more at every kernel boundary than kernels launched one by one by a host
-    # that runs ahead (measured: 4.05 against 3.90 ms a step at the 7B shape, 17.3 against
-    # 16.9 at the 32B shape; 0.97 against 1.7 at the 0.5B shape, where the host cannot keep
-    # up).  ``graph="auto"`` counts the calls into the kernel libraries that the model's
-    # first decode step makes and takes the graph unless the step's reading of the weights
-    # clearly outlasts the host's making of those calls.
-    HOST_SECONDS_PER_CALL = 12e-6
-    STREAMED_BYTES_PER_SECOND = 4.2e12
 
     def __init__(self, model: CausalLM, cache: CacheManager, ops, max_batch_tokens: int,
                  graph=False):
@@ -276,8 +267,13 @@ class StepFunction:
         # everything that changes from step to step (tokens, positions, block
         # tables) lives in device memory that is rewritten before the replay.
         # A model with a part that cannot be captured (``graph_safe`` False) runs
-        # eagerly whatever is asked for here.
+        # eagerly whatever is asked for here.  ``graph="auto"``: the first decode step
+        # runs eagerly and the calls into the kernel libraries that it makes are counted;
+        # from then on every decode step is replayed or launched call by call as the
+        # kernel set's rules say for that many calls, the model's weights and the cache
+        # that the step's requests hold (``ops.rules.graph_pays``).
         self.use_graph = graph if graph == "auto" else bool(graph)
+        self.auto_graph = graph == "auto"
         self._graphs: "collections.OrderedDict" = collections.OrderedDict()
         self.graph_replays = 0
         self.graph_captures = 0
@@ -291,18 +287,34 @@ class StepFunction:
         self.failed_steps = 0
         self.instruments = StepInstruments()
 
-    def _decode_choosing(self) -> torch.Tensor:
-        """``graph="auto"``: this decode step runs eagerly and its calls are counted."""
-        before = getattr(self.ops, "calls_made", None)
-        logits = self.model.forward(self.ctx)
-        if before is None:
-            self.use_graph = False
+    def cache_bytes_of_step(self) -> int:
+        """Bytes of cache that the step in ``ctx`` reads: for every group what its layers
+        keep per token, times the positions of each request that they still see."""
+        ctx, total = self.ctx, 0
+        for g in self.cache.groups:
+            per_token = len(g.entries) * g.spec.bytes_per_token(self.cache.dtype)
+            for b in range(ctx.n_reqs):
+                seen = ctx.host_start_pos[b] + ctx.host_q_start[b + 1] - ctx.host_q_start[b]
+                total += per_token * (min(seen, g.window) if g.window else seen)
+        return total
+
+    def _decode_auto(self) -> torch.Tensor:
+        """``graph="auto"``: the first decode step runs eagerly and its calls are counted;
+        then the rules decide, step by step."""
+        rules = getattr(self.ops, "rules", None)
+        counted = getattr(self.ops, "calls_made", None)
+        if counted is None or not hasattr(rules, "graph_pays"):
+            self.use_graph = self.auto_graph = False       # a kernel set that does not count
+            return self.model.forward(self.ctx)
+        if self.decode_calls is None:
+            logits = self.model.forward(self.ctx)
+            self.decode_calls = self.ops.calls_made - counted
+            self.use_graph = rules.graph_pays(self.decode_calls, self.model.weight_bytes_per_step(),
+                                              self.cache_bytes_of_step())
             return logits
-        self.decode_calls = self.ops.calls_made - before
-        host = self.decode_calls * self.HOST_SECONDS_PER_CALL
-        gpu = self.model.weight_bytes_per_step() / self.STREAMED_BYTES_PER_SECOND
-        self.use_graph = gpu < 1.25 * host
-        return logits
+        self.use_graph = rules.graph_pays(self.decode_calls, self.model.weight_bytes_per_step(),
+                                          self.cache_bytes_of_step())
+        return self._decode_with_graph() if self.use_graph else self.model.forward(self.ctx)
 
     def _decode_with_graph(self) -> torch.Tensor:
         ctx = self.ctx
@@ -426,9 +438,9 @@ class StepFunction:
         started = time.perf_counter()
         try:
             self.ctx.fill(valid, self.cache)
-            if (self.use_graph and self.model.graph_safe
+            if ((self.use_graph or self.auto_graph) and self.model.graph_safe
                     and all(len(e.tokens) == 1 and len(e.want) == 1 for e in valid)):
-                logits = self._decode_choosing() if self.use_graph == "auto" else self._decode_with_graph()
+                logits = self._decode_auto() if self.auto_graph else self._decode_with_graph()
             else:
                 logits = self.model.forward(self.ctx)
         except Exception as err:

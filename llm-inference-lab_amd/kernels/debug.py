@@ -51,6 +51,25 @@ class DispatchRules:
     # Debug only: a product that the tiled kernel cuts gets this many pieces whatever the
     # estimate says (0: the estimate decides).
     forced_tiled_pieces: int = 0
+    # ``graph="auto"`` (engine/step.py): what one call into the kernel libraries costs the
+    # host that makes it through ctypes, and the rate at which a decode step streams its
+    # weights and its cache.  A decode step replayed from a HIP graph costs the host
+    # nothing, but the GPU about a microsecond more at every kernel boundary than kernels
+    # launched one by one by a host that runs ahead (measured: 4.05 against 3.90 ms a step
+    # at the 7B shape, 17.3 against 16.9 at the 32B shape; 0.97 against 1.7 at the 0.5B
+    # shape, where the host cannot keep up).
+    host_seconds_per_call: float = 12e-6
+    streamed_bytes_per_second: float = 4.2e12
+    # the graph is taken unless the GPU's time outlasts the host's by this factor
+    graph_host_margin: float = 1.25
+
+    def graph_pays(self, calls: int, weight_bytes: float, cache_bytes: float) -> bool:
+        """Whether a decode step of ``calls`` library calls that reads ``weight_bytes`` of
+        weights and ``cache_bytes`` of cache should be replayed from a graph: yes, unless
+        the GPU's streaming clearly outlasts the host's making of the calls."""
+        host = calls * self.host_seconds_per_call
+        gpu = (weight_bytes + cache_bytes) / self.streamed_bytes_per_second
+        return gpu < self.graph_host_margin * host
 
 
 class KernelDebug:

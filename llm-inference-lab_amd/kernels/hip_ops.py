@@ -170,7 +170,9 @@ class HipOps:
         if head_dim % 16 != 0 or not 16 <= head_dim <= 256:
             raise UnsupportedSizeError(
                 f"attention kernels take head sizes that are multiples of 16 from 16 to 256, "
-                f"got {head_dim}")
+                f"got {head_dim} (in float32 too: the pages of keys and values are laid out in "
+                f"blocks of 16 numbers of a head for both dtypes, and the kernels are compiled "
+                f"per head size)")
         if num_heads % num_kv_heads != 0:
             raise UnsupportedSizeError(f"{num_heads} heads are not a multiple of {num_kv_heads} kv heads")
         self._attention_lib(head_dim)

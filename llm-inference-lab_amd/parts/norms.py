@@ -5,7 +5,7 @@ from typing import Dict, Optional
 
 import torch
 
-from ..weights.loader import TensorSpec, VECTOR
+from ..weights.loader import TensorSpec, VECTOR, INIT_NORM
 from .base import Norm
 from .registry import register_part
 
@@ -27,7 +27,7 @@ class RMSNorm(Norm):
         self.weight: Optional[torch.Tensor] = None
 
     def tensor_specs(self):
-        return {self.tensor_names["weight"]: TensorSpec((self.size,), VECTOR)}
+        return {self.tensor_names["weight"]: TensorSpec((self.size,), VECTOR, INIT_NORM)}
 
     def bind(self, tensors, ops, dtype):
         super().bind(tensors, ops, dtype)

@@ -32,10 +32,21 @@ VECTOR = "vector"
 INT_TABLE = "int"
 
 
+INIT_NORMAL = "normal"      # N(0, std): matrices, biases, learned vectors
+INIT_NORM = "norm"          # 1 + N(0, norm_std): the weight of a norm, which scales around one
+INIT_ZEROS = "zeros"
+INIT_ONES = "ones"
+
+
 @dataclasses.dataclass(frozen=True)
 class TensorSpec:
+    """What a part expects of a tensor of the model file: its shape, how it is kept
+    (``kind``), and how the random-weights mode draws it (``init``).  The part that owns
+    the tensor says all three; nothing is read off the tensor's name."""
+
     shape: Tuple[int, ...]
     kind: str = MATRIX
+    init: str = INIT_NORMAL
 
 
 def kept_dtype(kind: str, stored: torch.dtype, compute: torch.dtype) -> torch.dtype:

@@ -28,6 +28,11 @@ class EmuOps:
     def _count(self, name):
         self.calls[name] = self.calls.get(name, 0) + 1
 
+    @property
+    def calls_made(self):
+        """Calls so far, as the kernel set of the product counts them."""
+        return sum(self.calls.values())
+
     def check_attention_sizes(self, num_heads, num_kv_heads, head_dim, dtype):
         pass
 

@@ -113,9 +113,10 @@ def silu(z: torch.Tensor) -> torch.Tensor:
     return z / (1.0 + torch.exp(-z))
 
 
-def swiglu_mlp(x, gate_w, up_w, down_w):
-    """down( silu(x Wg^T) * (x Wu^T) )  (E:1234-1294)."""
-    return linear(silu(linear(x, gate_w)) * linear(x, up_w), down_w)
+def swiglu_mlp(x, gate_w, up_w, down_w, cast=None):
+    """down( silu(x Wg^T) * (x Wu^T) )  (E:1234-1294).  ``cast``: see ``decoder_layer``."""
+    act = silu(linear(x, gate_w)) * linear(x, up_w)
+    return linear(act if cast is None else cast(act), down_w)
 
 
 def layer_window(config: dict, layer: int) -> Optional[int]:
@@ -128,38 +129,50 @@ def layer_window(config: dict, layer: int) -> Optional[int]:
 
 
 def decoder_layer(x, positions, w: Dict[str, torch.Tensor], config: dict, layer: int,
-                  attention=causal_attention_dense):
+                  attention=causal_attention_dense, cast=None):
     """norm -> q/k/v (+bias) -> rope(q, k) -> attention -> o-proj -> add;
-    norm -> SwiGLU -> add  (E:1065-1122, E:1133-1296)."""
+    norm -> SwiGLU -> add  (E:1065-1122, E:1133-1296).
+
+    ``cast`` (None: nothing) is applied where the reference stores an activation in its
+    storage type ``T`` (its ``cast_T``: the output of a norm K:575-581, q and k after the
+    rotation and v K:620-630, the attention output K:846-852, the SwiGLU output K:1484);
+    the residual stream and the sums stay as they are.  With ``cast`` rounding to bfloat16
+    this is what a bfloat16 engine computes, up to the order of its sums: the tests measure
+    the price of those roundings with it."""
+    if cast is None:
+        cast = lambda t: t
     p = f"model.layers.{layer}."
     nq, nkv = config["num_attention_heads"], config["num_key_value_heads"]
     d = config.get("head_dim") or config["hidden_size"] // nq
     eps, theta = config["rms_norm_eps"], config["rope_theta"]
     t = x.shape[0]
-    n = rms_norm(x, w[p + "input_layernorm.weight"], eps)
+    n = cast(rms_norm(x, w[p + "input_layernorm.weight"], eps))
     q = linear(n, w[p + "self_attn.q_proj.weight"], w[p + "self_attn.q_proj.bias"]).view(t, nq, d)
     k = linear(n, w[p + "self_attn.k_proj.weight"], w[p + "self_attn.k_proj.bias"]).view(t, nkv, d)
-    v = linear(n, w[p + "self_attn.v_proj.weight"], w[p + "self_attn.v_proj.bias"]).view(t, nkv, d)
-    q = rope(q, positions, theta)
-    k = rope(k, positions, theta)
-    a = attention(q, k, v, positions, layer_window(config, layer)).reshape(t, nq * d)
+    v = cast(linear(n, w[p + "self_attn.v_proj.weight"], w[p + "self_attn.v_proj.bias"]).view(t, nkv, d))
+    q = cast(rope(q, positions, theta))
+    k = cast(rope(k, positions, theta))
+    a = cast(attention(q, k, v, positions, layer_window(config, layer)).reshape(t, nq * d))
     res = x + linear(a, w[p + "self_attn.o_proj.weight"])
-    n2 = rms_norm(res, w[p + "post_attention_layernorm.weight"], eps)
+    n2 = cast(rms_norm(res, w[p + "post_attention_layernorm.weight"], eps))
     return res + swiglu_mlp(n2, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"],
-                            w[p + "mlp.down_proj.weight"])
+                            w[p + "mlp.down_proj.weight"], cast)
 
 
 def forward_logits(ids: List[int], weights: Dict[str, torch.Tensor], config: dict,
-                   dtype=torch.float64, attention=causal_attention_dense) -> torch.Tensor:
+                   dtype=torch.float64, attention=causal_attention_dense, cast=None) -> torch.Tensor:
     """Logits [tokens, vocab] of one whole sequence; the head is the embedding
-    table iff tie_word_embeddings (E:299-303); final norm then head (E:1298-1319)."""
+    table iff tie_word_embeddings (E:299-303); final norm then head (E:1298-1319).
+    ``cast``: see ``decoder_layer``."""
     w = {k: v.to(dtype) for k, v in weights.items()}
     ids_t = torch.tensor(list(ids), dtype=torch.long)
     positions = torch.arange(len(ids), dtype=torch.long)
     x = embedding(w["model.embed_tokens.weight"], ids_t)
     for layer in range(config["num_hidden_layers"]):
-        x = decoder_layer(x, positions, w, config, layer, attention)
+        x = decoder_layer(x, positions, w, config, layer, attention, cast)
     x = rms_norm(x, w["model.norm.weight"], config["rms_norm_eps"])
+    if cast is not None:
+        x = cast(x)
     head = w["model.embed_tokens.weight"] if config["tie_word_embeddings"] else w["lm_head.weight"]
     return linear(x, head)
 

@@ -69,7 +69,7 @@ def test_spec_is_data_layer_by_layer():
     cfg = H.config_of("B")
     spec = get_architecture(cfg.architecture).build_spec(cfg)
     assert len(spec.blocks) == 3 and [e.block for e in spec.schedule] == [0, 1, 2]
-    assert [b.mixer.params["window"] for b in spec.blocks] == [None, 24, 24]
+    assert [b.parts["mixer"].params["window"] for b in spec.blocks] == [None, 24, 24]
     assert spec.head.tensors["weight"] == "lm_head.weight"
     tied = get_architecture("Qwen2ForCausalLM").build_spec(H.config_of("A"))
     assert tied.head.tensors["weight"] == tied.embedding.tensors["weight"]

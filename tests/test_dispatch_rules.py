@@ -97,3 +97,58 @@ def test_block_shapes_of_products_of_few_rows(core):
         assert nsb in (1, 2, 4, 8, 16) and kw >= 1 and nsb * kw <= 16, (epilogue, m, n, k, list(out))
         assert mb in (1, 2, 4) and 16 * mb <= max(16, 2 * m), (m, mb)
         assert stage in (0, 1) and qsplit == 1
+
+
+def test_when_a_decode_graph_pays():
+    """``graph="auto"``: the rule on measured cases.  At the 0.5B shape (151 calls a step, 1 GB
+    of weights) the host cannot keep up and the graph is taken, also with 3.2 GB of cache
+    behind 64 requests; at the 7B and 32B shapes the step streams for longer than the host
+    needs and is launched call by call; a small model behind a very long context is no
+    longer misjudged by its weights alone."""
+    from llm_inference_lab_amd.kernels.debug import DispatchRules
+    rules = DispatchRules()
+    assert rules.graph_pays(151, 0.988e9, 0.4e9)
+    assert rules.graph_pays(151, 0.988e9, 3.2e9)
+    assert not rules.graph_pays(171, 14.1e9, 1.9e9)
+    assert not rules.graph_pays(387, 64.0e9, 17e9)
+    assert rules.graph_pays(151, 0.988e9, 0.0) and not rules.graph_pays(151, 0.988e9, 12e9)
+
+
+def test_the_engine_counts_a_decode_step_and_decides_step_by_step():
+    """Over the kernel references on the CPU: the first decode step of ``graph="auto"`` runs
+    eagerly and its calls are counted; what the rules are asked is the number of calls, the
+    weights of one step and the cache that the step's requests hold at that moment, at
+    every decode step anew.  (The rules here always say no: a CPU has no graphs.)"""
+    import helpers as H
+    import llm_inference_lab_amd as lab
+    from emu_ops import EmuOps
+    from llm_inference_lab_amd.kernels.debug import DispatchRules
+
+    class Asked(DispatchRules):
+        def __init__(self):
+            super().__init__()
+            self.questions = []
+
+        def graph_pays(self, calls, weight_bytes, cache_bytes):
+            self.questions.append((calls, weight_bytes, cache_bytes))
+            return False
+
+    ops = EmuOps()
+    ops.rules = Asked()
+    engine = H.make_engine("B", 1, "f32", ops=ops, device="cpu", graph="auto", num_pages=24)
+    cfg = H.config_of("B")
+    a, b = engine.open("a"), engine.open("b")
+    engine.step([lab.StepEntry(a, H.random_ids(cfg, 30, 1), [29]), lab.StepEntry(b, H.random_ids(cfg, 7, 2), [6])])
+    assert engine.step_fn.decode_calls is None and ops.rules.questions == []      # a prefill step decides nothing
+    before = ops.calls_made
+    engine.step([lab.StepEntry(a, [1], [0]), lab.StepEntry(b, [2], [0])])
+    calls = ops.calls_made - before
+    assert engine.step_fn.decode_calls == calls > 0 and engine.step_fn.use_graph is False
+    engine.step([lab.StepEntry(a, [3], [0]), lab.StepEntry(b, [4], [0])])
+    engine.step([lab.StepEntry(a, [5], [0])])
+    assert [q[0] for q in ops.rules.questions] == [calls] * 3
+    assert all(q[1] == engine.model.weight_bytes_per_step() for q in ops.rules.questions)
+    # config B: one layer sees everything, two see the last 24 positions; 1 kv head of 32, float32
+    per_token = 2 * 32 * 4
+    seen = lambda n: per_token * (n + 2 * min(n, 24))
+    assert [q[2] for q in ops.rules.questions] == [seen(31) + seen(8), seen(32) + seen(9), seen(33)]

@@ -164,3 +164,11 @@ def test_schedule_may_repeat_a_block_and_share_a_cache():
 def CausalLMFromSpec(spec, cfg):
     from llm_inference_lab_amd.engine.model import CausalLM
     return CausalLM(spec)
+
+
+def test_another_block_arrangement_in_random_weights_mode(tmp_path):
+    """The toy architecture of tests/toy_parallel.py (a block with one norm and two parallel
+    sublayers, norm tensors called ``gain``) over the kernel references: the random-weights
+    mode draws its tensors as the parts say, the folder loads, every cut matches."""
+    import toy_parallel
+    toy_parallel.run("f32", str(tmp_path / "toy4"), ops=EmuOps(), device="cpu")

@@ -176,11 +176,19 @@ def test_greedy_generation_through_the_entry_point(name):
         assert m["rows_used"] == 0 and all(g["pages_used"] == 0 for g in m["groups"])
         if graph:
             assert engine.step_fn.graph_replays > 0
-    # bfloat16 follows the same tokens while the margins are clear of its rounding
+    # bfloat16 may part from the plain tokens only where the plain choice was closer than
+    # its rounding (twice the bound on a logit); from there on its own history differs
     engine = H.make_engine(name, 1, "bf16", max_batch_tokens=16)
     got = engine.generate(prompts, max_new_tokens=16, eos_token_id=[])
-    agree = sum(a == b for g, w in zip(got, want) for a, b in zip(g, w))
-    assert agree >= 0.8 * 16 * len(prompts), (got, want)
+    for prompt, g, w in zip(prompts, got, want):
+        assert len(g) == 16
+        logits = H.plain_logits(name, 1, prompt + w)
+        for i, (a, b) in enumerate(zip(g, w)):
+            if a != b:
+                top = logits[len(prompt) + i - 1].topk(2).values
+                assert float(top[0] - top[1]) <= 2 * H.TOL["bf16"], \
+                    f"bfloat16 strays at a clear choice (margin {float(top[0] - top[1]):.3f}): {g} vs {w}"
+                break
 
 
 @pytest.mark.parametrize("name,graph", [("A", False), ("B", True)])

@@ -39,6 +39,7 @@ def ragged_decode(name, dtype, graph, splits=None, prompts=(5, 60, 130, 250), de
     else:
         with engine.ops.debug.force(attention_splits=(cfg.head_dim, splits)):
             got = H.run_trace(engine, seqs, steps)
+    assert not any(bool(torch.isnan(g).any()) for g in got.values()), "a position's logits did not come back"
     bad = H.first_wrong(got, want, tolerance(name, dtype))
     assert bad is None, f"first wrong logits at (request, position, error) = {bad}"
     return engine
@@ -93,6 +94,7 @@ def test_more_graph_keys_than_are_kept(dtype):
     assert fn.graph_evictions > 0 and len(fn._graphs) <= fn.MAX_GRAPHS
     assert captures[0] > fn.MAX_GRAPHS and captures[1] > captures[0]        # dropped keys come back
     assert fn.graph_replays > 100
+    assert not any(bool(torch.isnan(g).any()) for g in got.values()), "a position's logits did not come back"
     bad = H.first_wrong(got, want, H.TOL[dtype])
     assert bad is None, f"first wrong logits at (request, position, error) = {bad}"
     m = engine.cache.metrics()

@@ -229,13 +229,14 @@ def toy_spec(cfg):
     norm = lambda n: PartSpec("rmsnorm", dict(size=h, eps=cfg.eps), dict(weight=n))
     ffn = lambda p: PartSpec("swiglu", dict(hidden_size=h, intermediate_size=2 * h),
                              dict(gate_weight=p + "gate", up_weight=p + "up", down_weight=p + "down"))
-    toy = BlockSpec("prenorm", mixer=PartSpec("toy_running_mean", dict(hidden_size=h), dict(weight="l0.mix")),
-                    feed_forward=ffn("l0."), norm1=norm("l0.n1"), norm2=norm("l0.n2"), params=dict(hidden_size=h))
-    attn = BlockSpec("prenorm", mixer=PartSpec(
+    toy = BlockSpec("prenorm", dict(
+        mixer=PartSpec("toy_running_mean", dict(hidden_size=h), dict(weight="l0.mix")),
+        feed_forward=ffn("l0."), norm1=norm("l0.n1"), norm2=norm("l0.n2")), params=dict(hidden_size=h))
+    attn = BlockSpec("prenorm", dict(mixer=PartSpec(
         "gqa_attention", dict(hidden_size=h, num_heads=2, num_kv_heads=1, head_dim=h // 2, qkv_bias=False,
                               position=None, window=None),
         dict(q_weight="l1.q", k_weight="l1.k", v_weight="l1.v", o_weight="l1.o")),
-        feed_forward=ffn("l1."), norm1=norm("l1.n1"), norm2=norm("l1.n2"), params=dict(hidden_size=h))
+        feed_forward=ffn("l1."), norm1=norm("l1.n1"), norm2=norm("l1.n2")), params=dict(hidden_size=h))
     sizes = dict(vocab_size=cfg.vocab_size, hidden_size=h)
     return ModelSpec("ToyForCausalLM", cfg.vocab_size, h, 4096,
                      PartSpec("token_embedding", sizes, dict(weight="embed")), (toy, attn),
@@ -274,8 +275,7 @@ def test_toy_mixer_with_state_is_registered_built_and_stepped(dtype):
         cfg = ToyConfig(vocab_size=97, hidden_size=64, eps=1e-5)
         from llm_inference_lab_amd.engine.model import CausalLM
         from llm_inference_lab_amd.weights import random_tensors
-        tensors = dict(random_tensors(CausalLM(toy_spec(cfg)).tensor_specs(), 3, torch.bfloat16,
-                                      is_norm=lambda n: n.endswith(("n1", "n2", "final"))))
+        tensors = dict(random_tensors(CausalLM(toy_spec(cfg)).tensor_specs(), 3, torch.bfloat16))
         for n in ("embed", "l1.q", "l1.k"):
             tensors[n] = (tensors[n].float() * 8).to(torch.bfloat16)
         engine = H.lab.Engine(config=cfg, tensors=tensors.items(), dtype=dtype, page_size=16, num_pages=16,
@@ -394,14 +394,14 @@ def toy2_spec(cfg):
     h = cfg.hidden_size
     norm = lambda n: PartSpec("rmsnorm", dict(size=h, eps=cfg.eps), dict(weight=n))
     block = BlockSpec(
-        "prenorm",
-        mixer=PartSpec("gqa_attention",
-                       dict(hidden_size=h, num_heads=2, num_kv_heads=2, head_dim=h // 2, qkv_bias=False,
-                            position=PartSpec("toy_half_rotary", dict(dim=h // 2, theta=cfg.theta)), window=None),
-                       dict(q_weight="q", k_weight="k", v_weight="v", o_weight="o")),
-        feed_forward=PartSpec("toy_top_one_experts", dict(hidden_size=h, num_experts=cfg.num_experts),
-                              dict(router="router", experts="expert")),
-        norm1=norm("n1"), norm2=norm("n2"), params=dict(hidden_size=h))
+        "prenorm", dict(
+            mixer=PartSpec("gqa_attention",
+                           dict(hidden_size=h, num_heads=2, num_kv_heads=2, head_dim=h // 2, qkv_bias=False,
+                                position=PartSpec("toy_half_rotary", dict(dim=h // 2, theta=cfg.theta)), window=None),
+                           dict(q_weight="q", k_weight="k", v_weight="v", o_weight="o")),
+            feed_forward=PartSpec("toy_top_one_experts", dict(hidden_size=h, num_experts=cfg.num_experts),
+                                  dict(router="router", experts="expert")),
+            norm1=norm("n1"), norm2=norm("n2")), params=dict(hidden_size=h))
     sizes = dict(vocab_size=cfg.vocab_size, hidden_size=h)
     return ModelSpec("Toy2ForCausalLM", cfg.vocab_size, h, 4096,
                      PartSpec("token_embedding", sizes, dict(weight="embed")), (block,),
@@ -444,8 +444,7 @@ def test_toy_routed_feed_forward_and_other_position_encoding(dtype):
         cfg = Toy2Config(vocab_size=61, hidden_size=64, num_experts=3, theta=100.0, eps=1e-6)
         from llm_inference_lab_amd.engine.model import CausalLM
         from llm_inference_lab_amd.weights import random_tensors
-        tensors = dict(random_tensors(CausalLM(toy2_spec(cfg)).tensor_specs(), 5, torch.bfloat16,
-                                      is_norm=lambda n: n in ("n1", "n2", "final")))
+        tensors = dict(random_tensors(CausalLM(toy2_spec(cfg)).tensor_specs(), 5, torch.bfloat16))
         for n in ("embed", "q", "k"):
             tensors[n] = (tensors[n].float() * 8).to(torch.bfloat16)
         # a decisive router: the best expert wins by a margin that bfloat16 rounding cannot turn
@@ -563,12 +562,12 @@ def toy3_spec(cfg):
     norm = lambda n: PartSpec("rmsnorm", dict(size=h, eps=cfg.eps), dict(weight=n))
     def block(p):
         return BlockSpec(
-            "prenorm",
-            mixer=PartSpec("toy_latent_mixer", dict(hidden_size=h, latent_size=cfg.latent_size),
-                           dict(down=p + "down", query=p + "query", up=p + "up")),
-            feed_forward=PartSpec("swiglu", dict(hidden_size=h, intermediate_size=2 * h),
-                                  dict(gate_weight=p + "gate", up_weight=p + "ffn_up", down_weight=p + "ffn_down")),
-            norm1=norm(p + "n1"), norm2=norm(p + "n2"), params=dict(hidden_size=h))
+            "prenorm", dict(
+                mixer=PartSpec("toy_latent_mixer", dict(hidden_size=h, latent_size=cfg.latent_size),
+                               dict(down=p + "down", query=p + "query", up=p + "up")),
+                feed_forward=PartSpec("swiglu", dict(hidden_size=h, intermediate_size=2 * h),
+                                      dict(gate_weight=p + "gate", up_weight=p + "ffn_up", down_weight=p + "ffn_down")),
+                norm1=norm(p + "n1"), norm2=norm(p + "n2")), params=dict(hidden_size=h))
     sizes = dict(vocab_size=cfg.vocab_size, hidden_size=h)
     return ModelSpec("Toy3ForCausalLM", cfg.vocab_size, h, cfg.max_positions,
                      PartSpec("toy_positional_embedding", dict(max_positions=cfg.max_positions, **sizes),
@@ -603,8 +602,7 @@ def test_toy_embedding_with_positions_and_mixer_with_a_cache_of_its_own_shape(dt
         cfg = Toy3Config(vocab_size=83, hidden_size=64, latent_size=24, max_positions=256, eps=1e-5)
         from llm_inference_lab_amd.engine.model import CausalLM
         from llm_inference_lab_amd.weights import random_tensors
-        tensors = dict(random_tensors(CausalLM(toy3_spec(cfg)).tensor_specs(), 7, torch.bfloat16,
-                                      is_norm=lambda n: n.endswith(("n1", "n2", "final"))))
+        tensors = dict(random_tensors(CausalLM(toy3_spec(cfg)).tensor_specs(), 7, torch.bfloat16))
         for n in tensors:
             if n in ("embed", "places") or n.endswith(("down", "query")) and "ffn" not in n:
                 tensors[n] = (tensors[n].float() * 8).to(torch.bfloat16)
@@ -630,3 +628,12 @@ def test_toy_embedding_with_positions_and_mixer_with_a_cache_of_its_own_shape(dt
         unregister_part("embedding", "toy_positional_embedding")
         unregister_part("mixer", "toy_latent_mixer")
         unregister_architecture("Toy3ForCausalLM")
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_toy_block_of_another_arrangement_in_random_weights_mode(dtype, tmp_path):
+    """A block kind with one norm and two parallel sublayers and a norm kind whose tensors
+    are not called norm (tests/toy_parallel.py): registered, written by the random-weights
+    mode, loaded and stepped without a change to the framework's files."""
+    import toy_parallel
+    toy_parallel.run(dtype, str(tmp_path / "toy4"))

@@ -34,13 +34,19 @@ _FLOORS = {}
 
 
 def rounding_floor(seed, name, seqs, want):
-    """Largest error of the emulated kernels (every request alone and whole) against plain."""
+    """What rounding to bfloat16 costs this configuration, measured without any code of the
+    product: the plain implementation with every stored activation rounded to bfloat16
+    where the reference rounds to its storage type (norm outputs, q, k, v, attention and
+    SwiGLU outputs; float64 sums), against the plain implementation without."""
     if seed not in _FLOORS:
-        from emu_ops import EmuOps
-        engine = H.make_engine(name, 2, "bf16", ops=EmuOps(), device="cpu", page_size=16, num_pages=64,
-                               max_requests=len(seqs))
-        got = H.run_trace(engine, seqs, H.steps_whole(seqs))
-        _FLOORS[seed] = H.max_error(got, want)
+        import torch
+        import plain_qwen2
+        cfg = H.config_of(name)
+        weights = {k: v.double() for k, v in H.make_tensors(cfg, 2).items()}
+        round_bf16 = lambda t: t.to(torch.bfloat16).to(t.dtype)
+        _FLOORS[seed] = max(
+            float((plain_qwen2.forward_logits(ids, weights, cfg.to_dict(), cast=round_bf16) - want[rid]).abs().max())
+            for rid, ids in seqs.items())
     return _FLOORS[seed]
 
 
@@ -64,10 +70,11 @@ def test_drawn_configuration(seed, cut, dtype):
     # The suite's bounds hold for logits of order 1 to 16 (configurations A to C).  A drawn
     # configuration with a tied head has logits up to 25, and deeper or wider ones round more
     # often.  float32: the bound grows with the largest logit beyond 8.  bfloat16: what the
-    # roundings of the kernels cost for this very configuration is measured with their
-    # emulation on the CPU (tests/emu_ops.py: float32 arithmetic, the same roundings); the
-    # GPU may be off by half as much again (other orders of its float32 sums), never by
-    # less than the suite's bound allows.
+    # roundings cost for this very configuration is measured with the plain implementation
+    # itself (``rounding_floor``: no code of the product, so a mistake of the engine cannot
+    # widen its own bound); the GPU may be off by half as much again (its probabilities are
+    # rounded too, its sums are float32 in other orders), never by less than the suite's
+    # bound allows.
     if dtype == "f32":
         bound = H.TOL[dtype] * max(1.0, max(float(w.abs().max()) for w in want.values()) / 8.0)
     else:
