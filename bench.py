@@ -20,9 +20,22 @@ back).  One JSON line is printed: decoded tokens a second as ``value``, plus
   difference below 1e-3 in float32 and 0.5 in bfloat16), and greedy tokens of two runs
   with fresh caches (identical), as the reference's bench does
   (rust/engine/benches/qwen2.rs:247-274, 317-369);
+* ``samples``: every point is timed three times (``--samples``), each time with fresh requests
+  and fresh cache pages, and the median counts (``value``, ``ms_per_step``, the prefill's
+  ``ms``); the smallest and the largest are printed beside it, as the reference's bench
+  reports mean / p50 / p95 over its iterations (rust/engine/benches/qwen2.rs:279-316);
+* ``measured``: what this very GPU gives to the simplest kernels (``csrc/measure.hip``, run
+  in a child process before anything else): a read stream and a copy over 4 GiB, and
+  waves that only issue matrix instructions (bfloat16 16x16x32 and float32 32x32x2).
+  ``roofline`` and ``prefill`` carry ``measured_peak`` and ``frac_measured`` beside the
+  fractions of the published peaks (8 TB/s; 2.5 PFLOP/s bfloat16, 157.3 TFLOP/s float32);
 * ``step_ms``: median and 95th percentile of single steps timed through GPU completion;
 * ``eager`` or ``graph``: the same decode steps the other way (launched kernel by kernel,
   or replayed from a HIP graph; ``--graph auto``, the default, lets the engine choose).
+
+``--profile``: for runs under ``rocprofv3``: collection is paused (rocTX) except around the
+timed steps, so that the profile holds those and not the filling of the caches
+(rust/engine/benches/qwen2.rs:110-114, 175-179, 297-301).
 
 ``--mixed``: many requests with prompts of different lengths go through the
 scheduler with a small token budget, so that portions of prompts run beside the
@@ -83,17 +96,10 @@ def prefill_flops(cfg, tokens):
 
 def random_weights_on_the_gpu(expected, seed):
     """Random weights of a large shape drawn on the GPU (the 65 GB of the 32B shape take
-    minutes on the host): N(0, 0.02), norm weights 1 + N(0, 0.1), in bfloat16."""
+    minutes on the host), by the product's own rule for every tensor."""
     import torch
-    from llm_inference_lab_amd.weights.loader import VECTOR
-    gen = torch.Generator(device="cuda:0")
-    gen.manual_seed(seed)
-    for name, spec in expected.items():
-        values = torch.randn(spec.shape, generator=gen, dtype=torch.bfloat16, device="cuda:0")
-        if spec.kind == VECTOR and "norm" in name:
-            yield name, (1.0 + 0.1 * values.float()).to(torch.bfloat16)
-        else:
-            yield name, values.mul_(0.02)
+    from llm_inference_lab_amd.weights import random_tensors
+    return random_tensors(expected, seed, torch.bfloat16, device="cuda:0")
 
 
 def make_engine(args, cfg, max_cache_tokens, max_requests, max_batch_tokens, max_seq_len):
@@ -110,14 +116,109 @@ def make_engine(args, cfg, max_cache_tokens, max_requests, max_batch_tokens, max
                       graph=False if args.no_graph else args.graph)
 
 
+class ProfilerBracket:
+    """``--profile``: the profiler collects inside ``with bracket:`` only.  rocTX's pause and
+    resume calls, which ``rocprofv3`` obeys; without the library, or without the flag,
+    nothing happens."""
+
+    def __init__(self, enabled):
+        self.lib = None
+        if enabled:
+            import ctypes
+            for name in ("librocprofiler-sdk-roctx.so", "/opt/rocm/lib/librocprofiler-sdk-roctx.so"):
+                try:
+                    self.lib = ctypes.CDLL(name)
+                    self.lib.roctxProfilerPause.argtypes = [ctypes.c_uint64]
+                    self.lib.roctxProfilerResume.argtypes = [ctypes.c_uint64]
+                    self.lib.roctxRangePushA.argtypes = [ctypes.c_char_p]
+                    break
+                except (OSError, AttributeError):
+                    self.lib = None
+            if self.lib is None:
+                print("bench.py: --profile: no rocTX library found, the whole run is collected", file=sys.stderr)
+            else:
+                self.lib.roctxProfilerPause(0)
+
+    def __enter__(self):
+        if self.lib is not None:
+            self.lib.roctxProfilerResume(0)
+            self.lib.roctxRangePushA(b"timed steps")
+        return self
+
+    def __exit__(self, *exc):
+        if self.lib is not None:
+            self.lib.roctxRangePop()
+            self.lib.roctxProfilerPause(0)
+        return False
+
+
+def spread(values, digits=4):
+    """Median, smallest and largest of the samples."""
+    ordered = sorted(values)
+    n = len(ordered)
+    median = ordered[n // 2] if n % 2 else 0.5 * (ordered[n // 2 - 1] + ordered[n // 2])
+    return {"median": round(median, digits), "min": round(ordered[0], digits), "max": round(ordered[-1], digits),
+            "n": n}
+
+
+def measured_peaks():
+    """What this GPU gives to the simplest kernels: GB/s of a read stream and of a copy over
+    4 GiB, TFLOP/s of waves that only issue matrix instructions.  Medians of five launches."""
+    import ctypes
+    import torch
+    from llm_inference_lab_amd.kernels import build
+    lib = ctypes.CDLL(build.measure_library())
+    vp, cs, ci = ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int
+    lib.llmlab_measure_read.argtypes = [vp, cs, vp, ci, vp]
+    lib.llmlab_measure_copy.argtypes = [vp, vp, cs, ci, vp]
+    lib.llmlab_measure_mfma.argtypes = [ci, ci, ci, vp, ctypes.POINTER(ctypes.c_double), vp]
+    torch.cuda.set_device(0)
+    stream = torch.cuda.current_stream().cuda_stream
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    size = 4 << 30
+    src = torch.empty(size, dtype=torch.uint8, device="cuda:0")
+    dst = torch.empty(size, dtype=torch.uint8, device="cuda:0")
+    src.random_(0, 255)
+    sink = torch.zeros(4096, dtype=torch.float32, device="cuda:0")
+
+    def timed(launch, repeats=5):
+        launch()
+        torch.cuda.synchronize()
+        times = []
+        for _ in range(repeats):
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record()
+            assert launch() == 0
+            end.record()
+            end.synchronize()
+            times.append(start.elapsed_time(end) * 1e-3)
+        return spread(times, 9)["median"]
+
+    out = {"stream_bytes": size, "compute_units": cus}
+    blocks = cus * 8
+    t = timed(lambda: lib.llmlab_measure_read(src.data_ptr(), size, sink.data_ptr(), blocks, stream))
+    out["hbm_read_gbs"] = round(size / t / 1e9, 1)
+    t = timed(lambda: lib.llmlab_measure_copy(src.data_ptr(), dst.data_ptr(), size, blocks, stream))
+    out["hbm_copy_gbs"] = round(2 * size / t / 1e9, 1)
+    for name, f32, iterations in (("mfma_bf16_tflops", 0, 20000), ("mfma_f32_tflops", 1, 5000)):
+        flops = ctypes.c_double(0.0)
+        t = timed(lambda: lib.llmlab_measure_mfma(f32, cus * 8, iterations, sink.data_ptr(), ctypes.byref(flops),
+                                                  stream))
+        out[name] = round(flops.value / t / 1e12, 1)
+    return out
+
+
 class Runs:
     """The timed runs over one engine."""
 
-    def __init__(self, engine, cfg, context, dtype):
+    def __init__(self, engine, cfg, context, dtype, samples=3, bracket=None, measured=None):
         import torch
         self.torch = torch
         self.engine, self.cfg, self.context, self.dtype = engine, cfg, context, dtype
         self.gen = torch.Generator().manual_seed(1234)
+        self.samples = max(1, int(samples))
+        self.bracket = bracket or ProfilerBracket(False)
+        self.measured = measured or {}
 
     def random_ids(self, n):
         return self.torch.randint(0, self.cfg.vocab_size, (n,), generator=self.gen).tolist()
@@ -150,22 +251,34 @@ class Runs:
         assert len(sched.active) == batch
         live_tokens = sum(r.computed for r in sched.active)
         self.sync()
-        t0 = time.perf_counter()
-        for _ in range(steps):
-            sched.step()
-        self.sync()
-        seconds = time.perf_counter() - t0
+        with self.bracket:
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                sched.step()
+            self.sync()
+            seconds = time.perf_counter() - t0
         assert len(sched.active) == batch, "a request ended inside the timed steps"
         live_tokens = (live_tokens + sum(r.computed for r in sched.active)) / 2
         done = sched.run()
         assert engine.cache.live_requests == 0 and all(r.error is None for r in done.values())
         return seconds, live_tokens
 
+    def decode_samples(self, batch, steps, warmup):
+        """``decode`` as often as ``--samples`` says, every time with fresh requests and pages:
+        (seconds of the median sample, live tokens, spread of ms a step)."""
+        runs = [self.decode(batch, steps, warmup) for _ in range(self.samples)]
+        ms = spread([sec / steps * 1e3 for sec, _ in runs])
+        return ms["median"] * steps / 1e3, runs[0][1], ms
+
     def roofline(self, seconds, steps, live_tokens):
         step_bytes = self.engine.weight_bytes_per_step() + live_tokens * self.engine.cache.bytes_per_token()
         achieved = step_bytes / (seconds / steps) / 1e9
-        return {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
-                "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4)}
+        out = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS,
+               "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4)}
+        if self.measured.get("hbm_read_gbs"):
+            out["measured_peak"] = self.measured["hbm_read_gbs"]
+            out["frac_measured"] = round(achieved / self.measured["hbm_read_gbs"], 4)
+        return out
 
     def step_latencies(self, batch, steps=32):
         """Single decode steps, each timed through GPU completion: (p50, p95) in ms."""
@@ -190,21 +303,37 @@ class Runs:
         times.sort()
         return round(times[len(times) // 2], 4), round(times[min(len(times) - 1, int(len(times) * 0.95))], 4)
 
-    def prefill(self, tokens=2048, repeats=4):
+    def prefill(self, tokens=2048, repeats=None):
+        """One prompt in one step, logits at its last place: one untimed run, then the median
+        of ``repeats`` (at least ``--samples``, at least three) with a fresh request each."""
         from llm_inference_lab_amd.engine.step import StepEntry
+        repeats = repeats or max(3, self.samples)
         times = []
-        for _ in range(repeats):
+        for i in range(repeats + 1):
             req = self.engine.open("prefill")
             ids = self.random_ids(tokens)
             self.sync()
-            t0 = time.perf_counter()
-            self.engine.step([StepEntry(req, ids, [tokens - 1])])
-            self.sync()
-            times.append(time.perf_counter() - t0)
+            if i == 0:
+                self.engine.step([StepEntry(req, ids, [tokens - 1])])
+                self.sync()
+            else:
+                with self.bracket:
+                    t0 = time.perf_counter()
+                    self.engine.step([StepEntry(req, ids, [tokens - 1])])
+                    self.sync()
+                    times.append(time.perf_counter() - t0)
             self.engine.close(req)
-        best = min(times[1:])
-        return {"value": round(tokens / best, 1), "tokens": tokens, "ms": round(best * 1e3, 3),
-                "frac": round(prefill_flops(self.cfg, tokens) / best / PEAK_FLOPS[self.dtype], 4)}
+        ms = spread([t * 1e3 for t in times], 3)
+        median = ms["median"] * 1e-3
+        flops = prefill_flops(self.cfg, tokens)
+        out = {"value": round(tokens / median, 1), "tokens": tokens, "ms": ms["median"],
+               "frac": round(flops / median / PEAK_FLOPS[self.dtype], 4), "ms_min": ms["min"], "ms_max": ms["max"],
+               "samples": ms["n"]}
+        key = "mfma_bf16_tflops" if self.dtype == "bf16" else "mfma_f32_tflops"
+        if self.measured.get(key):
+            out["measured_peak"] = self.measured[key]
+            out["frac_measured"] = round(flops / median / (self.measured[key] * 1e12), 4)
+        return out
 
     def validate(self, tokens=None, chunk=256):
         """Whole against portions at the last position of a long prompt, and two greedy runs
@@ -276,7 +405,8 @@ def mixed_run(args, cfg, engine=None):
         return seconds, steps
 
     one_run()                                   # warm-up: scratch buffers, graphs, kernel loading
-    seconds, steps = one_run()
+    timed = sorted(one_run() for _ in range(max(1, getattr(args, "samples", 1))))
+    seconds, steps = timed[len(timed) // 2]     # the median run; every run serves fresh requests
     prompt_tokens, new_tokens = sum(lengths), args.requests * args.outputs
     # every prompt token and every generated token but a request's last goes through the model once
     flops = sum(prefill_flops(cfg, n + args.outputs - 1) - 2 * cfg.hidden_size * cfg.vocab_size for n in lengths)
@@ -297,7 +427,8 @@ def mixed_run(args, cfg, engine=None):
             "outputs_per_request": args.outputs, "token_budget": args.chunk + args.requests,
             "page_size": PAGE, "weights_seed": 0,
         },
-        "seconds": round(seconds, 4), "generated_tokens_per_second": round(new_tokens / seconds, 1),
+        "seconds": round(seconds, 4), "seconds_min": round(timed[0][0], 4), "seconds_max": round(timed[-1][0], 4),
+        "samples": len(timed), "generated_tokens_per_second": round(new_tokens / seconds, 1),
         "flops_frac": round(flops / seconds / PEAK_FLOPS[args.dtype], 4),
     }
 
@@ -317,19 +448,20 @@ def child(*flags, timeout=420):
         return None
 
 
-def side_points(args):
+def side_points(args, measured):
     """The points of the default line that other shapes and the other dtype give, each from
     a child process of its own (run before this process touches the GPU)."""
     points, validation = {}, {}
     steps, warmup = str(max(8, args.steps // 2)), str(max(2, args.warmup // 2))
-    line = child("--side", "7b", "--steps", steps, "--warmup", warmup)
+    common = ["--steps", steps, "--warmup", warmup, "--samples", str(args.samples)]
+    line = child("--side", "7b", *common)
     if line is not None:
         points["decode_b8_7b"], points["hbm_frac_b8_7b"] = line["decode_b8"], line["hbm_frac_b8"]
         points["mixed_7b_tokens_per_second"] = line["mixed_tokens_per_second"]
-    line = child("--side", "32b", "--steps", steps, "--warmup", warmup)
+    line = child("--side", "32b", *common)
     if line is not None:
         points["decode_b8_32b"], points["hbm_frac_b8_32b"] = line["decode_b8"], line["hbm_frac_b8"]
-    line = child("--side", "f32", "--steps", steps, "--warmup", warmup)
+    line = child("--side", "f32", *common)
     if line is not None:
         for key in ("decode_b1", "decode_b8", "decode_b64", "prefill_tokens_per_second", "prefill_frac"):
             points[f"f32_{key}"] = line[key]
@@ -341,19 +473,22 @@ def side_run(args):
     """One child's work: ``--side 7b`` (decode at batch 8, context 4096, then the mixed run
     on the same engine), ``--side 32b`` (decode at batch 8, context 8192), ``--side f32``
     (the 0.5B shape in float32: validation, decode at batch 1 / 8 / 64, the prefill)."""
+    if args.side == "peaks":
+        print(json.dumps(measured_peaks()))
+        return
     import llm_inference_lab_amd as lab
     if args.side == "f32":
         args.shape, args.dtype = "0.5b", "f32"
         cfg = lab.Qwen2Config.from_dict(dict(SHAPES["0.5b"]))
         context = DEFAULT_CONTEXT["0.5b"]
         engine = make_engine(args, cfg, 64 * (context + PAGE), 64, FILL_TOKENS, context + PAGE)
-        runs = Runs(engine, cfg, context, "f32")
+        runs = Runs(engine, cfg, context, "f32", args.samples)
         out = {"validation": runs.validate()}
         for batch in (1, 8, 64):
             steps = max(4, args.steps // (1 if batch < 64 else 2))
-            seconds, _ = runs.decode(batch, steps, args.warmup)
+            seconds, _, _ = runs.decode_samples(batch, steps, args.warmup)
             out[f"decode_b{batch}"] = round(batch * steps / seconds, 1)
-        prefill = runs.prefill(repeats=3)
+        prefill = runs.prefill()
         out["prefill_tokens_per_second"], out["prefill_frac"] = prefill["value"], prefill["frac"]
         print(json.dumps(out))
         return
@@ -366,8 +501,8 @@ def side_run(args):
     mixed_tokens = sum(n + args.outputs + PAGE for n in lengths) if args.shape == "7b" else 0
     engine = make_engine(args, cfg, max(8 * (context + PAGE), mixed_tokens), max(8, args.requests),
                          FILL_TOKENS, max(context, max(lengths) + args.outputs) + PAGE)
-    runs = Runs(engine, cfg, context, "bf16")
-    seconds, live = runs.decode(8, args.steps, args.warmup)
+    runs = Runs(engine, cfg, context, "bf16", args.samples)
+    seconds, live, _ = runs.decode_samples(8, args.steps, args.warmup)
     out = {"decode_b8": round(8 * args.steps / seconds, 1),
            "hbm_frac_b8": runs.roofline(seconds, args.steps, live)["frac"]}
     if args.shape == "7b":
@@ -402,7 +537,16 @@ def main():
                     help="with --only-prefill: the length of the prompt (at most 8192, one step)")
     ap.add_argument("--only-prefill", action="store_true",
                     help="run nothing but the 2,048-token prefill (for profiling); prints its numbers")
-    ap.add_argument("--side", choices=["7b", "32b", "f32"], help=argparse.SUPPRESS)
+    ap.add_argument("--samples", type=int, default=3,
+                    help="how often every point is timed, each time with fresh requests; the median counts")
+    ap.add_argument("--profile", action="store_true",
+                    help="under rocprofv3: collect the timed steps only (rocTX pause / resume around them)")
+    ap.add_argument("--no-measured", action="store_true", help="skip the stream and matrix-instruction loops")
+    ap.add_argument("--force", action="append", default=[], metavar="KEY=VALUE",
+                    help="fix a choice of the kernels for the whole run, to compare variants: a keyword of "
+                         "engine.ops.debug.force, values separated by ':' (attention_splits=64:8, "
+                         "attention_merge_kernel=64, gemm_tile=129)")
+    ap.add_argument("--side", choices=["7b", "32b", "f32", "peaks"], help=argparse.SUPPRESS)
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
@@ -417,7 +561,10 @@ def main():
     # child process of its own, before this process touches the GPU.
     default_line = not (args.mixed or args.no_points or args.only_prefill) and args.shape == "0.5b" \
         and args.dtype == "bf16"
-    side, side_validation = side_points(args) if default_line else ({}, {})
+    measured = {}
+    if not (args.no_measured or args.mixed or args.profile):
+        measured = child("--side", "peaks", timeout=120) or {}
+    side, side_validation = side_points(args, measured) if default_line else ({}, {})
 
     import llm_inference_lab_amd as lab
 
@@ -431,7 +578,15 @@ def main():
     max_batch = max(batches)
     context = args.context or DEFAULT_CONTEXT[args.shape]
     engine = make_engine(args, cfg, max_batch * (context + PAGE), max_batch, FILL_TOKENS, context + PAGE)
-    runs = Runs(engine, cfg, context, args.dtype)
+    runs = Runs(engine, cfg, context, args.dtype, args.samples, ProfilerBracket(args.profile), measured)
+    if args.force:
+        forced = {}
+        for item in args.force:
+            key, _, value = item.partition("=")
+            numbers = [float(v) if "." in v else int(v) for v in value.split(":")]
+            forced[key] = numbers[0] if len(numbers) == 1 else tuple(numbers)
+        engine.forced_for_this_run = engine.ops.debug.force(**forced)    # (kept: it restores when collected)
+        engine.forced_for_this_run.__enter__()
 
     if args.only_prefill:
         if not 0 < args.prefill_tokens <= min(FILL_TOKENS, context):
@@ -443,7 +598,7 @@ def main():
     if not args.no_validate:
         validation[args.dtype] = runs.validate()
 
-    seconds, live_tokens = runs.decode(args.batch, args.steps, args.warmup)
+    seconds, live_tokens, ms_spread = runs.decode_samples(args.batch, args.steps, args.warmup)
     value = args.batch * args.steps / seconds
     result = {
         "metric": "decode_tokens_per_second", "value": round(value, 1), "unit": "tokens/s",
@@ -461,7 +616,10 @@ def main():
             "hip_graph_decode": bool(engine.step_fn.use_graph), "weights_seed": 0,
         },
         "roofline": runs.roofline(seconds, args.steps, live_tokens),
+        "samples": {"ms_per_step": ms_spread},
     }
+    if measured:
+        result["measured"] = measured
     if validation:
         result["validation"] = validation
     if not args.no_points:
@@ -473,8 +631,9 @@ def main():
             if b == args.batch:
                 points[f"decode_b{b}"] = round(value, 1)
                 continue
-            s, _ = runs.decode(b, half_steps, half_warmup)
+            s, _, spread_b = runs.decode_samples(b, half_steps, half_warmup)
             points[f"decode_b{b}"] = round(b * half_steps / s, 1)
+            result["samples"][f"decode_b{b}_ms_per_step"] = spread_b
         points.update(side)
         result["points"] = points
         p50, p95 = runs.step_latencies(args.batch)

@@ -45,6 +45,16 @@ constexpr float NEG_INF = -__builtin_huge_valf();
 // which is what a softmax wants of them)
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// Stores and loads of device scope: the value goes through the L2 of this die to memory
+// (and comes from there), so that blocks on different dies, each behind an L2 of its own,
+// can hand results to each other within one kernel without flushing those caches.
+__device__ __forceinline__ void store_device(float* p, float v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float load_device(const float* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // Maxima across the four lanes that hold the keys of one row, by the lane-swap
 // instructions of gfx950 instead of LDS permutes.  (No inline assembly for the
 // maxima themselves: the compiler does not see the wait states an MFMA result needs
@@ -71,6 +81,9 @@ struct AttnArgs {
   void* out;          // [rows, out_stride]
   float* o_part;      // [rows*nq, splits, D]      (splits > 1)
   float* ml_part;     // [rows*nq, splits, 2]
+  int* arrived;       // [reqs * nkv] counters, zero between launches: the split blocks of a
+                      // (request, kv head) count themselves here and the last one merges
+                      // (null: a kernel of its own merges)
   int q_stride, out_stride, table_stride, page_size;
   int nq, nkv, window, splits;
   int page_shift;     // log2(page_size); page sizes are powers of two
@@ -666,16 +679,76 @@ __device__ __forceinline__ void attention_tile(const AttnArgs& a, const int xblk
           ((bf16_t*)a.out)[(size_t)(r0 + t) * a.out_stride + (size_t)hh * D + dd] =
               (bf16_t)(den > 0.f ? num / den : 0.f);
         } else {
+          // (stores of device scope: written through to memory, where a block on another
+          // die finds them without a fence; see below)
           const size_t at = ((size_t)(r0 + t) * a.nq + hh) * a.splits + split;
-          a.o_part[at * D + dd] = num;
+          store_device(&a.o_part[at * D + dd], num);
           if (dd == 0) {
-            a.ml_part[at * 2] = mmax;
-            a.ml_part[at * 2 + 1] = den;
+            store_device(&a.ml_part[at * 2], mmax);
+            store_device(&a.ml_part[at * 2 + 1], den);
           }
         }
       }
     };
     merge(nw, a.splits == 1);
+    if constexpr (QB == 1) {        // (tiles of more rows are never split over blocks)
+    if (a.splits == 1 || a.arrived == nullptr) return;
+    // ---- the block that arrives last merges the splits of its (request, kv head):
+    //   out = sum_s w_s acc_s / sum_s w_s l_s,  w_s = 2^(m_s - max m)
+    // No fence: a fence of device scope writes back and invalidates the whole L2 of the
+    // die, which costs more than the kernel it saves.  Instead the partial results are
+    // stored and loaded with device scope (they pass the L2 of the die by), every thread
+    // waits until its stores are done, the block meets at a barrier, and then one thread
+    // counts the block in with an atomic of device scope.  Whoever reads splits - 1 there
+    // knows that all other blocks' results are in memory.  It sets the counter back to
+    // zero for the next launch.  Nobody waits for anybody: a block that is not the last
+    // simply ends.
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    __shared__ int s_last;
+    if (threadIdx.x == 0) {
+      int* counter = a.arrived + (size_t)b * a.nkv + kvh;
+      const int before = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      s_last = before == a.splits - 1;
+      if (s_last) __hip_atomic_store(counter, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (!s_last) return;
+    // maxima and denominators of all splits of the block's rows, through LDS: [row][split]
+    __shared__ float x_m[16 * MAX_KEY_SPLITS], x_l[16 * MAX_KEY_SPLITS];
+    const int S = a.splits;
+    for (int i = threadIdx.x; i < nrows * S; i += blockDim.x) {
+      const int r = i / S, sidx = i - r * S;
+      const int t = (row0 + r) / G, hh = kvh * G + (row0 + r) % G;
+      const size_t at = ((size_t)(r0 + t) * a.nq + hh) * S + sidx;
+      x_m[r * S + sidx] = load_device(&a.ml_part[at * 2]);
+      x_l[r * S + sidx] = load_device(&a.ml_part[at * 2 + 1]);
+    }
+    __syncthreads();
+    for (int idx = threadIdx.x; idx < nrows * D; idx += blockDim.x) {
+      const int r = idx / D, dd = idx - r * D;
+      const int t = (row0 + r) / G, hh = kvh * G + (row0 + r) % G;
+      const float* part = a.o_part + ((size_t)(r0 + t) * a.nq + hh) * S * D + dd;
+      float mmax = NEG_INF;
+      for (int u = 0; u < S; ++u) mmax = fmaxf(mmax, x_m[r * S + u]);
+      float num = 0.f, den = 0.f;
+      for (int u0 = 0; u0 < S; u0 += 8) {           // eight loads on their way at a time, summed in order
+        float v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) v[u] = load_device(part + (size_t)min(u0 + u, S - 1) * D);
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          if (u0 + u >= S) break;
+          const float mu = x_m[r * S + u0 + u];
+          const float wt = mu == NEG_INF ? 0.f : exp2f(mu - mmax);
+          num += wt * v[u];
+          den += wt * x_l[r * S + u0 + u];
+        }
+      }
+      ((bf16_t*)a.out)[(size_t)(r0 + t) * a.out_stride + (size_t)hh * D + dd] =
+          (bf16_t)(den > 0.f ? num / den : 0.f);
+    }
+    }
   }
 }
 
@@ -706,10 +779,12 @@ __global__ __launch_bounds__(256 * PH, (D <= 64 && PH == 1) ? 2 : 1) void attent
 // its partial sums on their way before the first is used (sixteen at a time: up to 64
 // splits cost one trip to memory), and the quarters meet in LDS in their order.  Up to
 // sixteen splits are one wave's work, and the block is launched with one.
-// A kernel of its own: within one kernel, results of blocks on other dies would
-// need device-wide fences, which cost far more than a launch (measured: the last
-// block to arrive, found by an atomic counter behind a fence, merging in place of this
-// kernel made the decode step of 24 layers 1.88 ms instead of 0.97).
+// A kernel of its own for more than a few splits: within one kernel, results of blocks on
+// other dies need either device-wide fences, which cost far more than a launch (measured:
+// the last block to arrive, found by an atomic counter behind a fence, merging in place of
+// this kernel made the decode step of 24 layers 1.88 ms instead of 0.97), or stores and
+// loads of device scope, a chain of trips to memory that pays with few splits only (see
+// launch_key_split_decode).
 constexpr int MERGE_WAVES = 4;
 __global__ __launch_bounds__(64 * MERGE_WAVES) void attention_merge_kernel(
     const float* __restrict__ o_part, const float* __restrict__ ml_part, bf16_t* __restrict__ out,
@@ -873,6 +948,11 @@ extern "C" void llmlab_debug_attention_splits(int splits) { g_force_splits = spl
 // staged keys in turn (0: chosen here).
 static int g_force_path = 0;
 extern "C" void llmlab_debug_attention_path(int path) { g_force_path = path; }
+// ... and who merges the key splits: 1 = the merge kernel even where the last block could.
+// -1 = the last block whatever the number of splits.
+static int g_force_merge_kernel = 0;
+extern "C" void llmlab_debug_attention_merge_kernel(int on) { g_force_merge_kernel = on; }
+constexpr int MERGE_IN_PLACE_SPLITS = 4;
 
 // The decode-like launch: a block of DECODE_WAVES waves per (request, kv head, split); a
 // wave gets about two steps of 32 keys, a block's waves merge in LDS, and only what is
@@ -880,7 +960,8 @@ extern "C" void llmlab_debug_attention_path(int path) { g_force_path = path; }
 // the filter of `a`, `ctx_len` is their longest context.
 static int launch_key_split_decode(AttnArgs a, int reqs, int live, int ctx_len, int window, int total_rows,
                                    int nq, int nkv, float* workspace, size_t workspace_floats, int num_cus,
-                                   const int* row_req, void* out, int out_stride, hipStream_t stream) {
+                                   const int* row_req, void* out, int out_stride, int* arrived,
+                                   size_t arrived_ints, hipStream_t stream) {
   const int visible = window > 0 ? min(window, ctx_len) : ctx_len;
   const int steps32 = (visible + 31) / 32 + 1;
   // A unit's memory rate is the limit, so the keys are spread over the units: as many
@@ -907,6 +988,16 @@ static int launch_key_split_decode(AttnArgs a, int reqs, int live, int ctx_len, 
   while (splits > 1 && per_split * splits > workspace_floats) --splits;
   if (splits < 1) splits = 1;
   a.splits = splits;
+  // Who merges the splits: with few splits the last block of each (request, kv head) to
+  // arrive, if the caller brought counters for them (zero now, zero again afterwards); else
+  // a kernel of its own.  The last block's way is a chain of trips to memory (its stores
+  // done, the counter, the other blocks' results) of about 2 us each, a kernel boundary
+  // costs less than two of them: measured at the 0.5B shape and context 4096, 64 requests
+  // in 2 splits take 1.743 ms a step against 1.781 with the kernel, 8 requests in 16
+  // splits 1.001 against 0.962.
+  const bool merge_in_place = splits > 1 && arrived != nullptr && (size_t)reqs * nkv <= arrived_ints &&
+                              g_force_merge_kernel == 0 && (splits <= MERGE_IN_PLACE_SPLITS || g_force_merge_kernel < 0);
+  a.arrived = merge_in_place ? arrived : nullptr;
   if (splits > 1) {
     a.o_part = workspace;
     a.ml_part = workspace + (size_t)total_rows * nq * splits * D;
@@ -918,7 +1009,7 @@ static int launch_key_split_decode(AttnArgs a, int reqs, int live, int ctx_len, 
   else
     hipLaunchKernelGGL((attention_bf16_kernel<1, true, 1>), grid, block, 0, stream, a);
   LLMLAB_LAUNCH_CHECK("attention(bfloat16, decode)");
-  if (splits > 1) {
+  if (splits > 1 && !merge_in_place) {
     hipLaunchKernelGGL(attention_merge_kernel, dim3(total_rows, nq), dim3(splits > 16 ? 64 * MERGE_WAVES : 64), 0, stream, a.o_part,
                        a.ml_part, (bf16_t*)out, out_stride, nq, splits, row_req, a.q_start, a.qlen_hi);
     LLMLAB_LAUNCH_CHECK("attention merge");
@@ -942,7 +1033,7 @@ extern "C" int llmlab_paged_attention(const void* q, int dtype, int q_stride, in
                                       int window, float scale, void* out, int out_stride,
                                       float* workspace, size_t workspace_floats, int total_rows,
                                       int num_cus, const int* row_req, int short_len, int n_short,
-                                      int short_ctx, hipStream_t stream) {
+                                      int short_ctx, int* arrived, size_t arrived_ints, hipStream_t stream) {
   LLMLAB_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0, "attention: %d heads, %d kv heads", nq, nkv);
   LLMLAB_REQUIRE(page_size >= 16 && (page_size & (page_size - 1)) == 0,
                  "attention: page size %d is not a power of two >= 16", page_size);
@@ -956,7 +1047,7 @@ extern "C" int llmlab_paged_attention(const void* q, int dtype, int q_stride, in
   if (num_cus <= 0) num_cus = 256;
   AttnArgs a;
   a.q = q; a.kc = kcache; a.vc = vcache; a.table = table; a.q_start = q_start; a.start_pos = start_pos;
-  a.out = out; a.o_part = nullptr; a.ml_part = nullptr;
+  a.out = out; a.o_part = nullptr; a.ml_part = nullptr; a.arrived = nullptr;
   a.q_stride = q_stride; a.out_stride = out_stride; a.table_stride = table_stride; a.page_size = page_size;
   a.nq = nq; a.nkv = nkv; a.window = window; a.splits = 1; a.scale = scale;
   a.page_shift = 0;
@@ -985,14 +1076,15 @@ extern "C" int llmlab_paged_attention(const void* q, int dtype, int q_stride, in
   const long max_rows = (long)max_q_len * G;
   if (max_rows <= 16)
     return launch_key_split_decode(a, reqs, reqs, max_ctx_len, window, total_rows, nq, nkv, workspace,
-                                   workspace_floats, num_cus, nullptr, out, out_stride, stream);
+                                   workspace_floats, num_cus, nullptr, out, out_stride, arrived, arrived_ints,
+                                   stream);
   int live = reqs;
   if (row_req != nullptr && n_short > 0 && n_short < reqs && (long)short_len * G <= 16) {
     AttnArgs s = a;
     s.qlen_hi = short_len;
     const int rc = launch_key_split_decode(s, reqs, n_short, short_ctx, window, total_rows, nq, nkv,
                                            workspace, workspace_floats, num_cus, row_req, out, out_stride,
-                                           stream);
+                                           arrived, arrived_ints, stream);
     if (rc) return rc;
     a.qlen_lo = short_len + 1;
     live = reqs - n_short;

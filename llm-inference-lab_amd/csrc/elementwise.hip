@@ -4,7 +4,7 @@
 
 extern "C" const char* llmlab_last_error() { return g_llmlab_error; }
 
-extern "C" int llmlab_abi_version() { return 5; }
+extern "C" int llmlab_abi_version() { return 6; }
 
 // --------------------------------------------------------------- embedding
 // out[r, :] = float(table[ids[r], :]); an id outside [0, vocab) is clamped (the

@@ -170,9 +170,48 @@ __global__ __launch_bounds__(64) void argmax_final_kernel(const float* __restric
   if (threadIdx.x == 0) out[b] = best.i;
 }
 
-// workspace: at least rows * ceil(vocab / 8192) * 2 words
+// Both stages in one kernel: every block leaves its (value, index) with stores of device
+// scope (written through to memory, past the L2 of its die), waits until they are done and
+// counts itself in at the row's counter; the block that arrives last picks among all of
+// them and sets the counter back to zero.  No fence, and nobody waits for anybody.
+__global__ __launch_bounds__(256) void argmax_one_pass_kernel(const float* __restrict__ logits,
+                                                              long row_stride, int vocab,
+                                                              float* pvals, int* pidx, int chunks,
+                                                              int* arrived, int* __restrict__ out) {
+  __shared__ Best red[17];
+  __shared__ int s_last;
+  const int b = blockIdx.y, ch = blockIdx.x;
+  const int begin = ch * ARGMAX_CHUNK;
+  const int count = min(ARGMAX_CHUNK, vocab - begin);
+  const Best best = block_argmax(logits + (size_t)b * row_stride + begin, count, 1.f, red);
+  if (threadIdx.x == 0) {
+    __hip_atomic_store(&pvals[(size_t)b * chunks + ch], best.v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(&pidx[(size_t)b * chunks + ch], best.i < 0 ? -1 : begin + best.i, __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+    __builtin_amdgcn_s_waitcnt(0);
+    const int before = __hip_atomic_fetch_add(&arrived[b], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    s_last = before == chunks - 1;
+    if (s_last) __hip_atomic_store(&arrived[b], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __syncthreads();
+  if (!s_last || threadIdx.x >= 64) return;
+  Best all{0.f, -1};
+  for (int i = threadIdx.x; i < chunks; i += 64)
+    all = better(all, Best{__hip_atomic_load(&pvals[(size_t)b * chunks + i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT),
+                           __hip_atomic_load(&pidx[(size_t)b * chunks + i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)});
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    Best o{__shfl_xor(all.v, off, WAVE), __shfl_xor(all.i, off, WAVE)};
+    all = better(all, o);
+  }
+  if (threadIdx.x == 0) out[b] = all.i;
+}
+
+// workspace: at least rows * ceil(vocab / 8192) * 2 words.  arrived (may be null: two
+// kernels then): at least `rows` counters that are zero now and are left zero.
 extern "C" int llmlab_argmax(const float* logits, long row_stride, int rows, int vocab, int* out,
-                             float* workspace, size_t workspace_floats, hipStream_t stream) {
+                             float* workspace, size_t workspace_floats, int* arrived, size_t arrived_ints,
+                             hipStream_t stream) {
   LLMLAB_REQUIRE(rows >= 0 && vocab > 0 && row_stride >= vocab, "argmax: bad sizes rows=%d vocab=%d",
                  rows, vocab);
   if (rows == 0) return 0;
@@ -182,6 +221,12 @@ extern "C" int llmlab_argmax(const float* logits, long row_stride, int rows, int
   LLMLAB_REQUIRE(rows <= 65535, "argmax: too many rows");
   float* pvals = workspace;
   int* pidx = (int*)(workspace + (size_t)rows * chunks);
+  if (arrived != nullptr && (size_t)rows <= arrived_ints && chunks > 1) {
+    hipLaunchKernelGGL(argmax_one_pass_kernel, dim3(chunks, rows), dim3(256), 0, stream, logits, row_stride,
+                       vocab, pvals, pidx, chunks, arrived, out);
+    LLMLAB_LAUNCH_CHECK("argmax (one pass)");
+    return 0;
+  }
   hipLaunchKernelGGL(argmax_partial_kernel, dim3(chunks, rows), dim3(256), 0, stream, logits, row_stride,
                      vocab, pvals, pidx, chunks);
   LLMLAB_LAUNCH_CHECK("argmax (partial)");

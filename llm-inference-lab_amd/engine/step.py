@@ -242,11 +242,19 @@ class StepContext:
             self.ops.gather_tokens(self._view("token_ids", self.max_rows), self._view("feed_dst", len(feeds)),
                                    feed_tensor, self._view("feed_src", len(feeds)), len(feeds))
 
+    ONE_COPY_INTS = 64 * 1024      # up to here the description and the block tables go in one copy
+
     def _upload(self, n_reqs: int) -> None:
-        self._dev[:self._meta_len].copy_(self._host[:self._meta_len], non_blocking=True)
-        for at in self._table_at:
-            n = n_reqs * self.max_pages
-            self._dev[at:at + n].copy_(self._host[at:at + n], non_blocking=True)
+        n = n_reqs * self.max_pages
+        end = self._table_at[-1] + n if self._table_at else self._meta_len
+        if end <= self.ONE_COPY_INTS:
+            # (the rows between the groups' tables that no request of this step uses go along:
+            # a copy more would cost more than their bytes)
+            self._dev[:end].copy_(self._host[:end], non_blocking=True)
+        else:
+            self._dev[:self._meta_len].copy_(self._host[:self._meta_len], non_blocking=True)
+            for at in self._table_at:
+                self._dev[at:at + n].copy_(self._host[at:at + n], non_blocking=True)
         if self._uploaded is not None:
             self._uploaded.record()
 

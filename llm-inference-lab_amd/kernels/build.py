@@ -2,7 +2,8 @@
 
 Two kinds of library: ``core`` (embedding, norm, rotary + cache write, matrix
 products, sampling) and ``attn_d<D>`` (attention for head size D; one per head
-size that a model needs); beside them the plain C++ references of the same operations,
+size that a model needs); beside them ``measure`` (stream and matrix-instruction loops for
+the benchmark's measured peaks) and the plain C++ references of the same operations,
 built with the host compiler for the tests.  A library's file name carries a hash of its sources
 and flags, so a library built from other sources is never loaded.  Libraries are
 kept in ``kernels/lib`` inside the package, or, if that folder cannot be written,
@@ -139,6 +140,15 @@ def attention_library(head_dim: int, force: bool = False) -> str:
     return _compile(f"attn_d{head_dim}", (ATTENTION_SOURCE,), (f"-DHEAD_DIM={head_dim}",), force)
 
 
+MEASURE_SOURCE = "measure.hip"
+
+
+def measure_library(force: bool = False) -> str:
+    """Stream and matrix-instruction loops that measure what the machine gives
+    (``csrc/measure.hip``).  The benchmark loads it; the product never does."""
+    return _compile("measure", (MEASURE_SOURCE,), (), force)
+
+
 REFERENCE_SOURCE = "reference.cpp"
 
 
@@ -190,5 +200,6 @@ def build_all(head_dims: Sequence[int] = DEFAULT_HEAD_DIMS, force: bool = True) 
     out = {"core": core_library(force)}
     for d in head_dims:
         out[f"attn_d{d}"] = attention_library(d, force)
+    out["measure"] = measure_library(force)
     out["reference"] = reference_library(force)
     return out

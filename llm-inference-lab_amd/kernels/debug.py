@@ -81,7 +81,9 @@ class KernelDebug:
               skinny_shape: Optional[Tuple[int, int, int, int]] = None,
               skinny_epilogue: Optional[int] = None,
               attention_splits: Optional[Tuple[int, int]] = None,
-              attention_path: Optional[Tuple[int, int]] = None, **rules):
+              attention_path: Optional[Tuple[int, int]] = None,
+              attention_merge_kernel: Optional[int] = None,
+              attention_merge_in_place: Optional[int] = None, **rules):
         """``gemm_tile``: 64 (64 x 64), 130 (64 x 128), 129 (128 x 128), 131 (128 x 256), 132 (256 x
         256) or 133 (192 x 256); -131: the choice among the first three; -256 and below: the
         tiles of two groups of waves (132, 133) from so many rows on.  ``skinny_shape``:
@@ -92,8 +94,10 @@ class KernelDebug:
         block split the keys of a tile of 32 rows, 2 = tiles of 32 rows per wave, 3 = late and
         early tiles in pairs, 4 = tiles of 16 rows per wave, 5 and 6 = 3 and 4 with two groups of
         waves that take the staged keys in turn; heads above 128 have no 5 and 6 and choose
-        for themselves).  Other keywords: fields of
-        ``DispatchRules`` for the time of the block."""
+        for themselves).  ``attention_merge_kernel`` / ``attention_merge_in_place``: a head size; the
+        key splits of decode attention are merged there by the kernel of its own, or by the
+        last block to arrive, whatever their number.
+        Other keywords: fields of ``DispatchRules`` for the time of the block."""
         ops = self._ops
         core = ops._core
         saved = dataclasses.replace(ops.rules)
@@ -101,8 +105,14 @@ class KernelDebug:
             if not hasattr(ops.rules, key):
                 raise TypeError(f"no dispatch rule named '{key}'")
             setattr(ops.rules, key, value)
-        lib = plib = None
+        lib = plib = mlib = None
         try:
+            if attention_merge_kernel is not None:
+                mlib = ops._attention_lib(int(attention_merge_kernel))
+                mlib.llmlab_debug_attention_merge_kernel(1)
+            elif attention_merge_in_place is not None:
+                mlib = ops._attention_lib(int(attention_merge_in_place))
+                mlib.llmlab_debug_attention_merge_kernel(-1)
             if attention_path is not None:
                 plib = ops._attention_lib(int(attention_path[0]))
                 plib.llmlab_debug_attention_path(int(attention_path[1]))
@@ -128,3 +138,5 @@ class KernelDebug:
                 lib.llmlab_debug_attention_splits(0)
             if plib is not None:
                 plib.llmlab_debug_attention_path(0)
+            if mlib is not None:
+                mlib.llmlab_debug_attention_merge_kernel(0)

@@ -67,6 +67,7 @@ class PackedWeight:
 
 class HipOps:
     WORKSPACE_FLOATS = 16 * 1024 * 1024      # 64 MiB of float32 scratch (split partial sums)
+    ARRIVED_INTS = 64 * 1024                 # arrival counters: one per (request, kv head) of a step
 
     def __init__(self, device="cuda:0"):
         if not torch.cuda.is_available():
@@ -81,12 +82,16 @@ class HipOps:
             self.device = torch.device("cuda", torch.cuda.current_device())
         self._core = self._load(build.core_library())
         self._declare_core()
-        if self._core.llmlab_abi_version() != 5:
+        if self._core.llmlab_abi_version() != 6:
             raise RuntimeError("kernel library and Python bindings disagree on the interface")
         self._attn: Dict[int, ctypes.CDLL] = {}
         self._shared: Dict[int, tuple] = {}
         self.num_cus = int(torch.cuda.get_device_properties(self.device).multi_processor_count)
         self.workspace = torch.empty(self.WORKSPACE_FLOATS, dtype=torch.float32, device=self.device)
+        # Counters by which blocks of one kernel find out which of them is the last to arrive
+        # (the key splits of decode attention, the pieces of the argmax).  Zero between
+        # launches: the block that reads the full count sets its counter back.
+        self.arrived = torch.zeros(self.ARRIVED_INTS, dtype=torch.int32, device=self.device)
         self.loaded_libraries = [self._core._name]
         self.calls_made = 0          # calls into the kernel libraries so far
         self.rules = DispatchRules()         # the measured thresholds of the dispatch, in one place
@@ -121,7 +126,8 @@ class HipOps:
         c.llmlab_packed_elements.restype = _c_long
         c.llmlab_pack_weight.argtypes = [_c_ptr, _c_ptr, _c_int, _c_int, _c_ptr]
         c.llmlab_pack_weight.restype = _c_int
-        c.llmlab_argmax.argtypes = [_c_ptr, _c_long, _c_int, _c_int, _c_ptr, _c_ptr, _c_size, _c_ptr]
+        c.llmlab_argmax.argtypes = [_c_ptr, _c_long, _c_int, _c_int, _c_ptr, _c_ptr, _c_size, _c_ptr, _c_size,
+                                    _c_ptr]
         c.llmlab_argmax.restype = _c_int
         c.llmlab_linear_qkv.argtypes = [_c_ptr, _c_ptr, _c_ptr, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_int,
                                         _c_ptr, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr, _c_ptr,
@@ -160,7 +166,7 @@ class HipOps:
             lib.llmlab_paged_attention.argtypes = [
                 _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_ptr, _c_ptr, _c_ptr, _c_int, _c_int, _c_ptr,
                 _c_ptr, _c_int, _c_int, _c_int, _c_int, _c_float, _c_ptr, _c_int, _c_ptr, _c_size,
-                _c_int, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_ptr]
+                _c_int, _c_int, _c_ptr, _c_int, _c_int, _c_int, _c_ptr, _c_size, _c_ptr]
             lib.llmlab_paged_attention.restype = _c_int
             self._attn[head_dim] = lib
             self.loaded_libraries.append(lib._name)
@@ -759,10 +765,13 @@ class HipOps:
             self._ptr(q_start), self._ptr(start_pos), n_reqs, max_q_len, max_ctx_len,
             int(window) if window else 0, float(scale), self._ptr(out), out.stride(0) if rows > 1 else
             out.shape[1], self._ptr(self.workspace), self.workspace.numel(), rows, self.num_cus,
-            self._ptr(row_req), short_len, n_short, short_ctx, self._stream(), lib=lib)
+            self._ptr(row_req), short_len, n_short, short_ctx, self._ptr(self.arrived), self.arrived.numel(),
+            self._stream(), lib=lib)
 
     # --------------------------------------------------------------- sampling
-    def argmax(self, logits, out) -> None:
+    def argmax(self, logits, out, one_pass: bool = True) -> None:
+        """``out[r]`` = the largest logit's index (the smallest among equals; -1 for a row
+        without a finite value).  ``one_pass=False``: in two kernels, without the counters."""
         self._need(logits, "logits", torch.float32, contiguous=False)
         self._need(out, "chosen tokens", torch.int32)
         rows, vocab = logits.shape
@@ -770,7 +779,8 @@ class HipOps:
             raise ValueError("argmax: logits rows must be contiguous and out must hold one token per row")
         self._call(self._core.llmlab_argmax,
             self._ptr(logits), logits.stride(0) if rows > 1 else vocab, rows, vocab, self._ptr(out),
-            self._ptr(self.workspace), self.workspace.numel(), self._stream())
+            self._ptr(self.workspace), self.workspace.numel(),
+            self._ptr(self.arrived) if one_pass else None, self.arrived.numel(), self._stream())
 
     def sample(self, logits, temperatures, uniforms, out) -> None:
         self._need(logits, "logits", torch.float32, contiguous=False)

@@ -22,21 +22,24 @@ from .safetensors_io import save_safetensors
 
 
 def random_tensors(expected: Dict[str, TensorSpec], seed: int, dtype: torch.dtype = torch.bfloat16,
-                   std: float = 0.02, norm_std: float = 0.1) -> Iterator[Tuple[str, torch.Tensor]]:
-    """One tensor per expected name, drawn as its ``TensorSpec.init`` says."""
+                   std: float = 0.02, norm_std: float = 0.1,
+                   device="cpu") -> Iterator[Tuple[str, torch.Tensor]]:
+    """One tensor per expected name, drawn as its ``TensorSpec.init`` says.  ``device``: where
+    they are drawn (a GPU's generator gives other numbers than the host's for the same
+    seed; a model folder is always written from the host's)."""
     for index, (name, spec) in enumerate(expected.items()):
-        gen = torch.Generator(device="cpu")
+        gen = torch.Generator(device=device)
         gen.manual_seed((int(seed) * 1000003 + index * 7919 + 12345) % (2 ** 63 - 1))
         if spec.kind == INT_TABLE:
-            yield name, torch.zeros(spec.shape, dtype=torch.int32)
+            yield name, torch.zeros(spec.shape, dtype=torch.int32, device=device)
             continue
         if spec.init == INIT_ZEROS:
-            yield name, torch.zeros(spec.shape, dtype=dtype)
+            yield name, torch.zeros(spec.shape, dtype=dtype, device=device)
             continue
         if spec.init == INIT_ONES:
-            yield name, torch.ones(spec.shape, dtype=dtype)
+            yield name, torch.ones(spec.shape, dtype=dtype, device=device)
             continue
-        values = torch.randn(spec.shape, generator=gen, dtype=torch.float32)
+        values = torch.randn(spec.shape, generator=gen, dtype=torch.float32, device=device)
         if spec.init == INIT_NORM:
             values = 1.0 + norm_std * values
         elif spec.init == INIT_NORMAL:

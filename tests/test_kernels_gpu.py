@@ -584,6 +584,18 @@ def run_attention(ops, emu, dtype, nq, nkv, d, page, window, reqs_spec, seed=30,
                         max_ctx, window, scale, got2, short)
     err = (got2.float().cpu() - want.float()).abs().max().item()
     assert err <= tol * max(1.0, want.float().abs().max().item()), f"attention error {err} (described step)"
+    # key splits are merged by the last block to arrive; the same with the kernel of its own,
+    # and the arrival counters are back at zero whoever merged
+    if dtype == torch.bfloat16:
+        for who in ("attention_merge_kernel", "attention_merge_in_place"):
+            got3 = torch.zeros(rows, nq * d, dtype=dtype, device=DEV)
+            with ops.debug.force(**{who: d}):
+                ops.paged_attention(qkv.to(DEV), nq, nkv, d, kc.to(DEV), vc.to(DEV), table.to(DEV), page,
+                                    q_start_t.to(DEV), start_pos_t.to(DEV), reqs, max(n for _, n in reqs_spec),
+                                    max_ctx, window, scale, got3, short)
+            err = (got3.float().cpu() - want.float()).abs().max().item()
+            assert err <= tol * max(1.0, want.float().abs().max().item()), f"attention error {err} ({who})"
+    assert int(ops.arrived.abs().sum()) == 0
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
@@ -642,10 +654,13 @@ def test_attention_merge_of_any_number_of_splits(ops, emu, splits):
                           seed=96, amplify=(0, length // 3, 30.0))
 
 
-@pytest.mark.parametrize("vocab", [1, 255, 256, 257, 4095, 4097, 151936])
-def test_argmax(ops, emu, vocab):
+@pytest.mark.parametrize("one_pass", [True, False])
+@pytest.mark.parametrize("vocab", [1, 255, 256, 257, 4095, 4097, 8193, 151936])
+def test_argmax(ops, emu, vocab, one_pass):
     """Vocabulary sizes and special rows of the reference's argmax tests
-    (rust/engine/src/runner/model/qwen2/engine.rs:2285-2358)."""
+    (rust/engine/src/runner/model/qwen2/engine.rs:2285-2358); in one kernel whose last block
+    picks among the blocks' results (three times in a row: its counters must come back to
+    zero), and in two kernels."""
     g = torch.Generator().manual_seed(vocab)
     logits = torch.randn(5, vocab, generator=g)
     logits[1, vocab - 1] = 100.0                      # maximum at the last index
@@ -655,9 +670,12 @@ def test_argmax(ops, emu, vocab):
     logits[4, :] = float("nan")                       # all NaN: -1
     want = torch.zeros(5, dtype=torch.int32)
     emu.argmax(logits, want)
-    got = torch.zeros(5, dtype=torch.int32, device=DEV)
-    ops.argmax(logits.to(DEV), got)
-    assert got.cpu().tolist() == want.tolist()
+    on_gpu = logits.to(DEV)
+    for _ in range(3):
+        got = torch.full((5,), -9, dtype=torch.int32, device=DEV)
+        ops.argmax(on_gpu, got, one_pass=one_pass)
+        assert got.cpu().tolist() == want.tolist()
+    assert int(ops.arrived.abs().sum()) == 0
     assert want[1] == vocab - 1 and want[3] == 0 and want[4] == -1
     if vocab > 300:
         assert want[2] == 7

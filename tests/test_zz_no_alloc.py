@@ -17,7 +17,7 @@ def _library():
     lib = ctypes.CDLL(build.core_library())
     vp, ci, cl, cs = ctypes.c_void_p, ctypes.c_int, ctypes.c_long, ctypes.c_size_t
     lib.llmlab_last_error.restype = ctypes.c_char_p
-    lib.llmlab_argmax.argtypes = [vp, cl, ci, ci, vp, vp, cs, vp]
+    lib.llmlab_argmax.argtypes = [vp, cl, ci, ci, vp, vp, cs, vp, cs, vp]
     lib.llmlab_argmax.restype = ci
     lib.llmlab_argmax_static.argtypes = [vp, cl, ci, ci, vp, vp]
     lib.llmlab_argmax_static.restype = ci
@@ -30,7 +30,7 @@ def _both(lib, logits, workspace):
     want = torch.full((rows,), -7, dtype=torch.int32, device=DEV)
     got = torch.full((rows,), -7, dtype=torch.int32, device=DEV)
     code = lib.llmlab_argmax(logits.data_ptr(), logits.stride(0), rows, vocab, want.data_ptr(),
-                             workspace.data_ptr(), workspace.numel(), stream)
+                             workspace.data_ptr(), workspace.numel(), None, 0, stream)     # (its two kernels)
     assert code == 0, lib.llmlab_last_error()
     code = lib.llmlab_argmax_static(logits.data_ptr(), logits.stride(0), rows, vocab, got.data_ptr(),
                                     stream)
