@@ -28,8 +28,8 @@
 // writes its merged partial result, and a second kernel merges the splits in their
 // order:  out = sum_s w_s acc_s / sum_s w_s l_s,  w_s = 2^(m_s - m).
 //
-// float32 kernel: one wave per (token, head), lanes over keys, plain FMA; true
-// 32-bit arithmetic.
+// float32 kernel: the same scheme on the float32 matrix instruction (true 32-bit
+// products and sums), in steps of 16 keys.
 #include "common.h"
 
 #ifndef HEAD_DIM
@@ -786,8 +786,9 @@ __global__ __launch_bounds__(256 * PH, (D <= 64 && PH == 1) ? 2 : 1) void attent
 // loads of device scope, a chain of trips to memory that pays with few splits only (see
 // launch_key_split_decode).
 constexpr int MERGE_WAVES = 4;
+template <typename T>
 __global__ __launch_bounds__(64 * MERGE_WAVES) void attention_merge_kernel(
-    const float* __restrict__ o_part, const float* __restrict__ ml_part, bf16_t* __restrict__ out,
+    const float* __restrict__ o_part, const float* __restrict__ ml_part, T* __restrict__ out,
     int out_stride, int nq, int splits, const int* __restrict__ row_req, const int* __restrict__ q_start,
     int qlen_hi) {
   constexpr int PER = (D + 63) / 64;
@@ -845,91 +846,236 @@ __global__ __launch_bounds__(64 * MERGE_WAVES) void attention_merge_kernel(
     float total = 0.f;
 #pragma unroll
     for (int q = 0; q < nw; ++q) total += s_num[q][dd];
-    if (dd < D) out[(size_t)row * out_stride + (size_t)head * D + dd] = (bf16_t)(total * inv);
+    if (dd < D) out[(size_t)row * out_stride + (size_t)head * D + dd] = (T)(total * inv);
   }
 }
 
-// ------------------------------------------------------------ f32, scalar
-// A block of NW waves per (token, head).  The waves take the chunks of 64 visible keys in
-// turn and merge at the end in LDS.  In a chunk every lane takes one key for the score
-// (q . k in 32 bits, the numbers of the head in order); the wave takes the chunk's maximum
-// and sum; for the values the lanes turn to the numbers of the head: lane c adds p_j v_j[c]
-// for the chunk's keys j, whose p_j, page and place go round by lane reads.
-template <int NW>
+// ------------------------------------------------------------ float32
+// True 32-bit arithmetic on the matrix cores: v_mfma_f32_16x16x4_f32 multiplies and sums
+// in float32 (no reduced-precision mode).  Same transposed scheme as the bfloat16 kernel,
+// in steps of 16 keys:
+//   S^T[key, row] = K . Q^T    A = keys (16 keys x 4 d), B = queries (4 d x 16 rows)
+//   O^T[d,  row]  = V^T . P^T  A = values (16 d x 4 keys), B = probabilities (4 keys x 16 rows)
+// An instruction contracts over four slots, one per group g of sixteen lanes.  Which d (or
+// key) sits in which slot is free as long as both operands agree, so lane (c, g) takes
+// the four consecutive numbers 16 M + 4 g .. + 3 of its key c (one 16-byte load in the
+// cache's order) and uses them in four instructions; for the second product the result
+// layout of S^T (lane (c, g): row c, keys 4 g .. 4 g + 3) already is the B operand, and
+// the values of keys 4 g .. 4 g + 3 at number c of a block of d are 16 consecutive bytes.
+// Scores, maxima, exponentials (the library's expf) and sums in float32.
+//
+// A tile is 16 QB rows ((token, head of the group) pairs of one request and kv head, so the
+// heads of a group share the keys they read).  SPLIT = false: every wave owns a tile and
+// walks all its keys (prompts).  SPLIT = true: the NW waves of a block share one tile and
+// split its keys, merge through LDS, and blockIdx.y also counts splits over blocks whose
+// partial results the merge kernel sums (decode steps; few rows behind a long history).
+template <int QB, bool SPLIT, int NW>
 __global__ __launch_bounds__(64 * NW) void attention_f32_kernel(AttnArgs a) {
-  constexpr int DPL = (D + 63) / 64;       // numbers of the head per lane
-  __shared__ float qs[D];
-  __shared__ float s_m[NW], s_l[NW];
-  __shared__ float s_o[NW][D];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int t = blockIdx.x, h = blockIdx.y, b = blockIdx.z;
-  const int r0 = a.q_start[b], qlen = a.q_start[b + 1] - r0;
-  if (t >= qlen) return;
-  const int G = a.nq / a.nkv, kvh = h / G;
-  const int p = a.start_pos[b] + t;
-  const int lo = a.window > 0 ? max(0, p - a.window + 1) : 0;
-  const int P = a.page_size;
-  const float* q = (const float*)a.q + (size_t)(r0 + t) * a.q_stride + (size_t)h * D;
+  constexpr int DQ = D / 16;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int c = lane & 15, g = lane >> 4;
+  const int b = blockIdx.z;
+  const int kvh = blockIdx.y / a.splits, split = blockIdx.y % a.splits;
+  const int G = a.nq / a.nkv;
+  const int r0 = a.q_start[b], qlen = a.q_start[b + 1] - r0, sp = a.start_pos[b];
+  const int rows_total = qlen * G;
+  if (qlen < a.qlen_lo || qlen > a.qlen_hi) return;                  // another launch's request
+  // tiles with the longest histories (the last rows) first
+  const int xblk = (int)(gridDim.x - 1 - blockIdx.x);
+  const int row0 = (SPLIT ? xblk : xblk * NW + wave) * (16 * QB);
+  if (row0 >= rows_total) {
+    if (!SPLIT || xblk * 16 * QB >= rows_total) return;              // (without SPLIT no wave waits for another)
+  }
+  const bool wave_live = row0 < rows_total;
+  const float* q = (const float*)a.q;
   const float* kc = (const float*)a.kc;
   const float* vc = (const float*)a.vc;
-  for (int dd = threadIdx.x; dd < D; dd += 64 * NW) qs[dd] = q[dd];
-  __syncthreads();
+  const int P = a.page_size, pshift = a.page_shift;
 
-  float o[DPL];
+  bool valid[QB];
+  int tok[QB], head[QB], pos[QB], lo[QB];
+  floatx4 qf[QB][DQ];
 #pragma unroll
-  for (int i = 0; i < DPL; ++i) o[i] = 0.f;
-  float m = NEG_INF, l = 0.f;
-  for (int j0 = lo + 64 * wave; j0 <= p; j0 += 64 * NW) {
-    const int j = j0 + lane;
-    const bool valid = j <= p;
-    const int jc = valid ? j : p;           // clamped: read, weight 0
-    const int page = a.table[(size_t)b * a.table_stride + (jc >> a.page_shift)];
-    const int off = jc & (P - 1);
-    const float* kp = kc + ((size_t)page * a.nkv + kvh) * P * D;
-    float dot = 0.f;
-#pragma unroll 16
-    for (int dd = 0; dd < D; ++dd) dot = fmaf(qs[dd], kp[kcache_index(off, dd, D)], dot);
-    const float s = valid ? dot * a.scale : NEG_INF;
-    const float m_new = fmaxf(m, wave_max(s));        // the chunk's first key is always visible
-    const float alpha = expf(m - m_new);              // m = -inf before the first chunk: exp(-inf) = 0
-    const float pr = valid ? expf(s - m_new) : 0.f;
-    l = l * alpha + wave_sum(pr);
+  for (int qb = 0; qb < QB; ++qb) {
+    const int rr = row0 + qb * 16 + c;
+    valid[qb] = wave_live && rr < rows_total;
+    tok[qb] = valid[qb] ? rr / G : 0;
+    head[qb] = kvh * G + (valid[qb] ? rr % G : 0);
+    pos[qb] = sp + tok[qb];
+    lo[qb] = a.window > 0 ? max(0, pos[qb] - a.window + 1) : 0;
+    const float* qp = q + (size_t)(r0 + tok[qb]) * a.q_stride + (size_t)head[qb] * D + g * 4;
 #pragma unroll
-    for (int i = 0; i < DPL; ++i) o[i] *= alpha;
-    m = m_new;
-    const int count = min(64, p - j0 + 1);
-    for (int jj = 0; jj < count; ++jj) {
-      const float pj = __shfl(pr, jj, WAVE);
-      const int pg = __shfl(page, jj, WAVE), of = __shfl(off, jj, WAVE);
-      const float* vp = vc + ((size_t)pg * a.nkv + kvh) * P * D;
+    for (int mb = 0; mb < DQ; ++mb)
+      qf[qb][mb] = valid[qb] ? *(const floatx4*)(qp + mb * 16) : floatx4{0.f, 0.f, 0.f, 0.f};
+  }
+  const int last_row = min(row0 + 16 * QB, rows_total) - 1;
+  const int p_first = sp + row0 / G, p_last = sp + last_row / G;
+  const int key_lo = a.window > 0 ? max(0, p_first - a.window + 1) : 0;
+  const int key_hi = wave_live ? p_last : -1;
+  const int full_lo = a.window > 0 ? max(0, p_last - a.window + 1) : 0;   // from here on inside every row's window
+  const int blk_lo = key_lo >> 4, blk_hi = key_hi >> 4;
+  const int per = (blk_hi - blk_lo + 1 + a.splits - 1) / a.splits;
+  int my0 = blk_lo + split * per;
+  int my1 = min(my0 + per, blk_hi + 1);
+  if constexpr (SPLIT) {
+    const int per_wave = (max(my1 - my0, 0) + NW - 1) / NW;
+    my0 += wave * per_wave;
+    my1 = min(my0 + per_wave, my1);
+  }
+
+  floatx4 o[QB][DQ];
+  float m[QB], lsum[QB];
 #pragma unroll
-      for (int i = 0; i < DPL; ++i) {
-        const int dd = lane + 64 * i;
-        if (dd < D) o[i] = fmaf(pj, vp[vcache_index(of, dd, D)], o[i]);
+  for (int qb = 0; qb < QB; ++qb) {
+    m[qb] = NEG_INF;
+    lsum[qb] = 0.f;
+#pragma unroll
+    for (int mb = 0; mb < DQ; ++mb) o[qb][mb] = floatx4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  struct Step {
+    floatx4 k[DQ], v[DQ];
+    bool ok;
+  };
+  auto compute = [&](int blk, const Step& f) {
+    if (!f.ok) return;                      // (the same for the whole wave)
+    const int kb = blk << 4;
+    const bool all_visible = kb + 15 <= p_first && kb >= full_lo;
+    const bool tail = kb + 15 > key_hi;
+#pragma unroll
+    for (int qb = 0; qb < QB; ++qb) {
+      floatx4 sc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int mb = 0; mb < DQ; ++mb)
+#pragma unroll
+        for (int t = 0; t < 4; ++t)
+          sc = __builtin_amdgcn_mfma_f32_16x16x4f32(f.k[mb][t], qf[qb][mb][t], sc, 0, 0, 0);
+      float sv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int j = kb + g * 4 + i;
+        const bool vis = all_visible || (valid[qb] && j <= pos[qb] && j >= lo[qb]);
+        sv[i] = vis ? sc[i] * a.scale : NEG_INF;
+      }
+      float mx = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
+      mx = max_across_32(mx);
+      mx = max_across_16(mx);
+      const float m_new = fmaxf(m[qb], mx);
+      // nothing visible so far (m_new = -inf): every weight is 0 and the sums stay 0
+      const float alpha = m_new == NEG_INF ? 1.f : expf(m[qb] - m_new);
+      float pv[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) pv[i] = sv[i] == NEG_INF ? 0.f : expf(sv[i] - m_new);
+      lsum[qb] = lsum[qb] * alpha + ((pv[0] + pv[1]) + (pv[2] + pv[3]));
+      m[qb] = m_new;
+#pragma unroll
+      for (int mb = 0; mb < DQ; ++mb) {
+        o[qb][mb] *= alpha;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          // (a position past the last one written holds whatever was there: kept out of
+          // the product although its weight is zero)
+          const float vv = (tail && kb + g * 4 + u > key_hi) ? 0.f : f.v[mb][u];
+          o[qb][mb] = __builtin_amdgcn_mfma_f32_16x16x4f32(vv, pv[u], o[qb][mb], 0, 0, 0);
+        }
       }
     }
+  };
+
+  // The next step's keys and values are on their way while this one is multiplied; the
+  // loads are unconditional (a load under a branch makes the compiler wait for all loads
+  // in flight where the branch ends): a step past the end reads the last one again, a
+  // page that is not there reads page 0, and the flag keeps it out of the sums.  The page
+  // numbers of 64 steps are read ahead, one step per lane.
+  for (int cb = my0; cb < my1; cb += 64) {
+    const int ce = min(cb + 64, my1);
+    int pages_v;
+    {
+      const int pos16 = (cb + lane) * 16;
+      const bool in = cb + lane < ce && pos16 <= key_hi && pos16 + 15 >= key_lo;
+      const int pg = a.table[(size_t)b * a.table_stride + min(pos16 >> pshift, a.table_stride - 1)];
+      pages_v = in ? pg : -1;
+    }
+    auto fetch = [&](int blk, Step& f) {
+      const int bl = min(blk, ce - 1);
+      const int page = __builtin_amdgcn_readlane(pages_v, bl - cb);
+      f.ok = blk < ce && page >= 0;
+      const size_t base = ((size_t)max(page, 0) * a.nkv + kvh) * P * D + (size_t)(((bl << 4) & (P - 1)) >> 4) * (16 * D);
+      const float* kp = kc + base + (size_t)((g >> 1) * 16 + c) * 8 + 4 * (g & 1);
+      const float* vp = vc + base + (size_t)(g * 16 + c) * 4;
+#pragma unroll
+      for (int mb = 0; mb < DQ; ++mb) {
+        f.k[mb] = *(const floatx4*)(kp + mb * 256);      // two octets of d further
+        f.v[mb] = *(const floatx4*)(vp + mb * 256);      // the next 16-wide block of d
+      }
+    };
+    Step cur, nxt;
+    fetch(cb, cur);
+    for (int blk = cb; blk < ce; ++blk) {
+      fetch(blk + 1, nxt);
+      __builtin_amdgcn_sched_barrier(0);
+      compute(blk, cur);
+      cur = nxt;
+    }
   }
-  if (lane == 0) {
-    s_m[wave] = m;
-    s_l[wave] = l;
-  }
+
+  if constexpr (!SPLIT) {
 #pragma unroll
-  for (int i = 0; i < DPL; ++i)
-    if (lane + 64 * i < D) s_o[wave][lane + 64 * i] = o[i];
-  __syncthreads();
-  float mmax = NEG_INF;
+    for (int qb = 0; qb < QB; ++qb) {
+      float l = lsum[qb];
+      l += __shfl_xor(l, 16, WAVE);
+      l += __shfl_xor(l, 32, WAVE);
+      if (!valid[qb]) continue;
+      const float inv = l > 0.f ? 1.f / l : 0.f;
+      float* dst = (float*)a.out + (size_t)(r0 + tok[qb]) * a.out_stride + (size_t)head[qb] * D + g * 4;
 #pragma unroll
-  for (int w = 0; w < NW; ++w) mmax = fmaxf(mmax, s_m[w]);
-  float ltot = 0.f;
+      for (int mb = 0; mb < DQ; ++mb) *(floatx4*)(dst + mb * 16) = o[qb][mb] * inv;
+    }
+  } else {
+    // ---- merge the waves of the block through LDS (see the bfloat16 kernel)
+    __shared__ float s_m[NW][16 * QB], s_l[NW][16 * QB];
+    __shared__ __attribute__((aligned(16))) float s_o[NW][16 * QB][D];
 #pragma unroll
-  for (int w = 0; w < NW; ++w) ltot += s_m[w] == NEG_INF ? 0.f : s_l[w] * expf(s_m[w] - mmax);
-  const float inv = ltot > 0.f ? 1.f / ltot : 0.f;
-  float* dst = (float*)a.out + (size_t)(r0 + t) * a.out_stride + (size_t)h * D;
-  for (int dd = threadIdx.x; dd < D; dd += 64 * NW) {
-    float tot = 0.f;
+    for (int qb = 0; qb < QB; ++qb) {
+      float l = lsum[qb];
+      l += __shfl_xor(l, 16, WAVE);
+      l += __shfl_xor(l, 32, WAVE);
+      if (g == 0) {
+        s_m[wave][qb * 16 + c] = m[qb];
+        s_l[wave][qb * 16 + c] = l;
+      }
 #pragma unroll
-    for (int w = 0; w < NW; ++w) tot += s_m[w] == NEG_INF ? 0.f : s_o[w][dd] * expf(s_m[w] - mmax);
-    dst[dd] = tot * inv;
+      for (int mb = 0; mb < DQ; ++mb) *(floatx4*)(&s_o[wave][qb * 16 + c][mb * 16 + g * 4]) = o[qb][mb];
+    }
+    __syncthreads();
+    const int nrows = min(16 * QB, rows_total - row0);
+    for (int idx = threadIdx.x; idx < nrows * D; idx += blockDim.x) {
+      const int r = idx / D, dd = idx - r * D;
+      float mmax = NEG_INF;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) mmax = fmaxf(mmax, s_m[w][r]);
+      float num = 0.f, den = 0.f;
+#pragma unroll
+      for (int w = 0; w < NW; ++w) {
+        const float wt = s_m[w][r] == NEG_INF ? 0.f : expf(s_m[w][r] - mmax);
+        num += wt * s_o[w][r][dd];
+        den += wt * s_l[w][r];
+      }
+      const int t = (row0 + r) / G, hh = kvh * G + (row0 + r) % G;
+      if (a.splits == 1) {
+        ((float*)a.out)[(size_t)(r0 + t) * a.out_stride + (size_t)hh * D + dd] = den > 0.f ? num / den : 0.f;
+      } else {
+        // (the merge kernel weighs the splits by powers of two: the maximum goes there in
+        // units of the binary exponent)
+        const size_t at = ((size_t)(r0 + t) * a.nq + hh) * a.splits + split;
+        a.o_part[at * D + dd] = num;
+        if (dd == 0) {
+          a.ml_part[at * 2] = mmax * 1.4426950408889634f;
+          a.ml_part[at * 2 + 1] = den;
+        }
+      }
+    }
   }
 }
 
@@ -1010,10 +1156,88 @@ static int launch_key_split_decode(AttnArgs a, int reqs, int live, int ctx_len, 
     hipLaunchKernelGGL((attention_bf16_kernel<1, true, 1>), grid, block, 0, stream, a);
   LLMLAB_LAUNCH_CHECK("attention(bfloat16, decode)");
   if (splits > 1 && !merge_in_place) {
-    hipLaunchKernelGGL(attention_merge_kernel, dim3(total_rows, nq), dim3(splits > 16 ? 64 * MERGE_WAVES : 64), 0, stream, a.o_part,
+    hipLaunchKernelGGL(attention_merge_kernel<bf16_t>, dim3(total_rows, nq), dim3(splits > 16 ? 64 * MERGE_WAVES : 64), 0, stream, a.o_part,
                        a.ml_part, (bf16_t*)out, out_stride, nq, splits, row_req, a.q_start, a.qlen_hi);
     LLMLAB_LAUNCH_CHECK("attention merge");
   }
+  return 0;
+}
+
+// float32.  Steps of at most 16 rows per request and kv head (decode) split the keys over
+// the waves of a block and over blocks, as many splits as still give every block a compute
+// unit of its own (the same rule as in bfloat16, for twice the bytes), and the merge kernel
+// sums the splits.  Few tiles of rows behind a long history take one block per tile whose
+// waves split the keys; everything else one wave per tile of 32 rows (16 for heads
+// above 128: registers).
+constexpr int F32_SPLIT_WAVES = D <= 64 ? 8 : 4;
+constexpr int F32_QB = D <= 128 ? 2 : 1;
+static int launch_f32_key_split(AttnArgs a, int reqs, int live, int ctx_len, int window, int total_rows,
+                                float* workspace, size_t workspace_floats, int num_cus, const int* row_req,
+                                hipStream_t stream) {
+  const int visible = window > 0 ? min(window, ctx_len) : ctx_len;
+  const int steps16 = (visible + 15) / 16 + 1;
+  int splits = (int)(num_cus / ((long)live * a.nkv));
+  const int most = (steps16 + 2 * F32_SPLIT_WAVES - 1) / (2 * F32_SPLIT_WAVES);     // two steps per wave at least
+  if (splits > most) splits = most;
+  if (splits > MAX_KEY_SPLITS) splits = MAX_KEY_SPLITS;
+  const size_t block_bytes = (size_t)visible * D * 2 * sizeof(float);
+  if (block_bytes < (384u << 10) || (splits <= 4 && block_bytes < (768u << 10))) splits = 1;
+  if (g_force_splits > 0) splits = min(g_force_splits, MAX_KEY_SPLITS);
+  if (splits < 1) splits = 1;
+  const size_t per_split = (size_t)total_rows * a.nq * (D + 2);
+  while (splits > 1 && per_split * splits > workspace_floats) --splits;
+  a.splits = splits;
+  if (splits > 1) {
+    a.o_part = workspace;
+    a.ml_part = workspace + (size_t)total_rows * a.nq * splits * D;
+  }
+  hipLaunchKernelGGL((attention_f32_kernel<1, true, F32_SPLIT_WAVES>), dim3(1, a.nkv * splits, reqs),
+                     dim3(64 * F32_SPLIT_WAVES), 0, stream, a);
+  LLMLAB_LAUNCH_CHECK("attention(float32, decode)");
+  if (splits > 1) {
+    hipLaunchKernelGGL(attention_merge_kernel<float>, dim3(total_rows, a.nq), dim3(splits > 16 ? 64 * MERGE_WAVES : 64),
+                       0, stream, a.o_part, a.ml_part, (float*)a.out, a.out_stride, a.nq, splits, row_req,
+                       a.q_start, a.qlen_hi);
+    LLMLAB_LAUNCH_CHECK("attention merge (float32)");
+  }
+  return 0;
+}
+
+static int launch_attention_f32(AttnArgs a, int reqs, int max_q_len, int max_ctx_len, int window, int total_rows,
+                                float* workspace, size_t workspace_floats, int num_cus, const int* row_req,
+                                int short_len, int n_short, int short_ctx, hipStream_t stream) {
+  LLMLAB_REQUIRE(a.q_stride % 4 == 0 && a.out_stride % 4 == 0 && ((uintptr_t)a.q % 16 == 0) &&
+                 ((uintptr_t)a.out % 16 == 0) && ((uintptr_t)a.kc % 16 == 0) && ((uintptr_t)a.vc % 16 == 0),
+                 "attention(float32): operands are not aligned for 16-byte loads");
+  const int G = a.nq / a.nkv;
+  const long max_rows = (long)max_q_len * G;
+  if (max_rows <= 16)
+    return launch_f32_key_split(a, reqs, reqs, max_ctx_len, window, total_rows, workspace, workspace_floats,
+                                num_cus, nullptr, stream);
+  int live = reqs;
+  if (row_req != nullptr && n_short > 0 && n_short < reqs && (long)short_len * G <= 16) {
+    // a mixed step: its requests of a few tokens by the launch that splits their keys
+    AttnArgs s = a;
+    s.qlen_hi = short_len;
+    const int rc = launch_f32_key_split(s, reqs, n_short, short_ctx, window, total_rows, workspace,
+                                        workspace_floats, num_cus, row_req, stream);
+    if (rc) return rc;
+    a.qlen_lo = short_len + 1;
+    live = reqs - n_short;
+  }
+  constexpr int ROWS = 16 * F32_QB;
+  const long tiles = (max_rows + ROWS - 1) / ROWS;
+  const bool long_history = (long)max_ctx_len >= 8L * max_q_len;
+  int path = g_force_path;        // (1: the waves of a block split the keys; anything else: a wave per tile)
+  if (path == 0) path = (tiles * a.nkv * live <= num_cus / 2 && long_history) ? 1 : 2;
+  if (path == 1) {
+    hipLaunchKernelGGL((attention_f32_kernel<F32_QB, true, F32_SPLIT_WAVES>), dim3((unsigned)tiles, a.nkv, reqs),
+                       dim3(64 * F32_SPLIT_WAVES), 0, stream, a);
+  } else {
+    hipLaunchKernelGGL((attention_f32_kernel<F32_QB, false, 4>), dim3((unsigned)((tiles + 3) / 4), a.nkv, reqs),
+                       dim3(256), 0, stream, a);
+  }
+  LLMLAB_LAUNCH_CHECK("attention(float32)");
   return 0;
 }
 
@@ -1054,21 +1278,9 @@ extern "C" int llmlab_paged_attention(const void* q, int dtype, int q_stride, in
   a.tiles = 0;
   a.qlen_lo = 0; a.qlen_hi = 0x7fffffff;
   while ((1 << a.page_shift) < page_size) ++a.page_shift;
-  if (dtype == DT_F32) {
-    // waves per (token, head): as many as the longest history has chunks of 64 keys for, up
-    // to 16; four at most where the rows alone fill the chip
-    dim3 grid(max_q_len, nq, reqs);
-    const int chunks = (max_ctx_len + 63) / 64;
-    const bool many_rows = (long)total_rows * nq >= 8L * num_cus;
-    if (chunks <= 2)
-      hipLaunchKernelGGL(attention_f32_kernel<1>, grid, dim3(64), 0, stream, a);
-    else if (chunks <= 16 || many_rows)
-      hipLaunchKernelGGL(attention_f32_kernel<4>, grid, dim3(256), 0, stream, a);
-    else
-      hipLaunchKernelGGL(attention_f32_kernel<16>, grid, dim3(1024), 0, stream, a);
-    LLMLAB_LAUNCH_CHECK("attention(float32)");
-    return 0;
-  }
+  if (dtype == DT_F32)
+    return launch_attention_f32(a, reqs, max_q_len, max_ctx_len, window, total_rows, workspace, workspace_floats,
+                                num_cus, row_req, short_len, n_short, short_ctx, stream);
   LLMLAB_REQUIRE(q_stride % 8 == 0 && ((uintptr_t)q % 16 == 0) && out_stride % 4 == 0 &&
                  ((uintptr_t)out % 8 == 0) && ((uintptr_t)kcache % 16 == 0) && ((uintptr_t)vcache % 16 == 0),
                  "attention(bfloat16): operands are not aligned for vector loads");

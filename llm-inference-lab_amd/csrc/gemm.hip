@@ -663,6 +663,11 @@ __global__ __launch_bounds__(512) void gemm_bf16_pingpong(const bf16_t* __restri
 }
 
 // ================================================================ float32
+// Debug interface: 1 = products of many rows by the plain FMA kernel instead of the matrix
+// cores (tests compare the two).
+static int g_f32_fma = 0;
+extern "C" void llmlab_debug_f32_fma(int on) { g_f32_fma = on; }
+
 // BM x BN outputs per block of 256 threads (16 x 16); thread (ty, tx) owns the TM = BM/16
 // rows ty*TM + i and the TN = BN/16 columns tx + 16*j, so for SWIGLU columns j = 0, 2, ..
 // are gate and j = 1, 3, .. the up values of the same outputs.  K steps of 8 through LDS
@@ -757,12 +762,134 @@ __global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__
   }
 }
 
+// Many rows in float32 on the matrix cores: v_mfma_f32_32x32x2_f32 multiplies and sums in
+// true 32 bits (no reduced-precision mode) at twice the rate of unpacked FMAs and with one
+// LDS read per operand and instruction.  BM x BN outputs per block of four waves (2 x 2);
+// both operands through LDS in steps of 16 of the inner size (rows padded to 17 floats:
+// the lanes of an instruction read one number each from 32 consecutive rows without
+// bank conflicts), the next step's numbers on their way from memory meanwhile.  The
+// product is taken transposed, C^T[n, m] = W x^T, so that a lane holds one row m of the
+// output and 16 of its columns, four and four next to each other, and for SWIGLU the gate
+// and the up value of an output in the same lane.
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float floatx16;
+template <int EPI, int BM, int BN>
+__global__ __launch_bounds__(256) void gemm_f32_mfma_kernel(const float* __restrict__ A,
+                                                             const float* __restrict__ W, EpiArgs e, int M,
+                                                             int N, int K, int vec) {
+  constexpr int KT = 16, LD = KT + 1;
+  constexpr int TM = BM / 64, TN = BN / 64;            // 32 x 32 tiles per wave along m and n
+  constexpr int LA = BM * KT / 4 / 256, LB = BN * KT / 4 / 256;     // 16-byte pieces per thread and step
+  __shared__ float Xs[BM * LD];
+  __shared__ float Ws[BN * LD];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave & 1, wn = wave >> 1;
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  const int r32 = lane & 31, kk = lane >> 5;
+  floatx16 acc[TN][TM];
+#pragma unroll
+  for (int j = 0; j < TN; ++j)
+#pragma unroll
+    for (int i = 0; i < TM; ++i)
+#pragma unroll
+      for (int x = 0; x < 16; ++x) acc[j][i][x] = 0.f;
+  floatx4 ra[LA], rb[LB];
+  // piece p of a tile: row p / 4, numbers 4 (p % 4) .. + 3 of the step
+  auto fetch = [&](int k0) {
+#pragma unroll
+    for (int x = 0; x < LA; ++x) {
+      const int p = tid + x * 256, row = p >> 2, kq = (p & 3) * 4;
+      const float* src = A + (size_t)min(m0 + row, M - 1) * K + k0 + kq;
+      if (vec && k0 + kq + 4 <= K) ra[x] = *(const floatx4*)src;
+      else
+#pragma unroll
+        for (int c = 0; c < 4; ++c) ra[x][c] = k0 + kq + c < K ? src[c] : 0.f;
+    }
+#pragma unroll
+    for (int x = 0; x < LB; ++x) {
+      const int p = tid + x * 256, row = p >> 2, kq = (p & 3) * 4;
+      const float* src = W + (size_t)min(n0 + row, N - 1) * K + k0 + kq;
+      if (vec && k0 + kq + 4 <= K) rb[x] = *(const floatx4*)src;
+      else
+#pragma unroll
+        for (int c = 0; c < 4; ++c) rb[x][c] = k0 + kq + c < K ? src[c] : 0.f;
+    }
+  };
+  fetch(0);
+  for (int k0 = 0; k0 < K; k0 += KT) {
+    __syncthreads();
+#pragma unroll
+    for (int x = 0; x < LA; ++x) {
+      const int p = tid + x * 256, row = p >> 2, kq = (p & 3) * 4;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) Xs[row * LD + kq + c] = ra[x][c];
+    }
+#pragma unroll
+    for (int x = 0; x < LB; ++x) {
+      const int p = tid + x * 256, row = p >> 2, kq = (p & 3) * 4;
+#pragma unroll
+      for (int c = 0; c < 4; ++c) Ws[row * LD + kq + c] = rb[x][c];
+    }
+    __syncthreads();
+    if (k0 + KT < K) fetch(k0 + KT);
+#pragma unroll
+    for (int s2 = 0; s2 < KT; s2 += 2) {
+      float wv[TN], xv[TM];
+#pragma unroll
+      for (int j = 0; j < TN; ++j) wv[j] = Ws[(wn * (BN / 2) + j * 32 + r32) * LD + s2 + kk];
+#pragma unroll
+      for (int i = 0; i < TM; ++i) xv[i] = Xs[(wm * (BM / 2) + i * 32 + r32) * LD + s2 + kk];
+#pragma unroll
+      for (int j = 0; j < TN; ++j)
+#pragma unroll
+        for (int i = 0; i < TM; ++i)
+          acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x2f32(wv[j], xv[i], acc[j][i], 0, 0, 0);
+    }
+  }
+  // lane (r32, kk) holds, of every 32 x 32 tile, output row m = r32 and the columns
+  // n = 8 (x / 4) + 4 kk + x % 4 for x = 0 .. 15
+#pragma unroll
+  for (int i = 0; i < TM; ++i) {
+    const int m = m0 + wm * (BM / 2) + i * 32 + r32;
+    if (m >= M) continue;
+#pragma unroll
+    for (int j = 0; j < TN; ++j) {
+      const int nb = n0 + wn * (BN / 2) + j * 32;
+      if constexpr (EPI == EPI_SWIGLU) {
+        // columns 0 .. 15 of the 32 are gate, 16 .. 31 the up values of the same outputs
+#pragma unroll
+        for (int x = 0; x < 8; ++x) {
+          const int o = (nb >> 5) * 16 + 8 * (x >> 2) + 4 * kk + (x & 3);
+          if (o < e.n_out) {
+            const float z = acc[j][i][x];
+            ((float*)e.out)[(size_t)m * e.ldo + o] = z / (1.f + expf(-z)) * acc[j][i][x + 8];
+          }
+        }
+      } else {
+#pragma unroll
+        for (int x = 0; x < 16; ++x) {
+          const int n = nb + 8 * (x >> 2) + 4 * kk + (x & 3);
+          if (n < N) epi_store<float, EPI>(e, m, n, acc[j][i][x]);
+        }
+      }
+    }
+  }
+}
+
 // The largest tile that still gives every compute unit a block.
 template <int EPI>
 static void launch_f32_tiled(const float* A, const float* W, const EpiArgs& e, int M, int N, int K,
                              int num_cus, hipStream_t stream) {
   const int vec = (K % 4 == 0) && ((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0);
   auto blocks = [&](int bm, int bn) { return (long)((M + bm - 1) / bm) * ((N + bn - 1) / bn); };
+  if (g_f32_fma == 0) {       // the matrix cores (the plain FMA kernels below stay as their reference)
+    if (blocks(128, 128) >= num_cus)
+      hipLaunchKernelGGL((gemm_f32_mfma_kernel<EPI, 128, 128>), dim3((N + 127) / 128, (M + 127) / 128), dim3(256),
+                         0, stream, A, W, e, M, N, K, vec);
+    else
+      hipLaunchKernelGGL((gemm_f32_mfma_kernel<EPI, 64, 64>), dim3((N + 63) / 64, (M + 63) / 64), dim3(256), 0,
+                         stream, A, W, e, M, N, K, vec);
+    return;
+  }
   if (blocks(128, 128) >= num_cus)
     hipLaunchKernelGGL((gemm_f32_kernel<EPI, 128, 128>), dim3((N + 127) / 128, (M + 127) / 128), dim3(256), 0,
                        stream, A, W, e, M, N, K, vec);

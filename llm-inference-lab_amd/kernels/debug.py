@@ -83,7 +83,7 @@ class KernelDebug:
               attention_splits: Optional[Tuple[int, int]] = None,
               attention_path: Optional[Tuple[int, int]] = None,
               attention_merge_kernel: Optional[int] = None,
-              attention_merge_in_place: Optional[int] = None, **rules):
+              attention_merge_in_place: Optional[int] = None, f32_fma: Optional[bool] = None, **rules):
         """``gemm_tile``: 64 (64 x 64), 130 (64 x 128), 129 (128 x 128), 131 (128 x 256), 132 (256 x
         256) or 133 (192 x 256); -131: the choice among the first three; -256 and below: the
         tiles of two groups of waves (132, 133) from so many rows on.  ``skinny_shape``:
@@ -97,7 +97,8 @@ class KernelDebug:
         for themselves).  ``attention_merge_kernel`` / ``attention_merge_in_place``: a head size; the
         key splits of decode attention are merged there by the kernel of its own, or by the
         last block to arrive, whatever their number.
-        Other keywords: fields of ``DispatchRules`` for the time of the block."""
+        ``f32_fma``: float32 products of many rows by the plain FMA kernel instead of the
+        matrix cores.  Other keywords: fields of ``DispatchRules`` for the time of the block."""
         ops = self._ops
         core = ops._core
         saved = dataclasses.replace(ops.rules)
@@ -118,6 +119,8 @@ class KernelDebug:
                 plib.llmlab_debug_attention_path(int(attention_path[1]))
             if gemm_tile is not None:
                 core.llmlab_debug_gemm_tile(int(gemm_tile))
+            if f32_fma is not None:
+                core.llmlab_debug_f32_fma(1 if f32_fma else 0)
             if skinny_shape is not None:
                 core.llmlab_debug_skinny_shape(*[int(v) for v in skinny_shape])
             if skinny_epilogue is not None:
@@ -130,6 +133,8 @@ class KernelDebug:
             ops.rules = saved
             if gemm_tile is not None:
                 core.llmlab_debug_gemm_tile(0)
+            if f32_fma is not None:
+                core.llmlab_debug_f32_fma(0)
             if skinny_shape is not None:
                 core.llmlab_debug_skinny_shape(0, 0, -1, 0)
             if skinny_epilogue is not None:

@@ -715,7 +715,7 @@ class HipOps:
         the chip, the portions to the tiled one.  Returns the most tokens a request may
         bring to count as short in such a step, or 0 if the step is not divided."""
         group = num_heads // num_kv_heads
-        if dtype == torch.bfloat16 and group <= 16 < max_q_len * group:
+        if group <= 16 < max_q_len * group:
             return 16 // group
         return 0
 

@@ -125,6 +125,38 @@ def test_linear_residual_and_logits(ops, emu, dtype, m, n, k):
     close(got, want, torch.float32, f"linear_logits {m}x{n}x{k}", want.abs().max().item())
 
 
+@pytest.mark.parametrize("fma", [False, True])
+@pytest.mark.parametrize("m,n,k", [(65, 130, 72), (200, 1152, 896), (300, 257, 137), (513, 384, 264), (129, 64, 1161),
+                                   (2048, 2304, 200), (1100, 4864, 96), (70, 33, 19)])
+def test_float32_products_of_many_rows(ops, emu, fma, m, n, k):
+    """The float32 products of more than 64 rows, on the matrix cores (both tiles: the large
+    one where its blocks fill the chip) and by the plain FMA kernel that stays beside them:
+    store with bias, add into the stream, SwiGLU pairs; inner sizes that are no multiple of
+    4 or of the step, edges inside a tile.  Both are true 32-bit products: the same bound."""
+    from llm_inference_lab_amd.parts.feed_forward import interleave_gate_up
+    x, w, bias = rnd((m, k), torch.float32, 5), rnd((n, k), torch.float32, 6, 0.1), rnd((n,), torch.float32, 7)
+    resid = rnd((m, n), torch.float32, 11)
+    with ops.debug.force(f32_fma=fma):
+        want = torch.empty(m, n)
+        emu.linear(x, w, want, bias)
+        got = torch.empty(m, n, device=DEV)
+        ops.linear(x.to(DEV), w.to(DEV), got, bias.to(DEV))
+        close(got, want, torch.float32, f"linear {m}x{n}x{k}", want.abs().max().item())
+        want = resid.clone()
+        emu.linear_residual(x, w, want)
+        got = resid.clone().to(DEV)
+        ops.linear_residual(x.to(DEV), w.to(DEV), got)
+        close(got, want, torch.float32, f"linear_residual {m}x{n}x{k}", want.abs().max().item())
+        inter = max(1, n // 3)
+        gate, up = rnd((inter, k), torch.float32, 13, 0.2), rnd((inter, k), torch.float32, 14, 0.2)
+        wgu = interleave_gate_up(gate, up)
+        want = torch.empty(m, inter)
+        emu.linear_swiglu(x, wgu, want)
+        got = torch.empty(m, inter, device=DEV)
+        ops.linear_swiglu(x.to(DEV), wgu.to(DEV), got)
+        close(got, want, torch.float32, f"linear_swiglu {m}x{inter}x{k}", want.abs().max().item())
+
+
 @pytest.mark.parametrize("tile", [64, 130, 129, 131, 132, 133])
 @pytest.mark.parametrize("m,n,k", [(65, 130, 72), (200, 1152, 896), (300, 257, 136), (513, 384, 264), (129, 64, 1160),
                                    (70, 300, 24), (130, 90, 40), (257, 520, 8)])
@@ -430,20 +462,21 @@ def test_values_of_four_positions_written_together(ops, emu, nq, nkv, d, page, h
         check_qkv_rope_cache(ops, emu, nq, nkv, d, page, hidden, rows_per, starts)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("window", [None, 40])
-def test_attention_of_a_mixed_step(ops, emu, window):
+def test_attention_of_a_mixed_step(ops, emu, window, dtype):
     """Portions of prompts beside decoding requests with long histories, one of which has a
     key that stands out far back."""
     spec = [(700, 1), (64, 300), (1500, 1), (0, 1), (31, 2), (200, 90), (999, 1)]
-    run_attention(ops, emu, torch.bfloat16, 14, 2, 64, 64, window, spec, seed=90, amplify=(2, 100 if window is None else 1480, 30.0))
-    run_attention(ops, emu, torch.bfloat16, 6, 3, 48, 16, window, spec[:5], seed=91)
-    run_attention(ops, emu, torch.bfloat16, 8, 1, 128, 32, window, spec[:4], seed=92)
+    run_attention(ops, emu, dtype, 14, 2, 64, 64, window, spec, seed=90, amplify=(2, 100 if window is None else 1480, 30.0))
+    run_attention(ops, emu, dtype, 6, 3, 48, 16, window, spec[:5], seed=91)
+    run_attention(ops, emu, dtype, 8, 1, 128, 32, window, spec[:4], seed=92)
 
 
 @pytest.mark.parametrize("window", [None, 40])
 @pytest.mark.parametrize("cus", [8, 16, 30, 60, 80, 100, 1000])
 @pytest.mark.parametrize("nq,nkv,d,page", [(14, 2, 64, 64), (6, 3, 48, 16), (8, 1, 128, 32), (2, 1, 256, 16)])
-def test_attention_tilings_of_many_rows(ops, emu, window, cus, nq, nkv, d, page):
+def test_attention_tilings_of_many_rows(ops, emu, window, cus, nq, nkv, d, page, dtype=torch.bfloat16):
     """The kernel variants for many tiles of rows (tiles of 128 rows, of 64, of 64 in
     pairs, keys split over the waves of a block) are chosen by the tiles per compute
     unit: told of fewer units than the chip has, a step of a few hundred rows takes
@@ -451,13 +484,22 @@ def test_attention_tilings_of_many_rows(ops, emu, window, cus, nq, nkv, d, page)
     real = ops.num_cus
     ops.num_cus = cus
     try:
-        run_attention(ops, emu, torch.bfloat16, nq, nkv, d, page, window, [(0, 300), (0, 200)], seed=93,
+        run_attention(ops, emu, dtype, nq, nkv, d, page, window, [(0, 300), (0, 200)], seed=93,
                       amplify=(0, 70, 30.0))
         # behind a history (never in pairs), and one request decoding beside
-        run_attention(ops, emu, torch.bfloat16, nq, nkv, d, page, window, [(500, 300), (64, 200), (900, 1)], seed=94,
+        run_attention(ops, emu, dtype, nq, nkv, d, page, window, [(500, 300), (64, 200), (900, 1)], seed=94,
                       amplify=(0, 130 if window is None else 770, 30.0))
     finally:
         ops.num_cus = real
+
+
+@pytest.mark.parametrize("window", [None, 40])
+@pytest.mark.parametrize("cus", [8, 1000])
+@pytest.mark.parametrize("nq,nkv,d,page", [(14, 2, 64, 64), (6, 3, 48, 16), (8, 1, 128, 32), (2, 1, 256, 16)])
+def test_attention_tilings_of_many_rows_float32(ops, emu, window, cus, nq, nkv, d, page):
+    """The float32 kernel's two launches for many rows: a wave per tile of rows, and (told
+    of a very large chip, behind a history) the waves of a block splitting a tile's keys."""
+    test_attention_tilings_of_many_rows(ops, emu, window, cus, nq, nkv, d, page, dtype=torch.float32)
 
 
 @pytest.mark.parametrize("window", [None, 40])
@@ -475,13 +517,19 @@ def test_attention_every_launch_of_many_rows(ops, emu, window, path, nq, nkv, d,
                       amplify=(0, 70, 30.0))
         run_attention(ops, emu, torch.bfloat16, nq, nkv, d, page, window, [(500, 300), (64, 200), (900, 1)], seed=97,
                       amplify=(0, 130 if window is None else 770, 30.0))
+        if path <= 2:      # float32 has these two: the waves of a block split the keys, or a wave per tile
+            run_attention(ops, emu, torch.float32, nq, nkv, d, page, window, [(0, 300), (0, 70), (0, 129)], seed=96,
+                          amplify=(0, 70, 30.0))
+            run_attention(ops, emu, torch.float32, nq, nkv, d, page, window, [(500, 300), (64, 200), (900, 1)],
+                          seed=97, amplify=(0, 130 if window is None else 770, 30.0))
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("start", [0, 3000])
-def test_attention_of_a_long_portion(ops, emu, start):
+def test_attention_of_a_long_portion(ops, emu, start, dtype):
     """2,048 tokens of a prompt at the 0.5B head counts, at its start and behind a
     history: enough tiles for the whole chip, as in a prefill step of the engine."""
-    run_attention(ops, emu, torch.bfloat16, 14, 2, 64, 64, None, [(start, 2048)], seed=95, amplify=(0, 1033, 30.0))
+    run_attention(ops, emu, dtype, 14, 2, 64, 64, None, [(start, 2048)], seed=95, amplify=(0, 1033, 30.0))
 
 
 def make_cache(num_pages, nkv, page, d, dtype, seed):
@@ -635,22 +683,24 @@ def test_attention_far_key_among_hundreds(ops, emu, dtype):
     run_attention(ops, emu, dtype, 14, 2, 64, 64, None, [(4000, 1), (2000, 1)], amplify=(1, 1999, 30.0))
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("d,length,key", [(64, 9000, 8000), (128, 5000, 70), (64, 20001, 11), (64, 40000, 33000)])
-def test_attention_one_request_over_a_long_history(ops, emu, d, length, key):
+def test_attention_one_request_over_a_long_history(ops, emu, d, length, key, dtype):
     """One decoded token of a single request: its keys are split over as many blocks
     as the merge takes (from 35 to the limit of 128 here), and one key far from both ends
     carries the answer."""
-    run_attention(ops, emu, torch.bfloat16, 4, 1, d, 64, None, [(length - 1, 1)], amplify=(0, key, 30.0))
+    run_attention(ops, emu, dtype, 4, 1, d, 64, None, [(length - 1, 1)], amplify=(0, key, 30.0))
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("splits", [1, 3, 16, 17, 50, 64, 65, 128])
-def test_attention_merge_of_any_number_of_splits(ops, emu, splits):
+def test_attention_merge_of_any_number_of_splits(ops, emu, splits, dtype):
     """The number of key splits is fixed from outside: one wave merges up to sixteen,
     four waves more, a lane holds the weights of two; splits past the end of a short
     history have no keys at all and must count for nothing."""
     for d, length in ((64, 700), (128, 3000), (48, 90)):
         with ops.debug.force(attention_splits=(d, splits)):
-            run_attention(ops, emu, torch.bfloat16, 6, 2, d, 16, None, [(length - 1, 1), (40, 1), (length // 2, 2)],
+            run_attention(ops, emu, dtype, 6, 2, d, 16, None, [(length - 1, 1), (40, 1), (length // 2, 2)],
                           seed=96, amplify=(0, length // 3, 30.0))
 
 
