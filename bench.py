@@ -551,6 +551,7 @@ def main():
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         sys.exit(2)
+    bracket = ProfilerBracket(args.profile)       # (pauses collection now: loading and filling are not collected)
     if args.graph == "on":
         args.graph = True
     if args.side:
@@ -578,7 +579,7 @@ def main():
     max_batch = max(batches)
     context = args.context or DEFAULT_CONTEXT[args.shape]
     engine = make_engine(args, cfg, max_batch * (context + PAGE), max_batch, FILL_TOKENS, context + PAGE)
-    runs = Runs(engine, cfg, context, args.dtype, args.samples, ProfilerBracket(args.profile), measured)
+    runs = Runs(engine, cfg, context, args.dtype, args.samples, bracket, measured)
     if args.force:
         forced = {}
         for item in args.force:

@@ -901,18 +901,21 @@ static void launch_f32_tiled(const float* A, const float* W, const EpiArgs& e, i
                        stream, A, W, e, M, N, K, vec);
 }
 
-// Few rows in float32 (decode steps, short portions): one wave owns NB = 4 rows of W and
-// its lanes split the inner size, four numbers a lane and step, so that a wave instruction
-// reads 1 KB of a row of W in a row (any inner size: one number at a time where rows are
-// not 16-byte aligned).  MB rows of x go with them (they stay in the caches); the MB x NB
-// sums meet by lane shuffles.  For SWIGLU the four rows are two gate rows and the up rows
-// of the same two outputs.  Still plain FMAs in 32 bits.
-template <int EPI, int MB>
-__global__ __launch_bounds__(64) void gemm_f32_rows_kernel(const float* __restrict__ A,
-                                                            const float* __restrict__ W, EpiArgs e, int M,
-                                                            int N, int K, int vec) {
+// Few rows in float32 (decode steps, short portions): a block owns NB = 4 rows of W, its KW
+// waves split the inner size, and a wave's lanes split its share, four numbers a lane and
+// step, so that a wave instruction reads 1 KB of a row of W in a row (any inner size: one
+// number at a time where rows are not 16-byte aligned).  Two steps are on their way from
+// memory at a time.  MB rows of x go with them (they stay in the caches); the MB x NB sums
+// meet by lane shuffles and, across the waves, in LDS in a fixed order.  For SWIGLU the four
+// rows are two gate rows and the up rows of the same two outputs.  Still plain FMAs in 32
+// bits.  (One wave per block left a narrow output, 224 blocks of the down product, with one
+// wave per compute unit walking 19 steps one after the other: 26 us for 17 MB.)
+template <int EPI, int MB, int KW>
+__global__ __launch_bounds__(64 * KW) void gemm_f32_rows_kernel(const float* __restrict__ A,
+                                                                 const float* __restrict__ W, EpiArgs e, int M,
+                                                                 int N, int K, int vec) {
   constexpr int NB = 4;
-  const int lane = threadIdx.x;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int m0 = blockIdx.y * MB;
   int rows_w[NB];
   if constexpr (EPI == EPI_SWIGLU) {
@@ -934,21 +937,38 @@ __global__ __launch_bounds__(64) void gemm_f32_rows_kernel(const float* __restri
 #pragma unroll
     for (int j = 0; j < NB; ++j) acc[i][j] = 0.f;
   if (vec) {
-    for (int k = lane * 4; k < K; k += 256) {
-      floatx4 w4[NB], x4[MB];
-#pragma unroll
-      for (int j = 0; j < NB; ++j) w4[j] = *(const floatx4*)(wp[j] + k);
-#pragma unroll
-      for (int i = 0; i < MB; ++i) x4[i] = *(const floatx4*)(xp[i] + k);
+    constexpr int STEP = 256 * KW;
+    auto mac = [&](const floatx4 (&w4)[NB], const floatx4 (&x4)[MB]) {
 #pragma unroll
       for (int i = 0; i < MB; ++i)
 #pragma unroll
         for (int j = 0; j < NB; ++j)
 #pragma unroll
           for (int c = 0; c < 4; ++c) acc[i][j] = fmaf(x4[i][c], w4[j][c], acc[i][j]);
+    };
+    int k = (wave * 64 + lane) * 4;
+    for (; k + STEP < K; k += 2 * STEP) {            // two steps at a time
+      floatx4 w4[2][NB], x4[2][MB];
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+#pragma unroll
+        for (int j = 0; j < NB; ++j) w4[u][j] = *(const floatx4*)(wp[j] + k + u * STEP);
+#pragma unroll
+        for (int i = 0; i < MB; ++i) x4[u][i] = *(const floatx4*)(xp[i] + k + u * STEP);
+      }
+      mac(w4[0], x4[0]);
+      mac(w4[1], x4[1]);
+    }
+    for (; k < K; k += STEP) {
+      floatx4 w4[NB], x4[MB];
+#pragma unroll
+      for (int j = 0; j < NB; ++j) w4[j] = *(const floatx4*)(wp[j] + k);
+#pragma unroll
+      for (int i = 0; i < MB; ++i) x4[i] = *(const floatx4*)(xp[i] + k);
+      mac(w4, x4);
     }
   } else {
-    for (int k = lane; k < K; k += 64) {
+    for (int k = wave * 64 + lane; k < K; k += 64 * KW) {
       float w1[NB], x1[MB];
 #pragma unroll
       for (int j = 0; j < NB; ++j) w1[j] = wp[j][k];
@@ -964,7 +984,28 @@ __global__ __launch_bounds__(64) void gemm_f32_rows_kernel(const float* __restri
   for (int i = 0; i < MB; ++i)
 #pragma unroll
     for (int j = 0; j < NB; ++j) acc[i][j] = wave_sum(acc[i][j]);
-  if (lane != 0) return;
+  if constexpr (KW > 1) {
+    __shared__ float red[KW][MB][NB];
+    if (lane == 0) {
+#pragma unroll
+      for (int i = 0; i < MB; ++i)
+#pragma unroll
+        for (int j = 0; j < NB; ++j) red[wave][i][j] = acc[i][j];
+    }
+    __syncthreads();
+    if (threadIdx.x != 0) return;
+#pragma unroll
+    for (int i = 0; i < MB; ++i)
+#pragma unroll
+      for (int j = 0; j < NB; ++j) {
+        float t = red[0][i][j];
+#pragma unroll
+        for (int w = 1; w < KW; ++w) t += red[w][i][j];
+        acc[i][j] = t;
+      }
+  } else {
+    if (lane != 0) return;
+  }
 #pragma unroll
   for (int i = 0; i < MB; ++i) {
     const int m = m0 + i;
@@ -986,20 +1027,35 @@ __global__ __launch_bounds__(64) void gemm_f32_rows_kernel(const float* __restri
   }
 }
 
+template <int EPI, int KW>
+static void launch_f32_rows_kw(const float* A, const float* W, const EpiArgs& e, int M, int N, int K, int vec,
+                               unsigned groups, hipStream_t stream) {
+  if (M == 1)
+    hipLaunchKernelGGL((gemm_f32_rows_kernel<EPI, 1, KW>), dim3(groups, 1), dim3(64 * KW), 0, stream, A, W, e, M, N, K, vec);
+  else if (M == 2)
+    hipLaunchKernelGGL((gemm_f32_rows_kernel<EPI, 2, KW>), dim3(groups, 1), dim3(64 * KW), 0, stream, A, W, e, M, N, K, vec);
+  else if (M <= 4)
+    hipLaunchKernelGGL((gemm_f32_rows_kernel<EPI, 4, KW>), dim3(groups, 1), dim3(64 * KW), 0, stream, A, W, e, M, N, K, vec);
+  else
+    hipLaunchKernelGGL((gemm_f32_rows_kernel<EPI, 8, KW>), dim3(groups, (M + 7) / 8), dim3(64 * KW), 0, stream, A, W, e,
+                       M, N, K, vec);
+}
+
+// Waves per block: as many as give every wave at least two steps of its own, up to 8, fewer
+// where the blocks alone already put several waves on every compute unit.
 template <int EPI>
-static void launch_f32_rows(const float* A, const float* W, const EpiArgs& e, int M, int N, int K,
+static void launch_f32_rows(const float* A, const float* W, const EpiArgs& e, int M, int N, int K, int num_cus,
                             hipStream_t stream) {
   const int vec = (K % 4 == 0) && ((uintptr_t)A % 16 == 0) && ((uintptr_t)W % 16 == 0);
   const unsigned groups = EPI == EPI_SWIGLU ? (unsigned)(N / 32) * 8 : (unsigned)((N + 3) / 4);
-  if (M == 1)
-    hipLaunchKernelGGL((gemm_f32_rows_kernel<EPI, 1>), dim3(groups, 1), dim3(64), 0, stream, A, W, e, M, N, K, vec);
-  else if (M == 2)
-    hipLaunchKernelGGL((gemm_f32_rows_kernel<EPI, 2>), dim3(groups, 1), dim3(64), 0, stream, A, W, e, M, N, K, vec);
-  else if (M <= 4)
-    hipLaunchKernelGGL((gemm_f32_rows_kernel<EPI, 4>), dim3(groups, 1), dim3(64), 0, stream, A, W, e, M, N, K, vec);
-  else
-    hipLaunchKernelGGL((gemm_f32_rows_kernel<EPI, 8>), dim3(groups, (M + 7) / 8), dim3(64), 0, stream, A, W, e, M, N,
-                       K, vec);
+  const long blocks = (long)groups * ((M + 7) / 8);
+  const int steps = (K + 255) / 256;
+  int kw = 1;
+  while (kw < 8 && steps >= 4 * kw && blocks * kw < 8L * num_cus) kw *= 2;
+  if (kw >= 8) launch_f32_rows_kw<EPI, 8>(A, W, e, M, N, K, vec, groups, stream);
+  else if (kw == 4) launch_f32_rows_kw<EPI, 4>(A, W, e, M, N, K, vec, groups, stream);
+  else if (kw == 2) launch_f32_rows_kw<EPI, 2>(A, W, e, M, N, K, vec, groups, stream);
+  else launch_f32_rows_kw<EPI, 1>(A, W, e, M, N, K, vec, groups, stream);
 }
 constexpr int F32_ROWS_MAX = 64;     // up to here the few-row kernel (the tiled one would run on N / 64 blocks)
 
@@ -1290,10 +1346,10 @@ extern "C" int llmlab_linear(const void* x, const void* w, int dtype, int epilog
     const float* W = (const float*)w;
     if (M <= F32_ROWS_MAX) {
       switch (epilogue) {
-        case EPI_STORE: launch_f32_rows<EPI_STORE>(A, W, e, M, N, K, stream); break;
-        case EPI_RESID: launch_f32_rows<EPI_RESID>(A, W, e, M, N, K, stream); break;
-        case EPI_F32: launch_f32_rows<EPI_F32>(A, W, e, M, N, K, stream); break;
-        default: launch_f32_rows<EPI_SWIGLU>(A, W, e, M, N, K, stream); break;
+        case EPI_STORE: launch_f32_rows<EPI_STORE>(A, W, e, M, N, K, num_cus, stream); break;
+        case EPI_RESID: launch_f32_rows<EPI_RESID>(A, W, e, M, N, K, num_cus, stream); break;
+        case EPI_F32: launch_f32_rows<EPI_F32>(A, W, e, M, N, K, num_cus, stream); break;
+        default: launch_f32_rows<EPI_SWIGLU>(A, W, e, M, N, K, num_cus, stream); break;
       }
       LLMLAB_LAUNCH_CHECK("linear(float32, few rows)");
       return 0;

@@ -210,6 +210,8 @@ class Engine:
                           "replays": fn.graph_replays, "evictions": fn.graph_evictions,
                           "kept": len(fn._graphs), "decode_calls": fn.decode_calls},
                "scratch": {"bytes": fn.ctx.scratch_bytes, "allocations": fn.ctx.scratch_allocations},
+               "launch_sequences": {"recorded": self.model.launches_recorded,
+                                    "replayed": self.model.launches_replayed},
                "kernel_calls": getattr(self.ops, "calls_made", None),
                "requests": self.request_instruments.snapshot(),
                "cache": self.cache.metrics()}

@@ -10,6 +10,7 @@ is a struct written for one architecture
 from __future__ import annotations
 
 import dataclasses
+import os
 from typing import Dict, List, Optional, Tuple
 
 import torch
@@ -44,6 +45,12 @@ class EntryView:
         return self.cache.get("v")
 
 
+def _same_pending(a, b) -> bool:
+    if a is None or b is None:
+        return a is b
+    return a.parts.data_ptr() == b.parts.data_ptr() and a.splits == b.splits and a.parts.shape == b.parts.shape
+
+
 class CausalLM:
     def __init__(self, spec: ModelSpec):
         spec.validate()
@@ -56,6 +63,12 @@ class CausalLM:
         self.ops = None
         self.dtype = None
         self.ranges = None         # profiler ranges (engine/profiling.py), off by default
+        # Launch sequences of the scheduled runs, kept by the shape of the step: see _run_block.
+        self.keep_launches = os.environ.get("LLMLAB_KEEP_LAUNCHES", "1") not in ("0", "")
+        self.verify_launches = os.environ.get("LLMLAB_VERIFY_LAUNCHES", "") not in ("0", "")
+        self._launches: List[Dict[tuple, object]] = [dict() for _ in self.entries]
+        self.launches_recorded = 0
+        self.launches_replayed = 0
 
     def parts(self):
         return [self.embedding, *self.blocks, self.final_norm, self.head]
@@ -155,9 +168,68 @@ class CausalLM:
         if self.ranges is not None:
             return self._forward_with_ranges(x, ctx)
         self.embedding.forward(ctx.token_ids, x, ctx)
-        for view in self.entries:
-            self.blocks[view.block].forward(x, ctx, view)
+        if self._launches_usable(ctx):
+            stamp = (ctx.n_rows, ctx.scratch_version, self.ops.fingerprint())
+            for view in self.entries:
+                self._run_block(self.blocks[view.block], x, ctx, view, stamp)
+        else:
+            for view in self.entries:
+                self.blocks[view.block].forward(x, ctx, view)
         return self._head(x, ctx)
+
+    MAX_KEPT_LAUNCHES = 256       # per scheduled run
+
+    def _launches_usable(self, ctx) -> bool:
+        return (self.keep_launches and hasattr(self.ops, "begin_recording") and hasattr(ctx, "scratch_version")
+                and hasattr(ctx, "pending"))
+
+    def _run_block(self, block, x, ctx, view, stamp) -> None:
+        """One scheduled run of a block.  Between the host's decision what to launch and the
+        launch itself lie shape checks, scratch lookups and argument marshalling that cost
+        the host more than the GPU needs for a small model's step.  A block whose parts all
+        say ``keeps_launches`` makes the same calls into the kernel libraries whenever the
+        step has the same number of rows, the scratch buffers have not moved, the sums
+        owed to the stream arrive in the same form and the kernel set's rules are the same;
+        so the calls of its first such run are written down (``HipOps.begin_recording``)
+        and made again from the list from then on.  Calls that depend on the step's data
+        (attention: requests, lengths) are kept as closures and evaluated anew
+        (``HipOps.live``).  ``LLMLAB_VERIFY_LAUNCHES=1``: at every replay the block's
+        Python code is run as well, without launching, and must make the very same calls.
+        The reference's host does this work in compiled code
+        (rust/engine/src/runner/model/qwen2/engine.rs:916-1130)."""
+        if not block.keeps_launches:
+            block.forward(x, ctx, view)
+            return
+        owed = ctx.pending
+        key = stamp + ((owed.parts.data_ptr(), owed.splits, tuple(owed.parts.shape)) if owed is not None else None,)
+        kept = self._launches[view.index]
+        hit = kept.get(key)
+        ops = self.ops
+        if hit is not None:
+            record, owed_after = hit
+            if self.verify_launches:
+                again = ops.begin_recording(dry=True)
+                try:
+                    block.forward(x, ctx, view)
+                finally:
+                    ops.end_recording()
+                if not again.same_as(record) or not _same_pending(ctx.pending, owed_after):
+                    raise AssertionError(f"schedule[{view.index}]: the calls kept for steps of {ctx.n_rows} rows "
+                                         f"are not the calls its parts would make now")
+            ops.replay(record)
+            ctx.pending = owed_after
+            self.launches_replayed += 1
+            return
+        record = ops.begin_recording()
+        try:
+            block.forward(x, ctx, view)
+        finally:
+            ops.end_recording()
+        if ctx.scratch_version == stamp[1]:        # (buffers that moved meanwhile: written down next time)
+            if len(kept) >= self.MAX_KEPT_LAUNCHES:
+                kept.clear()
+            kept[key] = (record, ctx.pending)
+            self.launches_recorded += 1
 
     def _head(self, x, ctx) -> Optional[torch.Tensor]:
         if ctx.n_want == 0:
@@ -174,8 +246,13 @@ class CausalLM:
         r = self.ranges
         with r.range("embedding"):
             self.embedding.forward(ctx.token_ids, x, ctx)
+        usable = self._launches_usable(ctx)
+        stamp = (ctx.n_rows, ctx.scratch_version, self.ops.fingerprint()) if usable else None
         for view in self.entries:
             with r.range(f"block {view.index}"):
-                self.blocks[view.block].forward(x, ctx, view)
+                if usable:
+                    self._run_block(self.blocks[view.block], x, ctx, view, stamp)
+                else:
+                    self.blocks[view.block].forward(x, ctx, view)
         with r.range("final norm + head"):
             return self._head(x, ctx)

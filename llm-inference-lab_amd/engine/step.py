@@ -107,6 +107,7 @@ class StepContext:
             for t, (page_size, window) in zip(self._table_at, groups)]
         self._uploaded = torch.cuda.Event() if pin else None
         self._scratch: Dict[Tuple[str, torch.dtype], torch.Tensor] = {}
+        self._views: Dict[tuple, torch.Tensor] = {}     # views of the scratch buffers handed out so far
         self.scratch_version = 0
         self.scratch_bytes = 0
         self.scratch_allocations = 0
@@ -142,6 +143,9 @@ class StepContext:
         unused): the page pool takes most of what the weights left, and a step that needs
         more scratch than remains fails with ``ScratchExhausted`` instead of somewhere in
         the allocator (rust/engine/src/runner/model/qwen2/workspace.rs:348-373)."""
+        hit = self._views.get((name, dtype, shape))      # (slicing and viewing anew costs microseconds a call)
+        if hit is not None:
+            return hit
         count = 1
         for s in shape:
             count *= int(s)
@@ -161,7 +165,11 @@ class StepContext:
             buf = torch.empty(max(count, 1), dtype=dtype, device=self.device)
             self._scratch[key] = buf
             self.scratch_version += 1
-        return buf[:count].view(shape)
+            self._views = {k: v for k, v in self._views.items() if (k[0], k[1]) != key}
+        view = buf[:count].view(shape)
+        if len(self._views) < 4096 and isinstance(shape, tuple):
+            self._views[(name, dtype, shape)] = view
+        return view
 
     def _memory_available(self) -> Optional[int]:
         if torch.device(self.device).type != "cuda":

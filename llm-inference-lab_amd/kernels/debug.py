@@ -107,6 +107,7 @@ class KernelDebug:
                 raise TypeError(f"no dispatch rule named '{key}'")
             setattr(ops.rules, key, value)
         lib = plib = mlib = None
+        ops.debug_epoch += 1
         try:
             if attention_merge_kernel is not None:
                 mlib = ops._attention_lib(int(attention_merge_kernel))
@@ -130,6 +131,7 @@ class KernelDebug:
                 lib.llmlab_debug_attention_splits(int(attention_splits[1]))
             yield ops
         finally:
+            ops.debug_epoch += 1
             ops.rules = saved
             if gemm_tile is not None:
                 core.llmlab_debug_gemm_tile(0)

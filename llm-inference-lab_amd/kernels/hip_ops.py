@@ -38,6 +38,9 @@ class KernelError(RuntimeError):
     pass
 
 
+_NO_HEADS = (None, None, None, None, 0, 0, None, None, 0, 0, 0)     # a few-row product without the q/k/v epilogue
+
+
 class PackedWeight:
     """A bfloat16 matrix [n, k] in the order the matrix cores read it: strips of 16
     rows, a strip a run of 1 KB tiles (16 rows x 32 columns, one MFMA B operand,
@@ -63,6 +66,31 @@ class PackedWeight:
 
     def element_size(self) -> int:
         return self.data.element_size()
+
+
+class LaunchRecord:
+    """The calls into the kernel libraries that a part made while it was recorded, so that
+    the same part under the same conditions can make them again without its Python code:
+    ``calls[i]`` is ``(function, argument list, library)``, or ``(None, callable, None)``
+    for a call that depends on the step's data and is made anew through its closure
+    (``HipOps.live``).  ``dry``: nothing is launched while recording (a recorded sequence is
+    only compared with one kept from before)."""
+
+    __slots__ = ("calls", "dry")
+
+    def __init__(self, dry: bool = False):
+        self.calls = []
+        self.dry = dry
+
+    def same_as(self, other: "LaunchRecord") -> bool:
+        if len(self.calls) != len(other.calls):
+            return False
+        for (fa, aa, _), (fb, ab, _) in zip(self.calls, other.calls):
+            if (fa is None) != (fb is None):
+                return False
+            if fa is not None and (fa is not fb or list(aa[:-1]) != list(ab[:-1])):     # (the last is the stream)
+                return False
+        return True
 
 
 class HipOps:
@@ -94,6 +122,8 @@ class HipOps:
         self.arrived = torch.zeros(self.ARRIVED_INTS, dtype=torch.int32, device=self.device)
         self.loaded_libraries = [self._core._name]
         self.calls_made = 0          # calls into the kernel libraries so far
+        self._record: Optional[LaunchRecord] = None
+        self.debug_epoch = 0         # counts the changes of forced kernel choices (kernels/debug.py)
         self.rules = DispatchRules()         # the measured thresholds of the dispatch, in one place
         self.debug = KernelDebug(self)       # forcing kernel choices from outside (tests, measurements)
 
@@ -245,9 +275,62 @@ class HipOps:
     def _call(self, fn, *args, lib=None) -> None:
         """One call into the kernel libraries; a failure raises with the library's message."""
         self.calls_made += 1
+        if self._record is not None:
+            self._record.calls.append((fn, list(args), lib))
+            if self._record.dry:
+                return
         code = fn(*args)
         if code != 0:
             self._check(code, lib)
+
+    # ------------------------------------------------- recorded launch sequences
+    def begin_recording(self, dry: bool = False) -> LaunchRecord:
+        """From now until ``end_recording`` every call into the kernel libraries is also
+        written down (``engine/model.py`` keeps the sequences of its blocks and replays
+        them for steps of the same shape)."""
+        if self._record is not None:
+            raise RuntimeError("a recording is already under way")
+        self._record = LaunchRecord(dry)
+        return self._record
+
+    def end_recording(self) -> Optional[LaunchRecord]:
+        record, self._record = self._record, None
+        return record
+
+    def live(self, launch) -> None:
+        """``launch()`` makes calls whose arguments depend on the step's data (how many
+        requests, how long their histories): while a sequence is recorded it is written
+        down as a closure, to be called anew at every replay, and its own calls are not."""
+        record = self._record
+        if record is None:
+            launch()
+            return
+        record.calls.append((None, launch, None))
+        if record.dry:
+            return
+        self._record = None
+        try:
+            launch()
+        finally:
+            self._record = record
+
+    def replay(self, record: LaunchRecord) -> None:
+        """Make a recorded sequence of calls again, on the current stream."""
+        stream = self._stream()
+        for fn, args, lib in record.calls:
+            if fn is None:
+                args()
+                continue
+            args[-1] = stream
+            self.calls_made += 1
+            code = fn(*args)
+            if code != 0:
+                self._check(code, lib)
+
+    def fingerprint(self):
+        """What the host-side choices of the kernel set depend on beside the shapes."""
+        import dataclasses
+        return (self.num_cus, self.debug_epoch, dataclasses.astuple(self.rules))
 
     def _check(self, code: int, lib=None) -> None:
         if code != 0:
@@ -398,8 +481,6 @@ class HipOps:
     def _skinny(self, x, norm, x_rows, norm_w, eps, w, bias, epilogue, out, m, n, k, ldo, n_out,
                 qkv=None, pending: Optional[PendingSums] = None, ksplit: int = 1,
                 part_stride: int = 0) -> None:
-        q = qkv or {}
-        table = q.get("table")
         if pending is not None:
             p = pending.parts
             if (p.dtype != torch.float32 or p.dim() != 3 or p.stride(2) != 1 or p.device != self.device
@@ -411,14 +492,18 @@ class HipOps:
             pend = (self._ptr(p), pending.splits, p.stride(1), p.stride(0))
         else:
             pend = (_c_ptr(0), 0, 0, 0)
+        if qkv is None:
+            heads = _NO_HEADS
+        else:
+            table, ptr = qkv["table"], self._ptr
+            heads = (ptr(qkv["inv_freq"]), ptr(qkv["positions"]), ptr(qkv["row_req"]), ptr(table),
+                     table.stride(0) if table is not None else 0, qkv["page_size"], ptr(qkv["k_cache"]),
+                     ptr(qkv["v_cache"]), qkv["nq"], qkv["nkv"], qkv["d"])
         self._call(self._core.llmlab_skinny_linear,
-            self._ptr(x), 1 if norm else 0, self._ptr(x_rows), self._ptr(norm_w),
-            _dt(norm_w) if norm_w is not None else 0, float(eps), self._ptr(w), self._ptr(bias),
-            _dt(bias) if bias is not None else 0, epilogue, self._ptr(out), m, n, k, ldo, n_out,
-            self._ptr(q.get("inv_freq")), self._ptr(q.get("positions")), self._ptr(q.get("row_req")),
-            self._ptr(table), table.stride(0) if table is not None else 0, q.get("page_size", 0),
-            self._ptr(q.get("k_cache")), self._ptr(q.get("v_cache")), q.get("nq", 0), q.get("nkv", 0),
-            q.get("d", 0), self.num_cus, pend[0], pend[1], pend[2], pend[3], int(ksplit),
+            x.data_ptr(), 1 if norm else 0, self._ptr(x_rows), self._ptr(norm_w),
+            _dt(norm_w) if norm_w is not None else 0, float(eps), w.data_ptr(), self._ptr(bias),
+            _dt(bias) if bias is not None else 0, epilogue, out.data_ptr(), m, n, k, ldo, n_out,
+            *heads, self.num_cus, pend[0], pend[1], pend[2], pend[3], int(ksplit),
             int(part_stride), self._stream())
 
     # --------------------------------------------- sums left in pieces (deferred)

@@ -143,11 +143,21 @@ class GQAAttention(Mixer):
                               ctx.positions, ctx.row_req, group.block_table, group.page_size,
                               k_cache, v_cache)
         out = ctx.scratch("attention.out", (rows, self.q_size), self.dtype)
-        ops.paged_attention(
-            q, self.num_heads, self.num_kv_heads, self.head_dim,
-            entry.k_cache, entry.v_cache, group.block_table, group.page_size,
-            ctx.q_start, ctx.start_pos, ctx.n_reqs, ctx.max_q_len, ctx.max_ctx_len,
-            self.window, self.scale, out, self._short_requests(ctx))
+
+        def attend():
+            # (how many requests, how long their portions and their histories are: read from
+            # the step's description when the launch is made, also when it is made again
+            # from a kept sequence of calls)
+            ops.paged_attention(
+                q, self.num_heads, self.num_kv_heads, self.head_dim,
+                entry.k_cache, entry.v_cache, group.block_table, group.page_size,
+                ctx.q_start, ctx.start_pos, ctx.n_reqs, ctx.max_q_len, ctx.max_ctx_len,
+                self.window, self.scale, out, self._short_requests(ctx))
+        live = getattr(ops, "live", None)
+        if live is not None:
+            live(attend)
+        else:
+            attend()
         if pending is not None:
             ops.linear_residual(out, self.w_o, residual, self.b_o, pending=pending)
             ctx.pending = None
@@ -180,6 +190,10 @@ class GQAAttention(Mixer):
                     longest = max(longest, ctx.host_start_pos[b] + n)
             ctx.memo[key] = (ctx.row_req, limit, count, longest) if 0 < count < ctx.n_reqs else None
         return ctx.memo[key]
+
+    @property
+    def keeps_launches(self):
+        return self.position is None or self.position.keeps_launches
 
     def kernel_libraries(self):
         return [("attention", self.head_dim)]

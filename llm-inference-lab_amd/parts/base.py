@@ -110,6 +110,15 @@ class Part:
         head_dim)``)."""
         return []
 
+    # True: everything ``forward`` does on the GPU goes through the kernel set's entry points,
+    # with arguments that depend on nothing but the number of rows of the step, the scratch
+    # buffers and the sums owed to the stream; what depends on the step's data beyond that
+    # is wrapped in ``ops.live(...)``.  The model may then write the calls of a run down and
+    # make them again without running ``forward`` (``CausalLM._run_block``).  False (the
+    # default, and right for any part that calls PyTorch or decides on the host from the
+    # step's data): ``forward`` runs every time.
+    keeps_launches = False
+
 
 class Norm(Part):
     # True: ``forward(x, out, None, pending=p)`` first makes the stream whole,
@@ -240,6 +249,10 @@ class Block(Part):
     @property
     def graph_safe(self):
         return all(p.graph_safe for p in self.parts())
+
+    @property
+    def keeps_launches(self):
+        return all(p.keeps_launches for p in self.parts())
 
     def kernel_libraries(self):
         return [lib for p in self.parts() for lib in p.kernel_libraries()]

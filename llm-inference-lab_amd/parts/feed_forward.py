@@ -65,6 +65,7 @@ class SwiGLU(FeedForward):
         self.w_down = ops.prepare_weight(tensors[t["down_weight"]].contiguous())
 
     takes_normed_input = True
+    keeps_launches = True
 
     def forward(self, h, residual, ctx):
         rows = h.shape[0]

@@ -19,6 +19,7 @@ class RMSNorm(Norm):
     are the same).  ``size`` and ``eps`` come from the caller."""
 
     folds_pending = True
+    keeps_launches = True
 
     def __init__(self, size: int, eps: float, tensors: Dict[str, str]):
         super().__init__(tensors)

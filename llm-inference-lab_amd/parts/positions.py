@@ -31,6 +31,8 @@ class RotaryEmbedding(PositionEncoding):
         self.inv_freq = (1.0 / (torch.tensor(self.theta, dtype=torch.float64) ** exponent)
                          ).to(torch.float32).to(ops.device)
 
+    keeps_launches = True      # (the frequency table goes to the kernels; ``apply`` depends on the rows only)
+
     def rotary_table(self):
         return self.inv_freq
 
@@ -41,6 +43,8 @@ class RotaryEmbedding(PositionEncoding):
 
 class NoPosition(PositionEncoding):
     """No position encoding: queries and keys are used as projected."""
+
+    keeps_launches = True
 
     def __init__(self, tensors: Optional[Dict[str, str]] = None, **_):
         super().__init__(tensors)

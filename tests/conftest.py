@@ -9,6 +9,11 @@ for p in (ROOT, os.path.join(ROOT, "tests")):
         sys.path.insert(0, p)
 
 
+# Every replay of a kept launch sequence (engine/model.py) is checked against the calls the
+# parts would make now.
+os.environ.setdefault("LLMLAB_VERIFY_LAUNCHES", "1")
+
+
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs an AMD GPU (run with -m gpu)")
 

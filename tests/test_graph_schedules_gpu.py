@@ -130,3 +130,36 @@ def test_a_long_history_beside_short_ones(dtype, graph):
     assert float((err ** 2).mean().sqrt()) <= TOL_REAL[dtype][1]
     if graph:
         assert engine.step_fn.graph_replays >= tail - 2
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
+@pytest.mark.parametrize("name", ["B", "R"])
+def test_kept_launch_sequences_change_nothing(name, dtype):
+    """A block's calls into the kernel libraries are written down at its first run for a
+    step of some number of rows and made again from the list afterwards (attention anew each
+    time, from the step's description).  Mixed steps whose row counts repeat with other
+    requests, other lengths and other histories behind them: bit for bit the logits of an
+    engine that runs every part's code every time, and within the bound of plain."""
+    cfg = H.config_of(name)
+    lengths = [150, 41, 97, 260, 33, 120]
+    seqs = {f"r{i}": H.random_ids(cfg, n, 7100 + i) for i, n in enumerate(lengths)}
+    want = {rid: H.plain_logits(name, 1, ids) for rid, ids in seqs.items()}
+    steps = H.steps_mixed(seqs, seed=3, max_live=4, budget=48)
+    steps += H.steps_prefill_then_decode({f"again{i}": ids for i, ids in enumerate(list(seqs.values())[:2])})
+    seqs.update({f"again{i}": ids for i, ids in enumerate(list(seqs.values())[:2])})
+    want.update({f"again{i}": want[f"r{i}"] for i in range(2)})
+    page = 64 if name == "R" else 16
+    runs = {}
+    for keep in (True, False):
+        engine = H.make_engine(name, 1, dtype, page_size=page, num_pages=60, max_requests=4, max_batch_tokens=512)
+        engine.model.keep_launches = keep
+        runs[keep] = H.run_trace(engine, seqs, steps)
+        m = engine.metrics()["launch_sequences"]
+        if keep:
+            assert m["recorded"] > 0 and m["replayed"] > 2 * m["recorded"]
+        else:
+            assert m == {"recorded": 0, "replayed": 0}
+    for rid in seqs:
+        assert torch.equal(runs[True][rid].nan_to_num(7.0), runs[False][rid].nan_to_num(7.0))
+    bad = H.first_wrong(runs[True], want, tolerance(name, dtype))
+    assert bad is None, f"first wrong logits at (request, position, error) = {bad}"
