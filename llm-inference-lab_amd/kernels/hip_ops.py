@@ -397,7 +397,7 @@ class HipOps:
             self._need(rows, "norm row indices", torch.int32)
             if rows.numel() != n_out:
                 raise ValueError("rmsnorm: one row index per output row")
-        pend = (_c_ptr(0), 0, 0)
+        pend = (None, 0, 0)
         if pending is not None:
             p = pending.parts
             if rows is not None or p.shape[1] != n_out or p.shape[2] != hidden or not p[0].is_contiguous():
@@ -491,7 +491,7 @@ class HipOps:
                 raise ValueError(f"pending sums are {p.shape[2]} wide, the rows they belong to {width}")
             pend = (self._ptr(p), pending.splits, p.stride(1), p.stride(0))
         else:
-            pend = (_c_ptr(0), 0, 0, 0)
+            pend = (None, 0, 0, 0)
         if qkv is None:
             heads = _NO_HEADS
         else:
