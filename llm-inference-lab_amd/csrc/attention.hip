@@ -862,7 +862,7 @@ __global__ __launch_bounds__(64 * MERGE_WAVES) void attention_merge_kernel(
 // cache's order) and uses them in four instructions; for the second product the result
 // layout of S^T (lane (c, g): row c, keys 4 g .. 4 g + 3) already is the B operand, and
 // the values of keys 4 g .. 4 g + 3 at number c of a block of d are 16 consecutive bytes.
-// Scores, maxima, exponentials (the library's expf) and sums in float32.
+// Scores, maxima, exponentials and sums in float32.
 //
 // A tile is 16 QB rows ((token, head of the group) pairs of one request and kv head, so the
 // heads of a group share the keys they read).  SPLIT = false: every wave owns a tile and
@@ -892,6 +892,7 @@ __global__ __launch_bounds__(64 * NW) void attention_f32_kernel(AttnArgs a) {
   const float* kc = (const float*)a.kc;
   const float* vc = (const float*)a.vc;
   const int P = a.page_size, pshift = a.page_shift;
+  const float scale2 = a.scale * 1.4426950408889634f;
 
   bool valid[QB];
   int tok[QB], head[QB], pos[QB], lo[QB];
@@ -951,27 +952,33 @@ __global__ __launch_bounds__(64 * NW) void attention_f32_kernel(AttnArgs a) {
 #pragma unroll
         for (int t = 0; t < 4; ++t)
           sc = __builtin_amdgcn_mfma_f32_16x16x4f32(f.k[mb][t], qf[qb][mb][t], sc, 0, 0, 0);
+      // scores in units of the binary exponent (score * scale * log2 e); the exponentials by
+      // the hardware's 2^x (one unit in the last place; a softmax asks no more of them)
       float sv[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int j = kb + g * 4 + i;
         const bool vis = all_visible || (valid[qb] && j <= pos[qb] && j >= lo[qb]);
-        sv[i] = vis ? sc[i] * a.scale : NEG_INF;
+        sv[i] = vis ? sc[i] * scale2 : NEG_INF;
       }
       float mx = fmaxf(fmaxf(sv[0], sv[1]), fmaxf(sv[2], sv[3]));
       mx = max_across_32(mx);
       mx = max_across_16(mx);
       const float m_new = fmaxf(m[qb], mx);
-      // nothing visible so far (m_new = -inf): every weight is 0 and the sums stay 0
-      const float alpha = m_new == NEG_INF ? 1.f : expf(m[qb] - m_new);
+      if (__any(m_new != m[qb])) {        // some row's maximum grew: rescale what is summed so far
+        // (nothing visible yet, m_new = -inf: the sums are 0 and stay 0)
+        const float alpha = m_new == NEG_INF ? 1.f : fast_exp2(m[qb] - m_new);
+        lsum[qb] *= alpha;
+#pragma unroll
+        for (int mb = 0; mb < DQ; ++mb) o[qb][mb] *= alpha;
+        m[qb] = m_new;
+      }
       float pv[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) pv[i] = sv[i] == NEG_INF ? 0.f : expf(sv[i] - m_new);
-      lsum[qb] = lsum[qb] * alpha + ((pv[0] + pv[1]) + (pv[2] + pv[3]));
-      m[qb] = m_new;
+      for (int i = 0; i < 4; ++i) pv[i] = sv[i] == NEG_INF ? 0.f : fast_exp2(sv[i] - m_new);
+      lsum[qb] += (pv[0] + pv[1]) + (pv[2] + pv[3]);
 #pragma unroll
       for (int mb = 0; mb < DQ; ++mb) {
-        o[qb][mb] *= alpha;
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
           // (a position past the last one written holds whatever was there: kept out of
@@ -983,7 +990,7 @@ __global__ __launch_bounds__(64 * NW) void attention_f32_kernel(AttnArgs a) {
     }
   };
 
-  // The next step's keys and values are on their way while this one is multiplied; the
+  // The next steps' keys and values are on their way while this one is multiplied; the
   // loads are unconditional (a load under a branch makes the compiler wait for all loads
   // in flight where the branch ends): a step past the end reads the last one again, a
   // page that is not there reads page 0, and the flag keeps it out of the sums.  The page
@@ -1010,13 +1017,33 @@ __global__ __launch_bounds__(64 * NW) void attention_f32_kernel(AttnArgs a) {
         f.v[mb] = *(const floatx4*)(vp + mb * 256);      // the next 16-wide block of d
       }
     };
-    Step cur, nxt;
-    fetch(cb, cur);
-    for (int blk = cb; blk < ce; ++blk) {
-      fetch(blk + 1, nxt);
+    // a ring of three: two steps are on their way while one is multiplied (a wave's step is
+    // about a microsecond of matrix instructions, a trip to memory takes longer, and a
+    // prompt gives a SIMD fewer than two waves to fill the wait with)
+    if constexpr (SPLIT) {       // (a wave's share of a split history is a few steps: one ahead is enough)
+      Step cur, nxt;
+      fetch(cb, cur);
+      for (int blk = cb; blk < ce; ++blk) {
+        fetch(blk + 1, nxt);
+        __builtin_amdgcn_sched_barrier(0);
+        compute(blk, cur);
+        cur = nxt;
+      }
+      continue;
+    }
+    Step r0, r1, r2;
+    fetch(cb, r0);
+    fetch(cb + 1, r1);
+    for (int blk = cb; blk < ce; blk += 3) {
+      fetch(blk + 2, r2);
       __builtin_amdgcn_sched_barrier(0);
-      compute(blk, cur);
-      cur = nxt;
+      compute(blk, r0);
+      fetch(blk + 3, r0);
+      __builtin_amdgcn_sched_barrier(0);
+      compute(blk + 1, r1);          // (a step past the end carries ok = false)
+      fetch(blk + 4, r1);
+      __builtin_amdgcn_sched_barrier(0);
+      compute(blk + 2, r2);
     }
   }
 
@@ -1058,7 +1085,7 @@ __global__ __launch_bounds__(64 * NW) void attention_f32_kernel(AttnArgs a) {
       float num = 0.f, den = 0.f;
 #pragma unroll
       for (int w = 0; w < NW; ++w) {
-        const float wt = s_m[w][r] == NEG_INF ? 0.f : expf(s_m[w][r] - mmax);
+        const float wt = s_m[w][r] == NEG_INF ? 0.f : exp2f(s_m[w][r] - mmax);
         num += wt * s_o[w][r][dd];
         den += wt * s_l[w][r];
       }
@@ -1066,12 +1093,10 @@ __global__ __launch_bounds__(64 * NW) void attention_f32_kernel(AttnArgs a) {
       if (a.splits == 1) {
         ((float*)a.out)[(size_t)(r0 + t) * a.out_stride + (size_t)hh * D + dd] = den > 0.f ? num / den : 0.f;
       } else {
-        // (the merge kernel weighs the splits by powers of two: the maximum goes there in
-        // units of the binary exponent)
         const size_t at = ((size_t)(r0 + t) * a.nq + hh) * a.splits + split;
         a.o_part[at * D + dd] = num;
         if (dd == 0) {
-          a.ml_part[at * 2] = mmax * 1.4426950408889634f;
+          a.ml_part[at * 2] = mmax;
           a.ml_part[at * 2 + 1] = den;
         }
       }
