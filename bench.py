@@ -172,6 +172,7 @@ def measured_peaks():
     lib.llmlab_measure_read.argtypes = [vp, cs, vp, ci, vp]
     lib.llmlab_measure_copy.argtypes = [vp, vp, cs, ci, vp]
     lib.llmlab_measure_mfma.argtypes = [ci, ci, ci, vp, ctypes.POINTER(ctypes.c_double), vp]
+    lib.llmlab_measure_barrier.argtypes = [ci, ci, vp, vp, ctypes.c_long, vp]
     torch.cuda.set_device(0)
     stream = torch.cuda.current_stream().cuda_stream
     cus = torch.cuda.get_device_properties(0).multi_processor_count
@@ -205,6 +206,16 @@ def measured_peaks():
         t = timed(lambda: lib.llmlab_measure_mfma(f32, cus * 8, iterations, sink.data_ptr(), ctypes.byref(flops),
                                                   stream))
         out[name] = round(flops.value / t / 1e12, 1)
+    # a device-wide barrier inside one kernel: 200 rounds of all compute units meeting at a
+    # counter, against the same launch with one round (the difference is the rounds alone)
+    flags = torch.zeros(2, dtype=torch.int32, device="cuda:0")
+
+    def barriers(rounds):
+        flags.zero_()
+        return lib.llmlab_measure_barrier(cus, rounds, flags.data_ptr(), flags.data_ptr() + 4, 1 << 22, stream)
+    many, one = timed(lambda: barriers(201)), timed(lambda: barriers(1))
+    if int(flags[1]) == 0:
+        out["grid_barrier_us"] = round((many - one) / 200 * 1e6, 2)
     return out
 
 

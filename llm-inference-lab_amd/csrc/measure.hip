@@ -9,6 +9,8 @@
 //   MFMA issue      waves that do nothing but matrix instructions on registers:
 //                   v_mfma_f32_16x16x32_bf16 (the engine's bfloat16 products) and
 //                   v_mfma_f32_32x32x2_f32 (32-bit products and sums)
+//   grid barrier    one block per compute unit, all meeting at a counter in memory again
+//                   and again: what a device-wide barrier inside a kernel would cost
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
@@ -95,7 +97,39 @@ __global__ __launch_bounds__(256) void mfma_f32_kernel(int iterations, float* __
   if (total == 12345.678f) sink[threadIdx.x] = total;
 }
 
+// What a device-wide barrier costs inside one kernel: every block counts itself in with an
+// atomic of device scope and reads the counter (device scope too, so the read passes the L2
+// of its die by) until all have arrived, `rounds` times.  The wait is bounded: a block that
+// has read the counter `spin_limit` times in one round without seeing it full sets `*failed`
+// and leaves, and so, each at its own limit, do the others.  One block per compute unit at
+// most, so that all of them are resident at once.
+__global__ __launch_bounds__(64) void barrier_rounds_kernel(int rounds, int* counter, int* failed,
+                                                            long spin_limit) {
+  if (threadIdx.x != 0) return;
+  for (int r = 0; r < rounds; ++r) {
+    const int full = (r + 1) * (int)gridDim.x;
+    __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    long spins = 0;
+    while (__hip_atomic_load(counter, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < full) {
+      if (++spins > spin_limit) {
+        __hip_atomic_store(failed, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        return;
+      }
+      __builtin_amdgcn_s_sleep(1);
+    }
+  }
+}
+
 static int check_launch() { return hipGetLastError() == hipSuccess ? 0 : 1; }
+
+// counter and failed: two ints that are zero now.  blocks: at most the number of compute units.
+extern "C" int llmlab_measure_barrier(int blocks, int rounds, int* counter, int* failed, long spin_limit,
+                                      hipStream_t stream) {
+  if (counter == nullptr || failed == nullptr || blocks <= 0 || blocks > 1024 || rounds <= 0 || spin_limit < 0)
+    return 1;
+  hipLaunchKernelGGL(barrier_rounds_kernel, dim3(blocks), dim3(64), 0, stream, rounds, counter, failed, spin_limit);
+  return check_launch();
+}
 
 // bytes: a multiple of 16; sink: at least 4 KB.  Reads `bytes` once.
 extern "C" int llmlab_measure_read(const void* src, size_t bytes, void* sink, int blocks, hipStream_t stream) {

@@ -852,3 +852,24 @@ def test_linear_partials_and_pending(ops, emu, m, n, k, splits):
         emu.fused_norm_logits(resid, None, nw, 1e-6, w3, want_l,
                               pending=type(pending)(want_parts, splits))
         close(logits, want_l, torch.float32, "pending under a fused norm", want_l.abs().max().item() * 4)
+
+
+def test_bounded_wait_of_the_measured_grid_barrier_gives_up():
+    """The benchmark's barrier loop (csrc/measure.hip) waits for all blocks at a counter; the
+    wait is bounded.  Told to give up at once (a spin limit of 0) with a counter that can
+    never fill (it starts far below zero), every block sets the flag and leaves; with room to
+    spin and a counter at zero all rounds complete and the flag stays clear."""
+    import ctypes
+    from llm_inference_lab_amd.kernels import build
+    lib = ctypes.CDLL(build.measure_library())
+    lib.llmlab_measure_barrier.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p,
+                                           ctypes.c_long, ctypes.c_void_p]
+    stream = torch.cuda.current_stream(DEV).cuda_stream
+    flags = torch.tensor([-1000000, 0], dtype=torch.int32, device=DEV)
+    assert lib.llmlab_measure_barrier(64, 3, flags.data_ptr(), flags.data_ptr() + 4, 0, stream) == 0
+    torch.cuda.synchronize(DEV)
+    assert flags.cpu().tolist() == [-1000000 + 64, 1]
+    flags = torch.zeros(2, dtype=torch.int32, device=DEV)
+    assert lib.llmlab_measure_barrier(64, 5, flags.data_ptr(), flags.data_ptr() + 4, 1 << 22, stream) == 0
+    torch.cuda.synchronize(DEV)
+    assert flags.cpu().tolist() == [5 * 64, 0]
