@@ -1123,7 +1123,7 @@ extern "C" void llmlab_debug_attention_path(int path) { g_force_path = path; }
 // -1 = the last block whatever the number of splits.
 static int g_force_merge_kernel = 0;
 extern "C" void llmlab_debug_attention_merge_kernel(int on) { g_force_merge_kernel = on; }
-constexpr int MERGE_IN_PLACE_SPLITS = 4;
+constexpr int MERGE_IN_PLACE_SPLITS = 2;
 
 // The decode-like launch: a block of DECODE_WAVES waves per (request, kv head, split); a
 // wave gets about two steps of 32 keys, a block's waves merge in LDS, and only what is
@@ -1159,13 +1159,14 @@ static int launch_key_split_decode(AttnArgs a, int reqs, int live, int ctx_len, 
   while (splits > 1 && per_split * splits > workspace_floats) --splits;
   if (splits < 1) splits = 1;
   a.splits = splits;
-  // Who merges the splits: with few splits the last block of each (request, kv head) to
-  // arrive, if the caller brought counters for them (zero now, zero again afterwards); else
-  // a kernel of its own.  The last block's way is a chain of trips to memory (its stores
+  // Who merges the splits: two splits the last block of each (request, kv head) to arrive,
+  // if the caller brought counters for them (zero now, zero again afterwards); more a
+  // kernel of its own.  The last block's way is a chain of trips to memory (its stores
   // done, the counter, the other blocks' results) of about 2 us each, a kernel boundary
-  // costs less than two of them: measured at the 0.5B shape and context 4096, 64 requests
-  // in 2 splits take 1.743 ms a step against 1.781 with the kernel, 8 requests in 16
-  // splits 1.001 against 0.962.
+  // costs less than two of them: measured at context 4096 of the 0.5B shape, 64 requests in
+  // 2 splits take 1.743 ms a step against 1.781 with the kernel, 8 requests in 16 splits
+  // 1.001 against 0.962; at the 32B shape, 8 requests in 4 splits, 55.4 us a layer against
+  // 47.3 + 4.7.
   const bool merge_in_place = splits > 1 && arrived != nullptr && (size_t)reqs * nkv <= arrived_ints &&
                               g_force_merge_kernel == 0 && (splits <= MERGE_IN_PLACE_SPLITS || g_force_merge_kernel < 0);
   a.arrived = merge_in_place ? arrived : nullptr;
