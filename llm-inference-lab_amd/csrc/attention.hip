@@ -1166,7 +1166,7 @@ static int launch_key_split_decode(AttnArgs a, int reqs, int live, int ctx_len, 
   // costs less than two of them: measured at context 4096 of the 0.5B shape, 64 requests in
   // 2 splits take 1.743 ms a step against 1.781 with the kernel, 8 requests in 16 splits
   // 1.001 against 0.962; at the 32B shape, 8 requests in 4 splits, 55.4 us a layer against
-  // 47.3 + 4.7.
+  // 51.6 + 4.8 (no difference).
   const bool merge_in_place = splits > 1 && arrived != nullptr && (size_t)reqs * nkv <= arrived_ints &&
                               g_force_merge_kernel == 0 && (splits <= MERGE_IN_PLACE_SPLITS || g_force_merge_kernel < 0);
   a.arrived = merge_in_place ? arrived : nullptr;
