@@ -12,7 +12,7 @@ back).  One JSON line is printed: decoded tokens a second as ``value``, plus
 * ``prefill``: one 2,048-token prompt in one step;
 * ``roofline``: bytes the decode step has to read over its time against 8 TB/s;
 * ``points``: decode at batch 1 and 64; the same shape in float32 (``f32_*``); decode at
-  batch 8 at the 7B shape (context 4096) and at the 32B shape (context 8192) with the
+  batch 8 and 1 at the 7B shape (context 4096) and at the 32B shape (context 8192) with the
   fraction of 8 TB/s each reaches, and the ``--mixed`` run at the 7B shape (all tokens a
   second): each of these comes from a child process of its own;
 * ``validation``: before anything is timed, the last-position logits of a 2,048-token
@@ -468,10 +468,12 @@ def side_points(args, measured):
     line = child("--side", "7b", *common)
     if line is not None:
         points["decode_b8_7b"], points["hbm_frac_b8_7b"] = line["decode_b8"], line["hbm_frac_b8"]
+        points["decode_b1_7b"], points["hbm_frac_b1_7b"] = line["decode_b1"], line["hbm_frac_b1"]
         points["mixed_7b_tokens_per_second"] = line["mixed_tokens_per_second"]
     line = child("--side", "32b", *common)
     if line is not None:
         points["decode_b8_32b"], points["hbm_frac_b8_32b"] = line["decode_b8"], line["hbm_frac_b8"]
+        points["decode_b1_32b"], points["hbm_frac_b1_32b"] = line["decode_b1"], line["hbm_frac_b1"]
     line = child("--side", "f32", *common)
     if line is not None:
         for key in ("decode_b1", "decode_b8", "decode_b64", "prefill_tokens_per_second", "prefill_frac"):
@@ -516,6 +518,9 @@ def side_run(args):
     seconds, live, _ = runs.decode_samples(8, args.steps, args.warmup)
     out = {"decode_b8": round(8 * args.steps / seconds, 1),
            "hbm_frac_b8": runs.roofline(seconds, args.steps, live)["frac"]}
+    seconds, live, _ = runs.decode_samples(1, args.steps, args.warmup)      # (a batch of 64 takes too long to fill)
+    out["decode_b1"] = round(args.steps / seconds, 1)
+    out["hbm_frac_b1"] = runs.roofline(seconds, args.steps, live)["frac"]
     if args.shape == "7b":
         out["mixed_tokens_per_second"] = mixed_run(args, cfg, engine)["value"]
     print(json.dumps(out))

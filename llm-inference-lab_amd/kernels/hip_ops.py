@@ -10,6 +10,7 @@ the current PyTorch stream, so they can be captured into a HIP graph.
 from __future__ import annotations
 
 import ctypes
+import dataclasses
 from typing import Dict, Optional
 
 import torch
@@ -329,7 +330,6 @@ class HipOps:
 
     def fingerprint(self):
         """What the host-side choices of the kernel set depend on beside the shapes."""
-        import dataclasses
         return (self.num_cus, self.debug_epoch, dataclasses.astuple(self.rules))
 
     def _check(self, code: int, lib=None) -> None:
