@@ -67,6 +67,7 @@ class CausalLM:
         self.keep_launches = os.environ.get("LLMLAB_KEEP_LAUNCHES", "1") not in ("0", "")
         self.verify_launches = os.environ.get("LLMLAB_VERIFY_LAUNCHES", "") not in ("0", "")
         self._launches: List[Dict[tuple, object]] = [dict() for _ in self.entries]
+        self._launches_version = None      # the scratch buffers' version the kept sequences belong to
         self.launches_recorded = 0
         self.launches_replayed = 0
 
@@ -169,7 +170,7 @@ class CausalLM:
             return self._forward_with_ranges(x, ctx)
         self.embedding.forward(ctx.token_ids, x, ctx)
         if self._launches_usable(ctx):
-            stamp = (ctx.n_rows, ctx.scratch_version, self.ops.fingerprint())
+            stamp = self._launch_stamp(ctx)
             for view in self.entries:
                 self._run_block(self.blocks[view.block], x, ctx, view, stamp)
         else:
@@ -178,6 +179,16 @@ class CausalLM:
         return self._head(x, ctx)
 
     MAX_KEPT_LAUNCHES = 256       # per scheduled run
+
+    def _launch_stamp(self, ctx) -> tuple:
+        """What the kept sequences of this step are filed under, beside the sums owed to the
+        stream.  Sequences written down before a scratch buffer moved hold pointers into
+        (and keep alive) the buffers of before: they are dropped as soon as that shows."""
+        if ctx.scratch_version != self._launches_version:
+            for kept in self._launches:
+                kept.clear()
+            self._launches_version = ctx.scratch_version
+        return (ctx.n_rows, ctx.scratch_version, self.ops.fingerprint())
 
     def _launches_usable(self, ctx) -> bool:
         return (self.keep_launches and hasattr(self.ops, "begin_recording") and hasattr(ctx, "scratch_version")
@@ -247,7 +258,7 @@ class CausalLM:
         with r.range("embedding"):
             self.embedding.forward(ctx.token_ids, x, ctx)
         usable = self._launches_usable(ctx)
-        stamp = (ctx.n_rows, ctx.scratch_version, self.ops.fingerprint()) if usable else None
+        stamp = self._launch_stamp(ctx) if usable else None
         for view in self.entries:
             with r.range(f"block {view.index}"):
                 if usable:

@@ -17,13 +17,110 @@ from llm_inference_lab_amd.cache import layout as cache_layout
 from llm_inference_lab_amd.parts import PendingSums
 
 
+class EmuRecord:
+    """The calls a part made while it was recorded (the counterpart of the product's
+    ``LaunchRecord``): ``(bound method, (args, kwargs), None)`` or ``(None, closure, None)``."""
+
+    def __init__(self, dry=False):
+        self.calls = []
+        self.dry = dry
+
+    @staticmethod
+    def _same(a, b):
+        if isinstance(a, torch.Tensor) or isinstance(b, torch.Tensor):
+            return (isinstance(a, torch.Tensor) and isinstance(b, torch.Tensor) and a.data_ptr() == b.data_ptr()
+                    and a.shape == b.shape and a.stride() == b.stride() and a.dtype == b.dtype)
+        if isinstance(a, PendingSums) or isinstance(b, PendingSums):
+            return (isinstance(a, PendingSums) and isinstance(b, PendingSums) and a.splits == b.splits
+                    and EmuRecord._same(a.parts, b.parts))
+        return a == b
+
+    def same_as(self, other):
+        if len(self.calls) != len(other.calls):
+            return False
+        for (fa, aa, _), (fb, ab, _) in zip(self.calls, other.calls):
+            if (fa is None) != (fb is None):
+                return False
+            if fa is None:
+                continue
+            if fa is not fb or len(aa[0]) != len(ab[0]) or sorted(aa[1]) != sorted(ab[1]):
+                return False
+            if not all(self._same(x, y) for x, y in zip(aa[0], ab[0])):
+                return False
+            if not all(self._same(aa[1][k], ab[1][k]) for k in aa[1]):
+                return False
+        return True
+
+
 class EmuOps:
+    # the operations that do work on tensors: written down while a part is recorded, as the
+    # product's kernel set writes down its calls into the kernel libraries
+    RECORDED = ("embed", "gather_tokens", "rmsnorm", "linear", "linear_residual", "linear_partials",
+                "add_pending", "linear_logits", "linear_swiglu", "fused_norm_qkv", "qkv_rope_cache",
+                "fused_norm_swiglu", "fused_norm_logits", "rope_inplace", "rope_kv_write",
+                "paged_attention", "argmax", "sample")
+
     def __init__(self, device="cpu", fuse=True):
         self.device = torch.device(device)
         self.calls = {}
         self.fuse = fuse
         import types
         self.rules = types.SimpleNamespace(min_steps_per_split=8)
+        self._record = None
+        self._depth = 0
+        for name in self.RECORDED:
+            setattr(self, name, self._recordable(getattr(self, name)))
+
+    # ----------------------------------------------- recorded sequences of calls
+    def _recordable(self, method):
+        def call(*args, **kwargs):
+            record = self._record
+            if record is not None and self._depth == 0:      # (an operation's own inner calls are its business)
+                record.calls.append((call, (args, kwargs), None))
+                if record.dry:      # (nothing is computed; what the caller is handed back all the same)
+                    return PendingSums(args[2], args[3]) if method.__name__ == "linear_partials" else None
+            self._depth += 1
+            try:
+                return method(*args, **kwargs)
+            finally:
+                self._depth -= 1
+        call.inner = method
+        return call
+
+    def begin_recording(self, dry=False):
+        assert self._record is None
+        self._record = EmuRecord(dry)
+        return self._record
+
+    def end_recording(self):
+        record, self._record = self._record, None
+        return record
+
+    def live(self, launch):
+        record = self._record
+        if record is None:
+            launch()
+            return
+        record.calls.append((None, launch, None))
+        if record.dry:
+            return
+        self._record = None
+        try:
+            launch()
+        finally:
+            self._record = record
+
+    def replay(self, record):
+        for fn, args, _ in record.calls:
+            if fn is None:
+                args()
+            else:
+                fn.inner(*args[0], **args[1])
+
+    def fingerprint(self):
+        plain = (int, float, str, bool, type(None))
+        rules = tuple(sorted((k, v if isinstance(v, plain) else id(v)) for k, v in vars(self.rules).items()))
+        return (self.fuse, rules, getattr(self, "num_cus", 0))
 
     def _count(self, name):
         self.calls[name] = self.calls.get(name, 0) + 1

@@ -172,3 +172,32 @@ def test_another_block_arrangement_in_random_weights_mode(tmp_path):
     mode draws its tensors as the parts say, the folder loads, every cut matches."""
     import toy_parallel
     toy_parallel.run("f32", str(tmp_path / "toy4"), ops=EmuOps(), device="cpu")
+
+
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_kept_launch_sequences_over_the_kernel_references(name):
+    """The model writes the calls of a block down at its first run for a step of some number
+    of rows and makes them again from the list afterwards, attention anew each time from the
+    step's description.  Steps of the same row counts with other requests, other lengths and
+    other pages behind them: bit for bit what an engine computes that runs every part's code
+    every time; and every replay is first checked call by call against what the parts would
+    do now (``LLMLAB_VERIFY_LAUNCHES``, set for all tests)."""
+    seqs = sequences_of(name, seed=3)
+    steps = H.steps_mixed(seqs, seed=5, max_live=3) + H.steps_prefill_then_decode(
+        {f"again{i}": ids for i, ids in enumerate(list(seqs.values())[:2])})
+    seqs.update({f"again{i}": ids for i, ids in enumerate(list(seqs.values())[:2])})
+    runs = {}
+    for keep in (True, False):
+        engine = engine_of(name, "bf16", page_size=16, num_pages=24, max_requests=4)
+        assert engine.model.verify_launches
+        engine.model.keep_launches = keep
+        runs[keep] = H.run_trace(engine, seqs, steps)
+        if keep:
+            assert engine.model.launches_recorded > 0
+            assert engine.model.launches_replayed > 2 * engine.model.launches_recorded
+        else:
+            assert engine.model.launches_recorded == engine.model.launches_replayed == 0
+    for rid in seqs:
+        assert torch.equal(runs[True][rid].nan_to_num(7.0), runs[False][rid].nan_to_num(7.0))
+    want = {rid: H.plain_logits(name, 1, ids) for rid, ids in seqs.items()}
+    assert H.first_wrong(runs[True], want, H.TOL["bf16"]) is None
