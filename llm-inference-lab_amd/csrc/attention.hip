@@ -714,8 +714,12 @@ __device__ __forceinline__ void attention_tile(const AttnArgs& a, const int xblk
     }
     __syncthreads();
     if (!s_last) return;
-    // maxima and denominators of all splits of the block's rows, through LDS: [row][split]
-    __shared__ float x_m[16 * MAX_KEY_SPLITS], x_l[16 * MAX_KEY_SPLITS];
+    // maxima and denominators of all splits of the block's rows, through LDS: [row][split];
+    // where the waves' own sums (done with behind the barriers above) leave room, in their place
+    constexpr bool FITS = (size_t)DECODE_WAVES * 16 * D >= (size_t)2 * 16 * MAX_KEY_SPLITS;
+    __shared__ float x_own[FITS ? 1 : 2 * 16 * MAX_KEY_SPLITS];
+    float* x_m = FITS ? &s_o[0][0][0] : x_own;
+    float* x_l = x_m + 16 * MAX_KEY_SPLITS;
     const int S = a.splits;
     for (int i = threadIdx.x; i < nrows * S; i += blockDim.x) {
       const int r = i / S, sidx = i - r * S;
