@@ -271,6 +271,7 @@ class StepFunction:
     """Owns the step's buffers; ``__call__`` runs one step."""
 
     MAX_GRAPHS = 16
+    CAPTURE_AT = 2           # a decode graph is captured when its key comes this many times
 
     def __init__(self, model: CausalLM, cache: CacheManager, ops, max_batch_tokens: int,
                  graph=False):
@@ -291,6 +292,7 @@ class StepFunction:
         self.use_graph = graph if graph == "auto" else bool(graph)
         self.auto_graph = graph == "auto"
         self._graphs: "collections.OrderedDict" = collections.OrderedDict()
+        self._seen: Dict[tuple, int] = {}         # how often a key without a graph has come
         self.graph_replays = 0
         self.graph_captures = 0
         self.graph_evictions = 0
@@ -351,6 +353,15 @@ class StepFunction:
         logits = self.model.forward(ctx)       # this step's result; also sizes every scratch buffer
         if key[2] != ctx.scratch_version:
             return logits                      # buffers moved: capture at the next step
+        # A capture costs milliseconds (a second forward and the making of the graph): it is
+        # made when a key comes the second time.  While requests end one after the other
+        # (the tail of a run) every key comes once or twice, and capturing each made those
+        # steps twice as slow as launching them from the kept sequences.
+        self._seen[key] = self._seen.get(key, 0) + 1
+        if len(self._seen) > 4 * self.MAX_GRAPHS:
+            self._seen.pop(next(iter(self._seen)))
+        if self._seen[key] < self.CAPTURE_AT:
+            return logits
         graph = torch.cuda.CUDAGraph()
         torch.cuda.synchronize(ctx.device)
         with torch.cuda.graph(graph):

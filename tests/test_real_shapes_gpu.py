@@ -136,7 +136,7 @@ def test_steps_of_many_decoding_requests_at_the_widths_of_larger_models(name, gr
         steps += [([(rid, 1, True) for rid in some], []) for _ in range(10)]
         replays = engine.step_fn.graph_replays
         got = H.run_trace(engine, some, steps)
-        if graph:
-            assert engine.step_fn.graph_replays - replays >= 8
+        if graph:       # (a key is captured when it comes the second time, after the buffers have settled)
+            assert engine.step_fn.graph_replays - replays >= 6
         check(name, "bf16", got, want, some)
     engine.cache.check()
