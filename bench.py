@@ -385,7 +385,20 @@ class Runs:
         return result
 
 
-def mixed_run(args, cfg, engine=None):
+def force_what_was_asked(engine, args):
+    """``--force KEY=VALUE``: kernel choices fixed for the whole run."""
+    if not getattr(args, "force", None):
+        return
+    forced = {}
+    for item in args.force:
+        key, _, value = item.partition("=")
+        numbers = [float(v) if "." in v else int(v) for v in value.split(":")]
+        forced[key] = numbers[0] if len(numbers) == 1 else tuple(numbers)
+    engine.forced_for_this_run = engine.ops.debug.force(**forced)    # (kept: it restores when collected)
+    engine.forced_for_this_run.__enter__()
+
+
+def mixed_run(args, cfg, engine=None, bracket=None):
     """Requests with prompts of 128..2048 tokens, all admitted at once; the scheduler cuts
     the prompts into portions under a budget of ``--chunk`` tokens a step, beside one
     token for every request that is decoding.  Timed from the first step to the last."""
@@ -398,6 +411,7 @@ def mixed_run(args, cfg, engine=None):
     if engine is None:
         engine = make_engine(args, cfg, sum(n + args.outputs + PAGE for n in lengths), args.requests,
                              args.chunk + args.requests, longest + PAGE)
+        force_what_was_asked(engine, args)
 
     def one_run():
         sched = engine.scheduler(max_batch_tokens=args.chunk + args.requests)
@@ -416,7 +430,8 @@ def mixed_run(args, cfg, engine=None):
         return seconds, steps
 
     one_run()                                   # warm-up: scratch buffers, graphs, kernel loading
-    timed = sorted(one_run() for _ in range(max(1, getattr(args, "samples", 1))))
+    with bracket or ProfilerBracket(False):
+        timed = sorted(one_run() for _ in range(max(1, getattr(args, "samples", 1))))
     seconds, steps = timed[len(timed) // 2]     # the median run; every run serves fresh requests
     prompt_tokens, new_tokens = sum(lengths), args.requests * args.outputs
     # every prompt token and every generated token but a request's last goes through the model once
@@ -589,21 +604,14 @@ def main():
     layers = args.layers or full_layers
     cfg = lab.Qwen2Config.from_dict(dict(SHAPES[args.shape], num_hidden_layers=layers))
     if args.mixed:
-        print(json.dumps(mixed_run(args, cfg)))
+        print(json.dumps(mixed_run(args, cfg, bracket=bracket)))
         return
     batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
     max_batch = max(batches)
     context = args.context or DEFAULT_CONTEXT[args.shape]
     engine = make_engine(args, cfg, max_batch * (context + PAGE), max_batch, FILL_TOKENS, context + PAGE)
     runs = Runs(engine, cfg, context, args.dtype, args.samples, bracket, measured)
-    if args.force:
-        forced = {}
-        for item in args.force:
-            key, _, value = item.partition("=")
-            numbers = [float(v) if "." in v else int(v) for v in value.split(":")]
-            forced[key] = numbers[0] if len(numbers) == 1 else tuple(numbers)
-        engine.forced_for_this_run = engine.ops.debug.force(**forced)    # (kept: it restores when collected)
-        engine.forced_for_this_run.__enter__()
+    force_what_was_asked(engine, args)
 
     if args.only_prefill:
         if not 0 < args.prefill_tokens <= min(FILL_TOKENS, context):

@@ -1,5 +1,5 @@
-// Matrix products for few rows (M <= 64: decode steps and short portions),
-// bfloat16, gfx950.  At this size a step is bound by launch count and by memory
+// Matrix products for few rows (decode steps and short portions; up to 1,024 rows of
+// a small matrix, in tiles of 16 to 64 rows), bfloat16, gfx950.  At this size a step is bound by launch count and by memory
 // latency, not by arithmetic, so one kernel does what the general path does in
 // three or four:
 //
@@ -488,6 +488,8 @@ static size_t skinny_lds_bytes(int nsb, int kw, int mb, int M, int K, int epi, b
 
 // Most LDS a block may take (a compute unit of gfx950 has 160 KB).
 static const size_t SK_LDS_LIMIT = 152 * 1024;
+// Most rows of a call (tiles of at most 64 rows, a block each per set of columns).
+constexpr int SK_MAX_ROWS = 1024;
 
 template <int MB, int EPI, bool NORM, bool STAGE>
 static int skinny_launch(const SkinnyArgs& a, int blocks, size_t lds, hipStream_t stream) {
@@ -625,7 +627,9 @@ static SkinnyShape skinny_choose(int epilogue, bool norm, int M, int N, int K, i
                                  int ksplit = 1) {
   SkinnyShape best{0, 0, false, 1, 1};
   double best_cost = 1e30;
-  const int mb_max = M <= 16 ? 1 : (M <= 32 ? 2 : 4);
+  // (q/k/v of more than 64 rows: tiles of 16 rows, measured; 576 rows of 1152 x 896 take
+  // 13.4 us so, 16.4 in tiles of 32 and 26 in tiles of 64)
+  const int mb_max = M <= 16 || (epilogue == SK_QKV && M > 64) ? 1 : (M <= 32 ? 2 : 4);
   for (int mb = mb_max; mb >= 1; mb >>= 1) {
     if (g_force_mb > 0 && (g_force_epi < 0 || g_force_epi == epilogue) && mb != g_force_mb &&
         !(g_force_mb > mb_max && mb == mb_max))
@@ -666,7 +670,7 @@ extern "C" int llmlab_skinny_linear(const void* x, int norm, const int* x_rows, 
                                     int num_cus, const float* pend, int pend_splits, int pend_ld,
                                     size_t pend_stride, int ksplit, size_t part_stride,
                                     hipStream_t stream) {
-  LLMLAB_REQUIRE(M >= 0 && M <= 64, "skinny_linear: takes at most 64 rows, got %d", M);
+  LLMLAB_REQUIRE(M >= 0 && M <= SK_MAX_ROWS, "skinny_linear: takes at most %d rows, got %d", SK_MAX_ROWS, M);
   LLMLAB_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "skinny_linear: bad sizes N=%d K=%d (K must be a multiple of 8)", N, K);
   LLMLAB_REQUIRE(epilogue >= 0 && epilogue <= 5, "skinny_linear: unknown epilogue %d", epilogue);
   LLMLAB_REQUIRE(pend_splits >= 0 && (pend_splits == 0 || (pend != nullptr && (norm || epilogue == SK_RESID))),

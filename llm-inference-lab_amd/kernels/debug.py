@@ -29,6 +29,15 @@ class DispatchRules:
     # once per tile of rows, stays below this many bytes in all (else norm + tiled product
     # wins: 64 rows of a 55 MB matrix take 38 us fused, 26 us in two kernels).
     fuse_read_bytes: float = 128e6
+    # Beyond 64 rows the few-row kernels (tiles of 16 rows, a block per tile and set of columns)
+    # still take a product, up to this many rows, while the matrix times the tiles stays below
+    # so many bytes: every tile streams the matrix for itself, and the tiles of a step that run
+    # at the same time miss the caches together.  Measured inside decode steps of 96 to 384
+    # requests: q/k/v and output product of the 0.5B shape (2 MB) gain up to 576 rows (a step of
+    # 96 requests 1.88 -> 1.52 ms, of 256 2.48 -> 2.40), of the 1.5B shape (6 MB) up to 128
+    # rows; 2560 x 2048 (10 MB) at 128 rows takes 23 us so and 17 through pieces.
+    few_rows_max: int = 1024
+    few_rows_read_bytes: float = 64e6
     # From 17 rows on, a matrix of this many bytes that adds into the stream is cut along its
     # inner size by the tiled kernel: the few-row kernel reads it once per tile of 16 rows
     # (64 rows of 3584 x 18944: 89 us against 34; of 1536 x 8960: 25 against 13).

@@ -433,7 +433,7 @@ class HipOps:
         ldo = out.stride(0) if m > 1 else max(out.stride(0), n_out)
         # few rows: the block kernel that splits K inside a block; from 17 rows on only
         # for narrow outputs (the tiled kernel has too few tiles there), measured
-        if x.dtype == torch.bfloat16 and (m <= 16 or (m <= self.skinny_max_rows and n < 8192)):
+        if x.dtype == torch.bfloat16 and (m <= 16 or (n < 8192 and self.few_rows_take(m, n, k))):
             self._skinny(x, False, None, None, 0.0, w, bias, epilogue, out, m, n, k, ldo, n_out,
                          pending=pending)
             return
@@ -461,20 +461,30 @@ class HipOps:
         self._linear(x, w_gate_up, out, None, EPI_SWIGLU, inter)
 
     # ----------------------------------------------- few rows: fused kernels
-    FUSED_MAX_ROWS = 64           # most rows the few-row kernels take at all
-    skinny_max_rows = 64          # plain products up to here may take the few-row kernel
-    fuse_max_rows = 64            # steps up to here may take the fused kernels
+    FUSED_MAX_ROWS = 1024         # most rows the few-row kernels take at all
+    FEW_ROWS = 64                 # up to here a product may take them whatever its matrix
     FUSE_TILE_ROWS = 16           # the few-row kernels cut the rows into tiles of so many
+
+    def few_rows_take(self, rows: int, outer: int, inner: int) -> bool:
+        """Whether a plain product of ``rows`` rows with an ``[outer, inner]`` matrix goes to the
+        few-row kernels: always up to 64 rows; beyond, up to ``rules.few_rows_max`` rows while
+        the matrix, read once per tile of 16 rows, stays below ``rules.few_rows_read_bytes``."""
+        if rows <= self.FEW_ROWS:
+            return True
+        tiles = (rows + self.FUSE_TILE_ROWS - 1) // self.FUSE_TILE_ROWS
+        return (rows <= min(self.rules.few_rows_max, self.FUSED_MAX_ROWS)
+                and 2.0 * outer * inner * tiles < self.rules.few_rows_read_bytes)
     STAGE_BYTES = 118 * 1024      # most LDS the staged rows of a fused kernel may take
 
     def can_fuse(self, rows: int, dtype, inner: int, outer: Optional[int] = None) -> bool:
         """Whether the fused few-row kernels take this step: bfloat16, few rows, a tile
         of rows (``inner`` wide) fits the staging buffer in LDS, and beyond one tile the
         matrix (``outer`` rows) is a small one."""
-        if dtype != torch.bfloat16 or not 0 < rows <= self.fuse_max_rows:
+        if dtype != torch.bfloat16 or not 0 < rows <= min(max(self.FEW_ROWS, self.rules.few_rows_max), self.FUSED_MAX_ROWS):
             return False
         tiles = (rows + self.FUSE_TILE_ROWS - 1) // self.FUSE_TILE_ROWS
-        if tiles > 1 and (outer is None or 2.0 * outer * inner * tiles >= self.rules.fuse_read_bytes):
+        limit = self.rules.fuse_read_bytes if rows <= self.FEW_ROWS else self.rules.few_rows_read_bytes
+        if tiles > 1 and (outer is None or 2.0 * outer * inner * tiles >= limit):
             return False
         return min(rows, self.FUSE_TILE_ROWS) * ((inner + 31) // 32 * 32 + 8) * 2 <= self.STAGE_BYTES
 
@@ -521,7 +531,7 @@ class HipOps:
 
     def pieces_by_tiles(self, rows: int, n: int, k: int) -> bool:
         """Whether a product left in pieces is cut by the tiled kernel (else by the few-row one)."""
-        return rows > self.FUSED_MAX_ROWS or (rows > self.FUSE_TILE_ROWS and 2.0 * n * k >= self.rules.tiled_pieces_bytes)
+        return rows > self.FEW_ROWS or (rows > self.FUSE_TILE_ROWS and 2.0 * n * k >= self.rules.tiled_pieces_bytes)
 
     def split_count(self, rows: int, dtype, n: int, k: int) -> int:
         """Into how many pieces along the inner size a few-row product ``[rows, k] x
@@ -659,6 +669,7 @@ class HipOps:
                           nkv=num_kv_heads, d=head_dim), pending=pending)
 
     QKV_ROPE_MAX_ROWS = 64        # up to here the few-row kernel, beyond it the tiled one
+    QKV_PIECES_MAX_ROWS = 384     # up to here a large matrix may go through pieces along its inner size
 
     def can_fuse_qkv_rope(self, rows: int, dtype, head_dim: int, n: Optional[int] = None,
                           k: Optional[int] = None) -> bool:
@@ -669,8 +680,30 @@ class HipOps:
             return False
         if rows <= self.QKV_ROPE_MAX_ROWS:
             return head_dim <= (128 if rows > 32 else 256)
+        if n is not None and k is not None and (self.few_rows_take(rows, n, k)
+                                                or self._qkv_pieces_plan(rows, n, k) is not None):
+            return True
         return (n is not None and k is not None
                 and self._core.llmlab_linear_tile(rows, n, k, self.num_cus) % head_dim == 0)
+
+    def _qkv_pieces_plan(self, rows: int, n: int, k: int):
+        """``(pieces, tile)`` if q/k/v of these sizes goes through pieces along the inner size
+        (then any head size does: the second kernel rotates whole rows), else None."""
+        if not (self.rules.qkv_pieces_min_rows <= rows <= self.QKV_PIECES_MAX_ROWS and self.pieces_by_tiles(rows, n, k)):
+            return None
+        if rows > self.FEW_ROWS and self.few_rows_take(rows, n, k):
+            return None
+        pieces, tile = self._linear_plan(rows, n, k)
+        if rows > self.FEW_ROWS and k >= 2 * 64 * self.rules.min_tiles_per_split:
+            # (65 to 384 rows: two pieces at least.  4608 x 3584 at 192 / 256 rows: 24 / 31 us
+            # against 33 / 39 whole; 2560 x 2048: 15 / 18.5 against 20.5; the estimate of
+            # the plan, made for products that add into the stream, says one)
+            pieces = max(pieces, 2)
+        if self.rules.forced_tiled_pieces:
+            pieces = max(1, min(self.rules.forced_tiled_pieces, (k + 63) // 64, self.MAX_SPLITS))
+        if pieces > 1 and pieces * rows * n <= self.workspace.numel():
+            return pieces, tile
+        return None
 
     def qkv_rope_cache(self, h, w_qkv, b_qkv, num_heads, num_kv_heads, head_dim, inv_freq, positions,
                        row_req, block_table, page_size, k_cache, v_cache, q_out) -> None:
@@ -684,29 +717,27 @@ class HipOps:
             raise ValueError(f"qkv_rope_cache: {rows} rows of {k}, heads of {head_dim} do not fit")
         self._qkv_checks("qkv_rope_cache", rows, w_qkv, b_qkv, num_heads, num_kv_heads, head_dim,
                          inv_freq, positions, row_req, block_table, page_size, k_cache, v_cache, q_out)
-        if self.rules.qkv_pieces_min_rows <= rows <= self.QKV_ROPE_MAX_ROWS and self.pieces_by_tiles(rows, n, k):
+        plan = self._qkv_pieces_plan(rows, n, k)
+        if plan is not None:
             # some rows of a large matrix: a head per block leaves most of the chip idle, so
             # the product is cut along K by the tiled kernel and a second kernel sums the
             # pieces, rotates and writes the cache (64 rows of 7168 x 5120: 26 us against 52
             # in one kernel, of 4608 x 3584: 19 against 24; the same at 24 rows, slower below)
-            pieces, tile = self._linear_plan(rows, n, k)
-            if self.rules.forced_tiled_pieces:
-                pieces = max(1, min(self.rules.forced_tiled_pieces, (k + 63) // 64, self.MAX_SPLITS))
-            if pieces > 1 and pieces * rows * n <= self.workspace.numel():
-                if b_qkv is not None:
-                    self._need(b_qkv, "bias")
-                parts = self.workspace[:pieces * rows * n].view(pieces, rows, n)
-                self._call(self._core.llmlab_linear_partials,
-                    self._ptr(h), self._ptr(w_qkv), self._ptr(parts), None, 0, rows, n, k, n, pieces,
-                    rows * n, tile, self._stream())
-                self._call(self._core.llmlab_qkv_from_pieces,
-                    self._ptr(parts), pieces, rows * n, n, self._ptr(b_qkv),
-                    _dt(b_qkv) if b_qkv is not None else 0, rows, num_heads, num_kv_heads, head_dim,
-                    self._ptr(inv_freq), self._ptr(positions), self._ptr(row_req), self._ptr(block_table),
-                    block_table.stride(0) if block_table is not None else 0, int(page_size),
-                    self._ptr(k_cache), self._ptr(v_cache), self._ptr(q_out), q_out.stride(0), self._stream())
-                return
-        if rows <= self.QKV_ROPE_MAX_ROWS:
+            pieces, tile = plan
+            if b_qkv is not None:
+                self._need(b_qkv, "bias")
+            parts = self.workspace[:pieces * rows * n].view(pieces, rows, n)
+            self._call(self._core.llmlab_linear_partials,
+                self._ptr(h), self._ptr(w_qkv), self._ptr(parts), None, 0, rows, n, k, n, pieces,
+                rows * n, tile, self._stream())
+            self._call(self._core.llmlab_qkv_from_pieces,
+                self._ptr(parts), pieces, rows * n, n, self._ptr(b_qkv),
+                _dt(b_qkv) if b_qkv is not None else 0, rows, num_heads, num_kv_heads, head_dim,
+                self._ptr(inv_freq), self._ptr(positions), self._ptr(row_req), self._ptr(block_table),
+                block_table.stride(0) if block_table is not None else 0, int(page_size),
+                self._ptr(k_cache), self._ptr(v_cache), self._ptr(q_out), q_out.stride(0), self._stream())
+            return
+        if rows <= self.QKV_ROPE_MAX_ROWS or self.few_rows_take(rows, n, k):
             self._skinny(h, False, None, None, 0.0, w_qkv, b_qkv, EPI_QKV, q_out, rows, n, k,
                          q_out.shape[1], n,
                          dict(inv_freq=inv_freq, positions=positions, row_req=row_req, table=block_table,

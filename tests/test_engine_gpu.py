@@ -65,6 +65,28 @@ def test_layers_of_real_size(dtype, cut):
     assert float((err ** 2).mean().sqrt()) <= TOL_REAL[dtype][1]
 
 
+@pytest.mark.parametrize("name", ["A", "B", "C", "R"])
+@pytest.mark.parametrize("cut", ["whole", "portions", "mixed"])
+def test_steps_of_many_rows_through_the_tiled_kernels(name, cut):
+    """Matrices as small as these keep the few-row kernels up to 1,024 rows of a step; with
+    that rule switched off every step of more than 64 rows takes the tiled kernels, as
+    the steps of a large model do.  Same logits."""
+    if name == "R":
+        cfg = H.config_of("R")
+        seqs = {f"r{i}": H.random_ids(cfg, n, 700 + i) for i, n in enumerate([3, 75, 140, 330])}
+        engine = H.make_engine("R", 1, "bf16", page_size=64, num_pages=12, max_requests=4, max_batch_tokens=512)
+        tol = TOL_REAL["bf16"][0]
+    else:
+        seqs = sequences_of(name)
+        engine = H.make_engine(name, 1, "bf16", page_size=16, num_pages=40, max_requests=4)
+        tol = H.TOL["bf16"]
+    want = {rid: H.plain_logits(name, 1, ids) for rid, ids in seqs.items()}
+    with engine.ops.debug.force(few_rows_max=64):
+        got = H.run_trace(engine, seqs, CUTS[cut](seqs))
+    bad = H.first_wrong(got, want, tol)
+    assert bad is None, f"first wrong logits at (request, position, error) = {bad}"
+
+
 @pytest.mark.parametrize("name", ["A", "B", "C"])
 @pytest.mark.parametrize("cut", ["decode", "portions", "mixed"])
 def test_sums_left_in_pieces_reach_every_reader(name, cut):

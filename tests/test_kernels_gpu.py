@@ -165,7 +165,7 @@ def test_every_tile_shape_of_the_tiled_products(ops, emu, tile, m, n, k):
     in all three dimensions (the chooser would pick only one of them per size)."""
     from llm_inference_lab_amd.parts.feed_forward import interleave_gate_up
     bf = torch.bfloat16
-    with ops.debug.force(gemm_tile=tile):
+    with ops.debug.force(gemm_tile=tile, few_rows_max=64):        # (small matrices: the few-row kernels would take them)
         x, w, bias = rnd((m, k), bf, 5), rnd((n, k), bf, 6, 0.1), rnd((n,), torch.float32, 7)
         pw = ops.prepare_weight(w.to(DEV))
         want = torch.empty(m, n, dtype=bf)
@@ -259,6 +259,52 @@ def test_few_row_products(ops, emu, m, n, k):
     close(got, want, torch.float32, "few-row residual", want.abs().max().item() * 4)
 
 
+@pytest.mark.parametrize("m", [65, 100, 333, 1024])
+@pytest.mark.parametrize("n,k,inter,vocab", [(896, 896, 320, 515), (90, 96, 128, 256), (65, 104, 72, 301)])
+def test_few_row_kernels_beyond_64_rows(ops, emu, m, n, k, inter, vocab):
+    """Small matrices keep the few-row kernels beyond 64 rows, in tiles of 16 rows that
+    separate blocks take (up to 1,024 rows; the rule that stops earlier for larger
+    matrices is taken away here): every epilogue, with and without the fused norm, rows
+    gathered for the logits among them."""
+    from llm_inference_lab_amd.parts.feed_forward import interleave_gate_up
+    bf = torch.bfloat16
+    with ops.debug.force(few_rows_read_bytes=1e15):
+        assert ops.few_rows_take(m, n, k) and ops.can_fuse(m, bf, k, max(n, 2 * inter, vocab))
+        x, w, bias = rnd((m, k), bf, 40), rnd((n, k), bf, 41, 0.05), rnd((n,), torch.float32, 42)
+        gu = interleave_gate_up(rnd((inter, k), bf, 52, 0.1), rnd((inter, k), bf, 53, 0.1))
+        head = rnd((vocab, k), bf, 54, 0.1)
+        pw, pgu, phead = (ops.prepare_weight(t.to(DEV)) for t in (w, gu, head))
+        calls = ops.calls_made
+        want = torch.empty(m, n, dtype=bf)
+        emu.linear(x, w, want, bias)
+        got = torch.empty(m, n, dtype=bf, device=DEV)
+        ops.linear(x.to(DEV), pw, got, bias.to(DEV))
+        close(got, want, bf, "linear", want.float().abs().max().item())
+        resid = rnd((m, n), torch.float32, 43)
+        want = resid.clone()
+        emu.linear_residual(x, w, want)
+        got = resid.clone().to(DEV)
+        ops.linear_residual(x.to(DEV), pw, got)
+        close(got, want, torch.float32, "residual", want.abs().max().item() * 4)
+        xs = rnd((m + 5, k), torch.float32, 50, 3.0)
+        nw = (1 + 0.1 * rnd((k,), torch.float32, 51)).to(bf)
+        want = torch.empty(m, inter, dtype=bf)
+        emu.fused_norm_swiglu(xs[:m], nw, 1e-5, gu, want)
+        got = torch.empty(m, inter, dtype=bf, device=DEV)
+        ops.fused_norm_swiglu(xs[:m].contiguous().to(DEV), nw.to(DEV), 1e-5, pgu, got)
+        close(got, want, bf, "fused norm + swiglu", want.float().abs().max().item())
+        idx = torch.randperm(m + 5, generator=torch.Generator().manual_seed(55))[:m].int()
+        want = torch.empty(m, vocab)
+        emu.fused_norm_logits(xs, idx, nw, 1e-5, head, want)
+        got = torch.empty(m, vocab, device=DEV)
+        ops.fused_norm_logits(xs.to(DEV), idx.to(DEV), nw.to(DEV), 1e-5, phead, got)
+        close(got, want, torch.float32, "fused norm + logits", want.abs().max().item() * 40)
+        assert ops.calls_made - calls == 4          # one kernel each
+    with pytest.raises(ValueError):
+        ops.fused_norm_swiglu(torch.zeros(1025, k, device=DEV), nw.to(DEV), 1e-5, pgu,
+                              torch.empty(1025, inter, dtype=bf, device=DEV))
+
+
 @pytest.mark.parametrize("mb", [1, 2, 4])
 @pytest.mark.parametrize("stage", [0, 1])
 @pytest.mark.parametrize("nsb,kw", [(1, 1), (1, 4), (1, 16), (2, 2), (2, 8), (4, 1), (4, 4), (8, 2), (16, 1)])
@@ -334,10 +380,13 @@ def test_fused_norm_products(ops, emu, wdtype, m, hidden, inter, vocab):
 
 @pytest.mark.parametrize("nq,nkv,d,page,hidden", [(4, 2, 16, 16, 64), (3, 1, 32, 32, 96), (14, 2, 64, 64, 896),
                                                  (6, 3, 48, 16, 72), (8, 8, 128, 64, 256), (2, 1, 256, 16, 64)])
-@pytest.mark.parametrize("rotate,rows_per", [(True, [5, 1, 9]), (False, [5, 1, 9]), (True, [17, 30, 16])])
+@pytest.mark.parametrize("rotate,rows_per", [(True, [5, 1, 9]), (False, [5, 1, 9]), (True, [17, 30, 16]),
+                                             (True, [70, 1, 130]), (True, [300, 90, 2])])
 def test_fused_norm_qkv_rope_write(ops, emu, nq, nkv, d, page, hidden, rotate, rows_per):
     bf = torch.bfloat16
-    starts, reqs, num_pages = [3, 40, 0], 3, 16
+    starts, reqs = [3, 40, 0], 3
+    needs = [(s0 + c + page - 1) // page for s0, c in zip(starts, rows_per)]
+    num_pages = 16 + sum(needs)
     rows = sum(rows_per)
     x = rnd((rows, hidden), torch.float32, 60, 2.0)
     nw = (1 + 0.1 * rnd((hidden,), torch.float32, 61)).to(bf)
@@ -345,7 +394,7 @@ def test_fused_norm_qkv_rope_write(ops, emu, nq, nkv, d, page, hidden, rotate, r
     w, b = rnd((n, hidden), bf, 62, 0.2), rnd((n,), bf, 63)
     positions = torch.cat([torch.arange(s, s + c) for s, c in zip(starts, rows_per)]).int()
     row_req = torch.cat([torch.full((c,), i) for i, c in enumerate(rows_per)]).int()
-    table = torch.full((reqs, 8), -1, dtype=torch.int32)
+    table = torch.full((reqs, max(8, max(needs))), -1, dtype=torch.int32)
     perm = torch.randperm(num_pages, generator=torch.Generator().manual_seed(64)).int()
     at = 0
     for i in range(reqs):
@@ -371,10 +420,15 @@ def test_fused_norm_qkv_rope_write(ops, emu, nq, nkv, d, page, hidden, rotate, r
 
 @pytest.mark.parametrize("nq,nkv,d,page,hidden", [(4, 2, 16, 16, 64), (14, 2, 64, 64, 896), (6, 3, 48, 16, 72),
                                                  (8, 8, 128, 64, 256), (2, 1, 256, 16, 64)])
-@pytest.mark.parametrize("rows_per", [[5, 1, 9], [20, 1, 1, 3], [17, 30, 16], [70, 1, 130], [300, 2, 2, 90]])
-def test_qkv_rope_cache_of_normed_rows(ops, emu, nq, nkv, d, page, hidden, rows_per):
+@pytest.mark.parametrize("rows_per,few_rows_max", [([5, 1, 9], 64), ([20, 1, 1, 3], 64), ([17, 30, 16], 64),
+                                                   ([70, 1, 130], 64), ([300, 2, 2, 90], 64),
+                                                   ([70, 1, 130], 1024), ([300, 2, 2, 90], 1024), ([1000, 24], 1024)])
+def test_qkv_rope_cache_of_normed_rows(ops, emu, nq, nkv, d, page, hidden, rows_per, few_rows_max):
+    """Up to 64 rows the few-row kernel; more rows the tiled kernel with rotation and cache
+    write in its epilogue, or (matrices as small as these, unless the rule is switched off)
+    the few-row kernel again in tiles of 16 rows."""
     # (heads of 128: the large tile, which this few rows would not get)
-    with ops.debug.force(gemm_tile=128 if d == 128 and sum(rows_per) > 64 else 0):
+    with ops.debug.force(gemm_tile=128 if d == 128 and sum(rows_per) > 64 else 0, few_rows_max=few_rows_max):
         check_qkv_rope_cache(ops, emu, nq, nkv, d, page, hidden, rows_per)
 
 
@@ -385,7 +439,7 @@ def test_qkv_rope_cache_of_normed_rows(ops, emu, nq, nkv, d, page, hidden, rows_
 def test_qkv_rope_cache_with_the_widest_tiles(ops, emu, nq, nkv, d, page, hidden, rows_per, tile):
     """The tiles of 256 columns and eight waves, which only large products get by
     themselves: heads of every size that divides them, a head of 256 among them."""
-    with ops.debug.force(gemm_tile=tile):
+    with ops.debug.force(gemm_tile=tile, few_rows_max=64):
         assert ops.can_fuse_qkv_rope(sum(rows_per), torch.bfloat16, d, (nq + 2 * nkv) * d, hidden)
         check_qkv_rope_cache(ops, emu, nq, nkv, d, page, hidden, rows_per)
 
@@ -458,7 +512,7 @@ def test_values_of_four_positions_written_together(ops, emu, nq, nkv, d, page, h
     to their page as one piece of 32 bytes per four numbers of a head, others number by number:
     requests whose rows and positions line up so (a prompt from its start, a portion that starts
     at a multiple of four), requests that do not, and short requests between them."""
-    with ops.debug.force(gemm_tile=tile):
+    with ops.debug.force(gemm_tile=tile, few_rows_max=64):
         check_qkv_rope_cache(ops, emu, nq, nkv, d, page, hidden, rows_per, starts)
 
 

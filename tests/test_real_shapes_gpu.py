@@ -73,12 +73,13 @@ def assert_large_matrix_rules_fire(ops, cfg):
     assert ops.split_count(8, bf, h, inter) == {3584: 1, 5120: 3}[h]
     # ... the fused norm + product kernels stop at one tile of rows ...
     assert ops.can_fuse(8, bf, h, qkv) and not ops.can_fuse(26, bf, h, 2 * inter) and not ops.can_fuse(64, bf, h, qkv)
-    # ... q/k/v of 24 to 64 rows goes through pieces, of more rows through the tiled epilogue
+    # ... q/k/v of 24 to 384 rows goes through pieces (two at least beyond 64 rows), of more
+    # rows through the tiled epilogue, and never through the few-row kernels beyond 64 rows
     assert ops.rules.qkv_pieces_min_rows <= 26 <= ops.QKV_ROPE_MAX_ROWS and ops.pieces_by_tiles(26, qkv, h)
     assert ops._linear_plan(26, qkv, h)[0] > 1 and ops._linear_plan(64, qkv, h)[0] > 1
-    # (a head of 128 needs the 128-wide tile for that; steps whose product gets the 64-wide
-    # one take the product, then the kernel that rotates and writes the cache)
-    assert ops.can_fuse_qkv_rope(512, bf, cfg.head_dim, qkv, h) and not ops.can_fuse_qkv_rope(140, bf, cfg.head_dim, qkv, h)
+    assert ops._qkv_pieces_plan(140, qkv, h) is not None and ops._qkv_pieces_plan(256, qkv, h)[0] >= 2
+    assert ops._qkv_pieces_plan(512, qkv, h) is None and not ops.few_rows_take(140, qkv, h)
+    assert ops.can_fuse_qkv_rope(512, bf, cfg.head_dim, qkv, h) and ops.can_fuse_qkv_rope(140, bf, cfg.head_dim, qkv, h)
     # ... and pieces of many rows are too large for a fused kernel to read in every block
     from llm_inference_lab_amd.parts import PendingSums
     pieces = PendingSums(torch.empty((ops.split_count(64, bf, h, inter), 64, h), device="meta"),
