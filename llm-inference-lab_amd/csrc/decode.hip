@@ -53,6 +53,8 @@
 // k = 8*(l/16)..+7; result element i: row 4*(l/16)+i, column l%16.
 #include <stdlib.h>
 
+#include <type_traits>
+
 #include "common.h"
 
 enum { SK_STORE = 0, SK_RESID = 1, SK_F32 = 2, SK_SWIGLU = 3, SK_QKV = 4, SK_PART = 5 };
@@ -102,6 +104,7 @@ __host__ __device__ constexpr int sk_ring(int mb, bool stage) {
   return stage ? SK_RING_STAGE : (mb >= 4 ? SK_RING_DIRECT / 2 : SK_RING_DIRECT);
 }
 
+constexpr int SK_STAGE_U_PIECES = 1;
 constexpr int SK_APAD = 8;   // padding of a staged row, in elements: 16-byte reads of 8 lanes cover all banks
 
 // floats of LDS before the staged rows (host and device must agree)
@@ -248,67 +251,112 @@ __global__ __launch_bounds__(MB >= 4 ? 512 : 1024) void skinny_block_kernel(Skin
     const int chunks = K >> 3, chunks_pad = steps * 4;
     int wpr = 1;
     while (2 * wpr * M <= nwaves) wpr *= 2;
-    for (int unit = wave; unit < M * wpr; unit += nwaves) {
-      const int r = unit / wpr, sub = unit - r * wpr;
-      bf16_t* dst = As + (size_t)r * lda;
-      if constexpr (NORM) {
-        const float* src = (const float*)a.x + (size_t)(a.x_rows ? a.x_rows[r] : r) * K;
-        float ssq = 0.f;
-        const size_t prow = (size_t)(a.x_rows ? a.x_rows[r] : r) * a.pend_ld;
-        for (int ch = sub * 64 + lane; ch < chunks; ch += 64 * wpr) {
-          floatx4 p = *(const floatx4*)(src + ch * 8), q = *(const floatx4*)(src + ch * 8 + 4);
-          // sums still owed to these rows: four pieces at a time, loads unconditional
-          // (past the last piece: the last one again, not added) so that they travel together
-          for (int sp0 = 0; sp0 < a.pend_splits; sp0 += 4) {
-            floatx4 pp[4], qq[4];
+    // A wave walks its part of a row U chunks at a time: the loads of all U (the row, the
+    // norm's weight, the pieces owed) are on their way before the first is used, so a part
+    // costs one trip to memory per U chunks and not one per chunk.  Loads are unconditional
+    // (a chunk past the end reads the last one again and is not stored).
+    auto stage_rows = [&](auto u_tag, auto w_tag) {
+      constexpr int U = decltype(u_tag)::value;
+      constexpr bool W_BF16 = decltype(w_tag)::value;     // (the norm's weight: no branch among the loads)
+      const int stride = 64 * wpr;
+      for (int unit = wave; unit < M * wpr; unit += nwaves) {
+        const int r = unit / wpr, sub = unit - r * wpr;
+        bf16_t* dst = As + (size_t)r * lda;
+        if constexpr (NORM) {
+          const float* src = (const float*)a.x + (size_t)(a.x_rows ? a.x_rows[r] : r) * K;
+          float ssq = 0.f;
+          const size_t prow = (size_t)(a.x_rows ? a.x_rows[r] : r) * a.pend_ld;
+          for (int ch0 = sub * 64 + lane; ch0 < chunks; ch0 += U * stride) {
+            floatx4 p[U], q[U], w0[U], w1[U];
+            bf16x8 w8[U];
+            int chs[U];
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              const float* src2 = a.pend + min(sp0 + j, a.pend_splits - 1) * a.pend_stride + prow + ch * 8;
-              pp[j] = *(const floatx4*)src2;
-              qq[j] = *(const floatx4*)(src2 + 4);
+            for (int u = 0; u < U; ++u) {
+              chs[u] = min(ch0 + u * stride, chunks - 1);
+              p[u] = *(const floatx4*)(src + chs[u] * 8);
+              q[u] = *(const floatx4*)(src + chs[u] * 8 + 4);
+              if constexpr (W_BF16) {
+                w8[u] = *(const bf16x8*)((const bf16_t*)a.norm_w + chs[u] * 8);
+              } else {
+                w0[u] = *(const floatx4*)((const float*)a.norm_w + chs[u] * 8);
+                w1[u] = *(const floatx4*)((const float*)a.norm_w + chs[u] * 8 + 4);
+              }
+            }
+            // sums still owed to these rows: four pieces at a time for every chunk, loads
+            // unconditional (past the last piece: the last one again, not added)
+            for (int sp0 = 0; sp0 < a.pend_splits; sp0 += 4) {
+              floatx4 pp[U][4], qq[U][4];
+#pragma unroll
+              for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                  const float* src2 = a.pend + min(sp0 + j, a.pend_splits - 1) * a.pend_stride + prow + chs[u] * 8;
+                  pp[u][j] = *(const floatx4*)src2;
+                  qq[u][j] = *(const floatx4*)(src2 + 4);
+                }
+#pragma unroll
+              for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                  const float on = sp0 + j < a.pend_splits ? 1.f : 0.f;
+                  p[u] += pp[u][j] * on;
+                  q[u] += qq[u][j] * on;
+                }
             }
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              const float on = sp0 + j < a.pend_splits ? 1.f : 0.f;
-              p += pp[j] * on;
-              q += qq[j] * on;
+            for (int u = 0; u < U; ++u) {
+              if (ch0 + u * stride >= chunks) break;
+              float wv[8];
+              if constexpr (W_BF16) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) wv[j] = (float)w8[u][j];
+              } else {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                  wv[j] = w0[u][j];
+                  wv[4 + j] = w1[u][j];
+                }
+              }
+              bf16x8 av;
+#pragma unroll
+              for (int j = 0; j < 4; ++j) {
+                ssq += p[u][j] * p[u][j] + q[u][j] * q[u][j];
+                av[j] = (bf16_t)(p[u][j] * wv[j]);
+                av[4 + j] = (bf16_t)(q[u][j] * wv[4 + j]);
+              }
+              *(bf16x8*)(dst + chs[u] * 8) = av;
             }
           }
-          float wv[8];
-          if (a.norm_w_bf16) {
-            const bf16x8 w8 = *(const bf16x8*)((const bf16_t*)a.norm_w + ch * 8);
-#pragma unroll
-            for (int j = 0; j < 8; ++j) wv[j] = (float)w8[j];
-          } else {
-            const floatx4 w0 = *(const floatx4*)((const float*)a.norm_w + ch * 8);
-            const floatx4 w1 = *(const floatx4*)((const float*)a.norm_w + ch * 8 + 4);
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-              wv[j] = w0[j];
-              wv[4 + j] = w1[j];
-            }
+          ssq = wave_sum(ssq);
+          if (lane == 0) {
+            if (wpr == 1) inv[r] = rsqrtf(ssq / (float)K + a.eps);
+            else s_ssq[unit] = ssq;       // (M * wpr <= 16 waves)
           }
-          bf16x8 av;
+        } else {
+          const bf16_t* src = (const bf16_t*)a.x + (size_t)r * K;
+          for (int ch0 = sub * 64 + lane; ch0 < chunks; ch0 += U * stride) {
+            bf16x8 v[U];
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            ssq += p[j] * p[j] + q[j] * q[j];
-            av[j] = (bf16_t)(p[j] * wv[j]);
-            av[4 + j] = (bf16_t)(q[j] * wv[4 + j]);
+            for (int u = 0; u < U; ++u) v[u] = *(const bf16x8*)(src + min(ch0 + u * stride, chunks - 1) * 8);
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+              if (ch0 + u * stride < chunks) *(bf16x8*)(dst + (ch0 + u * stride) * 8) = v[u];
           }
-          *(bf16x8*)(dst + ch * 8) = av;
         }
-        ssq = wave_sum(ssq);
-        if (lane == 0) {
-          if (wpr == 1) inv[r] = rsqrtf(ssq / (float)K + a.eps);
-          else s_ssq[unit] = ssq;       // (M * wpr <= 16 waves)
-        }
-      } else {
-        const bf16_t* src = (const bf16_t*)a.x + (size_t)r * K;
-        for (int ch = sub * 64 + lane; ch < chunks; ch += 64 * wpr)
-          *(bf16x8*)(dst + ch * 8) = *(const bf16x8*)(src + ch * 8);
+        if (sub == 0)
+          for (int ch = chunks + lane; ch < chunks_pad; ch += 64) *(bf16x8*)(dst + ch * 8) = zero;
       }
-      if (sub == 0)
-        for (int ch = chunks + lane; ch < chunks_pad; ch += 64) *(bf16x8*)(dst + ch * 8) = zero;
+    };
+    // (with pieces owed, two chunks' loads are as many registers as four without)
+    using two = std::integral_constant<int, SK_STAGE_U_PIECES>;
+    using four = std::integral_constant<int, 4>;
+    if (NORM && a.pend_splits > 0) {
+      if (a.norm_w_bf16) stage_rows(two{}, std::true_type{});
+      else stage_rows(two{}, std::false_type{});
+    } else if (NORM && !a.norm_w_bf16) {
+      stage_rows(four{}, std::false_type{});
+    } else {
+      stage_rows(four{}, std::true_type{});
     }
     __syncthreads();
     if constexpr (NORM) {
