@@ -110,10 +110,14 @@ def make_engine(args, cfg, max_cache_tokens, max_requests, max_batch_tokens, max
     if args.shape != "0.5b" and args.dtype == "bf16":
         expected = CausalLM(get_architecture(cfg.architecture).build_spec(cfg)).tensor_specs()
         tensors = random_weights_on_the_gpu(expected, 0)
-    return lab.Engine(config=cfg, seed=0, tensors=tensors, dtype=args.dtype, device="cuda:0", page_size=PAGE,
-                      max_cache_tokens=max_cache_tokens, max_requests=max_requests,
-                      max_batch_tokens=max_batch_tokens, max_seq_len=max_seq_len,
-                      graph=False if args.no_graph else args.graph)
+    engine = lab.Engine(config=cfg, seed=0, tensors=tensors, dtype=args.dtype, device="cuda:0", page_size=PAGE,
+                        max_cache_tokens=max_cache_tokens, max_requests=max_requests,
+                        max_batch_tokens=max_batch_tokens, max_seq_len=max_seq_len,
+                        graph=False if args.no_graph else args.graph)
+    del tensors
+    from llm_inference_lab_amd.engine import settle_collector
+    settle_collector()      # (as a serving process does: full collections cost 35 to 70 ms otherwise)
+    return engine
 
 
 class ProfilerBracket:

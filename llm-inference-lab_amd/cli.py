@@ -65,6 +65,7 @@ def main(argv: Optional[List[str]] = None) -> int:
         print("--max-new-tokens must be positive", file=sys.stderr)
         return 2
     from . import Engine, write_random_model
+    from .engine import settle_collector
     from .config.registry import architecture_of, read_config
     from .engine.step import StepEntry
 
@@ -114,6 +115,7 @@ def main(argv: Optional[List[str]] = None) -> int:
                     max_batch_tokens=args.max_batch_tokens,
                     max_seq_len=longest, graph=args.graph)
     load_seconds = time.perf_counter() - load_start
+    settle_collector()
 
     def trace(event):
         print(json.dumps(event), file=sys.stderr, flush=True)

@@ -32,11 +32,13 @@ class DispatchRules:
     # Beyond 64 rows the few-row kernels (tiles of 16 rows, a block per tile and set of columns)
     # still take a product, up to this many rows, while the matrix times the tiles stays below
     # so many bytes: every tile streams the matrix for itself, and the tiles of a step that run
-    # at the same time miss the caches together.  Measured inside decode steps of 96 to 384
-    # requests: q/k/v and output product of the 0.5B shape (2 MB) gain up to 576 rows (a step of
-    # 96 requests 1.88 -> 1.52 ms, of 256 2.48 -> 2.40), of the 1.5B shape (6 MB) up to 128
-    # rows; 2560 x 2048 (10 MB) at 128 rows takes 23 us so and 17 through pieces.
-    few_rows_max: int = 1024
+    # at the same time miss the caches together.  Measured inside decode steps of 96 / 128 /
+    # 192 / 256 / 320 requests of the 0.5B shape (q/k/v and output product, 2 MB each): 1.88 ->
+    # 1.64, 1.98 -> 1.76, 2.23 -> 2.14, 2.48 -> 2.41 ms, no difference from 320 on; of the 1.5B
+    # shape (6 MB) 3.04 -> 2.80 and 3.29 -> 3.06 at 96 and 128; 2560 x 2048 (10 MB) at 128 rows
+    # takes 23 us so and 17 through pieces.  Steps of 512-token portions beside decoding
+    # requests lose 7 % with a limit of 1024 rows and nothing with 256.
+    few_rows_max: int = 256
     few_rows_read_bytes: float = 64e6
     # From 17 rows on, a matrix of this many bytes that adds into the stream is cut along its
     # inner size by the tiled kernel: the few-row kernel reads it once per tile of 16 rows

@@ -268,7 +268,7 @@ def test_few_row_kernels_beyond_64_rows(ops, emu, m, n, k, inter, vocab):
     gathered for the logits among them."""
     from llm_inference_lab_amd.parts.feed_forward import interleave_gate_up
     bf = torch.bfloat16
-    with ops.debug.force(few_rows_read_bytes=1e15):
+    with ops.debug.force(few_rows_read_bytes=1e15, few_rows_max=1024):
         assert ops.few_rows_take(m, n, k) and ops.can_fuse(m, bf, k, max(n, 2 * inter, vocab))
         x, w, bias = rnd((m, k), bf, 40), rnd((n, k), bf, 41, 0.05), rnd((n,), torch.float32, 42)
         gu = interleave_gate_up(rnd((inter, k), bf, 52, 0.1), rnd((inter, k), bf, 53, 0.1))
