@@ -11,7 +11,7 @@ back).  One JSON line is printed: decoded tokens a second as ``value``, plus
 
 * ``prefill``: one 2,048-token prompt in one step;
 * ``roofline``: bytes the decode step has to read over its time against 8 TB/s;
-* ``points``: decode at batch 1 and 64; the same shape in float32 (``f32_*``); decode at
+* ``points``: decode at batch 1, 64 and 128; the same shape in float32 (``f32_*``); decode at
   batch 8 and 1 at the 7B shape (context 4096) and at the 32B shape (context 8192) with the
   fraction of 8 TB/s each reaches, and the ``--mixed`` run at the 7B shape (all tokens a
   second): each of these comes from a child process of its own;
@@ -610,7 +610,7 @@ def main():
     if args.mixed:
         print(json.dumps(mixed_run(args, cfg, bracket=bracket)))
         return
-    batches = [args.batch] if args.no_points else sorted({1, args.batch, 64})
+    batches = [args.batch] if args.no_points else sorted({1, args.batch, 64, 128})
     max_batch = max(batches)
     context = args.context or DEFAULT_CONTEXT[args.shape]
     engine = make_engine(args, cfg, max_batch * (context + PAGE), max_batch, FILL_TOKENS, context + PAGE)
@@ -656,7 +656,7 @@ def main():
         result["prefill"] = runs.prefill()
         points = {}
         half_steps, half_warmup = max(8, args.steps // 2), max(2, args.warmup // 2)
-        for b in (1, 64):
+        for b in (1, 64, 128):
             if b == args.batch:
                 points[f"decode_b{b}"] = round(value, 1)
                 continue
