@@ -102,6 +102,17 @@ def random_weights_on_the_gpu(expected, seed):
     return random_tensors(expected, seed, torch.bfloat16, device="cuda:0")
 
 
+def fits_the_gpu(cfg, batch, context, dtype, gpu_bytes=288e9, share=0.8):
+    """Whether the weights and the cache pages of ``batch`` requests of ``context`` tokens leave
+    a fifth of the GPU's memory to scratch buffers and the allocator."""
+    width = 2 if dtype == "bf16" else 4
+    h, i, v = cfg.hidden_size, cfg.intermediate_size, cfg.vocab_size
+    q, kv = cfg.num_attention_heads * cfg.head_dim, cfg.num_key_value_heads * cfg.head_dim
+    weights = cfg.num_hidden_layers * (h * (q + 2 * kv) + q * h + 3 * h * i) + (1 if cfg.tie_word_embeddings else 2) * h * v
+    cache = batch * (context + PAGE) * cfg.num_hidden_layers * 2 * kv
+    return (weights + cache) * width <= share * gpu_bytes
+
+
 def make_engine(args, cfg, max_cache_tokens, max_requests, max_batch_tokens, max_seq_len):
     import llm_inference_lab_amd as lab
     from llm_inference_lab_amd.config import get_architecture
@@ -234,6 +245,7 @@ class Runs:
         self.samples = max(1, int(samples))
         self.bracket = bracket or ProfilerBracket(False)
         self.measured = measured or {}
+        self.settled = set()
 
     def random_ids(self, n):
         return self.torch.randint(0, self.cfg.vocab_size, (n,), generator=self.gen).tolist()
@@ -263,6 +275,10 @@ class Runs:
             sched.step()                      # prefill in portions; ends with every request decoding
         for _ in range(warmup):
             sched.step()
+        if batch not in self.settled:       # (the launch sequences of this batch are kept by now)
+            from llm_inference_lab_amd.engine import settle_collector
+            settle_collector()
+            self.settled.add(batch)
         assert len(sched.active) == batch
         live_tokens = sum(r.computed for r in sched.active)
         self.sync()
@@ -611,8 +627,10 @@ def main():
         print(json.dumps(mixed_run(args, cfg, bracket=bracket)))
         return
     batches = [args.batch] if args.no_points else sorted({1, args.batch, 64, 128})
-    max_batch = max(batches)
     context = args.context or DEFAULT_CONTEXT[args.shape]
+    if not args.no_points and args.batch < 128 and not fits_the_gpu(cfg, 128, context, args.dtype):
+        batches.remove(128)             # (the 32B and 72B shapes: weights and the cache of 128 requests exceed the GPU)
+    max_batch = max(batches)
     engine = make_engine(args, cfg, max_batch * (context + PAGE), max_batch, FILL_TOKENS, context + PAGE)
     runs = Runs(engine, cfg, context, args.dtype, args.samples, bracket, measured)
     force_what_was_asked(engine, args)
@@ -657,6 +675,8 @@ def main():
         points = {}
         half_steps, half_warmup = max(8, args.steps // 2), max(2, args.warmup // 2)
         for b in (1, 64, 128):
+            if b not in batches:
+                continue
             if b == args.batch:
                 points[f"decode_b{b}"] = round(value, 1)
                 continue
