@@ -271,7 +271,8 @@ class StepFunction:
     """Owns the step's buffers; ``__call__`` runs one step."""
 
     MAX_GRAPHS = 16
-    CAPTURE_AT = 2           # a decode graph is captured when its key comes this many times
+    CAPTURE_AT = 2           # a decode graph is captured when its key comes this many times ...
+    CAPTURE_WINDOW = 32      # ... within so many decode steps
 
     def __init__(self, model: CausalLM, cache: CacheManager, ops, max_batch_tokens: int,
                  graph=False):
@@ -292,7 +293,8 @@ class StepFunction:
         self.use_graph = graph if graph == "auto" else bool(graph)
         self.auto_graph = graph == "auto"
         self._graphs: "collections.OrderedDict" = collections.OrderedDict()
-        self._seen: Dict[tuple, int] = {}         # how often a key without a graph has come
+        self._seen: Dict[tuple, tuple] = {}       # key without a graph -> (times it has come, at which step last)
+        self._decode_steps = 0                    # decode steps that asked for a graph
         self.graph_replays = 0
         self.graph_captures = 0
         self.graph_evictions = 0
@@ -343,6 +345,7 @@ class StepFunction:
             bucket *= 2
         ctx.max_ctx_len = min(bucket, self.cache.max_pages_per_request * self.cache.page_size)
         key = (ctx.n_reqs, ctx.max_ctx_len, ctx.scratch_version)
+        self._decode_steps += 1
         hit = self._graphs.get(key)
         if hit is not None:
             self._graphs.move_to_end(key)
@@ -354,14 +357,18 @@ class StepFunction:
         if key[2] != ctx.scratch_version:
             return logits                      # buffers moved: capture at the next step
         # A capture costs milliseconds (a second forward and the making of the graph): it is
-        # made when a key comes the second time.  While requests end one after the other
-        # (the tail of a run) every key comes once or twice, and capturing each made those
-        # steps twice as slow as launching them from the kept sequences.
-        self._seen[key] = self._seen.get(key, 0) + 1
+        # made when a key comes the second time within a few decode steps.  While requests
+        # end one after the other (the tail of a run) every key comes once, and again once
+        # in the next run's tail: capturing each made those steps twice as slow as launching
+        # them from the kept sequences, and pushed the graphs of the steady state out.
+        count, last = self._seen.pop(key, (0, -self.CAPTURE_WINDOW))
+        count = count + 1 if self._decode_steps - last <= self.CAPTURE_WINDOW else 1
+        self._seen[key] = (count, self._decode_steps)
         if len(self._seen) > 4 * self.MAX_GRAPHS:
             self._seen.pop(next(iter(self._seen)))
-        if self._seen[key] < self.CAPTURE_AT:
+        if count < self.CAPTURE_AT:
             return logits
+        self._seen.pop(key, None)
         graph = torch.cuda.CUDAGraph()
         torch.cuda.synchronize(ctx.device)
         with torch.cuda.graph(graph):
