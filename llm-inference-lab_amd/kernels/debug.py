@@ -44,10 +44,13 @@ class DispatchRules:
     # inner size by the tiled kernel: the few-row kernel reads it once per tile of 16 rows
     # (64 rows of 3584 x 18944: 89 us against 34; of 1536 x 8960: 25 against 13).
     tiled_pieces_bytes: float = 16e6
-    # Pieces beyond this many bytes are folded once by the norm kernel instead of being
+    # Pieces beyond this many bytes are folded once by a kernel of their own instead of being
     # added on the fly by every block of a fused kernel (32 rows of width 3584 in 7 pieces,
-    # 3.2 MB: 12 us a layer more in the fused kernels).
-    pieces_per_block_bytes: int = 1 << 20
+    # 3.2 MB: 12 us a layer more in the fused kernels; 8 rows of width 5120 in 3 pieces, 491 KB:
+    # a decode step of the 14B shape 7.82 -> 7.56 ms folded once, of the 32B shape 16.03 ->
+    # 15.97; 4 rows of the same, 246 KB: 6.70 -> 6.83, and the 115 to 131 KB of the 0.5B to 3B
+    # shapes at 8 rows 3 to 7 % slower folded once).
+    pieces_per_block_bytes: int = 400_000
     # A piece of a few-row product has at least this many K steps of 32 ...
     min_steps_per_split: int = 8
     # ... and of a many-row product this many K tiles of 64.
