@@ -76,6 +76,9 @@ class Request:
     error: Optional[Exception] = None
     finish_reason: Optional[str] = None        # "eos", "length", "error", "cancelled"
     in_flight: bool = False                    # a token of this request is chosen but not read yet
+    eos: Tuple[int, ...] = ()                  # end-of-sequence ids, temperature and seed: worked out once
+    temperature: float = 0.0
+    seed: int = 0
     arrival: float = 0.0
     admit_time: Optional[float] = None
     first_token_time: Optional[float] = None
@@ -104,7 +107,7 @@ class Request:
         return self.cache.computed_len if self.cache is not None else 0
 
 
-@dataclasses.dataclass
+@dataclasses.dataclass(slots=True)
 class Planned:
     request: Request
     count: int              # tokens of this step
@@ -113,13 +116,20 @@ class Planned:
 
 def plan_step(active: Sequence[Request], max_batch_tokens: int) -> List[Planned]:
     """Decode first, then prompts in order, under one token budget."""
-    runnable = [r for r in active if not r.finished and r.budget_left > 0]
-    decode_budget = min(sum(1 for r in runnable if r.decoding), max_batch_tokens)
+    # (plain attribute reads instead of the properties: this loop runs per request and step)
+    runnable, decoding = [], 0
+    for r in active:
+        if r.finish_reason is None and r.remaining - (1 if r.in_flight else 0) > 0:
+            runnable.append(r)
+            if r.in_flight or r.generated:
+                decoding += 1
+    decode_budget = min(decoding, max_batch_tokens)
     prefill_budget = max_batch_tokens - decode_budget
     plan: List[Planned] = []
     for r in runnable:
-        ready = r.computed
-        if r.decoding:
+        ready = r.cache.computed_len if r.cache is not None else 0
+        known = len(r.tokens) + (1 if r.in_flight else 0)
+        if r.in_flight or r.generated:
             if decode_budget == 0:
                 continue
             decode_budget -= 1
@@ -129,7 +139,7 @@ def plan_step(active: Sequence[Request], max_batch_tokens: int) -> List[Planned]
                 continue
             count = min(len(r.tokens) - ready, prefill_budget)
             prefill_budget -= count
-        plan.append(Planned(r, count, ready + count == r.known_len))
+        plan.append(Planned(r, count, ready + count == known))
     return plan
 
 
@@ -171,6 +181,8 @@ class Scheduler:
         self._next_id += 1
         request.tokens = request.prompt[:]
         request.remaining = request.sampling.new_tokens
+        request.eos = tuple(request.sampling.eos_ids(self._model_eos))
+        request.temperature, request.seed = request.sampling.effective_temperature, request.sampling.seed
         self.waiting.append(request)
         self.instruments.received()
         return request.request_id
@@ -299,13 +311,12 @@ class Scheduler:
                 else:
                     self._fail(p.request, err)
             yielding = [p.request for p in ran if p.yields_token]
-            phase = "decode" if all(p.request.decoding and p.count == 1 for p in plan) else "prefill"
+            phase = "decode" if all(p.count == 1 and (p.request.in_flight or p.request.generated) for p in plan) else "prefill"
             if yielding:
                 counters = [len(r.generated) + (1 if r.in_flight else 0) for r in yielding]
                 try:
                     handle = self.sampler.sample_async(
-                        result.logits, [r.sampling.effective_temperature for r in yielding],
-                        [r.sampling.seed for r in yielding], counters)
+                        result.logits, [r.temperature for r in yielding], [r.seed for r in yielding], counters)
                     started = (yielding, handle, t0, phase)
                 except Exception as err:
                     for r in yielding:
@@ -374,8 +385,7 @@ class Scheduler:
             self.instruments.first_token(now - r.arrival)
         if self.on_token is not None:
             self.on_token(r, token)
-        eos = r.sampling.eos_ids(self._model_eos)
-        if token in eos:
+        if token in r.eos:
             r.remaining = 0
             r.finish_reason = "eos"
         elif r.remaining == 0:

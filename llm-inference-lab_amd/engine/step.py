@@ -101,6 +101,7 @@ class StepContext:
         pin = (torch.device(device).type == "cuda")
         self._host = torch.zeros(at, dtype=torch.int32, pin_memory=pin)
         self._host_np = self._host.numpy()
+        self._counting = np.arange(max(r, b) + 1, dtype=np.int32)
         self._dev = torch.zeros(at, dtype=torch.int32, device=device)
         self._groups = [
             GroupView(self._dev[t:t + b * self.max_pages].view(b, self.max_pages), page_size, window)
@@ -198,7 +199,34 @@ class StepContext:
         self.host_q_start, self.host_start_pos, self.host_req_rows = [], [], []
         self.memo = {}
         max_q = max_ctx = 0
-        for b, e in enumerate(entries):
+        one_token_each = n_rows == n_reqs and all(len(e.tokens) == 1 for e in entries)
+        if one_token_each:
+            # a decode step: every array in one piece (a numpy store per number costs as much
+            # as the rest of the host's work on a request)
+            n = n_reqs
+            starts = [e.request.computed_len for e in entries]
+            slots = [e.request.row for e in entries]
+            count = self._counting[:n + 1]
+            h[o["token_ids"]:o["token_ids"] + n] = [e.tokens[0] for e in entries]
+            h[o["positions"]:o["positions"] + n] = starts
+            h[o["row_req"]:o["row_req"] + n] = count[:n]
+            h[o["q_start"]:o["q_start"] + n] = count[:n]
+            h[o["start_pos"]:o["start_pos"] + n] = starts
+            h[o["req_rows"]:o["req_rows"] + n] = slots
+            for b, e in enumerate(entries):
+                if e.source is not None:
+                    if feed_tensor is not None and feed_tensor is not e.source[0]:
+                        raise ValueError("all device-fed entries of a step share one source tensor")
+                    feed_tensor = e.source[0]
+                    feeds.append((b, int(e.source[1])))
+                for w in e.want:
+                    if w != 0:
+                        raise ValueError(f"request {e.request.request_id!r}: wanted place {w} is not "
+                                         f"among its 1 tokens of this step")
+                    want.append(b)
+            self.host_q_start, self.host_start_pos, self.host_req_rows = list(range(n)), starts, slots
+            max_q, max_ctx, row = 1, max(starts) + 1, n
+        for b, e in enumerate(() if one_token_each else entries):
             n = len(e.tokens)
             start = e.request.computed_len
             if n == 1:          # (a decoding request: no arrays for one number)
@@ -241,9 +269,9 @@ class StepContext:
         for gi, at in enumerate(self._table_at):
             table = h[at:at + self.max_reqs * self.max_pages].reshape(self.max_reqs, self.max_pages)
             table[:n_reqs, :used_pages] = cache.tables[gi][cache_rows, :used_pages]
-        for i, (dst, src) in enumerate(feeds):
-            h[o["feed_dst"] + i] = dst
-            h[o["feed_src"] + i] = src
+        if feeds:
+            h[o["feed_dst"]:o["feed_dst"] + len(feeds)] = [dst for dst, _ in feeds]
+            h[o["feed_src"]:o["feed_src"] + len(feeds)] = [src for _, src in feeds]
         self._upload(n_reqs)
         self._set_views()
         if feeds:
