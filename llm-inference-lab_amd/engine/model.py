@@ -62,6 +62,8 @@ class CausalLM:
         self.entries: List[EntryView] = [EntryView(i, e.block) for i, e in enumerate(spec.schedule)]
         self.ops = None
         self.dtype = None
+        self._weight_bytes = None          # worked out when first asked for, after the weights are bound
+        self._graph_safe = None
         self.ranges = None         # profiler ranges (engine/profiling.py), off by default
         # Launch sequences of the scheduled runs, kept by the shape of the step: see _run_block.
         self.keep_launches = os.environ.get("LLMLAB_KEEP_LAUNCHES", "1") not in ("0", "")
@@ -77,7 +79,9 @@ class CausalLM:
     @property
     def graph_safe(self) -> bool:
         """Whether a decode step of this model may be replayed from a captured graph."""
-        return all(p.graph_safe for p in self.parts())
+        if self._graph_safe is None:            # (asked at every step; the parts say it once)
+            self._graph_safe = all(p.graph_safe for p in self.parts())
+        return self._graph_safe
 
     def kernel_libraries(self):
         """What the parts want compiled before they are bound, each once."""
@@ -107,6 +111,7 @@ class CausalLM:
 
     def bind(self, tensors: Dict[str, torch.Tensor], ops, dtype: torch.dtype) -> None:
         self.ops, self.dtype = ops, dtype
+        self._weight_bytes = self._graph_safe = None
         self.embedding.bind(tensors, ops, dtype)
         for b in self.blocks:
             b.bind(tensors, ops, dtype)
@@ -117,8 +122,10 @@ class CausalLM:
     def weight_bytes_per_step(self) -> int:
         """Bytes of weights that one step reads once (every run of a block reads
         its block's weights; the embedding table is read by rows only)."""
-        total = sum(self.blocks[e.block].weight_bytes() for e in self.entries)
-        return total + self.final_norm.weight_bytes() + self.head.weight_bytes()
+        if self._weight_bytes is None:          # (asked at every decode step: the weights do not change once bound)
+            total = sum(self.blocks[e.block].weight_bytes() for e in self.entries)
+            self._weight_bytes = total + self.final_norm.weight_bytes() + self.head.weight_bytes()
+        return self._weight_bytes
 
     # ------------------------------------------------------------------ cache
     def cache_layout(self) -> Tuple[List[GroupLayout], Dict[int, dict]]:

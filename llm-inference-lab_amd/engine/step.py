@@ -109,6 +109,7 @@ class StepContext:
         self._uploaded = torch.cuda.Event() if pin else None
         self._scratch: Dict[Tuple[str, torch.dtype], torch.Tensor] = {}
         self._views: Dict[tuple, torch.Tensor] = {}     # views of the scratch buffers handed out so far
+        self._step_views: Dict[tuple, tuple] = {}       # views of the step's description by (rows, requests, wanted)
         self.scratch_version = 0
         self.scratch_bytes = 0
         self.scratch_allocations = 0
@@ -126,13 +127,17 @@ class StepContext:
         return self._dev[at:at + count]
 
     def _set_views(self) -> None:
-        self.token_ids = self._view("token_ids", self.n_rows)
-        self.positions = self._view("positions", self.n_rows)
-        self.row_req = self._view("row_req", self.n_rows)
-        self.q_start = self._view("q_start", self.n_reqs + 1)
-        self.start_pos = self._view("start_pos", self.n_reqs)
-        self.req_rows = self._view("req_rows", self.n_reqs)
-        self.want_rows = self._view("want_rows", self.n_want)
+        key = (self.n_rows, self.n_reqs, self.n_want)
+        views = self._step_views.get(key)          # (slicing seven tensors anew costs 10 us a step)
+        if views is None:
+            views = (self._view("token_ids", self.n_rows), self._view("positions", self.n_rows),
+                     self._view("row_req", self.n_rows), self._view("q_start", self.n_reqs + 1),
+                     self._view("start_pos", self.n_reqs), self._view("req_rows", self.n_reqs),
+                     self._view("want_rows", self.n_want))
+            if len(self._step_views) < 1024:
+                self._step_views[key] = views
+        (self.token_ids, self.positions, self.row_req, self.q_start, self.start_pos, self.req_rows,
+         self.want_rows) = views
 
     def group(self, index: int) -> GroupView:
         return self._groups[index]
@@ -339,11 +344,15 @@ class StepFunction:
         """Bytes of cache that the step in ``ctx`` reads: for every group what its layers
         keep per token, times the positions of each request that they still see."""
         ctx, total = self.ctx, 0
+        seen_all = sum(ctx.host_start_pos[:ctx.n_reqs]) + ctx.n_rows      # (without a window: one sum for all requests)
         for g in self.cache.groups:
             per_token = len(g.entries) * g.spec.bytes_per_token(self.cache.dtype)
+            if not g.window:
+                total += per_token * seen_all
+                continue
             for b in range(ctx.n_reqs):
                 seen = ctx.host_start_pos[b] + ctx.host_q_start[b + 1] - ctx.host_q_start[b]
-                total += per_token * (min(seen, g.window) if g.window else seen)
+                total += per_token * min(seen, g.window)
         return total
 
     def _decode_auto(self) -> torch.Tensor:

@@ -75,6 +75,7 @@ class Sampler:
         self._out_host = [torch.zeros(max_requests, dtype=torch.int32, pin_memory=self._cuda)
                           for _ in range(self.SLOTS)]
         self._done = [None] * self.SLOTS      # recorded after a slot's last copy to the host
+        self._views = {}
         self._slot = 0
 
     def sample_async(self, logits: torch.Tensor, temperatures: Sequence[float], seeds: Sequence[int],
@@ -85,26 +86,30 @@ class Sampler:
         self._slot = (self._slot + 1) % self.SLOTS
         slot = self._slot
         out, out_host = self._out[slot], self._out_host[slot]
+        views = self._views.get((slot, rows))       # (slices of the slot's buffers: made once per batch size)
+        if views is None:
+            views = self._views[(slot, rows)] = (out[:rows], out_host[:rows])
+        out_rows, out_host_rows = views
         if self._done[slot] is not None:
             # everything queued with this slot's buffers has run: they are free again
             self._done[slot].synchronize()
         if all(t <= 0.0 for t in temperatures):
-            self.ops.argmax(logits, out[:rows])
+            self.ops.argmax(logits, out_rows)
         else:
             host, dev = self._host[slot], self._dev[slot]
             h = host.numpy()
             h[0, :rows] = np.asarray(temperatures, dtype=np.float32)
             h[1, :rows] = np.asarray([uniform(s, c) for s, c in zip(seeds, counters)], dtype=np.float32)
             dev[:, :rows].copy_(host[:, :rows], non_blocking=True)
-            self.ops.sample(logits, dev[0, :rows], dev[1, :rows], out[:rows])
+            self.ops.sample(logits, dev[0, :rows], dev[1, :rows], out_rows)
         event = None
         if self._cuda:
-            out_host[:rows].copy_(out[:rows], non_blocking=True)
-            event = torch.cuda.Event()
+            out_host_rows.copy_(out_rows, non_blocking=True)
+            event = self._done[slot] or torch.cuda.Event()        # (the slot's event, recorded anew)
             event.record()
             self._done[slot] = event
         else:
-            out_host[:rows].copy_(out[:rows])
+            out_host_rows.copy_(out_rows)
         return PendingTokens(out, out_host, event, rows)
 
     def sample(self, logits: torch.Tensor, temperatures: Sequence[float], seeds: Sequence[int],
