@@ -120,6 +120,9 @@ class StepContext:
         self.host_q_start: List[int] = []
         self.host_start_pos: List[int] = []
         self.host_req_rows: List[int] = []
+        # (the whole arrays behind ``q_start`` and ``start_pos``, for a caller that checks once
+        # what it will use for steps of any number of requests)
+        self.all_q_start, self.all_start_pos = self._view("q_start", b + 1), self._view("start_pos", b)
         self._set_views()
 
     def _view(self, name: str, count: int) -> torch.Tensor:

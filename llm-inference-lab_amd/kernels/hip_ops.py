@@ -94,6 +94,37 @@ class LaunchRecord:
         return True
 
 
+class AttentionCall:
+    """An attention call with its unchanging arguments checked and laid out
+    (``HipOps.prepare_attention``)."""
+
+    __slots__ = ("ops", "lib", "args", "most_requests", "most_context", "row_req", "heads", "dtype")
+    N_REQS, MAX_Q, MAX_CTX, ROW_REQ, SHORT_LEN, N_SHORT, SHORT_CTX, STREAM = 12, 13, 14, 23, 24, 25, 26, 29
+
+    def __init__(self, ops, lib, args, most_requests, most_context, row_req, heads, dtype):
+        self.ops, self.lib, self.args = ops, lib, args
+        self.most_requests, self.most_context, self.row_req = most_requests, most_context, row_req
+        self.heads, self.dtype = heads, dtype
+
+    def launch(self, n_reqs: int, max_q_len: int, max_ctx_len: int, short=None) -> None:
+        if n_reqs > self.most_requests:
+            raise ValueError("attention: request arrays are shorter than the number of requests")
+        if max_ctx_len > self.most_context:
+            raise ValueError("attention: the block table is too narrow for the longest context")
+        a = self.args
+        a[self.N_REQS], a[self.MAX_Q], a[self.MAX_CTX] = n_reqs, max_q_len, max_ctx_len
+        if short is not None:
+            _, short_len, n_short, short_ctx = short
+            if (short_len != self.ops.attention_short_limit(self.heads[0], self.heads[1], self.dtype, max_q_len)
+                    or not 0 < n_short < n_reqs or short_ctx > max_ctx_len or self.row_req is None):
+                raise ValueError("attention: the description of the step's short requests does not fit")
+            a[self.ROW_REQ], a[self.SHORT_LEN], a[self.N_SHORT], a[self.SHORT_CTX] = self.row_req, short_len, n_short, short_ctx
+        else:
+            a[self.ROW_REQ], a[self.SHORT_LEN], a[self.N_SHORT], a[self.SHORT_CTX] = None, 0, 0, 0
+        a[self.STREAM] = self.ops._stream()
+        self.ops._call(self.lib.llmlab_paged_attention, *a, lib=self.lib)
+
+
 class HipOps:
     WORKSPACE_FLOATS = 16 * 1024 * 1024      # 64 MiB of float32 scratch (split partial sums)
     ARRIVED_INTS = 64 * 1024                 # arrival counters: one per (request, kv head) of a step
@@ -841,6 +872,17 @@ class HipOps:
         """``short``: ``(row_req, limit, count, longest)`` for a step in which ``count`` of the
         requests (not all) bring at most ``limit = attention_short_limit(...)`` tokens, the
         longest context among those being ``longest``."""
+        self.prepare_attention(qkv, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_table, page_size,
+                               q_start, start_pos, window, scale, out,
+                               short[0] if short is not None else None).launch(n_reqs, max_q_len, max_ctx_len, short)
+
+    def prepare_attention(self, qkv, num_heads, num_kv_heads, head_dim, k_cache, v_cache, block_table,
+                          page_size, q_start, start_pos, window, scale, out, row_req=None) -> "AttentionCall":
+        """Everything of an attention call that does not change while the same buffers serve
+        the same number of rows, checked and laid out once; ``launch`` then takes what a step
+        brings (how many requests, their longest portion and context, its short requests).
+        ``q_start`` and ``start_pos`` may be longer than a step's requests; ``row_req`` is
+        needed only if a step will name short requests."""
         lib = self._attention_lib(head_dim)
         rows = qkv.shape[0]
         self._need(qkv, "queries", contiguous=False)
@@ -859,30 +901,22 @@ class HipOps:
             raise ValueError("attention: the query rows are too narrow")
         if tuple(out.shape) != (rows, num_heads * head_dim):
             raise ValueError(f"attention: output {tuple(out.shape)} != ({rows}, {num_heads * head_dim})")
-        if q_start.numel() < n_reqs + 1 or start_pos.numel() < n_reqs or block_table.shape[0] < n_reqs:
-            raise ValueError("attention: request arrays are shorter than the number of requests")
-        if max_ctx_len > block_table.shape[1] * page_size:
-            raise ValueError("attention: the block table is too narrow for the longest context")
         if page_size < 16 or page_size & (page_size - 1):
             raise UnsupportedSizeError(f"page size {page_size} is not a power of two >= 16")
-        q_stride = qkv.stride(0) if rows > 1 else qkv.shape[1]
-        row_req, short_len, n_short, short_ctx = None, 0, 0, 0
-        if short is not None:
-            row_req, short_len, n_short, short_ctx = short
-            if (short_len != self.attention_short_limit(num_heads, num_kv_heads, qkv.dtype, max_q_len)
-                    or not 0 < n_short < n_reqs or short_ctx > max_ctx_len):
-                raise ValueError("attention: the description of the step's short requests does not fit")
+        if row_req is not None:
             self._need(row_req, "row -> request map", torch.int32)
             if row_req.numel() < rows:
                 raise ValueError("attention: one request index per row")
-        self._call(lib.llmlab_paged_attention,
-            self._ptr(qkv), _dt(qkv), q_stride, num_heads, num_kv_heads, self._ptr(k_cache),
-            self._ptr(v_cache), self._ptr(block_table), block_table.stride(0), page_size,
-            self._ptr(q_start), self._ptr(start_pos), n_reqs, max_q_len, max_ctx_len,
-            int(window) if window else 0, float(scale), self._ptr(out), out.stride(0) if rows > 1 else
-            out.shape[1], self._ptr(self.workspace), self.workspace.numel(), rows, self.num_cus,
-            self._ptr(row_req), short_len, n_short, short_ctx, self._ptr(self.arrived), self.arrived.numel(),
-            self._stream(), lib=lib)
+        q_stride = qkv.stride(0) if rows > 1 else qkv.shape[1]
+        args = [self._ptr(qkv), _dt(qkv), q_stride, num_heads, num_kv_heads, self._ptr(k_cache),
+                self._ptr(v_cache), self._ptr(block_table), block_table.stride(0), page_size,
+                self._ptr(q_start), self._ptr(start_pos), 0, 0, 0,
+                int(window) if window else 0, float(scale), self._ptr(out), out.stride(0) if rows > 1 else
+                out.shape[1], self._ptr(self.workspace), self.workspace.numel(), rows, self.num_cus,
+                None, 0, 0, 0, self._ptr(self.arrived), self.arrived.numel(), None]
+        return AttentionCall(self, lib, args, most_requests=min(q_start.numel() - 1, start_pos.numel(), block_table.shape[0]),
+                             most_context=block_table.shape[1] * page_size, row_req=self._ptr(row_req),
+                             heads=(num_heads, num_kv_heads), dtype=qkv.dtype)
 
     # --------------------------------------------------------------- sampling
     def argmax(self, logits, out, one_pass: bool = True) -> None:

@@ -144,15 +144,26 @@ class GQAAttention(Mixer):
                               k_cache, v_cache)
         out = ctx.scratch("attention.out", (rows, self.q_size), self.dtype)
 
+        prepare = getattr(ops, "prepare_attention", None)
+        prepared = []
+
         def attend():
             # (how many requests, how long their portions and their histories are: read from
             # the step's description when the launch is made, also when it is made again
-            # from a kept sequence of calls)
-            ops.paged_attention(
-                q, self.num_heads, self.num_kv_heads, self.head_dim,
-                entry.k_cache, entry.v_cache, group.block_table, group.page_size,
-                ctx.q_start, ctx.start_pos, ctx.n_reqs, ctx.max_q_len, ctx.max_ctx_len,
-                self.window, self.scale, out, self._short_requests(ctx))
+            # from a kept sequence of calls; what stays the same then is checked once)
+            if prepare is None:
+                ops.paged_attention(
+                    q, self.num_heads, self.num_kv_heads, self.head_dim,
+                    entry.k_cache, entry.v_cache, group.block_table, group.page_size,
+                    ctx.q_start, ctx.start_pos, ctx.n_reqs, ctx.max_q_len, ctx.max_ctx_len,
+                    self.window, self.scale, out, self._short_requests(ctx))
+                return
+            if not prepared:
+                prepared.append(prepare(
+                    q, self.num_heads, self.num_kv_heads, self.head_dim, entry.k_cache, entry.v_cache,
+                    group.block_table, group.page_size, getattr(ctx, "all_q_start", ctx.q_start),
+                    getattr(ctx, "all_start_pos", ctx.start_pos), self.window, self.scale, out, ctx.row_req))
+            prepared[0].launch(ctx.n_reqs, ctx.max_q_len, ctx.max_ctx_len, self._short_requests(ctx))
         live = getattr(ops, "live", None)
         if live is not None:
             live(attend)
