@@ -97,9 +97,14 @@ __device__ __forceinline__ float sk_silu(float z) { return z / (1.f + __expf(-z)
 
 // Loads of W (and of x where it is not staged) run R steps ahead of the MFMAs in a
 // ring of registers that is refilled slot by slot, so a wave always has R loads
-// in flight and never waits for all of them at once.  Measured at depths 4, 8 and
-// 12: no difference once the stream is continuous, so the shallow ring it is.
-constexpr int SK_RING_STAGE = 4, SK_RING_DIRECT = 4;
+// in flight and never waits for all of them at once.  Measured per decode step, staged
+// ring 4 / 6 / 8 / 12 / 16 deep: one request of the 7B shape 3.21 / 3.13 / 3.07 / 3.34 /
+// 3.76 ms, eight of the 32B shape 15.83 / 15.66 / 15.61 / 15.96 / 16.96, eight of the
+// 0.5B shape 0.963 / 0.976 / 0.962 / 1.010 / 1.162 (a block of 16 waves has 128
+// registers a lane; a wave with fewer steps than the ring is deep reads its last tile
+// again for nothing); the ring of the unstaged products 4 / 6 / 8 deep: 15.61 / 15.52 /
+// 15.51 and 0.965 / 0.959 / 0.971.
+constexpr int SK_RING_STAGE = 8, SK_RING_DIRECT = 6;
 __host__ __device__ constexpr int sk_ring(int mb, bool stage) {
   return stage ? SK_RING_STAGE : (mb >= 4 ? SK_RING_DIRECT / 2 : SK_RING_DIRECT);
 }
