@@ -1333,10 +1333,10 @@ extern "C" int llmlab_paged_attention(const void* q, int dtype, int q_stride, in
   }
   // The launch, from measurements of 64 to 4,096 tokens behind 0 and 4,096 keys, one to
   // eight requests, heads of 64 (14 over 2) and 128 (28 over 4, 40 over 8):
-  //   1  few tiles of rows behind a long history: the waves of a block split the keys of
+  //   1  few tiles of rows behind a history: the waves of a block split the keys of
   //      one tile of 32 rows and merge in LDS, so that the work still spreads over the
   //      chip (64 to 512 tokens behind 4,096 keys, heads of 64: 27 to 31 us against 41 to
-  //      46 for the next best; at the start of a prompt it is the slowest, 17 against 8)
+  //      46 for the next best; at the start of a short prompt it is the slowest)
   //   6  every wave owns 16 rows, the block's two groups of four waves take the staged
   //      keys in turn: for heads above 64, where a block of four waves is alone on its
   //      compute unit (2,048 tokens behind 4,096 keys, 28 heads of 128: 313 us against
@@ -1351,7 +1351,12 @@ extern "C" int llmlab_paged_attention(const void* q, int dtype, int q_stride, in
   constexpr bool TWO_GROUPS = D <= 128;      // (the staged keys and values of two groups at larger heads: more LDS than there is)
   const long blocks16 = ((max_rows + 63) / 64) * nkv * live;
   const long blocks32 = ((max_rows + 127) / 128) * nkv * live;
-  const bool long_history = (long)max_ctx_len >= 8L * max_q_len;
+  // (from how long a history on the key split of launch 1 pays, few tiles of rows given: 128
+  // to 512 tokens of 14 heads of 64 behind 512 / 1,536 / 2,560 keys take 12 to 14 / 17 to 19 /
+  // 21 to 24 us so and 13 to 16 / 21 to 24 / 29 to 32 with launch 6, at the start of a prompt
+  // 9 to 11 against 7 to 11; of 28 heads of 128 behind 1,024 / 1,536 / 2,560 keys 29 / 34 / 44
+  // against 25 / 32 / 47)
+  const bool long_history = (long)max_ctx_len - max_q_len >= (D <= 64 ? 384 : 1792);
   const bool triangle = window <= 0 && 16L * (max_ctx_len - max_q_len) <= max_q_len;
   int path = g_force_path;
   if (!TWO_GROUPS && (path == 5 || path == 6)) path = 0;
