@@ -1361,18 +1361,39 @@ extern "C" int llmlab_paged_attention(const void* q, int dtype, int q_stride, in
   int path = g_force_path;
   if (!TWO_GROUPS && (path == 5 || path == 6)) path = 0;
   if (path == 0) {
+    // (the rules below are fitted to sweeps of 1 to 64 requests of 32 to 16,384 tokens behind
+    // 0 to 8,192 keys at the three head shapes, 470 cases: they lose 0.7 % to the best launch
+    // of each case on average, and more than 7 % in 16 of them)
+    const bool short_rows = max_q_len <= 128;
     if (blocks16 <= num_cus / 2 && long_history) path = 1;
+    // larger heads, short prompts from their start that leave units idle: one group of waves
+    // (64 tokens of 28 heads of 128: 8.4 us against 9.8)
+    else if (D > 64 && triangle && short_rows && blocks16 <= num_cus) path = 4;
+    // ... and many short portions behind short histories: 32 rows a wave (8 requests of 64
+    // tokens, 40 heads of 128 over 8: 11 us against 18; of 128 tokens, 28 over 4: 14 against 19)
+    else if (D > 64 && D <= 128 && blocks16 > num_cus && max_ctx_len <= 1024 &&
+             (short_rows || (max_q_len <= 256 && triangle))) path = 2;
     else if (TWO_GROUPS && D > 64 && !(blocks16 >= 4L * num_cus && max_ctx_len <= 1024)) path = 6;
+    // heads of 64: two groups of waves when at most a tile of rows a unit is to be had, unless
+    // the prompts are short and at their start (16 requests of 64 tokens: 6.8 us with one
+    // group against 8.0), and for long portions up to three tiles a unit
+    else if (TWO_GROUPS && D <= 64 && blocks16 <= num_cus / 2 && max_ctx_len >= 384) path = 6;
     else if (TWO_GROUPS && D <= 64 && blocks16 > num_cus / 2 &&
-             (blocks16 <= num_cus || (blocks16 <= 3L * num_cus && triangle && max_q_len >= 1536))) path = 6;
+             ((blocks16 <= num_cus && (max_q_len >= 256 || !triangle)) ||
+              (blocks16 <= 3L * num_cus && max_q_len >= 1536))) path = 6;
     else if (blocks16 < num_cus) path = 4;
-    else if (D <= 128 && blocks32 >= 2L * num_cus) path = 2;
+    // 32 rows a wave once its blocks fill the chip twice; at heads of 64 a little earlier,
+    // but only for portions up to 1,024 tokens behind a history (8 requests of 512 tokens behind
+    // 2,048 keys: 75 us against 83; two prompts of 4,096 from their start: 161 against 132)
+    else if (D > 64 ? (D <= 128 && blocks32 >= 2L * num_cus)
+                    : (blocks32 >= (7L * num_cus) / 4 && max_q_len <= 1024 && !triangle)) path = 2;
     // not enough tiles to keep every unit busy with what the longest ones leave over:
     // pair late and early tiles (no window: then the loads add up evenly).  Only at the
     // start of a prompt: behind a history all tiles carry about the same load, and the
     // pairs only halve the blocks (2,048 tokens behind 8,192, head size 64: 246 us in
-    // pairs, 172 without)
-    else if (triangle && blocks16 >= (3L * num_cus) / 2) path = 3;
+    // pairs, 172 without); and only at larger heads (heads of 64: 8 requests of 256 tokens
+    // 13.6 us in pairs, 10.6 without; 2 of 1,024: 23.5 against 21.5)
+    else if (D > 64 && triangle && blocks16 >= (3L * num_cus) / 2) path = 3;
     else path = 4;
   }
   if (path == 1) {
