@@ -387,7 +387,10 @@ class Runs:
         engine.close(req)
         assert bool(self.torch.isfinite(whole).all() and self.torch.isfinite(portions).all()), "non-finite logits"
         err = float((whole - portions).abs().max())
-        same_token = int(whole.argmax()) == int(portions.argmax())
+        # the same choice from both, or one that the whole prompt's own logits prefer by no more
+        # than the two runs differ (random weights leave the best logits close together)
+        margin = float(whole.max() - whole[int(portions.argmax())])
+        same_token = margin <= 2 * err
         limit = 1e-3 if self.dtype == "f32" else 0.5
         prompts = [self.random_ids(n) for n in (5, 130, 700)]
         first = engine.generate(prompts, max_new_tokens=12, eos_token_id=[])
@@ -397,7 +400,7 @@ class Runs:
             for g in m["groups"]:
                 g.pop("pages_high_water")
         result = {"tokens": tokens, "chunk": chunk, "max_abs_logit_error": round(err, 6), "limit": limit,
-                  "same_token": same_token, "samples_identical": first == second,
+                  "same_token": same_token, "token_margin": round(margin, 6), "samples_identical": first == second,
                   "kv_released": initial == after}
         result["passed"] = err < limit and same_token and first == second and initial == after
         if not result["passed"]:
