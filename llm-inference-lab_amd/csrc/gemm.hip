@@ -1112,7 +1112,10 @@ static double tile_cost(int kind, int M, int N, int K, int num_cus, int pieces) 
   const TileModel& t = TILE_MODELS[kind];
   const double blocks = (double)((M + t.bm - 1) / t.bm) * ((N + t.bn - 1) / t.bn) * pieces;
   double rounds = blocks / (num_cus * t.resident);
-  if (t.whole_rounds) rounds = ceil(rounds - 1e-9);
+  // (the 64 x 64 tile beyond 64 rows: measured, a block more than the units hold costs a whole
+  // round: 256 rows of 4608 x 3584, 288 blocks, 32 us against 29 with 144 blocks of 64 x 128,
+  // and 192 rows, 216 blocks, 26 against 29)
+  if (t.whole_rounds || (kind == TILE_64 && M > 64)) rounds = ceil(rounds - 1e-9);
   const int nk = ((K + 63) / 64 + pieces - 1) / pieces;
   const double compute = (rounds > 1.0 ? rounds : 1.0) * (t.f + nk * t.tk);
   const double rate = blocks * t.stream < CHIP_STREAM ? blocks * t.stream : CHIP_STREAM;
@@ -1125,6 +1128,10 @@ static double tile_cost(int kind, int M, int N, int K, int num_cus, int pieces) 
 // 192 x 256; -131 = choose among the first three; -256 and below: the tiles of two groups
 // of waves from so many rows on).
 static int g_force_tile = 0, g_without_wide = 0, g_pp_min_rows = 512;
+// The 128 x 256 tile is weighed from so many rows on.  (By the product alone it would pay from
+// 768: 1,536 rows of 5120 x 27648 447 us against 543; inside prefill steps of 768 to 1,536
+// tokens of five shapes that is between 1.4 % faster and 1.3 % slower than from 2,048 on.)
+constexpr int WIDE_TILE_MIN_ROWS = 2048;
 constexpr int PP_MIN_INNER = 896;      // the shortest inner size the estimates of those tiles were fitted to
 extern "C" void llmlab_debug_gemm_tile(int tile) {
   g_force_tile = tile > 0 ? tile : 0;
@@ -1153,7 +1160,7 @@ static int choose_tile(int M, int N, int K, int num_cus) {
   // the shape of the model, of 4096 and 8192: 3 to 7 % faster at the larger shapes), and
   // an inner size of 1024 on: with 896 its one block per unit shows its start and its
   // epilogue, and steps of 4096 are 1.7 % slower with it.
-  const int kinds = M >= 2048 && K >= 1024 && !g_without_wide ? TILE_256 : TILE_128x256;
+  const int kinds = M >= WIDE_TILE_MIN_ROWS && K >= 1024 && !g_without_wide ? TILE_256 : TILE_128x256;
   double cost[TILE_KINDS];
   int best = 0;
   for (int kind = 0; kind < kinds; ++kind) {
@@ -1187,7 +1194,11 @@ static int choose_tile(int M, int N, int K, int num_cus) {
   // 3.5 / 5.8 % faster, 576 and 2048 unchanged).  (The same two groups of waves on a 128 x
   // 256 tile, 64 x 64 a wave, are as fast as the 128 x 256 tile above and no faster: a wave
   // then reads as many bytes from LDS per MFMA as there, and LDS is the limit of both.)
-  if (M >= g_pp_min_rows && K >= PP_MIN_INNER && !g_without_wide) {
+  // ... and from 129 rows on for a wide matrix, where one or two tiles of rows already fill the
+  // chip (192 / 256 / 384 rows of 55296 x 5120: 153 / 171 / 261 us against 187 / 199 / 274 with the
+  // best of the others; of 59136 x 8192: 229 / 263 / 392 against 305 / 316 / 437)
+  const bool pp_rows = M >= g_pp_min_rows || (g_pp_min_rows == 512 && M > 128 && N >= 16384);
+  if (pp_rows && K >= PP_MIN_INNER && !g_without_wide) {
     double least = tile_cost(best, M, N, K, num_cus, 1);
     for (int kind = TILE_256; kind <= TILE_192; ++kind) {
       const double c = tile_cost(kind, M, N, K, num_cus, 1);
