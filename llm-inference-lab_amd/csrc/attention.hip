@@ -1196,9 +1196,9 @@ static int launch_key_split_decode(AttnArgs a, int reqs, int live, int ctx_len, 
 // float32.  Steps of at most 16 rows per request and kv head (decode) split the keys over
 // the waves of a block and over blocks, as many splits as still give every block a compute
 // unit of its own (the same rule as in bfloat16, for twice the bytes), and the merge kernel
-// sums the splits.  Few tiles of rows behind a long history take one block per tile whose
-// waves split the keys; everything else one wave per tile of 32 rows (16 for heads
-// above 128: registers).
+// sums the splits.  Steps of more rows take one block per tile of 32 rows (16 for heads
+// above 128: registers) whose waves split the keys, or, once the tiles fill the chip, one
+// wave per tile (launch_attention_f32 says when).
 constexpr int F32_SPLIT_WAVES = D <= 64 ? 8 : 4;
 constexpr int F32_QB = D <= 128 ? 2 : 1;
 static int launch_f32_key_split(AttnArgs a, int reqs, int live, int ctx_len, int window, int total_rows,
@@ -1257,9 +1257,24 @@ static int launch_attention_f32(AttnArgs a, int reqs, int max_q_len, int max_ctx
   }
   constexpr int ROWS = 16 * F32_QB;
   const long tiles = (max_rows + ROWS - 1) / ROWS;
-  const bool long_history = (long)max_ctx_len >= 8L * max_q_len;
+  // Which launch, from a sweep of 1 to 32 requests of 64 to 8,192 tokens behind 0 to 4,096 keys
+  // (14 heads of 64 over 2, 28 of 128 over 4).  A block whose waves split the keys of a tile
+  // (1) wins wherever a wave per tile (2) would leave compute units idle or walk a long
+  // history alone: 512 tokens behind 1,024 keys at heads of 64 take 43 us so and 162 with a
+  // wave per tile, a prompt of 2,048 tokens 117 against 217.  A wave per tile wins once the
+  // tiles fill the chip and the keys are few (16 requests of 512 tokens from their start,
+  // heads of 64: 137 us against 187), at heads above 64 from half a tile a unit on (4
+  // requests of 256 tokens: 58 against 81).
   int path = g_force_path;        // (1: the waves of a block split the keys; anything else: a wave per tile)
-  if (path == 0) path = (tiles * a.nkv * live <= num_cus / 2 && long_history) ? 1 : 2;
+  if (path == 0) {
+    const long blocks = tiles * a.nkv * live;
+    if (D > 64) path = blocks <= num_cus / 2 ? 1 : 2;
+    else {
+      const int few_keys = blocks >= (7L * num_cus) / 2 ? 1024 : blocks >= (7L * num_cus) / 4 ? 768
+                           : blocks >= (7L * num_cus) / 8 ? 256 : 0;
+      path = max_ctx_len <= few_keys ? 2 : 1;
+    }
+  }
   if (path == 1) {
     hipLaunchKernelGGL((attention_f32_kernel<F32_QB, true, F32_SPLIT_WAVES>), dim3((unsigned)tiles, a.nkv, reqs),
                        dim3(64 * F32_SPLIT_WAVES), 0, stream, a);
