@@ -870,9 +870,10 @@ __global__ __launch_bounds__(64 * MERGE_WAVES) void attention_merge_kernel(
 //
 // A tile is 16 QB rows ((token, head of the group) pairs of one request and kv head, so the
 // heads of a group share the keys they read).  SPLIT = false: every wave owns a tile and
-// walks all its keys (prompts).  SPLIT = true: the NW waves of a block share one tile and
-// split its keys, merge through LDS, and blockIdx.y also counts splits over blocks whose
-// partial results the merge kernel sums (decode steps; few rows behind a long history).
+// walks all its keys (steps whose tiles fill the chip over few keys).  SPLIT = true: the NW
+// waves of a block share one tile and split its keys, merge through LDS (all other steps of
+// many rows), and blockIdx.y also counts splits over blocks whose partial results the merge
+// kernel sums (decode steps).
 template <int QB, bool SPLIT, int NW>
 __global__ __launch_bounds__(64 * NW) void attention_f32_kernel(AttnArgs a) {
   constexpr int DQ = D / 16;
