@@ -1153,6 +1153,11 @@ static int choose_tile(int M, int N, int K, int num_cus) {
   // 55296 x 5120: 127 against 157).
   const long wide = (N + 127) / 128;
   if (M <= 64 && wide >= num_cus) return TILE_64x128;
+  // ... and of a matrix of 32,768 to 65,536 rows the 128 x 256 tile (96 / 128 rows of 37888 x
+  // 3584: 81 / 77 us against 83 / 84; of 59136 x 8192: 195 / 201 against 200 / 209; a decode
+  // step of 128 requests of the 7B shape 6.99 -> 6.86 ms, of the 32B shape 24.8 -> 24.4; a
+  // vocabulary of 152,064 gains nothing from it)
+  if (M > 64 && M <= 128 && N >= 32768 && N <= 65536 && K >= 1024 && !g_without_wide) return TILE_128x256;
   if (M > 64 && M <= 128 && wide >= 3L * num_cus / 2) return TILE_128;
   // The 128 x 256 tile from 2048 rows on: with 576 and 1024 rows it wins or loses a few
   // percent by the product alone, and a prefill step of 1024 tokens as a whole is 1 to
