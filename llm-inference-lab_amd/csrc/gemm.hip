@@ -1270,6 +1270,18 @@ extern "C" void llmlab_linear_plan(int M, int N, int K, int num_cus, int max_pie
       }
     }
   }
+  // Two or three well-filled tiles of 128 rows of a matrix 5,120 to 16,383 wide: four pieces of
+  // the 128 x 128 tile, which the estimate prices too high there (with the norm that folds
+  // them, 384 rows of 8192 x 29568: 248 us against 365 whole with 64 x 128; of 5120 x 27648:
+  // 150 against 183 in two pieces; 256 rows of 8192 x 8192: 65 against 70; at 3,584 columns
+  // it loses as often as it wins).  Inside prefill steps of 256 / 320 / 384 tokens of the 14B
+  // shape 14.5 -> 14.2 / 16.5 -> 15.5 / 17.6 -> 16.7 ms, of the 32B shape 27.3 -> 27.0 / 34.0 ->
+  // 31.2 / 35.9 -> 33.8; at 192 rows the 32B shape loses 5 % with it, hence from 256 on.
+  if (M >= 256 && M <= 384 && 4 * M >= 3 * ((M + 127) / 128) * 128 && N >= 5120 && N < 16384 &&
+      g_force_tile == 0 && max_pieces >= 4 && (nk + 3) / 4 >= min_tiles_per_piece) {
+    best_kind = TILE_128;
+    best_pieces = 4;
+  }
   // One tile of rows in pieces: the small tile, if its blocks still find a compute unit
   // each (17 to 64 rows of matrices from 9 to 45 MB: 8.6 against 11.0, 12.4 against
   // 15.8, 15.1 against 18.8 us; with more blocks than units it is the slower one)

@@ -82,6 +82,10 @@ def test_limits_of_the_plan_are_kept(core):
     (192, 27648, 5120, (1, 1)),       # ... not where half the units would stay idle
     (192, 4608, 3584, (1, 0)),        # 216 blocks of 64 x 64 are one round (26 us against 29 with 64 x 128),
     (1536, 896, 896, (1, 1)),         # 336 are two: 64 x 128 (11.5 us against 13.3)
+    (384, 5120, 27648, (4, 2)),       # three tiles of 128 rows in four pieces (150 us against 183 in two of 64 x 128)
+    (256, 8192, 8192, (4, 2)),
+    (192, 5120, 27648, (4, 1)),       # ... from 256 rows on (a step of 192 requests of the 32B shape loses 5 % with them)
+    (272, 5120, 27648, (2, 1)),       # ... and only well-filled tiles
 ])
 def test_measured_decisions(core, m, n, k, want):
     assert plan(core, m, n, k) == want
