@@ -1234,6 +1234,23 @@ static int launch_f32_key_split(AttnArgs a, int reqs, int live, int ctx_len, int
   return 0;
 }
 
+// Which launch a float32 step of many rows takes: 1 = the waves of a block split the keys of a
+// tile, anything else = a wave per tile.  `blocks`: tiles of rows times kv heads times requests.
+static int choose_many_rows_launch_f32(long blocks, int max_q_len, int max_ctx_len, int num_cus, int forced) {
+  if (forced != 0) return forced;
+  // (how few the keys must be for a wave per tile, by how many times the tiles fill the chip)
+  int few_keys;
+  // (heads above 64: portions of 1,024 tokens and more keep the key split until their tiles fill
+  // the chip seven times, since the late tiles of a long portion walk many more keys than the
+  // early ones and a wave per tile leaves that uneven: one prompt of 1,024 tokens 148 us against
+  // 184, of 2,048 453 against 512, two of 1,024 290 against 305; four of 1,024 562 against 501)
+  if (D > 64) few_keys = blocks > (max_q_len >= 1024 ? 7L : 2L) * num_cus ? 0x7fffffff
+                         : blocks >= (7L * num_cus) / 4 && max_q_len < 1024 ? 128 : 0;
+  else few_keys = blocks >= 14L * num_cus ? 1024 : blocks >= 7L * num_cus ? 768 : blocks >= (7L * num_cus) / 2 ? 256
+                  : blocks >= (7L * num_cus) / 4 ? 128 : 0;
+  return max_ctx_len <= few_keys ? 2 : 1;
+}
+
 static int launch_attention_f32(AttnArgs a, int reqs, int max_q_len, int max_ctx_len, int window, int total_rows,
                                 float* workspace, size_t workspace_floats, int num_cus, const int* row_req,
                                 int short_len, int n_short, int short_ctx, hipStream_t stream) {
@@ -1264,18 +1281,9 @@ static int launch_attention_f32(AttnArgs a, int reqs, int max_q_len, int max_ctx
   // history alone: 512 tokens behind 1,024 keys at heads of 64 take 43 us so and 162 with a
   // wave per tile, a prompt of 2,048 tokens 117 against 217.  A wave per tile wins once the
   // tiles fill the chip and the keys are few (16 requests of 512 tokens from their start,
-  // heads of 64: 137 us against 187), at heads above 64 from half a tile a unit on (4
-  // requests of 256 tokens: 58 against 81).
-  int path = g_force_path;        // (1: the waves of a block split the keys; anything else: a wave per tile)
-  if (path == 0) {
-    const long blocks = tiles * a.nkv * live;
-    if (D > 64) path = blocks <= num_cus / 2 ? 1 : 2;
-    else {
-      const int few_keys = blocks >= (7L * num_cus) / 2 ? 1024 : blocks >= (7L * num_cus) / 4 ? 768
-                           : blocks >= (7L * num_cus) / 8 ? 256 : 0;
-      path = max_ctx_len <= few_keys ? 2 : 1;
-    }
-  }
+  // heads of 64: 137 us against 187), at heads above 64 from two tiles a unit on whatever the
+  // keys (4 requests of 256 tokens: 58 against 81).
+  const int path = choose_many_rows_launch_f32(tiles * a.nkv * live, max_q_len, max_ctx_len, num_cus, g_force_path);
   if (path == 1) {
     hipLaunchKernelGGL((attention_f32_kernel<F32_QB, true, F32_SPLIT_WAVES>), dim3((unsigned)tiles, a.nkv, reqs),
                        dim3(64 * F32_SPLIT_WAVES), 0, stream, a);
@@ -1285,6 +1293,95 @@ static int launch_attention_f32(AttnArgs a, int reqs, int max_q_len, int max_ctx
   }
   LLMLAB_LAUNCH_CHECK("attention(float32)");
   return 0;
+}
+
+constexpr bool TWO_GROUPS = D <= 128;      // (the staged keys and values of two groups at larger heads: more LDS than there is)
+
+// Which launch a step of many rows takes (bfloat16): `max_rows` (token, head of the group) pairs
+// at most per request and kv head, `live` requests, the longest portion and context, the window.
+static int choose_many_rows_launch(long max_rows, int nkv, int live, int max_q_len, int max_ctx_len, int window,
+                                   int num_cus, int forced) {
+  // The launch, from measurements of 64 to 4,096 tokens behind 0 and 4,096 keys, one to
+  // eight requests, heads of 64 (14 over 2) and 128 (28 over 4, 40 over 8):
+  //   1  few tiles of rows behind a history: the waves of a block split the keys of
+  //      one tile of 32 rows and merge in LDS, so that the work still spreads over the
+  //      chip (64 to 512 tokens behind 4,096 keys, heads of 64: 27 to 31 us against 41 to
+  //      46 for the next best; at the start of a short prompt it is the slowest)
+  //   6  every wave owns 16 rows, the block's two groups of four waves take the staged
+  //      keys in turn: for heads above 64, where a block of four waves is alone on its
+  //      compute unit (2,048 tokens behind 4,096 keys, 28 heads of 128: 313 us against
+  //      374 to 470 for the others), and for heads of 64 when the tiles of rows would
+  //      leave a SIMD with one wave or none, or the longest tile of a long prompt's
+  //      triangle decides (2,048 tokens from 0: 32 us against 38; four prompts of 512: 19
+  //      against 15, so not for those)
+  //   4  the same with one group of four waves (two blocks share a compute unit at heads
+  //      of 64)
+  //   2  32 rows per wave, when that still gives every compute unit two blocks
+  //   3  late and early tiles in pairs (see below)
+  const long blocks16 = ((max_rows + 63) / 64) * nkv * live;
+  const long blocks32 = ((max_rows + 127) / 128) * nkv * live;
+  // (from how long a history on the key split of launch 1 pays, few tiles of rows given: 128
+  // to 512 tokens of 14 heads of 64 behind 512 / 1,536 / 2,560 keys take 12 to 14 / 17 to 19 /
+  // 21 to 24 us so and 13 to 16 / 21 to 24 / 29 to 32 with launch 6, at the start of a prompt
+  // 9 to 11 against 7 to 11; of 28 heads of 128 behind 1,024 / 1,536 / 2,560 keys 29 / 34 / 44
+  // against 25 / 32 / 47)
+  const bool long_history = (long)max_ctx_len - max_q_len >= (D <= 64 ? 384 : 1792);
+  const bool triangle = window <= 0 && 16L * (max_ctx_len - max_q_len) <= max_q_len;
+  int path = forced;
+  if (!TWO_GROUPS && (path == 5 || path == 6)) path = 0;
+  if (path == 0) {
+    // (the rules below are fitted to sweeps of 1 to 64 requests of 32 to 16,384 tokens behind
+    // 0 to 8,192 keys at the three head shapes, 470 cases: they lose 0.7 % to the best launch
+    // of each case on average, and more than 7 % in 16 of them)
+    const bool short_rows = max_q_len <= 128;
+    if (blocks16 <= num_cus / 2 && long_history) path = 1;
+    // larger heads, short prompts from their start that leave units idle: one group of waves
+    // (64 tokens of 28 heads of 128: 8.4 us against 9.8)
+    else if (D > 64 && triangle && short_rows && blocks16 <= num_cus) path = 4;
+    // ... and many short portions behind short histories: 32 rows a wave (8 requests of 64
+    // tokens, 40 heads of 128 over 8: 11 us against 18; of 128 tokens, 28 over 4: 14 against 19)
+    else if (D > 64 && D <= 128 && blocks16 > num_cus && max_ctx_len <= 1024 &&
+             (short_rows || (max_q_len <= 256 && triangle))) path = 2;
+    else if (TWO_GROUPS && D > 64 && !(blocks16 >= 4L * num_cus && max_ctx_len <= 1024)) path = 6;
+    // heads of 64: two groups of waves when at most a tile of rows a unit is to be had, unless
+    // the prompts are short and at their start (16 requests of 64 tokens: 6.8 us with one
+    // group against 8.0), and for long portions up to three tiles a unit
+    else if (TWO_GROUPS && D <= 64 && blocks16 <= num_cus / 2 && max_ctx_len >= 384) path = 6;
+    else if (TWO_GROUPS && D <= 64 && blocks16 > num_cus / 2 &&
+             ((blocks16 <= num_cus && (max_q_len >= 256 || !triangle)) ||
+              (blocks16 <= 3L * num_cus && max_q_len >= 1536))) path = 6;
+    else if (blocks16 < num_cus) path = 4;
+    // 32 rows a wave once its blocks fill the chip twice; at heads of 64 a little earlier,
+    // but only for portions up to 1,024 tokens behind a history (8 requests of 512 tokens behind
+    // 2,048 keys: 75 us against 83; two prompts of 4,096 from their start: 161 against 132), and
+  // for prompts of 8,192 tokens and more (221 us against 235)
+    else if (D > 64 ? (D <= 128 && blocks32 >= 2L * num_cus)
+                    : (blocks32 >= (7L * num_cus) / 4 && ((max_q_len <= 1024 && !triangle) || max_q_len >= 8192))) path = 2;
+    // not enough tiles to keep every unit busy with what the longest ones leave over:
+    // pair late and early tiles (no window: then the loads add up evenly).  Only at the
+    // start of a prompt: behind a history all tiles carry about the same load, and the
+    // pairs only halve the blocks (2,048 tokens behind 8,192, head size 64: 246 us in
+    // pairs, 172 without); and only at larger heads (heads of 64: 8 requests of 256 tokens
+    // 13.6 us in pairs, 10.6 without; 2 of 1,024: 23.5 against 21.5)
+    else if (D > 64 && triangle && blocks16 >= (3L * num_cus) / 2) path = 3;
+    else path = 4;
+  }
+  return path;
+}
+
+// The launch that llmlab_paged_attention would take for a step of many rows of these sizes
+// (for tests and tuning; 0: the sizes make a decode step, whose keys are split over blocks).
+extern "C" int llmlab_attention_launch(int dtype, int nq, int nkv, int reqs, int max_q_len, int max_ctx_len, int window,
+                                       int num_cus) {
+  if (num_cus <= 0) num_cus = 256;
+  if (nq <= 0 || nkv <= 0 || nq % nkv != 0 || reqs <= 0 || max_q_len <= 0) return -1;
+  const long max_rows = (long)max_q_len * (nq / nkv);
+  if (max_rows <= 16) return 0;
+  if (dtype == DT_F32) {
+    constexpr int ROWS = 16 * F32_QB;
+    return choose_many_rows_launch_f32((max_rows + ROWS - 1) / ROWS * nkv * reqs, max_q_len, max_ctx_len, num_cus, 0);
+  }
+  return choose_many_rows_launch(max_rows, nkv, reqs, max_q_len, max_ctx_len, window, num_cus, 0);
 }
 
 // q rows are the step's packed rows; reqs requests; max_q_len / max_ctx_len are
@@ -1347,71 +1444,7 @@ extern "C" int llmlab_paged_attention(const void* q, int dtype, int q_stride, in
     a.qlen_lo = short_len + 1;
     live = reqs - n_short;
   }
-  // The launch, from measurements of 64 to 4,096 tokens behind 0 and 4,096 keys, one to
-  // eight requests, heads of 64 (14 over 2) and 128 (28 over 4, 40 over 8):
-  //   1  few tiles of rows behind a history: the waves of a block split the keys of
-  //      one tile of 32 rows and merge in LDS, so that the work still spreads over the
-  //      chip (64 to 512 tokens behind 4,096 keys, heads of 64: 27 to 31 us against 41 to
-  //      46 for the next best; at the start of a short prompt it is the slowest)
-  //   6  every wave owns 16 rows, the block's two groups of four waves take the staged
-  //      keys in turn: for heads above 64, where a block of four waves is alone on its
-  //      compute unit (2,048 tokens behind 4,096 keys, 28 heads of 128: 313 us against
-  //      374 to 470 for the others), and for heads of 64 when the tiles of rows would
-  //      leave a SIMD with one wave or none, or the longest tile of a long prompt's
-  //      triangle decides (2,048 tokens from 0: 32 us against 38; four prompts of 512: 19
-  //      against 15, so not for those)
-  //   4  the same with one group of four waves (two blocks share a compute unit at heads
-  //      of 64)
-  //   2  32 rows per wave, when that still gives every compute unit two blocks
-  //   3  late and early tiles in pairs (see below)
-  constexpr bool TWO_GROUPS = D <= 128;      // (the staged keys and values of two groups at larger heads: more LDS than there is)
-  const long blocks16 = ((max_rows + 63) / 64) * nkv * live;
-  const long blocks32 = ((max_rows + 127) / 128) * nkv * live;
-  // (from how long a history on the key split of launch 1 pays, few tiles of rows given: 128
-  // to 512 tokens of 14 heads of 64 behind 512 / 1,536 / 2,560 keys take 12 to 14 / 17 to 19 /
-  // 21 to 24 us so and 13 to 16 / 21 to 24 / 29 to 32 with launch 6, at the start of a prompt
-  // 9 to 11 against 7 to 11; of 28 heads of 128 behind 1,024 / 1,536 / 2,560 keys 29 / 34 / 44
-  // against 25 / 32 / 47)
-  const bool long_history = (long)max_ctx_len - max_q_len >= (D <= 64 ? 384 : 1792);
-  const bool triangle = window <= 0 && 16L * (max_ctx_len - max_q_len) <= max_q_len;
-  int path = g_force_path;
-  if (!TWO_GROUPS && (path == 5 || path == 6)) path = 0;
-  if (path == 0) {
-    // (the rules below are fitted to sweeps of 1 to 64 requests of 32 to 16,384 tokens behind
-    // 0 to 8,192 keys at the three head shapes, 470 cases: they lose 0.7 % to the best launch
-    // of each case on average, and more than 7 % in 16 of them)
-    const bool short_rows = max_q_len <= 128;
-    if (blocks16 <= num_cus / 2 && long_history) path = 1;
-    // larger heads, short prompts from their start that leave units idle: one group of waves
-    // (64 tokens of 28 heads of 128: 8.4 us against 9.8)
-    else if (D > 64 && triangle && short_rows && blocks16 <= num_cus) path = 4;
-    // ... and many short portions behind short histories: 32 rows a wave (8 requests of 64
-    // tokens, 40 heads of 128 over 8: 11 us against 18; of 128 tokens, 28 over 4: 14 against 19)
-    else if (D > 64 && D <= 128 && blocks16 > num_cus && max_ctx_len <= 1024 &&
-             (short_rows || (max_q_len <= 256 && triangle))) path = 2;
-    else if (TWO_GROUPS && D > 64 && !(blocks16 >= 4L * num_cus && max_ctx_len <= 1024)) path = 6;
-    // heads of 64: two groups of waves when at most a tile of rows a unit is to be had, unless
-    // the prompts are short and at their start (16 requests of 64 tokens: 6.8 us with one
-    // group against 8.0), and for long portions up to three tiles a unit
-    else if (TWO_GROUPS && D <= 64 && blocks16 <= num_cus / 2 && max_ctx_len >= 384) path = 6;
-    else if (TWO_GROUPS && D <= 64 && blocks16 > num_cus / 2 &&
-             ((blocks16 <= num_cus && (max_q_len >= 256 || !triangle)) ||
-              (blocks16 <= 3L * num_cus && max_q_len >= 1536))) path = 6;
-    else if (blocks16 < num_cus) path = 4;
-    // 32 rows a wave once its blocks fill the chip twice; at heads of 64 a little earlier,
-    // but only for portions up to 1,024 tokens behind a history (8 requests of 512 tokens behind
-    // 2,048 keys: 75 us against 83; two prompts of 4,096 from their start: 161 against 132)
-    else if (D > 64 ? (D <= 128 && blocks32 >= 2L * num_cus)
-                    : (blocks32 >= (7L * num_cus) / 4 && max_q_len <= 1024 && !triangle)) path = 2;
-    // not enough tiles to keep every unit busy with what the longest ones leave over:
-    // pair late and early tiles (no window: then the loads add up evenly).  Only at the
-    // start of a prompt: behind a history all tiles carry about the same load, and the
-    // pairs only halve the blocks (2,048 tokens behind 8,192, head size 64: 246 us in
-    // pairs, 172 without); and only at larger heads (heads of 64: 8 requests of 256 tokens
-    // 13.6 us in pairs, 10.6 without; 2 of 1,024: 23.5 against 21.5)
-    else if (D > 64 && triangle && blocks16 >= (3L * num_cus) / 2) path = 3;
-    else path = 4;
-  }
+  const int path = choose_many_rows_launch(max_rows, nkv, live, max_q_len, max_ctx_len, window, num_cus, g_force_path);
   if (path == 1) {
     const int steps32 = (max_ctx_len + 31) / 32 + 1;
     const int steps_per_wave = (steps32 + DECODE_WAVES - 1) / DECODE_WAVES;

@@ -174,3 +174,77 @@ def test_the_engine_counts_a_decode_step_and_decides_step_by_step():
     per_token = 2 * 32 * 4
     seen = lambda n: per_token * (n + 2 * min(n, 24))
     assert [q[2] for q in ops.rules.questions] == [seen(31) + seen(8), seen(32) + seen(9), seen(33)]
+
+
+# ----------------------------------------------------------------- attention
+def attention_library(head_dim):
+    if shutil.which("hipcc") is None and not build.hipcc_path():
+        pytest.skip("no hipcc to build the library with")
+    try:
+        lib = ctypes.CDLL(build.attention_library(head_dim))
+    except (OSError, RuntimeError) as err:
+        pytest.skip(f"the attention library does not load here: {err}")
+    lib.llmlab_attention_launch.restype = ctypes.c_int
+    return lib
+
+
+BF16, F32 = 1, 0        # (the dtype codes of the libraries)
+
+
+@pytest.mark.parametrize("head_dim,nq,nkv", [(64, 14, 2), (128, 28, 4), (256, 8, 8)])
+def test_attention_launch_is_one_the_head_size_has(head_dim, nq, nkv):
+    """Over steps drawn at random: a decode step is told apart, the launches with two groups of
+    waves and with 32 rows a wave only where the head size has them, pairs of tiles only at the
+    start of prompts without a window."""
+    lib = attention_library(head_dim)
+    rng = random.Random(head_dim)
+    group = nq // nkv
+    for _ in range(3000):
+        reqs = rng.choice([1, 2, 4, 8, 16, 64])
+        q = rng.choice([1, 2, 3, rng.randint(4, 64), rng.randint(65, 4096)])
+        ctx = q + rng.choice([0, rng.randint(0, 300), rng.randint(0, 9000)])
+        window = rng.choice([0, 0, 0, 128, 4096])
+        for dtype in (BF16, F32):
+            path = lib.llmlab_attention_launch(dtype, nq, nkv, reqs, q, ctx, window, CUS)
+            if q * group <= 16:
+                assert path == 0, (q, path)
+                continue
+            if dtype == F32:
+                assert path in (1, 2), (reqs, q, ctx, path)
+                continue
+            assert path in (1, 2, 3, 4, 6), (reqs, q, ctx, path)
+            if head_dim > 128:
+                assert path in (1, 3, 4)
+            if path == 3:
+                assert window == 0 and 16 * (ctx - q) <= q
+            if path == 1:
+                assert -(-q * group // 64) * nkv * reqs <= CUS // 2       # few tiles of rows only
+
+
+@pytest.mark.parametrize("head_dim,nq,nkv,dtype,reqs,q,behind,want", [
+    # (measured: see the comments in csrc/attention.hip; 1 = a block's waves split the keys of a tile of
+    # rows, 2 = 32 rows a wave, 4 = 16 rows a wave, 6 = 4 with two groups of waves a block)
+    (64, 14, 2, BF16, 1, 512, 1536, 1),      # a portion behind a history: 19 us against 32
+    (64, 14, 2, BF16, 1, 512, 256, 6),
+    (64, 14, 2, BF16, 1, 2048, 0, 6),        # a prompt from its start: 32 us against 38
+    (64, 14, 2, BF16, 1, 8192, 0, 2),        # a long one: 221 against 235
+    (64, 14, 2, BF16, 16, 64, 0, 4),         # many short prompts: 6.8 us against 8.0
+    (64, 14, 2, BF16, 8, 512, 2048, 2),      # 75 us against 83
+    (64, 14, 2, BF16, 2, 4096, 0, 4),        # 132 us against 161
+    (128, 28, 4, BF16, 1, 128, 1024, 6),     # 25 us against 29 with the key split
+    (128, 28, 4, BF16, 1, 128, 2560, 1),
+    (128, 28, 4, BF16, 8, 128, 0, 2),        # 14 us against 19
+    (128, 28, 4, BF16, 1, 64, 0, 4),         # 8.4 us against 9.8
+    (128, 28, 4, BF16, 1, 2048, 4096, 6),    # 313 us against 374 to 470
+    (64, 14, 2, F32, 1, 512, 1024, 1),       # 43 us against 162
+    (64, 14, 2, F32, 1, 2048, 0, 1),         # 117 against 217
+    (64, 14, 2, F32, 16, 512, 0, 2),         # 137 against 187
+    (128, 28, 4, F32, 4, 256, 0, 2),         # 58 against 81
+    (128, 28, 4, F32, 1, 256, 1024, 1),      # 77 against 226
+    (128, 28, 4, F32, 1, 1024, 0, 1),        # a long portion's tiles are uneven: 148 against 184
+    (128, 28, 4, F32, 2, 1024, 1024, 1),     # 620 against 656
+    (128, 28, 4, F32, 4, 1024, 0, 2),        # 501 against 562
+])
+def test_measured_attention_launches(head_dim, nq, nkv, dtype, reqs, q, behind, want):
+    lib = attention_library(head_dim)
+    assert lib.llmlab_attention_launch(dtype, nq, nkv, reqs, q, behind + q, 0, CUS) == want
