@@ -120,16 +120,28 @@ constexpr int DECODE_WAVES = D <= 64 ? 8 : (D <= 128 ? 4 : 2);
 // groups double the waves of a launch whose tiles of rows would leave a SIMD with one
 // wave or none: a wave's step is a chain (LDS, scores, maximum, exponentials, products)
 // that only another wave can fill.
+// LDS of the decode branch (the waves' sums, their maxima and denominators, the flag of the block
+// that arrives last, the splits' maxima where they do not fit in the sums' place): the kernel
+// declares it and hands it in, so that a kernel that runs two kinds of blocks has it once.
+template <int QB>
+constexpr int decode_lds_floats() {
+  return 2 * DECODE_WAVES * 16 * QB + DECODE_WAVES * 16 * QB * D + 4 +
+         (((size_t)DECODE_WAVES * 16 * D >= (size_t)2 * 16 * MAX_KEY_SPLITS) ? 0 : 2 * 16 * MAX_KEY_SPLITS);
+}
+
+// `xblk`, `by`, `bz`: the block's tile of rows, its (kv head, split) and its request (a kernel of
+// one kind of blocks passes its block indices).
 template <int QB, bool DECODE, int RING, int PH = 1>
-__device__ __forceinline__ void attention_tile(const AttnArgs& a, const int xblk) {
+__device__ __forceinline__ void attention_tile(const AttnArgs& a, const int xblk, const int by, const int bz,
+                                               float* dlds) {
   constexpr int DC = (D + 31) / 32;  // 32-wide chunks of d for Q.K
   constexpr int DB = D / 16;         // 16-wide blocks of d for P.V
   constexpr bool PIPE = DECODE;
   const int lane = threadIdx.x & 63, nw = blockDim.x >> 6;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);   // the same for all lanes: kept scalar
   const int c = lane & 15, g = lane >> 4;
-  const int b = blockIdx.z;
-  const int kvh = blockIdx.y / a.splits, split = blockIdx.y % a.splits;
+  const int b = bz;
+  const int kvh = by / a.splits, split = by % a.splits;
   const int G = a.nq / a.nkv;
   const int r0 = a.q_start[b], qlen = a.q_start[b + 1] - r0, sp = a.start_pos[b];
   const int rows_total = qlen * G;
@@ -645,8 +657,10 @@ __device__ __forceinline__ void attention_tile(const AttnArgs& a, const int xblk
   } else {
     // ---- merge the waves of the block through LDS
     //   acc = sum_w 2^(m_w - m) acc_w,  l = sum_w 2^(m_w - m) l_w,  m = max_w m_w
-    __shared__ float s_m[DECODE_WAVES][16 * QB], s_l[DECODE_WAVES][16 * QB];
-    __shared__ __attribute__((aligned(16))) float s_o[DECODE_WAVES][16 * QB][D];
+    float (*s_m)[16 * QB] = reinterpret_cast<float (*)[16 * QB]>(dlds);
+    float (*s_l)[16 * QB] = reinterpret_cast<float (*)[16 * QB]>(dlds + DECODE_WAVES * 16 * QB);
+    float (*s_o)[16 * QB][D] = reinterpret_cast<float (*)[16 * QB][D]>(dlds + 2 * DECODE_WAVES * 16 * QB);   // (16-byte aligned)
+    float* const after_sums = dlds + 2 * DECODE_WAVES * 16 * QB + DECODE_WAVES * 16 * QB * D;
 #pragma unroll
     for (int qb = 0; qb < QB; ++qb) {
       float l = lsum[qb];
@@ -705,7 +719,7 @@ __device__ __forceinline__ void attention_tile(const AttnArgs& a, const int xblk
     // simply ends.
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
-    __shared__ int s_last;
+    int& s_last = *reinterpret_cast<int*>(after_sums);
     if (threadIdx.x == 0) {
       int* counter = a.arrived + (size_t)b * a.nkv + kvh;
       const int before = __hip_atomic_fetch_add(counter, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -717,8 +731,7 @@ __device__ __forceinline__ void attention_tile(const AttnArgs& a, const int xblk
     // maxima and denominators of all splits of the block's rows, through LDS: [row][split];
     // where the waves' own sums (done with behind the barriers above) leave room, in their place
     constexpr bool FITS = (size_t)DECODE_WAVES * 16 * D >= (size_t)2 * 16 * MAX_KEY_SPLITS;
-    __shared__ float x_own[FITS ? 1 : 2 * 16 * MAX_KEY_SPLITS];
-    float* x_m = FITS ? &s_o[0][0][0] : x_own;
+    float* x_m = FITS ? &s_o[0][0][0] : after_sums + 4;
     float* x_l = x_m + 16 * MAX_KEY_SPLITS;
     const int S = a.splits;
     for (int i = threadIdx.x; i < nrows * S; i += blockDim.x) {
@@ -760,7 +773,29 @@ __device__ __forceinline__ void attention_tile(const AttnArgs& a, const int xblk
 // are dispatched first.
 template <int QB, bool DECODE, int RING = 1, int PH = 1>
 __global__ __launch_bounds__(DECODE ? 64 * DECODE_WAVES : 256 * PH, (!DECODE && D <= 64 && PH == 1) ? 2 : 1) void attention_bf16_kernel(AttnArgs a) {
-  attention_tile<QB, DECODE, RING, PH>(a, (int)(gridDim.x - 1 - blockIdx.x));
+  if constexpr (DECODE) {
+    __shared__ __attribute__((aligned(16))) float dlds[decode_lds_floats<QB>()];
+    attention_tile<QB, DECODE, RING, PH>(a, (int)(gridDim.x - 1 - blockIdx.x), (int)blockIdx.y, (int)blockIdx.z, dlds);
+  } else {
+    attention_tile<QB, DECODE, RING, PH>(a, (int)(gridDim.x - 1 - blockIdx.x), (int)blockIdx.y, (int)blockIdx.z, nullptr);
+  }
+}
+
+// A mixed step in one launch: the first `long_blocks` blocks of a request (x) are the tiles of
+// rows of a portion times the kv heads, each with the keys of its tile split over its waves; the
+// others are the (kv head, split) pairs of a request of a few tokens, whose keys are split over
+// blocks as in a decode step.  A block finds in its request's length which of the two it is
+// for and ends at once if it is for the other kind.  In two launches the decoding requests'
+// blocks, which stream their histories, wait for the portion's, which are a chain of small
+// products, although they need different parts of a compute unit.
+template <int QBL, int RL, int RS>
+__global__ __launch_bounds__(64 * DECODE_WAVES) void attention_bf16_mixed_kernel(AttnArgs al, AttnArgs as, int long_tiles) {
+  __shared__ __attribute__((aligned(16))) float dlds[decode_lds_floats<QBL>()];
+  const int x = (int)blockIdx.x, long_blocks = long_tiles * al.nkv;
+  if (x < long_blocks)
+    attention_tile<QBL, true, RL>(al, long_tiles - 1 - x / al.nkv, x % al.nkv, (int)blockIdx.z, dlds);
+  else
+    attention_tile<1, true, RS>(as, 0, x - long_blocks, (int)blockIdx.z, dlds);
 }
 
 // Two tiles of rows per block, one after the other: tile t from the end and tile t
@@ -772,7 +807,7 @@ __global__ __launch_bounds__(256 * PH, (D <= 64 && PH == 1) ? 2 : 1) void attent
   const int late = a.tiles - 1 - (int)blockIdx.x, early = (int)blockIdx.x;
   for (int pass = 0; pass < 2; ++pass) {
     if (pass == 1 && early >= late) break;
-    attention_tile<QB, false, 1, PH>(a, pass == 0 ? late : early);
+    attention_tile<QB, false, 1, PH>(a, pass == 0 ? late : early, (int)blockIdx.y, (int)blockIdx.z, nullptr);
     __syncthreads();
   }
 }
@@ -1134,10 +1169,17 @@ constexpr int MERGE_IN_PLACE_SPLITS = 2;
 // wave gets about two steps of 32 keys, a block's waves merge in LDS, and only what is
 // left is split over blocks; the merge kernel follows.  `live` requests (of `reqs`) pass
 // the filter of `a`, `ctx_len` is their longest context.
-static int launch_key_split_decode(AttnArgs a, int reqs, int live, int ctx_len, int window, int total_rows,
-                                   int nq, int nkv, float* workspace, size_t workspace_floats, int num_cus,
-                                   const int* row_req, void* out, int out_stride, int* arrived,
-                                   size_t arrived_ints, hipStream_t stream) {
+// A decode-like launch made ready: its arguments, the depth of its ring of key steps, and
+// whether a kernel of its own merges the splits afterwards.
+struct KeySplitLaunch {
+  AttnArgs a;
+  int ring;
+  bool merge_kernel;
+};
+
+static KeySplitLaunch prepare_key_split_decode(AttnArgs a, int reqs, int live, int ctx_len, int window, int total_rows,
+                                               int nq, int nkv, float* workspace, size_t workspace_floats, int num_cus,
+                                               int* arrived, size_t arrived_ints) {
   const int visible = window > 0 ? min(window, ctx_len) : ctx_len;
   const int steps32 = (visible + 31) / 32 + 1;
   // A unit's memory rate is the limit, so the keys are spread over the units: as many
@@ -1179,20 +1221,34 @@ static int launch_key_split_decode(AttnArgs a, int reqs, int live, int ctx_len, 
     a.o_part = workspace;
     a.ml_part = workspace + (size_t)total_rows * nq * splits * D;
   }
-  dim3 grid(1, nkv * splits, reqs), block(64 * DECODE_WAVES);
   const int steps_per_wave = ((steps32 + splits - 1) / splits + DECODE_WAVES - 1) / DECODE_WAVES;
-  if (steps_per_wave > 2)
-    hipLaunchKernelGGL((attention_bf16_kernel<1, true, 2>), grid, block, 0, stream, a);
-  else
-    hipLaunchKernelGGL((attention_bf16_kernel<1, true, 1>), grid, block, 0, stream, a);
-  LLMLAB_LAUNCH_CHECK("attention(bfloat16, decode)");
-  if (splits > 1 && !merge_in_place) {
-    hipLaunchKernelGGL(attention_merge_kernel<bf16_t>, dim3(total_rows, nq), dim3(splits > 16 ? 64 * MERGE_WAVES : 64), 0, stream, a.o_part,
-                       a.ml_part, (bf16_t*)out, out_stride, nq, splits, row_req, a.q_start, a.qlen_hi);
-    LLMLAB_LAUNCH_CHECK("attention merge");
-  }
+  return KeySplitLaunch{a, steps_per_wave > 2 ? 2 : 1, splits > 1 && !merge_in_place};
+}
+
+static int launch_split_merge(const KeySplitLaunch& k, int total_rows, int nq, const int* row_req, void* out,
+                              int out_stride, hipStream_t stream) {
+  if (!k.merge_kernel) return 0;
+  hipLaunchKernelGGL(attention_merge_kernel<bf16_t>, dim3(total_rows, nq), dim3(k.a.splits > 16 ? 64 * MERGE_WAVES : 64), 0,
+                     stream, k.a.o_part, k.a.ml_part, (bf16_t*)out, out_stride, nq, k.a.splits, row_req, k.a.q_start,
+                     k.a.qlen_hi);
+  LLMLAB_LAUNCH_CHECK("attention merge");
   return 0;
 }
+
+static int launch_key_split_decode(const KeySplitLaunch& k, int reqs, int total_rows, int nq, int nkv,
+                                   const int* row_req, void* out, int out_stride, hipStream_t stream) {
+  dim3 grid(1, nkv * k.a.splits, reqs), block(64 * DECODE_WAVES);
+  if (k.ring == 2)
+    hipLaunchKernelGGL((attention_bf16_kernel<1, true, 2>), grid, block, 0, stream, k.a);
+  else
+    hipLaunchKernelGGL((attention_bf16_kernel<1, true, 1>), grid, block, 0, stream, k.a);
+  LLMLAB_LAUNCH_CHECK("attention(bfloat16, decode)");
+  return launch_split_merge(k, total_rows, nq, row_req, out, out_stride, stream);
+}
+
+// 1: a mixed step always in two launches; -1: in one wherever a kernel for it exists (measurements)
+static int g_force_two_launches = 0;
+extern "C" void llmlab_debug_attention_two_launches(int on) { g_force_two_launches = on; }
 
 // float32.  Steps of at most 16 rows per request and kv head (decode) split the keys over
 // the waves of a block and over blocks, as many splits as still give every block a compute
@@ -1430,24 +1486,65 @@ extern "C" int llmlab_paged_attention(const void* q, int dtype, int q_stride, in
   const int G = nq / nkv;
   const long max_rows = (long)max_q_len * G;
   if (max_rows <= 16)
-    return launch_key_split_decode(a, reqs, reqs, max_ctx_len, window, total_rows, nq, nkv, workspace,
-                                   workspace_floats, num_cus, nullptr, out, out_stride, arrived, arrived_ints,
-                                   stream);
+    return launch_key_split_decode(prepare_key_split_decode(a, reqs, reqs, max_ctx_len, window, total_rows, nq, nkv,
+                                                            workspace, workspace_floats, num_cus, arrived, arrived_ints),
+                                   reqs, total_rows, nq, nkv, nullptr, out, out_stride, stream);
   int live = reqs;
-  if (row_req != nullptr && n_short > 0 && n_short < reqs && (long)short_len * G <= 16) {
+  const bool mixed = row_req != nullptr && n_short > 0 && n_short < reqs && (long)short_len * G <= 16;
+  KeySplitLaunch shorts{};
+  if (mixed) {
     AttnArgs s = a;
     s.qlen_hi = short_len;
-    const int rc = launch_key_split_decode(s, reqs, n_short, short_ctx, window, total_rows, nq, nkv,
-                                           workspace, workspace_floats, num_cus, row_req, out, out_stride,
-                                           arrived, arrived_ints, stream);
-    if (rc) return rc;
+    shorts = prepare_key_split_decode(s, reqs, n_short, short_ctx, window, total_rows, nq, nkv, workspace,
+                                      workspace_floats, num_cus, arrived, arrived_ints);
     a.qlen_lo = short_len + 1;
     live = reqs - n_short;
   }
   const int path = choose_many_rows_launch(max_rows, nkv, live, max_q_len, max_ctx_len, window, num_cus, g_force_path);
+  if (mixed && path != 1) {
+    const int rc = launch_key_split_decode(shorts, reqs, total_rows, nq, nkv, row_req, out, out_stride, stream);
+    if (rc) return rc;
+  }
   if (path == 1) {
     const int steps32 = (max_ctx_len + 31) / 32 + 1;
     const int steps_per_wave = (steps32 + DECODE_WAVES - 1) / DECODE_WAVES;
+    // Both kinds of blocks in one launch (see attention_bf16_mixed_kernel) where the portion's
+    // blocks leave half of the chip's places free, or all blocks together hardly exceed the
+    // places: every block of the one launch holds the registers of the portion's kind, so the
+    // decoding requests' blocks, which stream and want company on their unit, lose places
+    // (a unit holds one block at heads up to 64, two above).  Heads of 64, a portion of 128
+    // tokens behind 2,048 keys beside 63 requests decoding at 2,048: 28 us against 38 in two
+    // launches; a portion of 512 (224 blocks) beside 31 at 1,024: 27 against 30, beside 127 at
+    // 1,024: 68 against 59, hence not there.  Heads of 128, 128 tokens beside 63 at 2,048: 75
+    // against 90.
+    const int long_tiles = (int)((max_rows + 31) / 32);
+    bool one_launch = false;
+    if (mixed && g_force_two_launches <= 0) {
+      const long places = (D <= 64 ? 1L : 2L) * num_cus;
+      const long long_blocks = (long)long_tiles * nkv * live;
+      const long short_blocks = (long)nkv * shorts.a.splits * n_short;
+      one_launch = g_force_two_launches < 0 || 2 * long_blocks <= places || 4 * (long_blocks + short_blocks) <= 5 * places;
+    }
+    if (mixed && !one_launch) {
+      const int rc = launch_key_split_decode(shorts, reqs, total_rows, nq, nkv, row_req, out, out_stride, stream);
+      if (rc) return rc;
+    }
+    if (one_launch) {
+      const long gx = (long)long_tiles * nkv + (long)nkv * shorts.a.splits;
+      LLMLAB_REQUIRE(gx <= 0x7fffffffL, "attention: grid too large");
+      dim3 mgrid((unsigned)gx, 1, reqs), mblock(64 * DECODE_WAVES);
+      const bool deep = steps_per_wave > 2;
+      if (deep && shorts.ring == 2)
+        hipLaunchKernelGGL((attention_bf16_mixed_kernel<2, 2, 2>), mgrid, mblock, 0, stream, a, shorts.a, long_tiles);
+      else if (deep)
+        hipLaunchKernelGGL((attention_bf16_mixed_kernel<2, 2, 1>), mgrid, mblock, 0, stream, a, shorts.a, long_tiles);
+      else if (shorts.ring == 2)
+        hipLaunchKernelGGL((attention_bf16_mixed_kernel<2, 1, 2>), mgrid, mblock, 0, stream, a, shorts.a, long_tiles);
+      else
+        hipLaunchKernelGGL((attention_bf16_mixed_kernel<2, 1, 1>), mgrid, mblock, 0, stream, a, shorts.a, long_tiles);
+      LLMLAB_LAUNCH_CHECK("attention(bfloat16, mixed)");
+      return launch_split_merge(shorts, total_rows, nq, row_req, out, out_stride, stream);
+    }
     dim3 grid((unsigned)((max_rows + 31) / 32), nkv, reqs), block(64 * DECODE_WAVES);
     if (steps_per_wave > 2)
       hipLaunchKernelGGL((attention_bf16_kernel<2, true, 2>), grid, block, 0, stream, a);

@@ -97,7 +97,9 @@ class KernelDebug:
               attention_splits: Optional[Tuple[int, int]] = None,
               attention_path: Optional[Tuple[int, int]] = None,
               attention_merge_kernel: Optional[int] = None,
-              attention_merge_in_place: Optional[int] = None, f32_fma: Optional[bool] = None, **rules):
+              attention_merge_in_place: Optional[int] = None, attention_two_launches: Optional[int] = None,
+              attention_one_launch: Optional[int] = None,
+              f32_fma: Optional[bool] = None, **rules):
         """``gemm_tile``: 64 (64 x 64), 130 (64 x 128), 129 (128 x 128), 131 (128 x 256), 132 (256 x
         256) or 133 (192 x 256); -131: the choice among the first three; -256 and below: the
         tiles of two groups of waves (132, 133) from so many rows on.  ``skinny_shape``:
@@ -110,7 +112,9 @@ class KernelDebug:
         waves that take the staged keys in turn; heads above 128 have no 5 and 6 and choose
         for themselves).  ``attention_merge_kernel`` / ``attention_merge_in_place``: a head size; the
         key splits of decode attention are merged there by the kernel of its own, or by the
-        last block to arrive, whatever their number.
+        last block to arrive, whatever their number.  ``attention_two_launches`` / ``attention_one_launch``:
+        a head size; a mixed step's decoding requests and its portions get a launch each also
+        where one launch would serve both, or one launch wherever there is a kernel for both.
         ``f32_fma``: float32 products of many rows by the plain FMA kernel instead of the
         matrix cores.  Other keywords: fields of ``DispatchRules`` for the time of the block."""
         ops = self._ops
@@ -120,7 +124,7 @@ class KernelDebug:
             if not hasattr(ops.rules, key):
                 raise TypeError(f"no dispatch rule named '{key}'")
             setattr(ops.rules, key, value)
-        lib = plib = mlib = None
+        lib = plib = mlib = tlib = None
         ops.debug_epoch += 1
         try:
             if attention_merge_kernel is not None:
@@ -129,6 +133,12 @@ class KernelDebug:
             elif attention_merge_in_place is not None:
                 mlib = ops._attention_lib(int(attention_merge_in_place))
                 mlib.llmlab_debug_attention_merge_kernel(-1)
+            if attention_two_launches is not None:
+                tlib = ops._attention_lib(int(attention_two_launches))
+                tlib.llmlab_debug_attention_two_launches(1)
+            elif attention_one_launch is not None:
+                tlib = ops._attention_lib(int(attention_one_launch))
+                tlib.llmlab_debug_attention_two_launches(-1)
             if attention_path is not None:
                 plib = ops._attention_lib(int(attention_path[0]))
                 plib.llmlab_debug_attention_path(int(attention_path[1]))
@@ -161,3 +171,5 @@ class KernelDebug:
                 plib.llmlab_debug_attention_path(0)
             if mlib is not None:
                 mlib.llmlab_debug_attention_merge_kernel(0)
+            if tlib is not None:
+                tlib.llmlab_debug_attention_two_launches(0)

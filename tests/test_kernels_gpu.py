@@ -673,7 +673,7 @@ def run_attention(ops, emu, dtype, nq, nkv, d, page, window, reqs_spec, seed=30,
     assert err <= tol * max(1.0, want.float().abs().max().item()), f"attention error {err}"
 
     # the same step described as the engine describes it (which requests are short): a
-    # mixed step is then served by two launches
+    # mixed step is then served by two launches, or by one that runs both kinds of blocks
     limit = ops.attention_short_limit(nq, nkv, dtype, max(n for _, n in reqs_spec))
     short_reqs = [(s, n) for s, n in reqs_spec if n <= limit]
     short = None
@@ -689,7 +689,9 @@ def run_attention(ops, emu, dtype, nq, nkv, d, page, window, reqs_spec, seed=30,
     # key splits are merged by the last block to arrive; the same with the kernel of its own,
     # and the arrival counters are back at zero whoever merged
     if dtype == torch.bfloat16:
-        for who in ("attention_merge_kernel", "attention_merge_in_place"):
+        # (and a mixed step in a launch for each kind of request where one launch would serve both)
+        for who in ("attention_merge_kernel", "attention_merge_in_place", "attention_two_launches",
+                    "attention_one_launch"):
             got3 = torch.zeros(rows, nq * d, dtype=dtype, device=DEV)
             with ops.debug.force(**{who: d}):
                 ops.paged_attention(qkv.to(DEV), nq, nkv, d, kc.to(DEV), vc.to(DEV), table.to(DEV), page,
