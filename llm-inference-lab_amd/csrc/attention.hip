@@ -1425,6 +1425,33 @@ static int choose_many_rows_launch(long max_rows, int nkv, int live, int max_q_l
   return path;
 }
 
+// Whether the blocks of a mixed step's portions (keys split over the waves of a block) and of its
+// decoding requests go in one launch: see llmlab_paged_attention.
+static bool mixed_step_in_one_launch(long long_blocks, long short_blocks, int num_cus, int forced) {
+  if (forced > 0) return false;
+  if (forced < 0) return true;
+  const long places = (D <= 64 ? 1L : 2L) * num_cus;      // blocks of the portion's kind that the chip holds at a time
+  return 2 * long_blocks <= places || 4 * (long_blocks + short_blocks) <= 5 * places;
+}
+
+// How many attention launches a mixed step in bfloat16 takes (the merge of key splits not
+// counted): `n_short` of its requests decode behind at most `short_ctx` keys, the others bring
+// portions of at most `max_q_len` tokens (for tests and tuning; 0: not a mixed step).
+extern "C" int llmlab_attention_mixed_launches(int nq, int nkv, int reqs, int n_short, int max_q_len, int max_ctx_len,
+                                               int short_ctx, int window, int num_cus) {
+  if (num_cus <= 0) num_cus = 256;
+  if (nq <= 0 || nkv <= 0 || nq % nkv != 0 || n_short <= 0 || n_short >= reqs || max_q_len <= 0) return 0;
+  const long max_rows = (long)max_q_len * (nq / nkv);
+  if (max_rows <= 16) return 0;
+  const int live = reqs - n_short;
+  if (choose_many_rows_launch(max_rows, nkv, live, max_q_len, max_ctx_len, window, num_cus, 0) != 1) return 2;
+  AttnArgs a{};
+  const KeySplitLaunch shorts = prepare_key_split_decode(a, reqs, n_short, short_ctx, window, reqs, nq, nkv, nullptr,
+                                                         ~(size_t)0 >> 8, num_cus, nullptr, 0);
+  return mixed_step_in_one_launch((max_rows + 31) / 32 * nkv * live, (long)nkv * shorts.a.splits * n_short, num_cus, 0)
+             ? 1 : 2;
+}
+
 // The launch that llmlab_paged_attention would take for a step of many rows of these sizes
 // (for tests and tuning; 0: the sizes make a decode step, whose keys are split over blocks).
 extern "C" int llmlab_attention_launch(int dtype, int nq, int nkv, int reqs, int max_q_len, int max_ctx_len, int window,
@@ -1518,13 +1545,9 @@ extern "C" int llmlab_paged_attention(const void* q, int dtype, int q_stride, in
     // 1,024: 68 against 59, hence not there.  Heads of 128, 128 tokens beside 63 at 2,048: 75
     // against 90.
     const int long_tiles = (int)((max_rows + 31) / 32);
-    bool one_launch = false;
-    if (mixed && g_force_two_launches <= 0) {
-      const long places = (D <= 64 ? 1L : 2L) * num_cus;
-      const long long_blocks = (long)long_tiles * nkv * live;
-      const long short_blocks = (long)nkv * shorts.a.splits * n_short;
-      one_launch = g_force_two_launches < 0 || 2 * long_blocks <= places || 4 * (long_blocks + short_blocks) <= 5 * places;
-    }
+    const bool one_launch = mixed && mixed_step_in_one_launch((long)long_tiles * nkv * live,
+                                                              (long)nkv * shorts.a.splits * n_short, num_cus,
+                                                              g_force_two_launches);
     if (mixed && !one_launch) {
       const int rc = launch_key_split_decode(shorts, reqs, total_rows, nq, nkv, row_req, out, out_stride, stream);
       if (rc) return rc;

@@ -248,3 +248,25 @@ def test_attention_launch_is_one_the_head_size_has(head_dim, nq, nkv):
 def test_measured_attention_launches(head_dim, nq, nkv, dtype, reqs, q, behind, want):
     lib = attention_library(head_dim)
     assert lib.llmlab_attention_launch(dtype, nq, nkv, reqs, q, behind + q, 0, CUS) == want
+
+
+@pytest.mark.parametrize("head_dim,nq,nkv,portion,behind,decoding,their_keys,want", [
+    # (measured, one launch against two: see the comment in llmlab_paged_attention)
+    (64, 14, 2, 128, 2048, 63, 2048, 1),     # 28 us against 38
+    (64, 14, 2, 256, 1024, 31, 1024, 1),     # 21 against 27
+    (64, 14, 2, 512, 1536, 31, 1024, 1),     # 31 against 34
+    (64, 14, 2, 512, 1536, 127, 1024, 2),    # 70 against 63
+    (64, 14, 2, 512, 1536, 63, 512, 2),      # 43 against 40
+    (128, 28, 4, 128, 2048, 63, 2048, 1),    # 75 against 88
+    (128, 40, 8, 128, 2048, 127, 1024, 1),   # 145 against 164
+    (128, 28, 4, 512, 512, 63, 2048, 2),     # (the portion's launch is not the one with the key split)
+])
+def test_measured_launches_of_a_mixed_step(head_dim, nq, nkv, portion, behind, decoding, their_keys, want):
+    lib = attention_library(head_dim)
+    lib.llmlab_attention_mixed_launches.restype = ctypes.c_int
+    got = lib.llmlab_attention_mixed_launches(nq, nkv, decoding + 1, decoding, portion, behind + portion,
+                                              their_keys, 0, CUS)
+    assert got == want
+    # not a mixed step: nobody decodes, or everybody
+    assert lib.llmlab_attention_mixed_launches(nq, nkv, 4, 0, portion, behind + portion, 0, 0, CUS) == 0
+    assert lib.llmlab_attention_mixed_launches(nq, nkv, 4, 4, portion, behind + portion, their_keys, 0, CUS) == 0
