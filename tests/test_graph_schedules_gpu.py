@@ -133,6 +133,47 @@ def test_a_long_history_beside_short_ones(dtype, graph):
 
 
 @pytest.mark.parametrize("dtype", ["f32", "bf16"])
+def test_portions_behind_a_history_beside_decoding_requests(dtype):
+    """Layers of real size.  One request of 1,200 tokens comes in portions of 128 while three
+    others, with histories of 50, 300 and 700 tokens, decode one token a step beside it: from
+    the fourth portion on the portion's rows sit behind 384 keys and more, so its keys are split
+    over the waves of a block, and in bfloat16 the decoding requests' blocks then run in the
+    same attention launch.  Against the plain implementation, and bit for bit the logits of
+    an engine whose mixed steps take a launch for each kind of request."""
+    cfg = H.config_of("R")
+    long_len, portion = 1200, 128
+    steps_of_long = -(-long_len // portion)
+    peers = {"p0": 50, "p1": 300, "p2": 700}
+    seqs = {"long": H.random_ids(cfg, long_len, 6100)}
+    for i, (rid, n) in enumerate(peers.items()):
+        seqs[rid] = H.random_ids(cfg, n + steps_of_long, 6101 + i)
+    want = {rid: H.plain_logits("R", 1, ids) for rid, ids in seqs.items()}
+    steps = [([(rid, n, True)], []) for rid, n in peers.items()]
+    for at in range(0, long_len, portion):
+        steps.append(([("long", min(portion, long_len - at), True)] + [(rid, 1, True) for rid in peers], []))
+
+    def run(two_launches):
+        engine = H.make_engine("R", 1, dtype, graph=False, page_size=64, num_pages=40, max_requests=4,
+                               max_batch_tokens=768, max_seq_len=1280)
+        if two_launches:
+            with engine.ops.debug.force(attention_two_launches=cfg.head_dim):
+                return H.run_trace(engine, seqs, steps)
+        return H.run_trace(engine, seqs, steps)
+
+    if dtype == "bf16":      # (the schedule is one that the rule serves with one launch)
+        ops = H.make_engine("R", 1, dtype, page_size=64, num_pages=4, max_seq_len=128).ops
+        lib = ops._attention_lib(cfg.head_dim)
+        assert lib.llmlab_attention_mixed_launches(cfg.num_attention_heads, cfg.num_key_value_heads, 4, 3, portion,
+                                                   9 * portion, 709, 0, ops.num_cus) == 1
+    got = run(False)
+    bad = H.first_wrong(got, want, TOL_REAL[dtype][0])
+    assert bad is None, f"first wrong logits at (request, position, error) = {bad}"
+    other = run(True)
+    for rid in seqs:
+        assert torch.equal(got[rid], other[rid]), f"{rid}: one launch and two differ"
+
+
+@pytest.mark.parametrize("dtype", ["f32", "bf16"])
 @pytest.mark.parametrize("name", ["B", "R"])
 def test_kept_launch_sequences_change_nothing(name, dtype):
     """A block's calls into the kernel libraries are written down at its first run for a

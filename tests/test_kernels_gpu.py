@@ -690,10 +690,11 @@ def run_attention(ops, emu, dtype, nq, nkv, d, page, window, reqs_spec, seed=30,
     # and the arrival counters are back at zero whoever merged
     if dtype == torch.bfloat16:
         # (and a mixed step in a launch for each kind of request where one launch would serve both)
-        for who in ("attention_merge_kernel", "attention_merge_in_place", "attention_two_launches",
-                    "attention_one_launch"):
+        for who in (("attention_merge_kernel",), ("attention_merge_in_place",), ("attention_two_launches",),
+                    ("attention_one_launch",), ("attention_one_launch", "attention_merge_kernel"),
+                    ("attention_one_launch", "attention_merge_in_place")):
             got3 = torch.zeros(rows, nq * d, dtype=dtype, device=DEV)
-            with ops.debug.force(**{who: d}):
+            with ops.debug.force(**{w: d for w in who}):
                 ops.paged_attention(qkv.to(DEV), nq, nkv, d, kc.to(DEV), vc.to(DEV), table.to(DEV), page,
                                     q_start_t.to(DEV), start_pos_t.to(DEV), reqs, max(n for _, n in reqs_spec),
                                     max_ctx, window, scale, got3, short)
